@@ -1,0 +1,180 @@
+/*
+ * tship.h — C ABI of libtship.so, the native half of a TensorSharp.HIP backend for MI355X (gfx950).
+ *
+ * Conventions (the same ones the reference's GGML bridge uses between TensorSharp.GGML/GgmlNative.cs
+ * and TensorSharp.GGML.Native/ggml_ops.cpp):
+ *   - extern "C", cdecl, default visibility                              (ggml_ops.cpp:89-93, GgmlNative.cs:164)
+ *   - every call returns int: 1 = success, 0 = failure                   (GgmlNative.cs:471-479)
+ *   - on failure the message is kept per thread, read with TSHip_GetLastError()
+ *                                                                        (ggml_ops.cpp:211-224, :4683-4686)
+ *   - no C++ exception crosses the boundary                              (ggml_ops.cpp:4707-4722)
+ *   - the caller owns every tensor buffer; the library keeps no tensor pointer after a call returns
+ *   - calls are ordered on one library stream; functions that hand data to the host synchronise
+ *
+ * Tensor arguments are strided views (sizes and strides in ELEMENTS, outermost dimension first, exactly
+ * TensorSharp.Tensor's Sizes/Strides, TensorSharp/Tensor.cs:12-125).  `data` is a DEVICE pointer already
+ * advanced by StorageOffset.  Indices travel as float32 tensors, as everywhere in the reference
+ * (Seq2SeqSharp/Applications/Decoder.cs:708-715).
+ */
+#ifndef TSHIP_H
+#define TSHIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TSHIP_API __attribute__((visibility("default")))
+#define TSHIP_MAX_DIMS 6
+
+/* TensorSharp/DType.cs:6-13 */
+enum { TSHIP_F32 = 0, TSHIP_F16 = 1 };
+
+typedef struct TSHipTensor {
+    void*   data;                     /* device pointer (storage base + StorageOffset * element size) */
+    int32_t dtype;                    /* TSHIP_F32 or TSHIP_F16 */
+    int32_t ndim;                     /* 1..TSHIP_MAX_DIMS */
+    int64_t sizes[TSHIP_MAX_DIMS];
+    int64_t strides[TSHIP_MAX_DIMS];  /* in elements; 0 = expanded (broadcast) dimension */
+} TSHipTensor;
+
+/* ---- runtime: what HipAllocator / HipStorage need (TensorSharp/IAllocator.cs:13-20, Storage.cs:32-47,
+ *      modelled on TensorSharp.CUDA/CudaStorage.cs:35-173: synchronous device<->host copies) ---- */
+TSHIP_API const char* TSHip_GetLastError(void);                               /* cf. TSGgml_GetLastError */
+TSHIP_API int TSHip_GetDeviceCount(int* count);
+TSHIP_API int TSHip_Init(int device_id);                                      /* once per process; cf. ggml_ops.cpp:256-280 */
+TSHIP_API int TSHip_Malloc(void** ptr, size_t bytes);                         /* IAllocator.Allocate */
+TSHIP_API int TSHip_Free(void* ptr);                                          /* Storage.Destroy */
+TSHIP_API int TSHip_MemcpyH2D(void* dst, const void* src, size_t bytes);      /* Storage.CopyToStorage / SetElementsAsFloat */
+TSHIP_API int TSHip_MemcpyD2H(void* dst, const void* src, size_t bytes);      /* Storage.CopyFromStorage / GetElementsAsFloat */
+TSHIP_API int TSHip_MemcpyD2D(void* dst, const void* src, size_t bytes);
+TSHIP_API int TSHip_Memset(void* dst, int value, size_t bytes);
+TSHIP_API int TSHip_Synchronize(void);
+TSHIP_API int TSHip_GetMemInfo(size_t* free_bytes, size_t* total_bytes);      /* IAllocator.GetAllocatedMemoryRatio */
+
+/* ---- per-op surface: one entry per OpRegistry name the decode path issues (TensorSharp/Ops.cs:15-303).
+ *      Signatures follow the CPU handlers in TensorSharp/Cpu/CpuBasicOps.cs; `result` is always supplied
+ *      by the caller (the managed side allocates it with TensorResultBuilder.GetWriteTarget). ---- */
+
+/* "copy" (Ops.cs:24-34, TensorApplyCPU.cs:282-306); also float2half / half2float when dtypes differ
+ * (ComputeGraphTensor.cs:1427-1438, :1484-1495) */
+TSHIP_API int TSHip_Copy(const TSHipTensor* result, const TSHipTensor* src);
+/* "fill" */
+TSHIP_API int TSHip_Fill(const TSHipTensor* result, float value);
+/* "addmm": result = beta*src + alpha*m1*m2 (CpuBasicOps.cs:49-114) */
+TSHIP_API int TSHip_Addmm(const TSHipTensor* result, float beta, const TSHipTensor* src, float alpha,
+                          const TSHipTensor* m1, const TSHipTensor* m2);
+/* "addmmbatch" (CpuBasicOps.cs:116-184) */
+TSHIP_API int TSHip_AddmmBatch(const TSHipTensor* result, float beta, const TSHipTensor* src, float alpha,
+                               const TSHipTensor* m1, const TSHipTensor* m2);
+/* "indexselect": result[j,:] (+)= src[(int)indice[j],:], negative indices skipped (TensorApplyCPU.cs:1306-1333) */
+TSHIP_API int TSHip_IndexSelect(const TSHipTensor* result, const TSHipTensor* src, const TSHipTensor* indice, int is_add);
+/* "indexselectgrad": grad[(int)indice[j],:] += adj[j,:] in row order (TensorApplyCPU.cs:1336-1356) */
+TSHIP_API int TSHip_IndexSelectGrad(const TSHipTensor* grad, const TSHipTensor* adj, const TSHipTensor* indice);
+/* "rope" (CpuBasicOps.cs:1049-1066, TensorApplyCPU.cs:1148-1178): base 500000, adjacent pairs */
+TSHIP_API int TSHip_RoPE(const TSHipTensor* result, const TSHipTensor* src, int seq_len, int row_offset);
+/* same with the base as an argument (the reference has no such parameter) */
+TSHIP_API int TSHip_RoPEEx(const TSHipTensor* result, const TSHipTensor* src, int seq_len, int row_offset, float base);
+/* "rmsnorm" / "layernorm" (TensorApplyCPU.cs:1451-1496, :1360-1447); beta may be NULL */
+TSHIP_API int TSHip_RMSNorm(const TSHipTensor* result, const TSHipTensor* src, const TSHipTensor* gamma,
+                            const TSHipTensor* beta, float eps);
+TSHIP_API int TSHip_LayerNorm(const TSHipTensor* result, const TSHipTensor* src, const TSHipTensor* gamma,
+                              const TSHipTensor* beta, float eps);
+/* "softmax" over the last dimension (TensorApplyCPU.cs:1230-1268) */
+TSHIP_API int TSHip_Softmax(const TSHipTensor* result, const TSHipTensor* src);
+/* "argmax" along `dim`, float indices, first maximum wins (TensorApplyCPU.cs:339-360) */
+TSHIP_API int TSHip_Argmax(const TSHipTensor* result, const TSHipTensor* src, int dim);
+/* "topK": descending values + float indices with the reference's insertion rule (TensorApplyCPU.cs:1099-1146) */
+TSHIP_API int TSHip_TopK(const TSHipTensor* out_val, const TSHipTensor* out_idx, const TSHipTensor* src, int k);
+
+/* element-wise families (TensorApplyCPU.cs:378-673, :852-861, :1747-1801) */
+enum { TSHIP_ADD = 0, TSHIP_SUB = 1, TSHIP_MUL = 2, TSHIP_DIV = 3 };
+enum { TSHIP_RELU = 0, TSHIP_SILU = 1, TSHIP_LEAKYRELU = 2, TSHIP_EXP = 3, TSHIP_LOG = 4, TSHIP_NEG = 5,
+       TSHIP_SIGMOID = 6, TSHIP_TANH = 7, TSHIP_SQRT = 8, TSHIP_ABS = 9 };
+/* "addt" "subt" "mult" "divt": result = lhs op rhs (rhs may be an expanded view) */
+TSHIP_API int TSHip_BinaryTensor(int op, const TSHipTensor* result, const TSHipTensor* lhs, const TSHipTensor* rhs);
+/* "addv" "subv" "mulv" "divv": result = src op scalar */
+TSHIP_API int TSHip_BinaryScalar(int op, const TSHipTensor* result, const TSHipTensor* src, float scalar);
+/* "relu" "SiLU" "LeakyReLU" "exp" "log" "neg" "sigmoid" "tanh" "sqrt" "abs" */
+TSHIP_API int TSHip_Unary(int op, const TSHipTensor* result, const TSHipTensor* src);
+/* "buildtrimask" / "buildselftrimask" (TensorApplyCPU.cs:1016-1065) */
+TSHIP_API int TSHip_BuildTriMask(const TSHipTensor* result, float value, float masked_value);
+TSHIP_API int TSHip_BuildSelfTriMask(const TSHipTensor* result, const TSHipTensor* original_lengths,
+                                     int padded_seq_len, float value, float masked_value);
+/* "iscorrupted": *corrupted = 1 if any element is not finite (TensorApplyCPU.cs:1212-1228) */
+TSHIP_API int TSHip_IsCorrupted(const TSHipTensor* src, int* corrupted);
+
+/* Top-p sampling on the device, one row per sequence; semantics of ComputeGraphTensor.TopPSample
+ * (Seq2SeqSharp/Tools/ComputeGraphTensor.cs:2305-2403) with repeatPenalty = 0 and the random draw of row i
+ * replaced by uniforms[i].  probs [rows, K] f32, uniforms [rows] f32, result [rows,1] f32 (float indices). */
+TSHIP_API int TSHip_TopPSample(const TSHipTensor* result, const TSHipTensor* probs, const TSHipTensor* uniforms, float top_p);
+
+/* ---- fused GPTDecoder path: one object per model replica, preallocated compact KV cache, the whole
+ *      token loop on the device (replaces GPT.RunForwardOnSingleDevice, Seq2SeqSharp/Applications/GPT.cs:212-335,
+ *      Decoder.GPTDecode, Applications/Decoder.cs:648-794, and GPTDecoder.Decode, Networks/GPTDecoder.cs:153-191). ---- */
+typedef struct TSHipGptConfig {
+    int32_t n_layers, hidden, n_heads, n_kv_heads, ffn_dim, vocab;
+    int32_t attn_type;          /* 0 = MultiHeadAttention (fused QKV [h,3h], columns ordered [3][H][d]), 1 = GroupQueryAttention */
+    int32_t norm_type;          /* 0 = RMSNorm, 1 = LayerNorm */
+    int32_t act;                /* 0 ReLU, 1 SiLU, 2 LeakyReLU, 3 "SwiGLU" as the reference computes it (no SiLU on the gate),
+                                   4 = gated with SiLU (not a reference mode) */
+    int32_t n_experts;          /* > 1: layers 2.. use MoEFeedForward (Networks/GPTDecoder.cs:114-124) */
+    int32_t experts_per_token;
+    float   norm_eps;
+    float   rope_base;          /* the reference's literal is 500000 */
+    int32_t use_rope;
+    int32_t dtype;              /* TSHIP_F32 or TSHIP_F16: storage type of weights and KV cache */
+    int32_t max_batch;
+    int32_t max_seq_len;        /* KV cache capacity per sequence (prompt + generated) */
+} TSHipGptConfig;
+
+typedef struct TSHipGpt TSHipGpt;
+
+TSHIP_API int TSHip_GptCreate(const TSHipGptConfig* cfg, TSHipGpt** out);
+TSHIP_API int TSHip_GptDestroy(TSHipGpt* m);
+/* weights by the reference's saved parameter names, from host float32 arrays, shape as saved
+ * (WeightTensor.SetWeightArray, Seq2SeqSharp/Tools/WeightTensor.cs:504-520); converted to the model dtype
+ * with round-to-nearest-even (BasicTypesStructAsTypes.cs:800-840) */
+TSHIP_API int TSHip_GptSetWeight(TSHipGpt* m, const char* name, const float* host_data, int ndim, const int64_t* sizes);
+/* call once after the last TSHip_GptSetWeight: checks that every parameter is present */
+TSHIP_API int TSHip_GptFinalize(TSHipGpt* m);
+/* drop the KV cache contents (GPT.cs:236-247: a new dictionary per call) */
+TSHIP_API int TSHip_GptReset(TSHipGpt* m);
+/* prefill: ids [batch, prompt_len] int32 on the host, equal lengths; fills the cache and leaves the
+ * last-position logits on the device (Decoder.cs:679-716) */
+TSHIP_API int TSHip_GptPrefill(TSHipGpt* m, const int32_t* host_ids, int batch, int prompt_len);
+/* one decode step with the given tokens (Decoder.cs:661-678); leaves logits on the device */
+TSHIP_API int TSHip_GptDecode(TSHipGpt* m, const int32_t* host_ids, int batch);
+/* sampling modes */
+enum { TSHIP_GREEDY = 0, TSHIP_TOPP = 1 };
+/* choose next tokens from the logits on the device: softmax (after division by temperature when
+ * sampling and temperature != 1, Decoder.cs:720-732) then argmax or top-p; uniforms: host [batch] (top-p only) */
+TSHIP_API int TSHip_GptSample(TSHipGpt* m, int mode, float top_p, float temperature, const float* host_uniforms, int32_t* host_ids_out);
+/* n_steps of (sample from current logits -> decode the sampled tokens), all on the device; only token ids come
+ * back: host_ids_out [n_steps, batch].  host_uniforms [n_steps, batch] for top-p (else NULL).
+ * elapsed_ms (optional): device time of the loop measured with events on the library stream. */
+TSHIP_API int TSHip_GptGenerate(TSHipGpt* m, int n_steps, int mode, float top_p, float temperature,
+                                const float* host_uniforms, int32_t* host_ids_out, float* elapsed_ms);
+/* inspection for parity tests */
+TSHIP_API int TSHip_GptGetLogits(TSHipGpt* m, float* host_out /* [batch, vocab] */);
+TSHIP_API int TSHip_GptGetHidden(TSHipGpt* m, float* host_out /* [batch, hidden], after the final norm */);
+TSHIP_API int TSHip_GptGetSeqLen(TSHipGpt* m, int* len);
+/* KV cache rows of one layer as float32: which = 0 keys (after RoPE), 1 values; layout [batch, n_kv_heads, len, head_dim] */
+TSHIP_API int TSHip_GptGetKV(TSHipGpt* m, int layer, int which, float* host_out);
+/* install cache contents (same layout) and the sequence length: lets a benchmark start at a given context length */
+TSHIP_API int TSHip_GptSetKV(TSHipGpt* m, int layer, int which, const float* host_in, int batch, int len);
+TSHIP_API int TSHip_GptSetSeqLen(TSHipGpt* m, int batch, int len);
+/* routing of MoE layer `layer` at the last step: top_idx/top_val [rows, k], probs [rows, E] (host, float32) */
+TSHIP_API int TSHip_GptGetMoeRouting(TSHipGpt* m, int layer, float* top_idx, float* top_val, float* probs);
+/* per-kernel device times of one decode step (events around every launch on the library stream).
+ * names: buffer of n_max entries of 48 chars; ms: n_max floats; *n receives the number of launches. */
+TSHIP_API int TSHip_GptProfileDecode(TSHipGpt* m, const int32_t* host_ids, int batch, char* names, float* ms, int n_max, int* n);
+/* algorithmic bytes one decode step moves at the current sequence length (weights once, compact KV once) */
+TSHIP_API int TSHip_GptStepBytes(TSHipGpt* m, int batch, double* weight_bytes, double* kv_bytes);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TSHIP_H */

@@ -1,0 +1,937 @@
+// Fused GPTDecoder path: model object, weight loading/packing, prefill, decode step, on-device token loop.
+//
+// Replaces, for one model replica on one GPU, the reference's per-step stack
+//   GPT.RunForwardOnSingleDevice      Seq2SeqSharp/Applications/GPT.cs:212-335
+//   Decoder.GPTDecode                 Seq2SeqSharp/Applications/Decoder.cs:648-794
+//   GPTDecoder.Decode                 Seq2SeqSharp/Networks/GPTDecoder.cs:153-191
+//   GroupQueryAttention.Perform       Seq2SeqSharp/Layers/GroupQueryAttention.cs:114-233
+//   MultiHeadAttention.PerformClassic Seq2SeqSharp/Layers/MultiHeadAttention.cs:125-240
+//   PositionwiseFeedForward.Process   Seq2SeqSharp/Layers/PositionwiseFeedForward.cs:72-98
+// with a preallocated compact KV cache instead of concat-and-reallocate, and with only token ids
+// crossing PCIe per step.
+#include "tship_gpt_kernels.h"
+#include "tship_moe_kernels.h"
+#include "tship_sample_kernels.h"
+
+#include <cmath>
+#include <cstring>
+#include <map>
+#include <memory>
+#include <set>
+#include <vector>
+
+namespace tship {
+
+struct DevBuf {
+    void* p = nullptr;
+    size_t bytes = 0;
+    void alloc(size_t b) {
+        release();
+        if (b == 0) b = 256;
+        hipError_t e = hipMalloc(&p, b);
+        if (e != hipSuccess) {
+            (void)hipGetLastError(); p = nullptr;
+            throw Error("out of device memory: hipMalloc(" + std::to_string(b) + " bytes) failed");
+        }
+        bytes = b;
+        TSHIP_CHECK_HIP(hipMemsetAsync(p, 0, b, stream()));
+    }
+    void release() {
+        if (p) { (void)hipStreamSynchronize(stream()); (void)hipFree(p); p = nullptr; bytes = 0; }
+    }
+    ~DevBuf() { release(); }
+    DevBuf() {}
+    DevBuf(const DevBuf&) = delete;
+    DevBuf& operator=(const DevBuf&) = delete;
+    template <typename T> T* as() const { return (T*)p; }
+};
+
+// one GEMM operand: fp16 packed (KT x NT tiles) or fp32 row-major
+struct GemmW {
+    DevBuf buf;
+    int K = 0, N = 0;      // logical
+    int KT = 0, NT = 0;    // fp16 packed tile counts
+    long ld = 0;           // fp32 leading dimension
+    int KS = 1;            // split-K factor used at decode
+};
+
+struct LayerW {
+    DevBuf n1_g, n1_b, n2_g, n2_b;
+    GemmW qkv, wo, w13, w2;
+    DevBuf bqkv, bo, b1, b3, b2;
+    DevBuf kc, vc;
+    bool moe = false;
+    // MoE (Seq2SeqSharp/Layers/MoEFeedForward.cs:49-55)
+    DevBuf router, router_b;               // fp32 [h][E], [E]
+    std::vector<std::unique_ptr<GemmW>> e1, e2;   // per expert [h][4h], [4h][h]
+};
+
+struct Profiler {
+    std::vector<std::string> names;
+    std::vector<hipEvent_t> ev0, ev1;
+    ~Profiler() { for (auto e : ev0) (void)hipEventDestroy(e); for (auto e : ev1) (void)hipEventDestroy(e); }
+};
+
+}  // namespace tship
+
+using namespace tship;
+
+struct TSHipGpt {
+    TSHipGptConfig c;
+    bool f16;
+    int D, G, Nqkv, Bpad, BT;
+    long ldh, ldF;                 // leading dims of activation buffers (elements)
+    int F13;                       // columns of the first FFN GEMM output (F or 2F)
+    bool gated;
+    std::vector<std::unique_ptr<LayerW>> L;
+    DevBuf emb;                    // [V][h] model dtype
+    DevBuf fn_g, fn_b;             // final norm
+    GemmW head; DevBuf head_b;
+    DevBuf rope_cos, rope_sin;
+    std::set<std::string> expected, seen;
+    bool finalized = false;
+
+    // decode state
+    DevBuf x, xn, o, a, part_qkv, part_h, part_f, logits, ids, d_pos, hidden;
+    DevBuf moe_ws;
+    int pos = 0;                   // host mirror of *d_pos
+    int cur_batch = 0;
+    Profiler* prof = nullptr;
+
+    size_t esz() const { return f16 ? 2 : 4; }
+};
+
+namespace tship {
+
+template <typename... KArgs, typename... Args>
+static void launch(TSHipGpt* m, const char* name, void (*kernel)(KArgs...), dim3 grid, dim3 block, Args... args) {
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    if (m && m->prof) {
+        TSHIP_CHECK_HIP(hipEventCreate(&e0));
+        TSHIP_CHECK_HIP(hipEventCreate(&e1));
+        m->prof->names.push_back(name);
+        m->prof->ev0.push_back(e0);
+        m->prof->ev1.push_back(e1);
+    }
+    hipExtLaunchKernelGGL(kernel, grid, block, 0, stream(), e0, e1, 0, args...);
+    TSHIP_CHECK_HIP(hipGetLastError());
+}
+
+static int pick_ks_f16(int NT, int KT) {
+    int target = 2 * std::max(n_compute_units(), 64);
+    int ks = std::max(1, target / std::max(NT, 1));
+    ks = std::min(ks, std::max(1, KT / 8));
+    return std::min(ks, 16);
+}
+static int pick_ks_f32(int N, int K) {
+    int target = 2 * std::max(n_compute_units(), 64);
+    int ks = std::max(1, target / (int)ceil_div(N, 64));
+    ks = std::min(ks, std::max(1, K / 64));
+    return std::min(ks, 16);
+}
+
+static void upload_f32(DevBuf& dst, const float* host, size_t n) {
+    dst.alloc(n * sizeof(float));
+    TSHIP_CHECK_HIP(hipMemcpyAsync(dst.p, host, n * sizeof(float), hipMemcpyHostToDevice, stream()));
+    TSHIP_CHECK_HIP(hipStreamSynchronize(stream()));
+}
+
+// allocate the destination of a GEMM weight with logical shape [K][N]
+static void gemmw_alloc(TSHipGpt* m, GemmW& w, int K, int N) {
+    if (w.buf.p) return;
+    w.K = K; w.N = N;
+    if (m->f16) {
+        w.KT = (int)ceil_div(K, 16); w.NT = (int)ceil_div(N, 32);
+        w.buf.alloc((size_t)w.KT * w.NT * 512 * sizeof(half_t));
+        w.KS = pick_ks_f16(w.NT, w.KT);
+    } else {
+        w.ld = N;
+        w.buf.alloc((size_t)K * N * sizeof(float));
+        w.KS = pick_ks_f32(N, K);
+    }
+}
+
+// copy host fp32 [K][n_src] into columns of a GEMM weight (packing for fp16)
+static void gemmw_fill(TSHipGpt* m, GemmW& w, const float* host, int K, int n_src, int mode, int n_off) {
+    TSHIP_REQUIRE(K == w.K, "weight row count does not match the model configuration");
+    DevBuf tmp;
+    upload_f32(tmp, host, (size_t)K * n_src);
+    if (m->f16) {
+        long total = (long)n_src * w.KT * 2;
+        pack_w_kernel<<<(unsigned)ceil_div(total, 256), 256, 0, stream()>>>(tmp.as<float>(), n_src, K, n_src, w.buf.as<half_t>(), w.KT, mode, n_off);
+    } else {
+        TSHIP_REQUIRE(mode == PACK_PLAIN, "internal: interleave is an fp16-only layout");
+        long total = (long)K * n_src;
+        copy_cols_kernel<float><<<(unsigned)ceil_div(total, 256), 256, 0, stream()>>>(tmp.as<float>(), n_src, K, n_src, w.buf.as<float>(), w.ld, n_off);
+    }
+    TSHIP_CHECK_HIP(hipGetLastError());
+    TSHIP_CHECK_HIP(hipStreamSynchronize(stream()));
+}
+
+static void expect_shape(const char* name, int ndim, const int64_t* sizes, std::initializer_list<int64_t> want) {
+    bool ok = (size_t)ndim == want.size();
+    if (ok) { int i = 0; for (auto w : want) ok = ok && sizes[i++] == w; }
+    if (!ok) {
+        std::string s = std::string("weight '") + name + "' has shape [";
+        for (int i = 0; i < ndim; ++i) s += (i ? "," : "") + std::to_string(sizes[i]);
+        s += "], expected [";
+        int i = 0; for (auto w : want) s += (i++ ? "," : "") + std::to_string(w);
+        throw Error(s + "]");
+    }
+}
+
+static void build_expected(TSHipGpt* m) {
+    auto& c = m->c;
+    auto& e = m->expected;
+    bool ln = c.norm_type == 1;
+    auto norm = [&](const std::string& p) { e.insert(p + ".m_alpha"); if (ln) e.insert(p + ".m_beta"); };
+    e.insert("TgtEmbeddings");
+    for (int i = 0; i < c.n_layers; ++i) {
+        std::string a = "GPTDecoder.SelfAttn_" + std::to_string(i);
+        norm(a + ".layerNormQ");
+        if (c.attn_type == 1) for (auto s : {"Q", "Qb", "K", "Kb", "V", "Vb"}) e.insert(a + "." + s);
+        else { e.insert(a + ".QKV"); e.insert(a + ".QKVb"); }
+        e.insert(a + ".W0"); e.insert(a + ".b0");
+        if (c.n_experts > 1 && i > 1) {
+            std::string f = "GPTDecoder.MoEFFN_" + std::to_string(i);
+            for (auto s : {"layerNorm.m_alpha", "layerNorm.m_beta", "m_Router", "m_RouterBias", "m_Whd1", "m_Whd2"}) e.insert(f + "." + s);
+        } else {
+            std::string f = "GPTDecoder.PosFFN_" + std::to_string(i);
+            norm(f + ".layerNorm2");
+            e.insert(f + ".feedForwardLayer1.m_Whd"); e.insert(f + ".feedForwardLayer1.m_Bd");
+            e.insert(f + ".feedForwardLayer2.m_Whd"); e.insert(f + ".feedForwardLayer2.m_Bd");
+            if (m->gated) { e.insert(f + ".feedForwardLayer3.m_Whd"); e.insert(f + ".feedForwardLayer3.m_Bd"); }
+        }
+    }
+    norm("GPTDecoder.layerNorm");
+    e.insert("FeedForward_Decoder_0.m_Whd"); e.insert("FeedForward_Decoder_0.m_Bd");
+}
+
+static void set_weight(TSHipGpt* m, const std::string& name, const float* host, int ndim, const int64_t* sizes) {
+    auto& c = m->c;
+    TSHIP_REQUIRE(m->expected.count(name), "unknown weight name for this configuration: " + name);
+    const int h = c.hidden, H = c.n_heads, Gk = c.n_kv_heads, D = m->D, F = c.ffn_dim, V = c.vocab;
+    long count = 1; for (int i = 0; i < ndim; ++i) count *= sizes[i];
+    auto vec = [&](DevBuf& dst, int64_t n) { expect_shape(name.c_str(), ndim, sizes, {1, n}); upload_f32(dst, host, (size_t)n); };
+    auto vec_into = [&](DevBuf& dst, int64_t total, int64_t off, int64_t n) {
+        expect_shape(name.c_str(), ndim, sizes, {1, n});
+        if (!dst.p) dst.alloc((size_t)total * sizeof(float));
+        TSHIP_CHECK_HIP(hipMemcpyAsync(dst.as<float>() + off, host, (size_t)n * sizeof(float), hipMemcpyHostToDevice, stream()));
+        TSHIP_CHECK_HIP(hipStreamSynchronize(stream()));
+    };
+    if (name == "TgtEmbeddings") {
+        expect_shape(name.c_str(), ndim, sizes, {V, h});
+        DevBuf tmp; upload_f32(tmp, host, (size_t)V * h);
+        m->emb.alloc((size_t)V * h * m->esz());
+        long total = (long)V * h;
+        if (m->f16) copy_cols_kernel<half_t><<<(unsigned)ceil_div(total, 256), 256, 0, stream()>>>(tmp.as<float>(), h, V, h, m->emb.as<half_t>(), h, 0);
+        else copy_cols_kernel<float><<<(unsigned)ceil_div(total, 256), 256, 0, stream()>>>(tmp.as<float>(), h, V, h, m->emb.as<float>(), h, 0);
+        TSHIP_CHECK_HIP(hipGetLastError());
+        TSHIP_CHECK_HIP(hipStreamSynchronize(stream()));
+    } else if (name == "GPTDecoder.layerNorm.m_alpha") vec(m->fn_g, h);
+    else if (name == "GPTDecoder.layerNorm.m_beta") vec(m->fn_b, h);
+    else if (name == "FeedForward_Decoder_0.m_Whd") {
+        expect_shape(name.c_str(), ndim, sizes, {h, V});
+        gemmw_alloc(m, m->head, h, V); m->head.KS = 1;
+        gemmw_fill(m, m->head, host, h, V, PACK_PLAIN, 0);
+    } else if (name == "FeedForward_Decoder_0.m_Bd") vec(m->head_b, V);
+    else {
+        // GPTDecoder.<kind>_<i>.<field>
+        size_t us = name.find('_'), dot = name.find('.', us);
+        TSHIP_REQUIRE(us != std::string::npos && dot != std::string::npos, "cannot parse weight name: " + name);
+        int li = std::stoi(name.substr(us + 1, dot - us - 1));
+        TSHIP_REQUIRE(li >= 0 && li < c.n_layers, "layer index out of range in weight name: " + name);
+        LayerW& L = *m->L[li];
+        std::string kind = name.substr(0, us), field = name.substr(dot + 1);
+        if (kind == "GPTDecoder.SelfAttn") {
+            if (field == "layerNormQ.m_alpha") vec(L.n1_g, h);
+            else if (field == "layerNormQ.m_beta") vec(L.n1_b, h);
+            else if (field == "QKV") { expect_shape(name.c_str(), ndim, sizes, {h, 3 * h}); gemmw_alloc(m, L.qkv, h, m->Nqkv); gemmw_fill(m, L.qkv, host, h, 3 * h, PACK_PLAIN, 0); }
+            else if (field == "QKVb") vec(L.bqkv, 3 * h);
+            else if (field == "Q") { expect_shape(name.c_str(), ndim, sizes, {h, H * D}); gemmw_alloc(m, L.qkv, h, m->Nqkv); gemmw_fill(m, L.qkv, host, h, H * D, PACK_PLAIN, 0); }
+            else if (field == "K") { expect_shape(name.c_str(), ndim, sizes, {h, Gk * D}); gemmw_alloc(m, L.qkv, h, m->Nqkv); gemmw_fill(m, L.qkv, host, h, Gk * D, PACK_PLAIN, H * D); }
+            else if (field == "V") { expect_shape(name.c_str(), ndim, sizes, {h, Gk * D}); gemmw_alloc(m, L.qkv, h, m->Nqkv); gemmw_fill(m, L.qkv, host, h, Gk * D, PACK_PLAIN, H * D + Gk * D); }
+            else if (field == "Qb") vec_into(L.bqkv, m->Nqkv, 0, H * D);
+            else if (field == "Kb") vec_into(L.bqkv, m->Nqkv, H * D, Gk * D);
+            else if (field == "Vb") vec_into(L.bqkv, m->Nqkv, H * D + Gk * D, Gk * D);
+            else if (field == "W0") { expect_shape(name.c_str(), ndim, sizes, {h, h}); gemmw_alloc(m, L.wo, h, h); gemmw_fill(m, L.wo, host, h, h, PACK_PLAIN, 0); }
+            else if (field == "b0") vec(L.bo, h);
+            else throw Error("unknown attention field: " + name);
+        } else if (kind == "GPTDecoder.PosFFN") {
+            bool inter = m->f16 && m->gated;     // fp16: W1/W3 interleaved by 16 columns; fp32: [W1 | W3]
+            if (field == "layerNorm2.m_alpha") vec(L.n2_g, h);
+            else if (field == "layerNorm2.m_beta") vec(L.n2_b, h);
+            else if (field == "feedForwardLayer1.m_Whd") {
+                expect_shape(name.c_str(), ndim, sizes, {h, F});
+                gemmw_alloc(m, L.w13, h, m->F13); if (m->f16) L.w13.KS = 1;
+                gemmw_fill(m, L.w13, host, h, F, inter ? PACK_INTERLEAVE16 : PACK_PLAIN, 0);
+            } else if (field == "feedForwardLayer3.m_Whd") {
+                expect_shape(name.c_str(), ndim, sizes, {h, F});
+                gemmw_alloc(m, L.w13, h, m->F13); if (m->f16) L.w13.KS = 1;
+                gemmw_fill(m, L.w13, host, h, F, inter ? PACK_INTERLEAVE16 : PACK_PLAIN, inter ? 16 : F);
+            } else if (field == "feedForwardLayer1.m_Bd") vec(L.b1, F);
+            else if (field == "feedForwardLayer3.m_Bd") vec(L.b3, F);
+            else if (field == "feedForwardLayer2.m_Whd") { expect_shape(name.c_str(), ndim, sizes, {F, h}); gemmw_alloc(m, L.w2, F, h); gemmw_fill(m, L.w2, host, F, h, PACK_PLAIN, 0); }
+            else if (field == "feedForwardLayer2.m_Bd") vec(L.b2, h);
+            else throw Error("unknown feed-forward field: " + name);
+        } else if (kind == "GPTDecoder.MoEFFN") {
+            const int E = c.n_experts;
+            if (field == "layerNorm.m_alpha") vec(L.n2_g, h);
+            else if (field == "layerNorm.m_beta") vec(L.n2_b, h);
+            else if (field == "m_Router") { expect_shape(name.c_str(), ndim, sizes, {h, E}); upload_f32(L.router, host, (size_t)h * E); }
+            else if (field == "m_RouterBias") vec(L.router_b, E);
+            else if (field == "m_Whd1") {
+                expect_shape(name.c_str(), ndim, sizes, {E, h, 4 * h});
+                for (int e = 0; e < E; ++e) { gemmw_alloc(m, *L.e1[e], h, 4 * h); L.e1[e]->KS = 1; gemmw_fill(m, *L.e1[e], host + (size_t)e * h * 4 * h, h, 4 * h, PACK_PLAIN, 0); }
+            } else if (field == "m_Whd2") {
+                expect_shape(name.c_str(), ndim, sizes, {E, 4 * h, h});
+                for (int e = 0; e < E; ++e) { gemmw_alloc(m, *L.e2[e], 4 * h, h); L.e2[e]->KS = 1; gemmw_fill(m, *L.e2[e], host + (size_t)e * h * 4 * h, 4 * h, h, PACK_PLAIN, 0); }
+            } else throw Error("unknown MoE field: " + name);
+        } else throw Error("unknown weight name: " + name);
+    }
+    (void)count;
+    m->seen.insert(name);
+}
+
+// ------------------------------------------------------------------------------------------------
+// kernel dispatch helpers
+// ------------------------------------------------------------------------------------------------
+static void run_resid_norm(TSHipGpt* m, const char* name, int rows, ResidNormArgs a) {
+    if (m->f16) launch(m, name, resid_norm_kernel<half_t>, dim3(rows), dim3(256), a);
+    else launch(m, name, resid_norm_kernel<float>, dim3(rows), dim3(256), a);
+}
+
+// Y = X * W for <= 128 rows.  fp16: MFMA kernel; epilogue per `epi`.  fp32: tiled GEMM into partials.
+static void run_skinny(TSHipGpt* m, const char* name, const GemmW& w, const void* X, long ldx, int rows, int epi, SkinnyArgs e) {
+    TSHIP_REQUIRE(m->f16, "internal: run_skinny is the fp16 path");
+    e.W = w.buf.as<half_t>(); e.KT = w.KT; e.NT = w.NT; e.X = (const half_t*)X; e.ldx = (int)ldx;
+    e.KS = (epi == EPI_PARTIAL) ? w.KS : 1; e.rows_valid = rows;
+    dim3 grid(w.NT * e.KS), block(256);
+    const int BT = m->BT;
+#define TSHIP_SK(BTV)                                                                                       \
+    if (epi == EPI_PARTIAL) launch(m, name, skinny_gemm_f16_kernel<BTV, EPI_PARTIAL>, grid, block, e);      \
+    else if (epi == EPI_F32_BIAS) launch(m, name, skinny_gemm_f16_kernel<BTV, EPI_F32_BIAS>, grid, block, e); \
+    else launch(m, name, skinny_gemm_f16_kernel<BTV, EPI_ACT16>, grid, block, e);
+    if (BT == 1) { TSHIP_SK(1) } else if (BT == 2) { TSHIP_SK(2) } else { TSHIP_SK(4) }
+#undef TSHIP_SK
+}
+
+static void run_gemm_f32(TSHipGpt* m, const char* name, const GemmW& w, const float* X, long ldx, int rows, float* out, long ld_out,
+                         long split_stride, int KS, const float* bias = nullptr) {
+    F32GemmArgs g;
+    g.bias = KS == 1 ? bias : nullptr;
+    g.A = X; g.lda = ldx; g.B = w.buf.as<float>(); g.ldb = w.ld; g.C = out; g.ldc = ld_out; g.split_stride = split_stride;
+    g.M = rows; g.N = w.N; g.K = w.K; g.KS = KS;
+    dim3 grid((unsigned)ceil_div(w.N, 64), (unsigned)ceil_div(rows, 64), KS);
+    launch(m, name, gemm_f32_kernel, grid, dim3(256), g);
+}
+
+typedef void (*AttnKernel)(AttnArgs);
+template <typename CT, typename AT, int D>
+static AttnKernel pick_attn_g(int G, bool prefill) {
+    switch (G) {
+        case 1: return prefill ? attn_prefill_kernel<CT, AT, D, 1> : attn_decode_kernel<CT, AT, D, 1>;
+        case 2: return prefill ? attn_prefill_kernel<CT, AT, D, 2> : attn_decode_kernel<CT, AT, D, 2>;
+        case 4: return prefill ? attn_prefill_kernel<CT, AT, D, 4> : attn_decode_kernel<CT, AT, D, 4>;
+        default: throw Error("query heads per KV head must be 1, 2 or 4");
+    }
+}
+template <typename CT, typename AT>
+static AttnKernel pick_attn_d(int D, int G, bool prefill) {
+    switch (D) {
+        case 16: return pick_attn_g<CT, AT, 16>(G, prefill);
+        case 32: return pick_attn_g<CT, AT, 32>(G, prefill);
+        case 64: return pick_attn_g<CT, AT, 64>(G, prefill);
+        case 128: return pick_attn_g<CT, AT, 128>(G, prefill);
+        default: throw Error("head_dim must be 16, 32, 64 or 128");
+    }
+}
+static AttnKernel pick_attn(TSHipGpt* m, bool prefill) {
+    return m->f16 ? pick_attn_d<half_t, half_t>(m->D, m->G, prefill) : pick_attn_d<float, float>(m->D, m->G, prefill);
+}
+template <typename CT>
+static AttnKernel pick_kvw_t(int D) {
+    switch (D) {
+        case 16: return kv_write_kernel<CT, 16>;
+        case 32: return kv_write_kernel<CT, 32>;
+        case 64: return kv_write_kernel<CT, 64>;
+        case 128: return kv_write_kernel<CT, 128>;
+        default: throw Error("head_dim must be 16, 32, 64 or 128");
+    }
+}
+static AttnKernel pick_kvw(TSHipGpt* m) { return m->f16 ? pick_kvw_t<half_t>(m->D) : pick_kvw_t<float>(m->D); }
+
+static AttnArgs attn_args(TSHipGpt* m, LayerW& L) {
+    AttnArgs a; std::memset(&a, 0, sizeof(a));
+    a.bias = L.bqkv.as<float>(); a.H = m->c.n_heads; a.Hkv = m->c.n_kv_heads;
+    a.kcache = L.kc.p; a.vcache = L.vc.p; a.max_len = m->c.max_seq_len;
+    if (m->c.use_rope) { a.rope_cos = m->rope_cos.as<float>(); a.rope_sin = m->rope_sin.as<float>(); }
+    a.d_pos = m->d_pos.as<int>();
+    a.scale = 1.0f / (float)std::sqrt((double)m->D);   // GroupQueryAttention.cs:193
+    return a;
+}
+
+// ------------------------------------------------------------------------------------------------
+// MoE feed-forward at decode (MoEFeedForward.Process, Seq2SeqSharp/Layers/MoEFeedForward.cs:76-181)
+// ------------------------------------------------------------------------------------------------
+static void run_moe_ffn(TSHipGpt* m, LayerW& L, int rows, const ResidNormArgs& pre);
+static void moe_alloc(TSHipGpt* m);
+static void moe_get_routing(TSHipGpt* m, int layer, float* top_idx, float* top_val, float* probs);
+static void sample_tokens(TSHipGpt* m, int mode, float top_p, float temperature, const float* host_uniforms, const float* dev_uniforms, int B, int* gen_out);
+
+// ------------------------------------------------------------------------------------------------
+// decode step: tokens (device int32 [batch]) -> logits (device fp32 [batch][vocab])
+// ------------------------------------------------------------------------------------------------
+static void decode_step(TSHipGpt* m, const int* d_ids, int B) {
+    auto& c = m->c;
+    const int h = c.hidden, F = c.ffn_dim;
+    const long hp = round_up(h, 32), qp = round_up(m->Nqkv, 32);
+    ResidNormArgs rn; std::memset(&rn, 0, sizeof(rn));
+    rn.x = m->x.as<float>(); rn.ldx = h; rn.h = h; rn.eps = c.norm_eps; rn.norm_type = c.norm_type;
+    rn.xn = m->xn.p; rn.ldxn = m->ldh;
+
+    // embedding gather * sqrt(h) and the first layer's attention norm
+    {
+        ResidNormArgs a = rn;
+        a.ids = d_ids; a.emb = m->emb.p; a.emb_f16 = m->f16; a.emb_scale = (float)std::sqrt((double)h);
+        a.gamma = m->L[0]->n1_g.as<float>(); a.beta = m->L[0]->n1_b.as<float>();
+        run_resid_norm(m, "embed_norm", B, a);
+    }
+    for (int l = 0; l < c.n_layers; ++l) {
+        LayerW& L = *m->L[l];
+        // QKV projection -> split-K partials
+        long qstride = (long)m->Bpad * qp;
+        if (m->f16) {
+            SkinnyArgs e; std::memset(&e, 0, sizeof(e));
+            e.out = m->part_qkv.as<float>(); e.ld_out = (int)qp; e.split_stride = qstride;
+            run_skinny(m, "gemm_qkv", L.qkv, m->xn.p, m->ldh, B, EPI_PARTIAL, e);
+        } else {
+            run_gemm_f32(m, "gemm_qkv", L.qkv, m->xn.as<float>(), m->ldh, B, m->part_qkv.as<float>(), qp, qstride, L.qkv.KS);
+        }
+        // RoPE, cache append, attention
+        {
+            AttnArgs a = attn_args(m, L);
+            a.qkv = m->part_qkv.as<float>(); a.KS = L.qkv.KS; a.split_stride = qstride; a.ldq = qp;
+            a.out = m->o.p; a.ld_out = m->ldh;
+            launch(m, "attn_decode", pick_attn(m, false), dim3(c.n_kv_heads, B), dim3(256), a);
+        }
+        // output projection -> partials
+        long hstride = (long)m->Bpad * hp;
+        if (m->f16) {
+            SkinnyArgs e; std::memset(&e, 0, sizeof(e));
+            e.out = m->part_h.as<float>(); e.ld_out = (int)hp; e.split_stride = hstride;
+            run_skinny(m, "gemm_wo", L.wo, m->o.p, m->ldh, B, EPI_PARTIAL, e);
+        } else {
+            run_gemm_f32(m, "gemm_wo", L.wo, m->o.as<float>(), m->ldh, B, m->part_h.as<float>(), hp, hstride, L.wo.KS);
+        }
+        // x += attn_out + b0 ; feed-forward norm
+        ResidNormArgs a2 = rn;
+        a2.part = m->part_h.as<float>(); a2.KS = L.wo.KS; a2.split_stride = hstride; a2.ld_part = hp; a2.bias = L.bo.as<float>();
+        a2.gamma = L.n2_g.as<float>(); a2.beta = L.n2_b.as<float>();
+        const float* next_g = (l + 1 < c.n_layers) ? m->L[l + 1]->n1_g.as<float>() : m->fn_g.as<float>();
+        const float* next_b = (l + 1 < c.n_layers) ? m->L[l + 1]->n1_b.as<float>() : m->fn_b.as<float>();
+        if (L.moe) {
+            a2.norm_type = 1;          // MoEFeedForward always uses LayerNormalization (MoEFeedForward.cs:49)
+            run_moe_ffn(m, L, B, a2);
+            // x already updated by the MoE combine; next norm
+            ResidNormArgs a3 = rn;
+            a3.gamma = next_g; a3.beta = next_b;
+            if (l + 1 == c.n_layers) a3.advance_pos = m->d_pos.as<int>();
+            run_resid_norm(m, "norm_next", B, a3);
+            continue;
+        }
+        run_resid_norm(m, "resid_norm_ffn", B, a2);
+        // FFN up (and gate) projection
+        if (m->f16) {
+            SkinnyArgs e; std::memset(&e, 0, sizeof(e));
+            e.bias = L.b1.as<float>(); e.bias2 = L.b3.as<float>(); e.out16 = m->a.as<half_t>(); e.ld16 = (int)m->ldF;
+            e.act = c.act; e.gated = m->gated; e.n_valid = F;
+            run_skinny(m, "gemm_ffn13", L.w13, m->xn.p, m->ldh, B, EPI_ACT16, e);
+        } else {
+            long fp = m->F13, fstride = (long)m->Bpad * fp;
+            run_gemm_f32(m, "gemm_ffn13", L.w13, m->xn.as<float>(), m->ldh, B, m->part_f.as<float>(), fp, fstride, L.w13.KS);
+            long tot = (long)B * F;
+            launch(m, "ffn_act", ffn_act_kernel<float>, dim3((unsigned)ceil_div(tot, 256)), dim3(256), (const float*)m->part_f.as<float>(), L.w13.KS,
+                   fstride, fp, (const float*)L.b1.as<float>(), (const float*)L.b3.as<float>(), F, (int)m->gated, (int)c.act, m->a.as<float>(), m->ldF, (long)B);
+        }
+        // FFN down projection -> partials
+        if (m->f16) {
+            SkinnyArgs e; std::memset(&e, 0, sizeof(e));
+            e.out = m->part_h.as<float>(); e.ld_out = (int)hp; e.split_stride = hstride;
+            run_skinny(m, "gemm_ffn2", L.w2, m->a.p, m->ldF, B, EPI_PARTIAL, e);
+        } else {
+            run_gemm_f32(m, "gemm_ffn2", L.w2, m->a.as<float>(), m->ldF, B, m->part_h.as<float>(), hp, hstride, L.w2.KS);
+        }
+        // x += ffn_out + b2 ; next layer's attention norm, or the final norm
+        ResidNormArgs a3 = rn;
+        a3.part = m->part_h.as<float>(); a3.KS = L.w2.KS; a3.split_stride = hstride; a3.ld_part = hp; a3.bias = L.b2.as<float>();
+        a3.gamma = next_g; a3.beta = next_b;
+        if (l + 1 == c.n_layers) a3.advance_pos = m->d_pos.as<int>();
+        run_resid_norm(m, l + 1 == c.n_layers ? "resid_norm_final" : "resid_norm_attn", B, a3);
+    }
+    // vocabulary projection (only the new position exists at decode)
+    const long Vp = round_up(c.vocab, 32);
+    if (m->f16) {
+        SkinnyArgs e; std::memset(&e, 0, sizeof(e));
+        e.out = m->logits.as<float>(); e.ld_out = (int)Vp; e.bias = m->head_b.as<float>(); e.n_valid = c.vocab;
+        run_skinny(m, "gemm_head", m->head, m->xn.p, m->ldh, B, EPI_F32_BIAS, e);
+    } else {
+        run_gemm_f32(m, "gemm_head", m->head, m->xn.as<float>(), m->ldh, B, m->logits.as<float>(), Vp, 0, 1, m->head_b.as<float>());
+    }
+    m->pos += 1;
+}
+
+// ------------------------------------------------------------------------------------------------
+// prefill: whole prompts, causal attention, cache filled for every position, logits of the last position
+// ------------------------------------------------------------------------------------------------
+static void prefill(TSHipGpt* m, const int32_t* host_ids, int B, int Tp) {
+    auto& c = m->c;
+    const int h = c.hidden, F = c.ffn_dim;
+    const long R = (long)B * Tp, Rp = round_up(R, 128);
+    const long qp = round_up(m->Nqkv, 32);
+    TSHIP_REQUIRE(m->pos == 0, "TSHip_GptPrefill: the cache is not empty; call TSHip_GptReset first");
+    TSHIP_REQUIRE(Tp >= 1 && Tp < c.max_seq_len, "TSHip_GptPrefill: prompt length exceeds max_seq_len");
+    DevBuf ids, px, pxn, pqkv, po, pa, pf, rowmap;
+    ids.alloc(R * sizeof(int));
+    TSHIP_CHECK_HIP(hipMemcpyAsync(ids.p, host_ids, R * sizeof(int), hipMemcpyHostToDevice, stream()));
+    px.alloc((size_t)Rp * h * sizeof(float));
+    pxn.alloc((size_t)Rp * m->ldh * m->esz());
+    pqkv.alloc((size_t)Rp * qp * sizeof(float));
+    po.alloc((size_t)Rp * m->ldh * m->esz());
+    bool any_dense = false; for (auto& L : m->L) any_dense = any_dense || !L->moe;
+    if (any_dense) pa.alloc((size_t)Rp * m->ldF * m->esz());
+    if (!m->f16 && any_dense) pf.alloc((size_t)Rp * m->F13 * sizeof(float));
+
+    ResidNormArgs rn; std::memset(&rn, 0, sizeof(rn));
+    rn.x = px.as<float>(); rn.ldx = h; rn.h = h; rn.eps = c.norm_eps; rn.norm_type = c.norm_type;
+    rn.xn = pxn.p; rn.ldxn = m->ldh;
+    {
+        ResidNormArgs a = rn;
+        a.ids = ids.as<int>(); a.emb = m->emb.p; a.emb_f16 = m->f16; a.emb_scale = (float)std::sqrt((double)h);
+        a.gamma = m->L[0]->n1_g.as<float>(); a.beta = m->L[0]->n1_b.as<float>();
+        run_resid_norm(m, "p_embed_norm", (int)R, a);
+    }
+    auto big = [&](const char* name, const GemmW& w, const void* X, long ldx, int epi, BigArgs e) {
+        e.W = w.buf.as<half_t>(); e.KT = w.KT; e.NT = w.NT; e.X = (const half_t*)X; e.ldx = (int)ldx; e.R = (int)R;
+        dim3 grid((unsigned)ceil_div(w.NT, 4), (unsigned)(Rp / 128));
+        if (epi == BEPI_F32_BIAS) launch(m, name, big_gemm_f16_kernel<BEPI_F32_BIAS>, grid, dim3(256), e);
+        else if (epi == BEPI_RESID) launch(m, name, big_gemm_f16_kernel<BEPI_RESID>, grid, dim3(256), e);
+        else launch(m, name, big_gemm_f16_kernel<BEPI_ACT16>, grid, dim3(256), e);
+    };
+    DevBuf zero_bias; zero_bias.alloc((size_t)std::max<long>(std::max<long>(qp, m->F13), round_up(h, 32)) * sizeof(float));
+    for (int l = 0; l < c.n_layers; ++l) {
+        LayerW& L = *m->L[l];
+        AttnArgs aa = attn_args(m, L);
+        aa.qkv = pqkv.as<float>(); aa.KS = 1; aa.split_stride = 0; aa.ldq = qp; aa.pos0 = 0; aa.Tq = Tp;
+        aa.out = po.p; aa.ld_out = m->ldh;
+        if (m->f16) {
+            BigArgs e; std::memset(&e, 0, sizeof(e));
+            e.out = pqkv.as<float>(); e.ld_out = (int)qp; e.bias = L.bqkv.as<float>(); e.n_valid = m->Nqkv;
+            big("p_gemm_qkv", L.qkv, pxn.p, m->ldh, BEPI_F32_BIAS, e);
+            aa.bias = zero_bias.as<float>();      // bias already added by the GEMM epilogue
+        } else {
+            run_gemm_f32(m, "p_gemm_qkv", L.qkv, pxn.as<float>(), m->ldh, (int)R, pqkv.as<float>(), qp, 0, 1);
+        }
+        launch(m, "p_kv_write", pick_kvw(m), dim3(Tp, B), dim3(256), aa);
+        launch(m, "p_attn", pick_attn(m, true), dim3(Tp, c.n_kv_heads, B), dim3(256), aa);
+        ResidNormArgs a2 = rn;
+        a2.gamma = L.n2_g.as<float>(); a2.beta = L.n2_b.as<float>();
+        if (m->f16) {
+            BigArgs e; std::memset(&e, 0, sizeof(e));
+            e.out = px.as<float>(); e.ld_out = h; e.bias = L.bo.as<float>(); e.n_valid = h;
+            big("p_gemm_wo", L.wo, po.p, m->ldh, BEPI_RESID, e);
+        } else {
+            run_gemm_f32(m, "p_gemm_wo", L.wo, po.as<float>(), m->ldh, (int)R, pqkv.as<float>(), qp, 0, 1);
+            a2.part = pqkv.as<float>(); a2.KS = 1; a2.ld_part = qp; a2.bias = L.bo.as<float>();
+        }
+        if (L.moe) throw Error("TSHip_GptPrefill: MoE layers are prefilled token by token; use TSHip_GptDecode");
+        run_resid_norm(m, "p_norm_ffn", (int)R, a2);
+        ResidNormArgs a3 = rn;
+        if (l + 1 < c.n_layers) { a3.gamma = m->L[l + 1]->n1_g.as<float>(); a3.beta = m->L[l + 1]->n1_b.as<float>(); }
+        else a3.xn = nullptr;
+        if (m->f16) {
+            BigArgs e; std::memset(&e, 0, sizeof(e));
+            e.bias = L.b1.as<float>(); e.bias2 = L.b3.as<float>(); e.out16 = pa.as<half_t>(); e.ld16 = (int)m->ldF;
+            e.act = c.act; e.gated = m->gated; e.n_valid = F;
+            big("p_gemm_ffn13", L.w13, pxn.p, m->ldh, BEPI_ACT16, e);
+            BigArgs e2; std::memset(&e2, 0, sizeof(e2));
+            e2.out = px.as<float>(); e2.ld_out = h; e2.bias = L.b2.as<float>(); e2.n_valid = h;
+            big("p_gemm_ffn2", L.w2, pa.p, m->ldF, BEPI_RESID, e2);
+        } else {
+            run_gemm_f32(m, "p_gemm_ffn13", L.w13, pxn.as<float>(), m->ldh, (int)R, pf.as<float>(), m->F13, 0, 1);
+            long tot = R * F;
+            launch(m, "p_ffn_act", ffn_act_kernel<float>, dim3((unsigned)ceil_div(tot, 256)), dim3(256), (const float*)pf.as<float>(), 1, 0L,
+                   (long)m->F13, (const float*)L.b1.as<float>(), (const float*)L.b3.as<float>(), F, (int)m->gated, (int)c.act, pa.as<float>(), m->ldF, R);
+            run_gemm_f32(m, "p_gemm_ffn2", L.w2, pa.as<float>(), m->ldF, (int)R, pqkv.as<float>(), qp, 0, 1);
+            a3.part = pqkv.as<float>(); a3.KS = 1; a3.ld_part = qp; a3.bias = L.b2.as<float>();
+        }
+        if (l + 1 < c.n_layers || !m->f16) run_resid_norm(m, "p_norm_attn", (int)R, a3);
+    }
+    // last position of every sequence (Decoder.cs:705-716) -> final norm -> vocabulary projection
+    std::vector<int> map(B);
+    for (int b = 0; b < B; ++b) map[b] = Tp * (b + 1) - 1;
+    rowmap.alloc(B * sizeof(int));
+    TSHIP_CHECK_HIP(hipMemcpyAsync(rowmap.p, map.data(), B * sizeof(int), hipMemcpyHostToDevice, stream()));
+    {
+        ResidNormArgs a = rn;
+        a.row_map = rowmap.as<int>(); a.xn = m->xn.p; a.ldxn = m->ldh;
+        a.gamma = m->fn_g.as<float>(); a.beta = m->fn_b.as<float>();
+        run_resid_norm(m, "p_final_norm", B, a);
+    }
+    const long Vp = round_up(c.vocab, 32);
+    if (m->f16) {
+        SkinnyArgs e; std::memset(&e, 0, sizeof(e));
+        e.out = m->logits.as<float>(); e.ld_out = (int)Vp; e.bias = m->head_b.as<float>(); e.n_valid = c.vocab;
+        run_skinny(m, "gemm_head", m->head, m->xn.p, m->ldh, B, EPI_F32_BIAS, e);
+    } else {
+        run_gemm_f32(m, "gemm_head", m->head, m->xn.as<float>(), m->ldh, B, m->logits.as<float>(), Vp, 0, 1, m->head_b.as<float>());
+    }
+    m->pos = Tp;
+    TSHIP_CHECK_HIP(hipMemcpyAsync(m->d_pos.p, &m->pos, sizeof(int), hipMemcpyHostToDevice, stream()));
+    TSHIP_CHECK_HIP(hipStreamSynchronize(stream()));
+    m->cur_batch = B;
+}
+
+}  // namespace tship
+
+#include "tship_gpt_extra.h"
+
+// =================================================================================================
+// exported functions
+// =================================================================================================
+extern "C" {
+
+TSHIP_API int TSHip_GptCreate(const TSHipGptConfig* cfg, TSHipGpt** out) {
+    TSHIP_BEGIN
+    TSHIP_REQUIRE(cfg && out, "TSHip_GptCreate: null argument");
+    ensure_init();
+    const TSHipGptConfig& c = *cfg;
+    TSHIP_REQUIRE(c.n_layers > 0 && c.hidden > 0 && c.n_heads > 0 && c.n_kv_heads > 0 && c.vocab > 0, "TSHip_GptCreate: sizes must be positive");
+    TSHIP_REQUIRE(c.hidden % c.n_heads == 0, "TSHip_GptCreate: hidden must be divisible by n_heads");
+    TSHIP_REQUIRE(c.n_heads % c.n_kv_heads == 0, "TSHip_GptCreate: n_heads must be divisible by n_kv_heads");
+    TSHIP_REQUIRE(c.attn_type == 1 || c.n_kv_heads == c.n_heads, "TSHip_GptCreate: MultiHeadAttention needs n_kv_heads == n_heads");
+    TSHIP_REQUIRE(c.hidden <= 8192, "TSHip_GptCreate: hidden up to 8192 is supported");
+    TSHIP_REQUIRE(c.dtype == TSHIP_F32 || c.dtype == TSHIP_F16, "TSHip_GptCreate: dtype must be f32 or f16");
+    TSHIP_REQUIRE(c.max_batch >= 1 && c.max_batch <= 128, "TSHip_GptCreate: max_batch must be in 1..128");
+    TSHIP_REQUIRE(c.max_seq_len >= 2, "TSHip_GptCreate: max_seq_len too small");
+    TSHIP_REQUIRE(c.act >= 0 && c.act <= 4, "TSHip_GptCreate: unknown activation");
+    TSHIP_REQUIRE(c.norm_type == 0 || c.norm_type == 1, "TSHip_GptCreate: unknown norm type");
+    std::unique_ptr<TSHipGpt> m(new TSHipGpt());
+    m->c = c;
+    m->f16 = c.dtype == TSHIP_F16;
+    m->D = c.hidden / c.n_heads;
+    m->G = c.n_heads / c.n_kv_heads;
+    TSHIP_REQUIRE(m->D == 16 || m->D == 32 || m->D == 64 || m->D == 128, "TSHip_GptCreate: head_dim must be 16, 32, 64 or 128");
+    TSHIP_REQUIRE(m->G == 1 || m->G == 2 || m->G == 4, "TSHip_GptCreate: query heads per KV head must be 1, 2 or 4");
+    m->Nqkv = (c.n_heads + 2 * c.n_kv_heads) * m->D;
+    m->BT = c.max_batch <= 32 ? 1 : (c.max_batch <= 64 ? 2 : 4);
+    m->Bpad = m->BT * 32;
+    m->gated = (c.act == 3 || c.act == 4);
+    m->F13 = m->gated ? 2 * c.ffn_dim : c.ffn_dim;
+    if (c.n_experts > 1) {
+        TSHIP_REQUIRE(c.experts_per_token >= 1 && c.experts_per_token <= c.n_experts && c.n_experts <= 64, "TSHip_GptCreate: bad MoE sizes");
+        TSHIP_REQUIRE(!m->gated, "TSHip_GptCreate: the reference's MoE experts are two-matrix MLPs; a gated activation has no third matrix");
+    }
+    const long h4 = 4L * c.hidden;
+    m->ldh = round_up(c.hidden, 16);
+    m->ldF = round_up(std::max<long>(c.ffn_dim, c.n_experts > 1 ? h4 : 0), 16);
+    const int h = c.hidden;
+    for (int i = 0; i < c.n_layers; ++i) {
+        m->L.emplace_back(new LayerW());
+        LayerW& L = *m->L.back();
+        L.moe = c.n_experts > 1 && i > 1;      // Networks/GPTDecoder.cs:114-124
+        if (L.moe) for (int e = 0; e < c.n_experts; ++e) { L.e1.emplace_back(new GemmW()); L.e2.emplace_back(new GemmW()); }
+        size_t cache_bytes = (size_t)c.max_batch * c.n_kv_heads * c.max_seq_len * m->D * m->esz();
+        L.kc.alloc(cache_bytes); L.vc.alloc(cache_bytes);
+    }
+    build_expected(m.get());
+    // rotary table, computed exactly as the reference's expression (TensorApplyCPU.cs:1161-1164):
+    // theta = (float)pow(base, -2 i / cols); cos/sin of the float product theta * m, evaluated in double
+    if (c.use_rope) {
+        const int D = m->D;
+        std::vector<float> cs((size_t)c.max_seq_len * D / 2), sn(cs.size());
+        for (int i = 0; i < D / 2; ++i) {
+            float theta = (float)std::pow((double)c.rope_base, -2.0 * (double)i / (double)D);
+            for (int p = 0; p < c.max_seq_len; ++p) {
+                float tm = theta * (float)p;
+                cs[(size_t)p * (D / 2) + i] = (float)std::cos((double)tm);
+                sn[(size_t)p * (D / 2) + i] = (float)std::sin((double)tm);
+            }
+        }
+        upload_f32(m->rope_cos, cs.data(), cs.size());
+        upload_f32(m->rope_sin, sn.data(), sn.size());
+    }
+    // decode buffers
+    const long hp = round_up(h, 32), qp = round_up(m->Nqkv, 32), Vp = round_up(c.vocab, 32);
+    m->x.alloc((size_t)m->Bpad * h * sizeof(float));
+    m->xn.alloc((size_t)m->Bpad * m->ldh * m->esz());
+    m->o.alloc((size_t)m->Bpad * m->ldh * m->esz());
+    m->a.alloc((size_t)m->Bpad * m->ldF * m->esz());
+    m->part_qkv.alloc((size_t)16 * m->Bpad * qp * sizeof(float));
+    m->part_h.alloc((size_t)16 * m->Bpad * hp * sizeof(float));
+    if (!m->f16) m->part_f.alloc((size_t)16 * m->Bpad * m->F13 * sizeof(float));
+    m->logits.alloc((size_t)m->Bpad * Vp * sizeof(float));
+    m->ids.alloc((size_t)m->Bpad * sizeof(int));
+    m->d_pos.alloc(sizeof(int));
+    m->hidden.alloc((size_t)m->Bpad * h * sizeof(float));
+    if (c.n_experts > 1) moe_alloc(m.get());
+    TSHIP_CHECK_HIP(hipStreamSynchronize(stream()));
+    *out = m.release();
+    TSHIP_END
+}
+
+TSHIP_API int TSHip_GptDestroy(TSHipGpt* m) {
+    TSHIP_BEGIN
+    if (m) { (void)hipStreamSynchronize(stream()); delete m; }
+    TSHIP_END
+}
+
+TSHIP_API int TSHip_GptSetWeight(TSHipGpt* m, const char* name, const float* host_data, int ndim, const int64_t* sizes) {
+    TSHIP_BEGIN
+    TSHIP_REQUIRE(m && name && host_data && sizes, "TSHip_GptSetWeight: null argument");
+    TSHIP_REQUIRE(ndim >= 1 && ndim <= 3, "TSHip_GptSetWeight: ndim must be 1..3");
+    set_weight(m, name, host_data, ndim, sizes);
+    TSHIP_END
+}
+
+TSHIP_API int TSHip_GptFinalize(TSHipGpt* m) {
+    TSHIP_BEGIN
+    TSHIP_REQUIRE(m, "TSHip_GptFinalize: null model");
+    for (auto& n : m->expected)
+        if (!m->seen.count(n)) throw Error("TSHip_GptFinalize: weight '" + n + "' was never set");
+    // RMSNorm has no beta (Layers/RMSNormalization.cs:33-37): keep null pointers there
+    m->finalized = true;
+    TSHIP_END
+}
+
+TSHIP_API int TSHip_GptReset(TSHipGpt* m) {
+    TSHIP_BEGIN
+    TSHIP_REQUIRE(m, "TSHip_GptReset: null model");
+    m->pos = 0; m->cur_batch = 0;
+    TSHIP_CHECK_HIP(hipMemsetAsync(m->d_pos.p, 0, sizeof(int), stream()));
+    TSHIP_CHECK_HIP(hipStreamSynchronize(stream()));
+    TSHIP_END
+}
+
+TSHIP_API int TSHip_GptPrefill(TSHipGpt* m, const int32_t* host_ids, int batch, int prompt_len) {
+    TSHIP_BEGIN
+    TSHIP_REQUIRE(m && host_ids, "TSHip_GptPrefill: null argument");
+    TSHIP_REQUIRE(m->finalized, "TSHip_GptPrefill: call TSHip_GptFinalize first");
+    TSHIP_REQUIRE(batch >= 1 && batch <= m->c.max_batch, "TSHip_GptPrefill: batch out of range");
+    for (long i = 0; i < (long)batch * prompt_len; ++i)
+        TSHIP_REQUIRE(host_ids[i] >= 0 && host_ids[i] < m->c.vocab, "TSHip_GptPrefill: token id out of range");
+    bool any_moe = false; for (auto& L : m->L) any_moe = any_moe || L->moe;
+    if (any_moe) {
+        // token-by-token: the MoE layer is built for decode-sized row counts
+        std::vector<int32_t> col(batch);
+        for (int t = 0; t < prompt_len; ++t) {
+            for (int b = 0; b < batch; ++b) col[b] = host_ids[(long)b * prompt_len + t];
+            TSHIP_CHECK_HIP(hipMemcpyAsync(m->ids.p, col.data(), batch * sizeof(int), hipMemcpyHostToDevice, stream()));
+            TSHIP_CHECK_HIP(hipStreamSynchronize(stream()));
+            if (t == 0) TSHIP_REQUIRE(m->pos == 0, "TSHip_GptPrefill: the cache is not empty; call TSHip_GptReset first");
+            decode_step(m, m->ids.as<int>(), batch);
+        }
+        TSHIP_CHECK_HIP(hipStreamSynchronize(stream()));
+        m->cur_batch = batch;
+    } else {
+        prefill(m, host_ids, batch, prompt_len);
+    }
+    TSHIP_END
+}
+
+TSHIP_API int TSHip_GptDecode(TSHipGpt* m, const int32_t* host_ids, int batch) {
+    TSHIP_BEGIN
+    TSHIP_REQUIRE(m && host_ids, "TSHip_GptDecode: null argument");
+    TSHIP_REQUIRE(m->finalized, "TSHip_GptDecode: call TSHip_GptFinalize first");
+    TSHIP_REQUIRE(batch >= 1 && batch <= m->c.max_batch, "TSHip_GptDecode: batch out of range");
+    TSHIP_REQUIRE(m->cur_batch == 0 || m->cur_batch == batch, "TSHip_GptDecode: batch differs from the cached sequences");
+    TSHIP_REQUIRE(m->pos + 1 <= m->c.max_seq_len, "TSHip_GptDecode: KV cache is full (max_seq_len)");
+    for (int i = 0; i < batch; ++i) TSHIP_REQUIRE(host_ids[i] >= 0 && host_ids[i] < m->c.vocab, "TSHip_GptDecode: token id out of range");
+    TSHIP_CHECK_HIP(hipMemcpyAsync(m->ids.p, host_ids, batch * sizeof(int), hipMemcpyHostToDevice, stream()));
+    TSHIP_CHECK_HIP(hipStreamSynchronize(stream()));
+    decode_step(m, m->ids.as<int>(), batch);
+    TSHIP_CHECK_HIP(hipStreamSynchronize(stream()));
+    m->cur_batch = batch;
+    TSHIP_END
+}
+
+TSHIP_API int TSHip_GptSample(TSHipGpt* m, int mode, float top_p, float temperature, const float* host_uniforms, int32_t* host_ids_out) {
+    TSHIP_BEGIN
+    TSHIP_REQUIRE(m && host_ids_out, "TSHip_GptSample: null argument");
+    TSHIP_REQUIRE(m->cur_batch > 0, "TSHip_GptSample: no logits yet; prefill or decode first");
+    const int B = m->cur_batch;
+    sample_tokens(m, mode, top_p, temperature, host_uniforms, nullptr, B, nullptr);
+    TSHIP_CHECK_HIP(hipMemcpyAsync(host_ids_out, m->ids.p, B * sizeof(int), hipMemcpyDeviceToHost, stream()));
+    TSHIP_CHECK_HIP(hipStreamSynchronize(stream()));
+    TSHIP_END
+}
+
+TSHIP_API int TSHip_GptGenerate(TSHipGpt* m, int n_steps, int mode, float top_p, float temperature,
+                                const float* host_uniforms, int32_t* host_ids_out, float* elapsed_ms) {
+    TSHIP_BEGIN
+    TSHIP_REQUIRE(m && host_ids_out, "TSHip_GptGenerate: null argument");
+    TSHIP_REQUIRE(m->cur_batch > 0, "TSHip_GptGenerate: no logits yet; prefill first");
+    TSHIP_REQUIRE(n_steps >= 1, "TSHip_GptGenerate: n_steps must be positive");
+    TSHIP_REQUIRE(m->pos + n_steps <= m->c.max_seq_len, "TSHip_GptGenerate: KV cache too small for n_steps (max_seq_len)");
+    TSHIP_REQUIRE(mode == TSHIP_GREEDY || (mode == TSHIP_TOPP && host_uniforms), "TSHip_GptGenerate: top-p needs the uniform stream");
+    const int B = m->cur_batch;
+    DevBuf gen, uni;
+    gen.alloc((size_t)n_steps * B * sizeof(int));
+    if (mode == TSHIP_TOPP) {
+        uni.alloc((size_t)n_steps * B * sizeof(float));
+        TSHIP_CHECK_HIP(hipMemcpyAsync(uni.p, host_uniforms, (size_t)n_steps * B * sizeof(float), hipMemcpyHostToDevice, stream()));
+    }
+    hipEvent_t e0, e1;
+    TSHIP_CHECK_HIP(hipEventCreate(&e0));
+    TSHIP_CHECK_HIP(hipEventCreate(&e1));
+    TSHIP_CHECK_HIP(hipStreamSynchronize(stream()));
+    TSHIP_CHECK_HIP(hipEventRecord(e0, stream()));
+    for (int s = 0; s < n_steps; ++s) {
+        sample_tokens(m, mode, top_p, temperature, nullptr, mode == TSHIP_TOPP ? uni.as<float>() + (size_t)s * B : nullptr, B,
+                      gen.as<int>() + (size_t)s * B);
+        decode_step(m, m->ids.as<int>(), B);
+    }
+    TSHIP_CHECK_HIP(hipEventRecord(e1, stream()));
+    TSHIP_CHECK_HIP(hipStreamSynchronize(stream()));
+    float ms = 0.0f;
+    TSHIP_CHECK_HIP(hipEventElapsedTime(&ms, e0, e1));
+    (void)hipEventDestroy(e0); (void)hipEventDestroy(e1);
+    if (elapsed_ms) *elapsed_ms = ms;
+    TSHIP_CHECK_HIP(hipMemcpy(host_ids_out, gen.p, (size_t)n_steps * B * sizeof(int), hipMemcpyDeviceToHost));
+    TSHIP_END
+}
+
+TSHIP_API int TSHip_GptGetLogits(TSHipGpt* m, float* host_out) {
+    TSHIP_BEGIN
+    TSHIP_REQUIRE(m && host_out, "TSHip_GptGetLogits: null argument");
+    TSHIP_REQUIRE(m->cur_batch > 0, "TSHip_GptGetLogits: no logits yet");
+    const long Vp = round_up(m->c.vocab, 32);
+    TSHIP_CHECK_HIP(hipStreamSynchronize(stream()));
+    TSHIP_CHECK_HIP(hipMemcpy2D(host_out, (size_t)m->c.vocab * sizeof(float), m->logits.p, (size_t)Vp * sizeof(float),
+                                (size_t)m->c.vocab * sizeof(float), m->cur_batch, hipMemcpyDeviceToHost));
+    TSHIP_END
+}
+
+TSHIP_API int TSHip_GptGetHidden(TSHipGpt* m, float* host_out) {
+    TSHIP_BEGIN
+    TSHIP_REQUIRE(m && host_out, "TSHip_GptGetHidden: null argument");
+    TSHIP_REQUIRE(m->cur_batch > 0, "TSHip_GptGetHidden: nothing computed yet");
+    const int B = m->cur_batch, h = m->c.hidden;
+    TSHIP_CHECK_HIP(hipStreamSynchronize(stream()));
+    if (m->f16) {
+        std::vector<half_t> tmp((size_t)B * m->ldh);
+        TSHIP_CHECK_HIP(hipMemcpy(tmp.data(), m->xn.p, tmp.size() * sizeof(half_t), hipMemcpyDeviceToHost));
+        for (int b = 0; b < B; ++b) for (int i = 0; i < h; ++i) host_out[(size_t)b * h + i] = (float)tmp[(size_t)b * m->ldh + i];
+    } else {
+        TSHIP_CHECK_HIP(hipMemcpy2D(host_out, (size_t)h * sizeof(float), m->xn.p, (size_t)m->ldh * sizeof(float), (size_t)h * sizeof(float), B, hipMemcpyDeviceToHost));
+    }
+    TSHIP_END
+}
+
+TSHIP_API int TSHip_GptGetSeqLen(TSHipGpt* m, int* len) {
+    TSHIP_BEGIN
+    TSHIP_REQUIRE(m && len, "TSHip_GptGetSeqLen: null argument");
+    TSHIP_CHECK_HIP(hipStreamSynchronize(stream()));
+    int dev = 0;
+    TSHIP_CHECK_HIP(hipMemcpy(&dev, m->d_pos.p, sizeof(int), hipMemcpyDeviceToHost));
+    TSHIP_REQUIRE(dev == m->pos, "internal: device and host sequence positions disagree");
+    *len = m->pos;
+    TSHIP_END
+}
+
+TSHIP_API int TSHip_GptGetKV(TSHipGpt* m, int layer, int which, float* host_out) {
+    TSHIP_BEGIN
+    TSHIP_REQUIRE(m && host_out, "TSHip_GptGetKV: null argument");
+    TSHIP_REQUIRE(layer >= 0 && layer < m->c.n_layers && (which == 0 || which == 1), "TSHip_GptGetKV: bad layer or selector");
+    const int B = m->cur_batch, G = m->c.n_kv_heads, D = m->D, T = m->pos; const long ML = m->c.max_seq_len;
+    TSHIP_CHECK_HIP(hipStreamSynchronize(stream()));
+    const char* base = (const char*)(which ? m->L[layer]->vc.p : m->L[layer]->kc.p);
+    std::vector<char> tmp((size_t)T * D * m->esz());
+    for (int b = 0; b < B; ++b) for (int g = 0; g < G; ++g) {
+        TSHIP_CHECK_HIP(hipMemcpy(tmp.data(), base + ((size_t)b * G + g) * ML * D * m->esz(), tmp.size(), hipMemcpyDeviceToHost));
+        float* dst = host_out + ((size_t)b * G + g) * T * D;
+        if (m->f16) { const half_t* s = (const half_t*)tmp.data(); for (long i = 0; i < (long)T * D; ++i) dst[i] = (float)s[i]; }
+        else std::memcpy(dst, tmp.data(), tmp.size());
+    }
+    TSHIP_END
+}
+
+TSHIP_API int TSHip_GptSetSeqLen(TSHipGpt* m, int batch, int len) {
+    TSHIP_BEGIN
+    TSHIP_REQUIRE(m, "TSHip_GptSetSeqLen: null model");
+    TSHIP_REQUIRE(batch >= 1 && batch <= m->c.max_batch && len >= 0 && len < m->c.max_seq_len, "TSHip_GptSetSeqLen: out of range");
+    m->pos = len; m->cur_batch = batch;
+    TSHIP_CHECK_HIP(hipMemcpyAsync(m->d_pos.p, &m->pos, sizeof(int), hipMemcpyHostToDevice, stream()));
+    TSHIP_CHECK_HIP(hipStreamSynchronize(stream()));
+    TSHIP_END
+}
+
+TSHIP_API int TSHip_GptSetKV(TSHipGpt* m, int layer, int which, const float* host_in, int batch, int len) {
+    TSHIP_BEGIN
+    TSHIP_REQUIRE(m && host_in, "TSHip_GptSetKV: null argument");
+    TSHIP_REQUIRE(layer >= 0 && layer < m->c.n_layers && (which == 0 || which == 1), "TSHip_GptSetKV: bad layer or selector");
+    TSHIP_REQUIRE(batch >= 1 && batch <= m->c.max_batch && len >= 0 && len <= m->c.max_seq_len, "TSHip_GptSetKV: out of range");
+    const int G = m->c.n_kv_heads, D = m->D; const long ML = m->c.max_seq_len;
+    char* base = (char*)(which ? m->L[layer]->vc.p : m->L[layer]->kc.p);
+    std::vector<char> tmp((size_t)len * D * m->esz());
+    for (int b = 0; b < batch; ++b) for (int g = 0; g < G; ++g) {
+        const float* src = host_in + ((size_t)b * G + g) * len * D;
+        if (m->f16) { half_t* d = (half_t*)tmp.data(); for (long i = 0; i < (long)len * D; ++i) d[i] = (half_t)src[i]; }
+        else std::memcpy(tmp.data(), src, tmp.size());
+        TSHIP_CHECK_HIP(hipMemcpy(base + ((size_t)b * G + g) * ML * D * m->esz(), tmp.data(), tmp.size(), hipMemcpyHostToDevice));
+    }
+    TSHIP_END
+}
+
+TSHIP_API int TSHip_GptGetMoeRouting(TSHipGpt* m, int layer, float* top_idx, float* top_val, float* probs) {
+    TSHIP_BEGIN
+    TSHIP_REQUIRE(m, "TSHip_GptGetMoeRouting: null model");
+    TSHIP_REQUIRE(layer >= 0 && layer < m->c.n_layers && m->L[layer]->moe, "TSHip_GptGetMoeRouting: not an MoE layer");
+    moe_get_routing(m, layer, top_idx, top_val, probs);
+    TSHIP_END
+}
+
+TSHIP_API int TSHip_GptProfileDecode(TSHipGpt* m, const int32_t* host_ids, int batch, char* names, float* ms, int n_max, int* n) {
+    TSHIP_BEGIN
+    TSHIP_REQUIRE(m && host_ids && names && ms && n, "TSHip_GptProfileDecode: null argument");
+    TSHIP_REQUIRE(m->finalized && batch >= 1 && batch <= m->c.max_batch, "TSHip_GptProfileDecode: bad state or batch");
+    TSHIP_REQUIRE(m->pos + 1 <= m->c.max_seq_len, "TSHip_GptProfileDecode: KV cache is full");
+    TSHIP_CHECK_HIP(hipMemcpyAsync(m->ids.p, host_ids, batch * sizeof(int), hipMemcpyHostToDevice, stream()));
+    TSHIP_CHECK_HIP(hipStreamSynchronize(stream()));
+    Profiler prof;
+    m->prof = &prof;
+    try { decode_step(m, m->ids.as<int>(), batch); } catch (...) { m->prof = nullptr; throw; }
+    m->prof = nullptr;
+    TSHIP_CHECK_HIP(hipStreamSynchronize(stream()));
+    m->cur_batch = batch;
+    int cnt = (int)prof.names.size();
+    *n = cnt;
+    for (int i = 0; i < cnt && i < n_max; ++i) {
+        float t = 0.0f;
+        TSHIP_CHECK_HIP(hipEventElapsedTime(&t, prof.ev0[i], prof.ev1[i]));
+        ms[i] = t;
+        std::strncpy(names + (size_t)i * 48, prof.names[i].c_str(), 47);
+        names[(size_t)i * 48 + 47] = 0;
+    }
+    TSHIP_END
+}
+
+TSHIP_API int TSHip_GptStepBytes(TSHipGpt* m, int batch, double* weight_bytes, double* kv_bytes) {
+    TSHIP_BEGIN
+    TSHIP_REQUIRE(m && weight_bytes && kv_bytes, "TSHip_GptStepBytes: null argument");
+    auto& c = m->c;
+    const double s = (double)m->esz();
+    const double h = c.hidden, Hd = (double)c.n_heads * m->D, Gd = (double)c.n_kv_heads * m->D, F = c.ffn_dim, V = c.vocab;
+    double params = 0.0;
+    for (int l = 0; l < c.n_layers; ++l) {
+        params += h * Hd + 2.0 * h * Gd + Hd * h;
+        if (m->L[l]->moe) params += h * c.n_experts + (double)std::min(c.n_experts, batch * c.experts_per_token) * 2.0 * h * 4.0 * h;
+        else params += (m->gated ? 3.0 : 2.0) * h * F;
+    }
+    params += h * V;
+    *weight_bytes = s * params + (double)batch * h * s;
+    *kv_bytes = s * (double)c.n_layers * batch * Gd * 2.0 * (double)(m->pos + 1);
+    TSHIP_END
+}
+
+}  // extern "C"

@@ -1,0 +1,145 @@
+// Host side of the MoE feed-forward and of token sampling for the fused GPTDecoder path.
+// Included by tship_gpt.hip after the model object is defined.
+#pragma once
+
+namespace tship {
+
+struct MoeLayout {
+    size_t xn32, probs, top_val, top_idx, counts, lists, slot, xg, mid, y, wtab1, wtab2, zero, total;
+    long ld4h, ldy;
+};
+
+static MoeLayout moe_layout(TSHipGpt* m) {
+    auto& c = m->c;
+    MoeLayout o; size_t at = 0;
+    auto take = [&](size_t bytes) { size_t r = at; at += round_up((long)bytes, 256); return r; };
+    const long h = c.hidden, E = c.n_experts, k = c.experts_per_token, Bp = m->Bpad;
+    o.ld4h = round_up(4 * h, 16); o.ldy = round_up(h, 32);
+    o.xn32 = take(Bp * h * 4); o.probs = take(Bp * E * 4); o.top_val = take(Bp * k * 4); o.top_idx = take(Bp * k * 4);
+    o.counts = take(E * 4); o.lists = take(E * Bp * 4); o.slot = take(Bp * k * 4);
+    o.xg = take(E * Bp * m->ldh * m->esz());
+    o.mid = take(E * Bp * o.ld4h * m->esz());
+    o.y = take(E * Bp * o.ldy * 4);
+    o.wtab1 = take(E * sizeof(void*)); o.wtab2 = take(E * sizeof(void*));
+    o.zero = take(std::max<long>(4 * h, 64) * 4);
+    o.total = at;
+    return o;
+}
+
+static void moe_alloc(TSHipGpt* m) {
+    TSHIP_REQUIRE(m->c.hidden <= 4096, "TSHip_GptCreate: MoE layers support hidden up to 4096");
+    m->moe_ws.alloc(moe_layout(m).total);
+}
+
+static void moe_get_routing(TSHipGpt* m, int layer, float* top_idx, float* top_val, float* probs) {
+    (void)layer;   // the workspace holds the routing of the MoE layer that ran last; callers run one layer at a time
+    MoeLayout o = moe_layout(m);
+    const int B = m->cur_batch, k = m->c.experts_per_token, E = m->c.n_experts;
+    TSHIP_CHECK_HIP(hipStreamSynchronize(stream()));
+    char* base = (char*)m->moe_ws.p;
+    if (top_idx) TSHIP_CHECK_HIP(hipMemcpy(top_idx, base + o.top_idx, (size_t)B * k * 4, hipMemcpyDeviceToHost));
+    if (top_val) TSHIP_CHECK_HIP(hipMemcpy(top_val, base + o.top_val, (size_t)B * k * 4, hipMemcpyDeviceToHost));
+    if (probs) TSHIP_CHECK_HIP(hipMemcpy(probs, base + o.probs, (size_t)B * E * 4, hipMemcpyDeviceToHost));
+}
+
+// `pre` carries the pending attention output (split-K partials + bias) and the LayerNorm parameters
+static void run_moe_ffn(TSHipGpt* m, LayerW& L, int rows, const ResidNormArgs& pre) {
+    auto& c = m->c;
+    MoeLayout o = moe_layout(m);
+    char* base = (char*)m->moe_ws.p;
+    const int h = c.hidden, E = c.n_experts, k = c.experts_per_token, Bp = m->Bpad;
+    float* xn32 = (float*)(base + o.xn32); float* probs = (float*)(base + o.probs);
+    float* top_val = (float*)(base + o.top_val); float* top_idx = (float*)(base + o.top_idx);
+    int* counts = (int*)(base + o.counts); int* lists = (int*)(base + o.lists); int* slot = (int*)(base + o.slot);
+    float* y = (float*)(base + o.y); float* zero = (float*)(base + o.zero);
+
+    MoeRouterArgs r; std::memset(&r, 0, sizeof(r));
+    r.x = pre.x; r.ldx = pre.ldx; r.h = h;
+    r.part = pre.part; r.KS = pre.KS; r.split_stride = pre.split_stride; r.ld_part = pre.ld_part; r.bias = pre.bias;
+    r.gamma = pre.gamma; r.beta = pre.beta; r.eps = pre.eps;
+    r.router = L.router.as<float>(); r.router_b = L.router_b.as<float>(); r.E = E; r.k = k;
+    r.xn32 = xn32; r.probs = probs; r.top_val = top_val; r.top_idx = top_idx;
+    launch(m, "moe_router", moe_router_kernel, dim3(rows), dim3(64), r);
+    launch(m, "moe_lists", moe_lists_kernel, dim3(1), dim3(64), (const float*)top_idx, rows, k, E, Bp, counts, lists, slot);
+    const long xg_stride = (long)Bp * m->ldh, mid_stride = (long)Bp * o.ld4h, y_stride = (long)Bp * o.ldy;
+    if (m->f16) {
+        half_t* xg = (half_t*)(base + o.xg); half_t* mid = (half_t*)(base + o.mid);
+        launch(m, "moe_gather", moe_gather_kernel<half_t>, dim3(rows, E), dim3(256), (const float*)xn32, h, (const int*)counts, (const int*)lists, Bp, xg,
+               m->ldh, xg_stride);
+        // pointer tables are written once per layer object (weights never move)
+        std::vector<const half_t*> t1(E), t2(E);
+        for (int e = 0; e < E; ++e) { t1[e] = L.e1[e]->buf.as<half_t>(); t2[e] = L.e2[e]->buf.as<half_t>(); }
+        TSHIP_CHECK_HIP(hipMemcpyAsync(base + o.wtab1, t1.data(), E * sizeof(void*), hipMemcpyHostToDevice, stream()));
+        TSHIP_CHECK_HIP(hipMemcpyAsync(base + o.wtab2, t2.data(), E * sizeof(void*), hipMemcpyHostToDevice, stream()));
+        TSHIP_CHECK_HIP(hipStreamSynchronize(stream()));
+        SkinnyArgs e1; std::memset(&e1, 0, sizeof(e1));
+        e1.W = t1[0]; e1.KT = L.e1[0]->KT; e1.NT = L.e1[0]->NT; e1.X = xg; e1.ldx = (int)m->ldh; e1.KS = 1;
+        e1.bias = zero; e1.out16 = mid; e1.ld16 = (int)o.ld4h; e1.act = c.act; e1.gated = 0; e1.n_valid = 4 * h;
+        e1.Wtab = (const half_t* const*)(base + o.wtab1); e1.x_estride = xg_stride; e1.out16_estride = mid_stride; e1.rows_tab = counts;
+        SkinnyArgs e2; std::memset(&e2, 0, sizeof(e2));
+        e2.W = t2[0]; e2.KT = L.e2[0]->KT; e2.NT = L.e2[0]->NT; e2.X = mid; e2.ldx = (int)o.ld4h; e2.KS = 1;
+        e2.bias = zero; e2.out = y; e2.ld_out = (int)o.ldy; e2.n_valid = h;
+        e2.Wtab = (const half_t* const*)(base + o.wtab2); e2.x_estride = mid_stride; e2.out_estride = y_stride; e2.rows_tab = counts;
+        dim3 g1(e1.NT, E), g2(e2.NT, E);
+        if (m->BT == 1) {
+            launch(m, "moe_gemm1", skinny_gemm_f16_kernel<1, EPI_ACT16>, g1, dim3(256), e1);
+            launch(m, "moe_gemm2", skinny_gemm_f16_kernel<1, EPI_F32_BIAS>, g2, dim3(256), e2);
+        } else if (m->BT == 2) {
+            launch(m, "moe_gemm1", skinny_gemm_f16_kernel<2, EPI_ACT16>, g1, dim3(256), e1);
+            launch(m, "moe_gemm2", skinny_gemm_f16_kernel<2, EPI_F32_BIAS>, g2, dim3(256), e2);
+        } else {
+            launch(m, "moe_gemm1", skinny_gemm_f16_kernel<4, EPI_ACT16>, g1, dim3(256), e1);
+            launch(m, "moe_gemm2", skinny_gemm_f16_kernel<4, EPI_F32_BIAS>, g2, dim3(256), e2);
+        }
+    } else {
+        float* xg = (float*)(base + o.xg); float* mid = (float*)(base + o.mid);
+        launch(m, "moe_gather", moe_gather_kernel<float>, dim3(rows, E), dim3(256), (const float*)xn32, h, (const int*)counts, (const int*)lists, Bp, xg,
+               m->ldh, xg_stride);
+        for (int e = 0; e < E; ++e) {
+            // fp32 models: every expert runs on `rows` rows; rows past the expert's count hold stale finite data
+            // and are never read back
+            float* mid_e = mid + e * mid_stride;
+            run_gemm_f32(m, "moe_gemm1", *L.e1[e], xg + e * xg_stride, m->ldh, rows, mid_e, o.ld4h, 0, 1);
+            long tot = (long)rows * 4 * h;
+            launch(m, "moe_act", ffn_act_kernel<float>, dim3((unsigned)ceil_div(tot, 256)), dim3(256), (const float*)mid_e, 1, 0L, o.ld4h,
+                   (const float*)zero, (const float*)zero, 4 * h, 0, (int)c.act, mid_e, o.ld4h, (long)rows);
+            run_gemm_f32(m, "moe_gemm2", *L.e2[e], mid_e, o.ld4h, rows, y + e * y_stride, o.ldy, 0, 1);
+        }
+    }
+    launch(m, "moe_combine", moe_combine_kernel, dim3(rows), dim3(256), pre.x, pre.ldx, h, (const float*)y, o.ldy, y_stride, (const float*)probs,
+           (const float*)top_idx, (const int*)slot, k, E);
+}
+
+// next tokens from the logits on the device -> m->ids (and gen_out); greedy or top-p
+static void sample_tokens(TSHipGpt* m, int mode, float top_p, float temperature, const float* host_uniforms, const float* dev_uniforms, int B,
+                          int* gen_out) {
+    const long Vp = round_up(m->c.vocab, 32);
+    if (mode == TSHIP_GREEDY) {
+        launch(m, "greedy", greedy_kernel, dim3(B), dim3(256), (const float*)m->logits.as<float>(), Vp, m->c.vocab, m->ids.as<int>(), gen_out);
+        return;
+    }
+    TSHIP_REQUIRE(mode == TSHIP_TOPP, "unknown sampling mode");
+    TSHIP_REQUIRE(m->c.vocab <= 65535, "top-p sampling supports vocabularies up to 65535");
+    TSHIP_REQUIRE(temperature > 0.0f, "temperature must be positive");
+    const long Vs = round_up(m->c.vocab, 64);
+    static thread_local DevBuf scratch, uni;
+    size_t need = (size_t)m->Bpad * Vs * 5 * 4;
+    if (scratch.bytes < need) scratch.alloc(need);
+    if (!dev_uniforms) {
+        TSHIP_REQUIRE(host_uniforms, "top-p sampling needs one uniform draw per row");
+        if (uni.bytes < (size_t)B * 4) uni.alloc((size_t)m->Bpad * 4);
+        TSHIP_CHECK_HIP(hipMemcpyAsync(uni.p, host_uniforms, (size_t)B * 4, hipMemcpyHostToDevice, stream()));
+        dev_uniforms = uni.as<float>();
+    }
+    TopPArgs a; std::memset(&a, 0, sizeof(a));
+    a.in = m->logits.as<float>(); a.ld = Vp; a.V = m->c.vocab; a.in_is_logits = 1;
+    a.uniforms = dev_uniforms; a.top_p = top_p; a.Vs = Vs;
+    char* s = (char*)scratch.p; size_t one = (size_t)m->Bpad * Vs * 4;
+    a.keysA = (unsigned*)s; a.keysB = (unsigned*)(s + one); a.idxA = (int*)(s + 2 * one); a.idxB = (int*)(s + 3 * one); a.accp = (float*)(s + 4 * one);
+    a.next_ids = m->ids.as<int>(); a.gen_out = gen_out;
+    // Decoder.cs:720-723 divides the logits by the temperature (fp32 division) before the softmax
+    a.temperature = temperature;
+    launch(m, "topp", topp_kernel, dim3(B), dim3(256), a);
+}
+
+}  // namespace tship

@@ -1,0 +1,634 @@
+// Device kernels of the fused GPTDecoder path (gfx950).  Included by tship_gpt.hip only.
+//
+// Data layout in HBM
+//   residual stream x      fp32 [rows][hidden]
+//   GEMM inputs            model activation type AT (fp16 or fp32) [rows padded][K padded], zero padded
+//   fp16 weights           "P32" packed: tile (nt, kt) = 32 output columns x 16 k, 1 KiB, stored as the
+//                          A-operand fragment of v_mfma_f32_32x32x16_f16: lane l holds column nt*32 + l%32,
+//                          k = kt*16 + 8*(l/32) .. +7.  All k-tiles of one column tile are contiguous, so a
+//                          wavefront streams one contiguous range with 16-byte loads.
+//   fp32 weights           row-major [K][N] as the reference stores them
+//   KV cache               [layer][batch][kv_head][max_len][head_dim], keys after RoPE, head_dim contiguous
+//   GEMM outputs           fp32 split-K partials [split][rows][N]; the consumer kernel adds them up in split
+//                          order together with the bias, so results do not depend on scheduling.
+#pragma once
+
+#include "tship_internal.h"
+
+namespace tship {
+
+__device__ __forceinline__ float act_apply(int act, float w) {
+    // TensorSharp/TensorApplyCPU.cs:1747-1801; act 3 is the reference's "SwiGLU" gate: no activation
+    // (Seq2SeqSharp/Layers/PositionwiseFeedForward.cs:100-116)
+    if (act == 0) return w < 0.0f ? 0.0f : w;
+    if (act == 1 || act == 4) return w / (1.0f + __expf(-w));
+    if (act == 2) return w < 0.0f ? 0.01f * w : w;
+    return w;
+}
+
+template <typename T> __device__ __forceinline__ float to_f32(T v) { return (float)v; }
+template <typename T> __device__ __forceinline__ T from_f32(float v) { return (T)v; }
+
+// ------------------------------------------------------------------------------------------------
+// weight packing (runs once per tensor at load time)
+// ------------------------------------------------------------------------------------------------
+enum { PACK_PLAIN = 0, PACK_INTERLEAVE16 = 1 };
+
+// src fp32 row-major [K][N] (ld) -> dst P32.  One thread per (source column, group of 8 k).
+// PACK_PLAIN: destination column = n_off + n.  PACK_INTERLEAVE16: destination column =
+// (n/16)*32 + n_off + n%16 with n_off in {0,16}: column tile j then holds 16 columns of the first matrix
+// followed by the same 16 columns of the second, so a gated FFN epilogue finds both factors in one tile.
+__global__ void pack_w_kernel(const float* __restrict__ src, long ld, int K, int N, half_t* __restrict__ dst, int KT,
+                              int mode, int n_off) {
+    long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    long total = (long)N * KT * 2;
+    if (idx >= total) return;
+    int n = (int)(idx % N);
+    int kg = (int)(idx / N);
+    int nd = mode == PACK_PLAIN ? n_off + n : (n / 16) * 32 + n_off + (n % 16);
+    int nt = nd / 32, lane = (nd % 32) + 32 * (kg & 1), kt = kg >> 1;
+    half8 v;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        int k = kg * 8 + j;
+        v[j] = (half_t)(k < K ? src[(long)k * ld + n] : 0.0f);
+    }
+    *(half8*)(dst + (((long)nt * KT + kt) * 64 + lane) * 8) = v;
+}
+
+// fp32 -> T copy of a [rows][cols] matrix into a wider destination at a column offset
+template <typename T>
+__global__ void copy_cols_kernel(const float* __restrict__ src, long ld_src, long rows, long cols, T* __restrict__ dst, long ld_dst,
+                                 long col_off) {
+    long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= rows * cols) return;
+    long r = idx / cols, c = idx % cols;
+    dst[r * ld_dst + col_off + c] = (T)src[r * ld_src + c];
+}
+
+// ------------------------------------------------------------------------------------------------
+// decode GEMM, fp16 weights: Y[b][n] = sum_k X[b][k] * W[k][n] for <= 128 rows, MFMA 32x32x16.
+// A block owns one 32-column tile and one k-split; its 4 wavefronts split the k range again and are
+// reduced through LDS.  HBM-bound: every weight byte is read exactly once with 16-byte loads.
+// ------------------------------------------------------------------------------------------------
+enum { EPI_PARTIAL = 0, EPI_F32_BIAS = 1, EPI_ACT16 = 2 };
+
+struct SkinnyArgs {
+    const half_t* W; int KT; int NT;
+    const half_t* X; int ldx;
+    int KS;
+    float* out; int ld_out; long split_stride;
+    const float* bias; const float* bias2;
+    half_t* out16; int ld16;
+    int act; int gated; int n_valid; int rows_valid;
+    // optional batch of independent problems (MoE experts) on blockIdx.y: weights from a pointer table,
+    // activations / outputs at a fixed stride, row counts read on the device
+    const half_t* const* Wtab; long x_estride; long out_estride; long out16_estride; const int* rows_tab;
+};
+
+template <int BT, int EPI>
+__global__ __launch_bounds__(256) void skinny_gemm_f16_kernel(SkinnyArgs a) {
+    constexpr int U = 8;
+    __shared__ float red[4][BT * 32][33];
+    if (a.Wtab) {
+        const int e = blockIdx.y;
+        a.rows_valid = a.rows_tab[e];
+        if (a.rows_valid == 0) return;
+        a.W = a.Wtab[e]; a.X += e * a.x_estride;
+        if (a.out) a.out += e * a.out_estride;
+        if (a.out16) a.out16 += e * a.out16_estride;
+    }
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    const int nt = blockIdx.x / a.KS, ks = blockIdx.x % a.KS;
+    const int per = (a.KT + a.KS - 1) / a.KS;
+    const int k0 = ks * per, k1 = min(a.KT, k0 + per);
+    const int pw = (max(k1 - k0, 0) + 3) / 4;
+    const int wk0 = k0 + w * pw, wk1 = min(k1, wk0 + pw);
+
+    floatx16 acc[BT];
+#pragma unroll
+    for (int bt = 0; bt < BT; ++bt)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[bt][v] = 0.0f;
+
+    const half_t* wp = a.W + ((long)nt * a.KT * 64 + lane) * 8;
+    const half_t* xp = a.X + (long)(lane & 31) * a.ldx + (lane >> 5) * 8;
+    for (int kt = wk0; kt < wk1; kt += U) {
+        half8 wf[U];
+        half8 xf[U][BT];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            if (kt + u < wk1) {
+                wf[u] = *(const half8*)(wp + (long)(kt + u) * 512);
+#pragma unroll
+                for (int bt = 0; bt < BT; ++bt) xf[u][bt] = *(const half8*)(xp + (long)bt * 32 * a.ldx + (kt + u) * 16);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            if (kt + u < wk1) {
+#pragma unroll
+                for (int bt = 0; bt < BT; ++bt) acc[bt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf[u], xf[u][bt], acc[bt], 0, 0, 0);
+            }
+        }
+    }
+    // accumulator lane l, register v holds column nt*32 + 8*(v/4) + 4*(l/32) + v%4 of batch row bt*32 + l%32
+#pragma unroll
+    for (int bt = 0; bt < BT; ++bt)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) red[w][bt * 32 + (lane & 31)][8 * (v / 4) + 4 * (lane >> 5) + (v % 4)] = acc[bt][v];
+    __syncthreads();
+
+    const int n = threadIdx.x & 31, bq = threadIdx.x >> 5;
+    for (int b = bq; b < BT * 32; b += 8) {
+        if (b >= a.rows_valid) break;
+        float s = (red[0][b][n] + red[1][b][n]) + (red[2][b][n] + red[3][b][n]);
+        if (EPI == EPI_PARTIAL) {
+            a.out[ks * a.split_stride + (long)b * a.ld_out + nt * 32 + n] = s;
+        } else if (EPI == EPI_F32_BIAS) {
+            int col = nt * 32 + n;
+            if (col < a.n_valid) a.out[(long)b * a.ld_out + col] = s + a.bias[col];
+        } else {
+            if (a.gated) {
+                if (n < 16) {
+                    float c = (red[0][b][n + 16] + red[1][b][n + 16]) + (red[2][b][n + 16] + red[3][b][n + 16]);
+                    int f = nt * 16 + n;
+                    if (f < a.n_valid) a.out16[(long)b * a.ld16 + f] = (half_t)(act_apply(a.act, s + a.bias[f]) * (c + a.bias2[f]));
+                }
+            } else {
+                int f = nt * 32 + n;
+                if (f < a.n_valid) a.out16[(long)b * a.ld16 + f] = (half_t)act_apply(a.act, s + a.bias[f]);
+            }
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// prefill GEMM, fp16 weights: many rows.  Block tile 128 rows x 128 columns; each wavefront owns one
+// 32-column weight tile (streamed from HBM/L2 as packed fragments) and 4 row tiles.  MFMA-bound.
+// ------------------------------------------------------------------------------------------------
+enum { BEPI_F32_BIAS = 0, BEPI_RESID = 1, BEPI_ACT16 = 2 };
+
+struct BigArgs {
+    const half_t* W; int KT; int NT;
+    const half_t* X; int ldx; int R;
+    float* out; int ld_out;
+    const float* bias; const float* bias2;
+    half_t* out16; int ld16;
+    int act; int gated; int n_valid;
+};
+
+template <int EPI>
+__global__ __launch_bounds__(256) void big_gemm_f16_kernel(BigArgs a) {
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    const int nt = blockIdx.x * 4 + w;
+    if (nt >= a.NT) return;
+    const int row0 = blockIdx.y * 128;
+    floatx16 acc[4];
+#pragma unroll
+    for (int rt = 0; rt < 4; ++rt)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[rt][v] = 0.0f;
+    const half_t* wp = a.W + ((long)nt * a.KT * 64 + lane) * 8;
+    const half_t* xp = a.X + (long)(row0 + (lane & 31)) * a.ldx + (lane >> 5) * 8;
+#pragma unroll 2
+    for (int kt = 0; kt < a.KT; ++kt) {
+        half8 wf = *(const half8*)(wp + (long)kt * 512);
+        half8 xf[4];
+#pragma unroll
+        for (int rt = 0; rt < 4; ++rt) xf[rt] = *(const half8*)(xp + (long)rt * 32 * a.ldx + kt * 16);
+#pragma unroll
+        for (int rt = 0; rt < 4; ++rt) acc[rt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf, xf[rt], acc[rt], 0, 0, 0);
+    }
+#pragma unroll
+    for (int rt = 0; rt < 4; ++rt) {
+        const int row = row0 + rt * 32 + (lane & 31);
+        if (row >= a.R) continue;
+        if (EPI == BEPI_ACT16 && a.gated) {
+#pragma unroll
+            for (int v = 0; v < 8; ++v) {
+                int nl = 8 * (v / 4) + 4 * (lane >> 5) + (v % 4);
+                int f = nt * 16 + nl;
+                if (f < a.n_valid)
+                    a.out16[(long)row * a.ld16 + f] = (half_t)(act_apply(a.act, acc[rt][v] + a.bias[f]) * (acc[rt][v + 8] + a.bias2[f]));
+            }
+        } else {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                int col = nt * 32 + 8 * (v / 4) + 4 * (lane >> 5) + (v % 4);
+                if (col >= a.n_valid) continue;
+                float s = acc[rt][v] + a.bias[col];
+                if (EPI == BEPI_F32_BIAS) a.out[(long)row * a.ld_out + col] = s;
+                else if (EPI == BEPI_RESID) a.out[(long)row * a.ld_out + col] = s + a.out[(long)row * a.ld_out + col];
+                else a.out16[(long)row * a.ld16 + col] = (half_t)act_apply(a.act, s);
+            }
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// fp32 GEMM (fp32 models: prefill and decode): C[ks][M][N] = A[M][K-range ks] * B[K-range][N], 64x64 tile,
+// k accumulated sequentially inside a split.
+// ------------------------------------------------------------------------------------------------
+struct F32GemmArgs {
+    const float* A; long lda; const float* B; long ldb; float* C; long ldc; long split_stride;
+    int M, N, K, KS;
+    const float* bias;     // optional, added when the result is final (KS == 1)
+};
+
+__global__ __launch_bounds__(256) void gemm_f32_kernel(F32GemmArgs a) {
+    __shared__ float As[16][64 + 4];
+    __shared__ float Bs[16][64 + 4];
+    const int t = threadIdx.x, tx = t & 15, ty = t >> 4;
+    const int col0 = blockIdx.x * 64, row0 = blockIdx.y * 64, ks = blockIdx.z;
+    const int kper = (int)round_up(ceil_div(a.K, a.KS), 16);
+    const int kb = ks * kper, ke = min(a.K, kb + kper);
+    float acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = 0.0f;
+    const int am = t >> 2, ak = (t & 3) * 4;
+    const int bk = t >> 4, bn = (t & 15) * 4;
+    for (int k0 = kb; k0 < ke; k0 += 16) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            int r = row0 + am, k = k0 + ak + j;
+            As[ak + j][am] = (r < a.M && k < ke) ? a.A[(long)r * a.lda + k] : 0.0f;
+            int kk = k0 + bk, c = col0 + bn + j;
+            Bs[bk][bn + j] = (kk < ke && c < a.N) ? a.B[(long)kk * a.ldb + c] : 0.0f;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int k = 0; k < 16; ++k) {
+            float av[4], bv[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) { av[i] = As[k][ty * 4 + i]; bv[i] = Bs[k][tx * 4 + i]; }
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(av[i], bv[j], acc[i][j]);
+        }
+        __syncthreads();
+    }
+    float* C = a.C + ks * a.split_stride;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        int r = row0 + ty * 4 + i;
+        if (r >= a.M) continue;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            int c = col0 + tx * 4 + j;
+            if (c < a.N) C[(long)r * a.ldc + c] = a.bias ? acc[i][j] + a.bias[c] : acc[i][j];
+        }
+    }
+}
+
+// FFN activation for paths whose GEMM has no fused epilogue: out[r][f] = act(sum part[.][r][f] + b1[f])
+// (* (sum part[.][r][F+f] + b3[f]) when gated)
+template <typename AT>
+__global__ void ffn_act_kernel(const float* __restrict__ part, int KS, long split_stride, long ldp, const float* __restrict__ b1,
+                               const float* __restrict__ b3, int F, int gated, int act, AT* __restrict__ out, long ld_out, long R) {
+    long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= R * F) return;
+    long r = idx / F; int f = (int)(idx % F);
+    float s = 0.0f;
+    for (int k = 0; k < KS; ++k) s += part[k * split_stride + r * ldp + f];
+    s = act_apply(act, s + b1[f]);
+    if (gated) {
+        float c = 0.0f;
+        for (int k = 0; k < KS; ++k) c += part[k * split_stride + r * ldp + F + f];
+        s *= (c + b3[f]);
+    }
+    out[r * ld_out + f] = (AT)s;
+}
+
+// ------------------------------------------------------------------------------------------------
+// residual update + normalisation, one block per row.
+//   source   : embedding gather x = E[id] * scale  (TensorUtils.CreateTokensEmbeddings, Utils/TensorUtils.cs:147-156)
+//              or x += (sum of split-K partials + bias)   (g.Affine then graph.Add with the layer input)
+//              or x as it is
+//   then RMSNorm (TensorApplyCPU.cs:1451-1496) or LayerNorm (:1360-1447) -> xn in the activation type.
+// ------------------------------------------------------------------------------------------------
+struct ResidNormArgs {
+    float* x; long ldx; int h;
+    const int* ids; const void* emb; int emb_f16; float emb_scale;
+    const float* part; int KS; long split_stride; long ld_part; const float* bias;
+    const float* gamma; const float* beta; float eps; int norm_type;
+    void* xn; long ldxn;
+    const int* row_map;     // optional: block r works on row row_map[r] of x and writes row r of xn
+    int* advance_pos;       // optional: block 0 increments this device counter (end of a decode step)
+};
+
+template <typename AT>
+__global__ __launch_bounds__(256) void resid_norm_kernel(ResidNormArgs a) {
+    constexpr int NPT = 32;   // hidden <= 8192
+    __shared__ float sred[4];
+    const int r = blockIdx.x, t = threadIdx.x;
+    const long xr = a.row_map ? a.row_map[r] : r;
+    float v[NPT];
+    float sum = 0.0f, sq = 0.0f;
+    long erow = a.ids ? (long)a.ids[r] : 0;
+#pragma unroll
+    for (int i = 0; i < NPT; ++i) {
+        int c = t + i * 256;
+        float val = 0.0f;
+        if (c < a.h) {
+            if (a.ids) {
+                float e = a.emb_f16 ? (float)((const half_t*)a.emb)[erow * a.h + c] : ((const float*)a.emb)[erow * a.h + c];
+                val = e * a.emb_scale;
+            } else {
+                val = a.x[xr * a.ldx + c];
+            }
+            if (a.part) {
+                float s = a.part[(long)r * a.ld_part + c];
+                for (int k = 1; k < a.KS; ++k) s += a.part[k * a.split_stride + (long)r * a.ld_part + c];
+                val = (s + a.bias[c]) + val;
+            }
+            if (a.ids || a.part) a.x[xr * a.ldx + c] = val;
+            sum += val; sq += val * val;
+        }
+        v[i] = val;
+    }
+    if (a.advance_pos && r == 0 && t == 0) *a.advance_pos += 1;
+    if (!a.xn) return;
+    AT* out = (AT*)a.xn + (long)r * a.ldxn;
+    if (a.norm_type == 0) {
+        float tot = block_sum_256(sq, sred);
+        float rms = sqrtf(tot / (float)a.h + a.eps);
+#pragma unroll
+        for (int i = 0; i < NPT; ++i) {
+            int c = t + i * 256;
+            if (c < a.h) {
+                float y = a.gamma[c] * (v[i] / rms);
+                if (a.beta) y += a.beta[c];
+                out[c] = (AT)y;
+            }
+        }
+    } else {
+        float mean = block_sum_256(sum, sred) / (float)a.h;
+        float d2 = 0.0f;
+#pragma unroll
+        for (int i = 0; i < NPT; ++i) {
+            int c = t + i * 256;
+            if (c < a.h) { float d = v[i] - mean; d2 += d * d; }
+        }
+        float sigma = sqrtf(a.eps + block_sum_256(d2, sred) / (float)a.h);
+#pragma unroll
+        for (int i = 0; i < NPT; ++i) {
+            int c = t + i * 256;
+            if (c < a.h) {
+                float y = a.gamma[c] * ((v[i] - mean) / sigma);
+                if (a.beta) y += a.beta[c];
+                out[c] = (AT)y;
+            }
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// attention
+// ------------------------------------------------------------------------------------------------
+struct AttnArgs {
+    // q/k/v source: fp32 [KS][rows][ldq] partial sums + bias; columns: H*D queries, then Hkv*D keys, then Hkv*D values
+    const float* qkv; int KS; long split_stride; long ldq; const float* bias;
+    int H, Hkv;
+    void* kcache; void* vcache; long max_len;      // [batch][Hkv][max_len][D]
+    const float* rope_cos; const float* rope_sin;  // [max_len][D/2]; null = no rotary embedding
+    const int* d_pos;                              // decode: number of cached positions, read on the device
+    int pos0;                                      // prefill: cache offset of the first query row
+    int Tq;                                        // prefill: query rows per sequence
+    void* out; long ld_out;                        // [rows][H*D] in the activation type
+    float scale;
+};
+
+// rotary embedding of one (even, odd) pair, two roundings per output like the reference's C# expression
+// (TensorSharp/TensorApplyCPU.cs:1166-1173)
+__device__ __forceinline__ void rope_pair(float x0, float x1, float c, float s, float& y0, float& y1) {
+#pragma clang fp contract(off)
+    y0 = x0 * c - x1 * s;
+    y1 = x1 * c + x0 * s;
+}
+
+// Single-query attention of G query heads that share one KV head over T cached positions.
+// Lanes are grouped LPR to a cache row (16-byte loads, head_dim contiguous); every lane group keeps its own
+// online-softmax state over the rows it visits; the groups of all 4 wavefronts are merged at the end.
+// sQ: LDS [G][D] queries, already rotated and scaled.  Result (fp32) is written to sOut [G][D] in LDS.
+template <typename CT, int D, int G>
+__device__ __forceinline__ void attn_core(const float* sQ, const CT* Kb, const CT* Vb, int T, float* sM,
+                                          float* sL, float* sAcc, float* sOut) {
+    constexpr int EPL = 16 / (int)sizeof(CT);
+    constexpr int LPR = D / EPL;
+    constexpr int RPW = 64 / LPR;
+    constexpr int NW = 4;
+    constexpr int NG = NW * RPW;
+    constexpr int UR = 4;
+    typedef CT vec_t __attribute__((ext_vector_type(EPL)));
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int sub = lane % LPR, rg = lane / LPR;
+
+    float q[G][EPL];
+#pragma unroll
+    for (int g = 0; g < G; ++g)
+#pragma unroll
+        for (int e = 0; e < EPL; ++e) q[g][e] = sQ[g * D + sub * EPL + e];
+    float m[G], l[G], acc[G][EPL];
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+        m[g] = -INFINITY; l[g] = 0.0f;
+#pragma unroll
+        for (int e = 0; e < EPL; ++e) acc[g][e] = 0.0f;
+    }
+    for (int base = wave * RPW; base < T; base += NW * RPW * UR) {
+        vec_t kv[UR], vv[UR];
+        bool ok[UR];
+#pragma unroll
+        for (int u = 0; u < UR; ++u) {
+            int t = base + u * NW * RPW + rg;
+            ok[u] = t < T;
+            if (ok[u]) {
+                kv[u] = *(const vec_t*)(Kb + (long)t * D + sub * EPL);
+                vv[u] = *(const vec_t*)(Vb + (long)t * D + sub * EPL);
+            } else {
+#pragma unroll
+                for (int e = 0; e < EPL; ++e) { kv[u][e] = (CT)0.0f; vv[u][e] = (CT)0.0f; }
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < UR; ++u) {
+            float s[G];
+#pragma unroll
+            for (int g = 0; g < G; ++g) {
+                float d = 0.0f;
+#pragma unroll
+                for (int e = 0; e < EPL; ++e) d = fmaf(q[g][e], (float)kv[u][e], d);
+#pragma unroll
+                for (int o = LPR / 2; o > 0; o >>= 1) d += __shfl_xor(d, o, 64);
+                s[g] = d;
+            }
+            if (ok[u]) {
+#pragma unroll
+                for (int g = 0; g < G; ++g) {
+                    float mn = fmaxf(m[g], s[g]);
+                    float corr = __expf(m[g] - mn);
+                    float p = __expf(s[g] - mn);
+                    l[g] = l[g] * corr + p;
+#pragma unroll
+                    for (int e = 0; e < EPL; ++e) acc[g][e] = acc[g][e] * corr + p * (float)vv[u][e];
+                    m[g] = mn;
+                }
+            }
+        }
+    }
+    const int gi = wave * RPW + rg;
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+        if (sub == 0) { sM[gi * G + g] = m[g]; sL[gi * G + g] = l[g]; }
+#pragma unroll
+        for (int e = 0; e < EPL; ++e) sAcc[(gi * G + g) * D + sub * EPL + e] = acc[g][e];
+    }
+    __syncthreads();
+    for (int idx = threadIdx.x; idx < G * D; idx += 256) {
+        int g = idx / D, d = idx % D;
+        float M = -INFINITY;
+        for (int i = 0; i < NG; ++i) M = fmaxf(M, sM[i * G + g]);
+        float L = 0.0f, O = 0.0f;
+        for (int i = 0; i < NG; ++i) {
+            float wgt = __expf(sM[i * G + g] - M);    // groups that saw no row have m = -inf -> weight 0
+            L += sL[i * G + g] * wgt;
+            O += sAcc[(i * G + g) * D + d] * wgt;
+        }
+        sOut[idx] = O / L;
+    }
+    __syncthreads();
+}
+
+template <typename CT, int D, int G>
+struct AttnSmem {
+    static constexpr int EPL = 16 / (int)sizeof(CT);
+    static constexpr int NG = 4 * (64 / (D / EPL));
+    float in[(G + 2) * D];
+    float q[G * D];
+    float m[NG * G];
+    float l[NG * G];
+    float acc[NG * G * D];
+    float out[G * D];
+};
+
+// decode step: grid (Hkv, batch).  Sums the QKV split-K partials, applies RoPE at position pos, appends the new
+// key/value to the cache in place, then attends over pos+1 positions.
+// Replaces: AsContiguous head split, RoPE, GQA Expand, Concate(cache), MulBatch, Softmax, MulBatch, transpose
+// (Seq2SeqSharp/Layers/GroupQueryAttention.cs:121-224, Layers/MultiHeadAttention.cs:133-230).
+template <typename CT, typename AT, int D, int G>
+__global__ __launch_bounds__(256) void attn_decode_kernel(AttnArgs a) {
+    __shared__ AttnSmem<CT, D, G> sm;
+    const int kvh = blockIdx.x, b = blockIdx.y, t = threadIdx.x;
+    const int pos = *a.d_pos;
+    const int HD = a.H * D, GD = a.Hkv * D;
+    for (int idx = t; idx < (G + 2) * D; idx += 256) {
+        int col;
+        if (idx < G * D) col = kvh * G * D + idx;
+        else if (idx < (G + 1) * D) col = HD + kvh * D + (idx - G * D);
+        else col = HD + GD + kvh * D + (idx - (G + 1) * D);
+        float s = a.qkv[(long)b * a.ldq + col];
+        for (int k = 1; k < a.KS; ++k) s += a.qkv[k * a.split_stride + (long)b * a.ldq + col];
+        sm.in[idx] = s + a.bias[col];
+    }
+    __syncthreads();
+    CT* Kb = (CT*)a.kcache + ((long)b * a.Hkv + kvh) * a.max_len * D;
+    CT* Vb = (CT*)a.vcache + ((long)b * a.Hkv + kvh) * a.max_len * D;
+    for (int p = t; p < (G + 1) * D / 2; p += 256) {
+        int vec = p / (D / 2), i = p % (D / 2);
+        float x0 = sm.in[vec * D + 2 * i], x1 = sm.in[vec * D + 2 * i + 1], y0 = x0, y1 = x1;
+        if (a.rope_cos) rope_pair(x0, x1, a.rope_cos[(long)pos * (D / 2) + i], a.rope_sin[(long)pos * (D / 2) + i], y0, y1);
+        if (vec < G) { sm.q[vec * D + 2 * i] = a.scale * y0; sm.q[vec * D + 2 * i + 1] = a.scale * y1; }
+        else { Kb[(long)pos * D + 2 * i] = (CT)y0; Kb[(long)pos * D + 2 * i + 1] = (CT)y1; }
+    }
+    for (int d = t; d < D; d += 256) Vb[(long)pos * D + d] = (CT)sm.in[(G + 1) * D + d];
+    __threadfence_block();
+    __syncthreads();
+    attn_core<CT, D, G>(sm.q, Kb, Vb, pos + 1, sm.m, sm.l, sm.acc, sm.out);
+    AT* out = (AT*)a.out + (long)b * a.ld_out + kvh * G * D;
+    for (int idx = t; idx < G * D; idx += 256) out[idx] = (AT)sm.out[idx];
+}
+
+// prefill, step 1: grid (Tq, batch).  Rotates the keys of every position and writes keys and values into the cache.
+template <typename CT, int D>
+__global__ __launch_bounds__(256) void kv_write_kernel(AttnArgs a) {
+    const int tq = blockIdx.x, b = blockIdx.y, t = threadIdx.x;
+    const long row = (long)b * a.Tq + tq;
+    const int pos = a.pos0 + tq;
+    const int HD = a.H * D, GD = a.Hkv * D;
+    CT* Kb = (CT*)a.kcache + (long)b * a.Hkv * a.max_len * D;
+    CT* Vb = (CT*)a.vcache + (long)b * a.Hkv * a.max_len * D;
+    for (int p = t; p < GD / 2; p += 256) {
+        int kvh = p / (D / 2), i = p % (D / 2);
+        int col = HD + kvh * D + 2 * i;
+        float x0 = a.qkv[row * a.ldq + col] + a.bias[col], x1 = a.qkv[row * a.ldq + col + 1] + a.bias[col + 1], y0 = x0, y1 = x1;
+        if (a.rope_cos) rope_pair(x0, x1, a.rope_cos[(long)pos * (D / 2) + i], a.rope_sin[(long)pos * (D / 2) + i], y0, y1);
+        CT* dst = Kb + ((long)kvh * a.max_len + pos) * D + 2 * i;
+        dst[0] = (CT)y0; dst[1] = (CT)y1;
+    }
+    for (int p = t; p < GD; p += 256) {
+        int kvh = p / D, d = p % D;
+        int col = HD + GD + p;
+        Vb[((long)kvh * a.max_len + pos) * D + d] = (CT)(a.qkv[row * a.ldq + col] + a.bias[col]);
+    }
+}
+
+// prefill, step 2: grid (Tq, Hkv, batch).  Causal attention of query row tq over cache positions 0..pos0+tq.
+// The reference adds -30000 to masked scores (TensorApplyCPU.cs:1016-1036, Decoder.cs:685-686); exp(-30000 - max)
+// is exactly 0 in fp32, so leaving masked positions out gives the same sums.
+template <typename CT, typename AT, int D, int G>
+__global__ __launch_bounds__(256) void attn_prefill_kernel(AttnArgs a) {
+    __shared__ AttnSmem<CT, D, G> sm;
+    const int tq = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z, t = threadIdx.x;
+    const long row = (long)b * a.Tq + tq;
+    const int pos = a.pos0 + tq;
+    for (int p = t; p < G * D / 2; p += 256) {
+        int vec = p / (D / 2), i = p % (D / 2);
+        int col = (kvh * G + vec) * D + 2 * i;
+        float x0 = a.qkv[row * a.ldq + col] + a.bias[col], x1 = a.qkv[row * a.ldq + col + 1] + a.bias[col + 1], y0 = x0, y1 = x1;
+        if (a.rope_cos) rope_pair(x0, x1, a.rope_cos[(long)pos * (D / 2) + i], a.rope_sin[(long)pos * (D / 2) + i], y0, y1);
+        sm.q[vec * D + 2 * i] = a.scale * y0; sm.q[vec * D + 2 * i + 1] = a.scale * y1;
+    }
+    __syncthreads();
+    const CT* Kb = (const CT*)a.kcache + ((long)b * a.Hkv + kvh) * a.max_len * D;
+    const CT* Vb = (const CT*)a.vcache + ((long)b * a.Hkv + kvh) * a.max_len * D;
+    attn_core<CT, D, G>(sm.q, Kb, Vb, pos + 1, sm.m, sm.l, sm.acc, sm.out);
+    AT* out = (AT*)a.out + row * a.ld_out + kvh * G * D;
+    for (int idx = t; idx < G * D; idx += 256) out[idx] = (AT)sm.out[idx];
+}
+
+// ------------------------------------------------------------------------------------------------
+// sampling on the device
+// ------------------------------------------------------------------------------------------------
+// Greedy: argmax over a row of logits, lowest index among equal maxima (TensorApplyCPU.cs:339-360 applied to the
+// softmax output; softmax is monotone, so the winner is the same up to ties created by rounding of the division).
+__global__ __launch_bounds__(256) void greedy_kernel(const float* __restrict__ logits, long ld, int V, int* __restrict__ next_ids,
+                                                     int* __restrict__ gen_out) {
+    __shared__ float sv[4];
+    __shared__ int si[4];
+    const int b = blockIdx.x, t = threadIdx.x;
+    const float* row = logits + (long)b * ld;
+    float best = -INFINITY; int bi = 0x7fffffff;
+    for (int i = t; i < V; i += 256) {
+        float v = row[i];
+        if (v > best || (v == best && i < bi)) { best = v; bi = i; }
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        float ov = __shfl_xor(best, o, 64); int oi = __shfl_xor(bi, o, 64);
+        if (ov > best || (ov == best && oi < bi)) { best = ov; bi = oi; }
+    }
+    if ((t & 63) == 0) { sv[t >> 6] = best; si[t >> 6] = bi; }
+    __syncthreads();
+    if (t == 0) {
+        for (int w = 1; w < 4; ++w) if (sv[w] > best || (sv[w] == best && si[w] < bi)) { best = sv[w]; bi = si[w]; }
+        if (bi == 0x7fffffff) bi = 0;   // a row of NaNs: the reference's scan never moves off index 0
+        next_ids[b] = bi;
+        if (gen_out) gen_out[b] = bi;
+    }
+}
+
+}  // namespace tship

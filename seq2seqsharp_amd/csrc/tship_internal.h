@@ -1,0 +1,88 @@
+// Internal helpers shared by the translation units of libtship.so: per-thread error string,
+// boundary macros that keep C++ exceptions inside the library, the library stream, small device helpers.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+#include <hip/hip_ext.h>
+
+#include <cstdint>
+#include <cstdio>
+#include <stdexcept>
+#include <string>
+
+#include "../../include/tship.h"
+
+namespace tship {
+
+void set_last_error(const std::string& msg);
+
+struct Error : std::runtime_error {
+    explicit Error(const std::string& m) : std::runtime_error(m) {}
+};
+
+#define TSHIP_CHECK_HIP(expr)                                                                         \
+    do {                                                                                              \
+        hipError_t _e = (expr);                                                                       \
+        if (_e != hipSuccess)                                                                         \
+            throw ::tship::Error(std::string(#expr) + " failed: " + hipGetErrorString(_e));           \
+    } while (0)
+
+#define TSHIP_REQUIRE(cond, msg)                                                                      \
+    do {                                                                                              \
+        if (!(cond)) throw ::tship::Error(std::string(msg));                                          \
+    } while (0)
+
+// Every exported function is wrapped: 1 on success, 0 on failure with the message stored per thread.
+#define TSHIP_BEGIN try {
+#define TSHIP_END                                                                                     \
+    return 1;                                                                                         \
+    }                                                                                                 \
+    catch (const std::exception& e) {                                                                 \
+        ::tship::set_last_error(e.what());                                                            \
+        return 0;                                                                                     \
+    }                                                                                                 \
+    catch (...) {                                                                                     \
+        ::tship::set_last_error("unknown native exception");                                          \
+        return 0;                                                                                     \
+    }
+
+// The library's ordered stream (created by TSHip_Init, default priority).
+hipStream_t stream();
+void ensure_init();
+int n_compute_units();
+
+typedef _Float16 half_t;
+typedef half_t half8 __attribute__((ext_vector_type(8)));
+typedef half_t half4 __attribute__((ext_vector_type(4)));
+typedef half_t half2v __attribute__((ext_vector_type(2)));
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+__host__ __device__ static inline long round_up(long v, long m) { return (v + m - 1) / m * m; }
+__host__ __device__ static inline long ceil_div(long a, long b) { return (a + b - 1) / b; }
+
+// ------------------------------------------------------------------------------------------------
+// reductions
+// ------------------------------------------------------------------------------------------------
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+    return v;
+}
+// 256-thread block sum; s is LDS scratch of 4 floats; every thread gets the result
+__device__ __forceinline__ float block_sum_256(float v, float* s) {
+    v = wave_sum(v);
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) s[threadIdx.x >> 6] = v;
+    __syncthreads();
+    return (s[0] + s[1]) + (s[2] + s[3]);
+}
+
+
+}  // namespace tship

@@ -1,0 +1,150 @@
+// MoE feed-forward kernels (decode-sized row counts).
+// MoEFeedForward.Process, Seq2SeqSharp/Layers/MoEFeedForward.cs:76-181: LayerNorm -> router Affine -> + (-65000)
+// -> Softmax -> TopK -> per-expert token lists (ascending token order) -> gather -> expert MLP -> scale by the
+// expert's softmax probability -> scatter-add in expert-major order -> residual.
+//
+// The routing decision is index work, so the arithmetic that feeds it is done in the reference's own operation
+// order: LayerNorm sums in 8-lane partial sums (TensorApplyCPU.cs:1381-1409), the router dot product serially
+// over k with separately rounded product and sum (SGEMM.cs:482-549), exp evaluated in double
+// (TensorApplyCPU.cs:1246), TopK by the reference's insertion rule (TensorApplyCPU.cs:1099-1146).
+#pragma once
+
+#include "tship_internal.h"
+
+namespace tship {
+
+struct MoeRouterArgs {
+    float* x; long ldx; int h;
+    const float* part; int KS; long split_stride; long ld_part; const float* bias;   // pending attention output
+    const float* gamma; const float* beta; float eps;
+    const float* router; const float* router_b; int E; int k;
+    float* xn32; float* probs; float* top_val; float* top_idx;
+};
+
+__device__ __forceinline__ float tree8(float v) {
+    // ((l0+l1)+(l2+l3))+((l4+l5)+(l6+l7)) across 8 adjacent lanes
+    v += __shfl_xor(v, 1, 64);
+    v += __shfl_xor(v, 2, 64);
+    v += __shfl_xor(v, 4, 64);
+    return v;
+}
+
+__global__ __launch_bounds__(64) void moe_router_kernel(MoeRouterArgs a) {
+#pragma clang fp contract(off)
+    __shared__ float sx[4096];
+    __shared__ float sxn[4096];
+    __shared__ float sr[64];
+    __shared__ float s_stat[2];
+    const int r = blockIdx.x, t = threadIdx.x, h = a.h;
+    for (int c = t; c < h; c += 64) {
+        float v = a.x[(long)r * a.ldx + c];
+        if (a.part) {
+            float s = a.part[(long)r * a.ld_part + c];
+            for (int k = 1; k < a.KS; ++k) s += a.part[k * a.split_stride + (long)r * a.ld_part + c];
+            v = (s + a.bias[c]) + v;
+            a.x[(long)r * a.ldx + c] = v;
+        }
+        sx[c] = v;
+    }
+    __syncthreads();
+    if (t < 8) {
+        float lane = 0.0f;
+        int i = 0;
+        for (; i < h - 8; i += 8) lane += sx[i + t];
+        float sum = tree8(lane);
+        for (; i < h; ++i) sum += sx[i];
+        float mean = sum / (float)h;
+        float sq = 0.0f;
+        for (i = 0; i < h - 8; i += 8) {
+            float d = sx[i + t] - mean;
+            sq += tree8(d * d);
+        }
+        for (; i < h; ++i) { float d = sx[i] - mean; sq += d * d; }
+        float sigma = sqrtf(a.eps + sq / (float)h);
+        if (t == 0) { s_stat[0] = mean; s_stat[1] = sigma; }
+    }
+    __syncthreads();
+    const float mean = s_stat[0], sigma = s_stat[1];
+    for (int c = t; c < h; c += 64) {
+        float y = a.gamma[c] * ((sx[c] - mean) / sigma);
+        y += a.beta[c];
+        sxn[c] = y;
+        a.xn32[(long)r * h + c] = y;
+    }
+    __syncthreads();
+    if (t < a.E) {
+        float acc = a.router_b[t];
+        for (int l = 0; l < h; ++l) {
+            float xv = sxn[l];
+            if (xv != 0.0f) acc += xv * a.router[(long)l * a.E + t];
+        }
+        sr[t] = acc + (-65000.0f);
+    }
+    __syncthreads();
+    if (t == 0) {
+        const int E = a.E, k = a.k;
+        float mx = sr[0];
+        for (int e = 1; e < E; ++e) mx = fmaxf(mx, sr[e]);
+        float sum = 0.0f;
+        for (int e = 0; e < E; ++e) { float ex = (float)exp((double)(sr[e] - mx)); sr[e] = ex; sum += ex; }
+        float* pr = a.probs + (long)r * E;
+        for (int e = 0; e < E; ++e) { sr[e] = sr[e] / sum; pr[e] = sr[e]; }
+        float* ov = a.top_val + (long)r * k; float* oi = a.top_idx + (long)r * k;
+        for (int i = 0; i < k; ++i) { ov[i] = -1.70141e+38f; oi[i] = -1.70141e+38f; }
+        for (int e = 0; e < E; ++e) {
+            float data = sr[e];
+            if (data < ov[k - 1]) continue;
+            int j = k - 2;
+            for (; j >= 0; --j) {
+                if (data > ov[j]) { ov[j + 1] = ov[j]; oi[j + 1] = oi[j]; }
+                else { ov[j + 1] = data; oi[j + 1] = (float)e; break; }
+            }
+            if (j < 0) { ov[0] = data; oi[0] = (float)e; }
+        }
+    }
+}
+
+// per-expert token lists in ascending token order (MoEFeedForward.cs:92-105); slot[i*k+j] = position of token i in
+// the list of its j-th expert
+__global__ void moe_lists_kernel(const float* __restrict__ top_idx, int rows, int k, int E, int max_rows, int* __restrict__ counts,
+                                 int* __restrict__ lists, int* __restrict__ slot) {
+    int e = threadIdx.x;
+    if (e >= E) return;
+    int n = 0;
+    for (int i = 0; i < rows; ++i)
+        for (int j = 0; j < k; ++j)
+            if ((int)top_idx[i * k + j] == e) { lists[e * max_rows + n] = i; slot[i * k + j] = n; ++n; }
+    counts[e] = n;
+}
+
+// IndexSelect(inputNorm, tokenIdx_e) for every expert (MoEFeedForward.cs:155): grid (max_rows, E)
+template <typename AT>
+__global__ __launch_bounds__(256) void moe_gather_kernel(const float* __restrict__ xn32, int h, const int* __restrict__ counts,
+                                                          const int* __restrict__ lists, int max_rows, AT* __restrict__ xg, long ld, long estride) {
+    const int j = blockIdx.x, e = blockIdx.y;
+    if (j >= counts[e]) return;
+    const int tok = lists[e * max_rows + j];
+    AT* dst = xg + e * estride + (long)j * ld;
+    for (int c = threadIdx.x; c < h; c += 256) dst[c] = (AT)xn32[(long)tok * h + c];
+}
+
+// EltMul by the expert's probability, scatter-add in expert-major order into zeros, then input + result
+// (MoEFeedForward.cs:167-178; IndexSelectGrad, TensorApplyCPU.cs:1336-1356): one block per token
+__global__ __launch_bounds__(256) void moe_combine_kernel(float* __restrict__ x, long ldx, int h, const float* __restrict__ y, long ldy, long estride,
+                                                           const float* __restrict__ probs, const float* __restrict__ top_idx, const int* __restrict__ slot,
+                                                           int k, int E) {
+#pragma clang fp contract(off)
+    const int i = blockIdx.x;
+    for (int c = threadIdx.x; c < h; c += 256) {
+        float out = 0.0f;
+        for (int e = 0; e < E; ++e)
+            for (int j = 0; j < k; ++j)
+                if ((int)top_idx[i * k + j] == e) {
+                    float sc = y[e * estride + (long)slot[i * k + j] * ldy + c] * probs[i * E + e];
+                    out += sc;
+                }
+        x[(long)i * ldx + c] = x[(long)i * ldx + c] + out;
+    }
+}
+
+}  // namespace tship

@@ -1,0 +1,177 @@
+"""Host-side mirror of the reference's GPT decode loop over the fused C-ABI path.
+
+`HipGpt` plays the role of Seq2SeqSharp's GPT.RunForwardOnSingleDevice + Decoder.GPTDecode
+(Seq2SeqSharp/Applications/GPT.cs:212-335, Applications/Decoder.cs:648-794): prompts in, token ids out,
+KV cache kept on the device.  Every method is a thin call into libtship.so; nothing is computed here.
+"""
+import ctypes as C
+
+import numpy as np
+
+from ._lib import TSHipGptConfig, check, lib
+
+GREEDY, TOPP = 0, 1
+F32, F16 = 0, 1
+
+_proto_done = False
+
+
+def _protos():
+    global _proto_done
+    if _proto_done:
+        return
+    L = lib()
+    vp = C.c_void_p
+    L.TSHip_Init.argtypes = [C.c_int]
+    L.TSHip_GptCreate.argtypes = [C.POINTER(TSHipGptConfig), C.POINTER(vp)]
+    L.TSHip_GptDestroy.argtypes = [vp]
+    L.TSHip_GptSetWeight.argtypes = [vp, C.c_char_p, vp, C.c_int, C.POINTER(C.c_int64)]
+    L.TSHip_GptFinalize.argtypes = [vp]
+    L.TSHip_GptReset.argtypes = [vp]
+    L.TSHip_GptPrefill.argtypes = [vp, vp, C.c_int, C.c_int]
+    L.TSHip_GptDecode.argtypes = [vp, vp, C.c_int]
+    L.TSHip_GptSample.argtypes = [vp, C.c_int, C.c_float, C.c_float, vp, vp]
+    L.TSHip_GptGenerate.argtypes = [vp, C.c_int, C.c_int, C.c_float, C.c_float, vp, vp, C.POINTER(C.c_float)]
+    L.TSHip_GptGetLogits.argtypes = [vp, vp]
+    L.TSHip_GptGetHidden.argtypes = [vp, vp]
+    L.TSHip_GptGetSeqLen.argtypes = [vp, C.POINTER(C.c_int)]
+    L.TSHip_GptGetKV.argtypes = [vp, C.c_int, C.c_int, vp]
+    L.TSHip_GptSetKV.argtypes = [vp, C.c_int, C.c_int, vp, C.c_int, C.c_int]
+    L.TSHip_GptSetSeqLen.argtypes = [vp, C.c_int, C.c_int]
+    L.TSHip_GptGetMoeRouting.argtypes = [vp, C.c_int, vp, vp, vp]
+    L.TSHip_GptProfileDecode.argtypes = [vp, vp, C.c_int, vp, vp, C.c_int, C.POINTER(C.c_int)]
+    L.TSHip_GptStepBytes.argtypes = [vp, C.c_int, C.POINTER(C.c_double), C.POINTER(C.c_double)]
+    L.TSHip_Synchronize.argtypes = []
+    _proto_done = True
+
+
+def _ptr(a):
+    return None if a is None else a.ctypes.data_as(C.c_void_p)
+
+
+class HipGpt:
+    """One GPTDecoder replica on one GPU with a preallocated KV cache."""
+
+    def __init__(self, cfg, weights, max_batch=None, max_seq_len=None, device=0):
+        """cfg: dict (see seq2seqsharp_amd.synth); weights: dict or iterable of (name, float32 array)
+        under the reference's saved parameter names."""
+        _protos()
+        L = lib()
+        check(L.TSHip_Init(device))
+        self.cfg = dict(cfg)
+        self.max_batch = int(max_batch or cfg.get("batch", 1))
+        self.max_seq_len = int(max_seq_len or (cfg.get("prompt", 16) + cfg.get("steps", 16) + 1))
+        c = TSHipGptConfig(cfg["n_layers"], cfg["hidden"], cfg["n_heads"], cfg["n_kv_heads"], cfg["ffn_dim"], cfg["vocab"],
+                           cfg["attn_type"], cfg["norm_type"], cfg["act"], cfg.get("n_experts", 1),
+                           cfg.get("experts_per_token", 1), cfg.get("norm_eps", 1e-6), cfg.get("rope_base", 500000.0),
+                           cfg.get("use_rope", 1), F16 if cfg.get("dtype", "f32") == "f16" else F32,
+                           self.max_batch, self.max_seq_len)
+        h = C.c_void_p()
+        check(L.TSHip_GptCreate(C.byref(c), C.byref(h)))
+        self.h = h
+        items = weights.items() if hasattr(weights, "items") else weights
+        for name, w in items:
+            w = np.ascontiguousarray(w, dtype=np.float32)
+            sizes = (C.c_int64 * w.ndim)(*w.shape)
+            check(L.TSHip_GptSetWeight(self.h, name.encode(), _ptr(w), w.ndim, sizes))
+        check(L.TSHip_GptFinalize(self.h))
+        self.batch = 0
+
+    def close(self):
+        if getattr(self, "h", None):
+            lib().TSHip_GptDestroy(self.h)
+            self.h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def reset(self):
+        check(lib().TSHip_GptReset(self.h))
+        self.batch = 0
+
+    def prefill(self, ids):
+        ids = np.ascontiguousarray(ids, dtype=np.int32)
+        B, T = ids.shape
+        check(lib().TSHip_GptPrefill(self.h, _ptr(ids), B, T))
+        self.batch = B
+
+    def decode(self, ids):
+        ids = np.ascontiguousarray(ids, dtype=np.int32).reshape(-1)
+        check(lib().TSHip_GptDecode(self.h, _ptr(ids), ids.size))
+        self.batch = ids.size
+
+    def sample(self, mode=GREEDY, top_p=0.0, temperature=1.0, uniforms=None):
+        out = np.empty((self.batch,), np.int32)
+        u = None if uniforms is None else np.ascontiguousarray(uniforms, dtype=np.float32)
+        check(lib().TSHip_GptSample(self.h, mode, top_p, temperature, _ptr(u), _ptr(out)))
+        return out
+
+    def generate(self, n_steps, mode=GREEDY, top_p=0.0, temperature=1.0, uniforms=None):
+        """Returns (ids [n_steps, batch], device milliseconds of the loop)."""
+        out = np.empty((n_steps, self.batch), np.int32)
+        u = None if uniforms is None else np.ascontiguousarray(uniforms, dtype=np.float32)
+        ms = C.c_float(0.0)
+        check(lib().TSHip_GptGenerate(self.h, n_steps, mode, top_p, temperature, _ptr(u), _ptr(out), C.byref(ms)))
+        return out, ms.value
+
+    def logits(self):
+        out = np.empty((self.batch, self.cfg["vocab"]), np.float32)
+        check(lib().TSHip_GptGetLogits(self.h, _ptr(out)))
+        return out
+
+    def hidden(self):
+        out = np.empty((self.batch, self.cfg["hidden"]), np.float32)
+        check(lib().TSHip_GptGetHidden(self.h, _ptr(out)))
+        return out
+
+    def seq_len(self):
+        n = C.c_int(0)
+        check(lib().TSHip_GptGetSeqLen(self.h, C.byref(n)))
+        return n.value
+
+    def get_kv(self, layer, which):
+        """[batch, n_kv_heads, len, head_dim] float32; which = 0 keys (after RoPE), 1 values."""
+        T = self.seq_len()
+        d = self.cfg["hidden"] // self.cfg["n_heads"]
+        out = np.empty((self.batch, self.cfg["n_kv_heads"], T, d), np.float32)
+        check(lib().TSHip_GptGetKV(self.h, layer, which, _ptr(out)))
+        return out
+
+    def set_kv(self, layer, which, data):
+        data = np.ascontiguousarray(data, dtype=np.float32)
+        B, G, T, d = data.shape
+        check(lib().TSHip_GptSetKV(self.h, layer, which, _ptr(data), B, T))
+
+    def set_seq_len(self, batch, length):
+        check(lib().TSHip_GptSetSeqLen(self.h, batch, length))
+        self.batch = batch
+
+    def moe_routing(self, layer):
+        k, E = self.cfg["experts_per_token"], self.cfg["n_experts"]
+        ti = np.empty((self.batch, k), np.float32)
+        tv = np.empty((self.batch, k), np.float32)
+        pr = np.empty((self.batch, E), np.float32)
+        check(lib().TSHip_GptGetMoeRouting(self.h, layer, _ptr(ti), _ptr(tv), _ptr(pr)))
+        return ti, tv, pr
+
+    def profile_decode(self, ids, n_max=4096):
+        """One decode step with device events around every kernel: list of (kernel name, milliseconds)."""
+        ids = np.ascontiguousarray(ids, dtype=np.int32).reshape(-1)
+        names = C.create_string_buffer(48 * n_max)
+        ms = np.zeros((n_max,), np.float32)
+        n = C.c_int(0)
+        check(lib().TSHip_GptProfileDecode(self.h, _ptr(ids), ids.size, C.cast(names, C.c_void_p), _ptr(ms), n_max, C.byref(n)))
+        self.batch = ids.size
+        out = []
+        for i in range(min(n.value, n_max)):
+            out.append((names.raw[i * 48:(i + 1) * 48].split(b"\0", 1)[0].decode(), float(ms[i])))
+        return out
+
+    def step_bytes(self, batch=None):
+        """Algorithmic bytes of one decode step at the current length: (weight bytes, KV bytes)."""
+        w, k = C.c_double(0), C.c_double(0)
+        check(lib().TSHip_GptStepBytes(self.h, batch or self.batch, C.byref(w), C.byref(k)))
+        return w.value, k.value
