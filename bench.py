@@ -1,0 +1,166 @@
+#!/usr/bin/env python3
+"""Benchmark of the GPTDecoder decode loop on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config cfg2_1b_gqa_f16] [--no-cpu-baseline]
+
+A "step" is one decode step of the whole batch (one new token per sequence) on synthetic data:
+seeded N(0, 0.02) weights of the named architecture and uniform-random prompts, KV cache filled by a real
+prefill of the prompts.  Prints ONE JSON line: decode tokens/s (whole batch), the roofline of the
+dominant kernel (the weight-streaming decode GEMM of the FFN up/gate projection) measured live with device
+events, and the CPU baseline (the oracle's restatement of the reference's CPU backend, single thread,
+timed on a bounded sample on this host).
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, vendor figure
+MFMA_FP16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 matrix, vendor figure
+
+
+def algorithmic_prefill_flops(cfg, B, Tp):
+    h, H, G, F, V, L = cfg["hidden"], cfg["n_heads"], cfg["n_kv_heads"], cfg["ffn_dim"], cfg["vocab"], cfg["n_layers"]
+    d = h // H
+    nW = 3 if cfg["act"] in (3, 4) else 2
+    per_tok = L * (h * H * d + 2 * h * G * d + H * d * h + nW * h * F)
+    return 2.0 * B * Tp * per_tok + 2.0 * B * h * V + L * B * H * d * float(Tp) * Tp * 2.0
+
+
+def cpu_baseline(cfg, gpu, weights, next_ids, budget_note):
+    """One decode step of the CPU oracle (kind "port": a restatement of the reference's CPU path), single
+    thread, at the benchmark's shape, on the KV cache the GPU prefill produced.  Also returns the logit
+    difference between that step and the GPU's, a full-size parity number."""
+    from oracle import ts_oracle as O
+    O.set_threads(1)
+    B = gpu.batch
+    H, G = cfg["n_heads"], cfg["n_kv_heads"]
+    d = cfg["hidden"] // H
+    T = gpu.seq_len()
+    orc = O.OracleGpt(cfg, weights)
+    for l in range(cfg["n_layers"]):
+        k = gpu.get_kv(l, 0)                      # [B, G, T, d]
+        v = gpu.get_kv(l, 1)
+        # the reference caches K/V expanded to all query heads, K transposed (GroupQueryAttention.cs:156-188)
+        ke = np.repeat(k, H // G, axis=1).transpose(0, 1, 3, 2).reshape(B * H, d, T)
+        ve = np.repeat(v, H // G, axis=1).reshape(B * H, T, d)
+        orc.set_cache(l, 0, ke, B * H, T, d)
+        orc.set_cache(l, 1, ve, B * H, T, d)
+    seqs = np.ascontiguousarray(next_ids.reshape(B, 1), dtype=np.int32)
+    t0 = time.perf_counter()
+    _, lg = orc.step(seqs, use_cache=True)
+    dt = time.perf_counter() - t0
+    return {"value": B / dt, "unit": "tokens/s", "cores": 1, "kind": "port",
+            "sample": "1 decode step of the whole batch at KV length %d (%s), %.1f s" % (T, budget_note, dt)}, lg
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=256)
+    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--config", default="cfg2_1b_gqa_f16")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-topp", action="store_true")
+    ap.add_argument("--prompt", type=int, default=0, help="override the prompt length")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build drives one GPU per process and measures one GPU; --gpus %d is not supported "
+              "(each GPU would hold a full replica and its own batch rows, with no per-step exchange)" % args.gpus, file=sys.stderr)
+        sys.exit(2)
+
+    from seq2seqsharp_amd import synth
+    from seq2seqsharp_amd.gpt import GREEDY, TOPP, HipGpt
+
+    cfg = dict(synth.CONFIGS[args.config])
+    if args.prompt:
+        cfg["prompt"] = args.prompt
+    B, Tp, K, W = cfg["batch"], cfg["prompt"], args.steps, args.warmup
+    t0 = time.perf_counter()
+    weights = synth.make_weights(cfg, seed=0)
+    gpu = HipGpt(cfg, weights, max_batch=B, max_seq_len=Tp + 2 * (W + K) + 8)
+    t_load = time.perf_counter() - t0
+    prompts = synth.make_prompts(cfg, seed=1)
+
+    # prefill (timed separately)
+    gpu.prefill(prompts[:, :8])            # touch every kernel once
+    gpu.reset()
+    t0 = time.perf_counter()
+    gpu.prefill(prompts)
+    t_prefill = time.perf_counter() - t0
+    prefill_tok_s = B * Tp / t_prefill
+    prefill_tflops = algorithmic_prefill_flops(cfg, B, Tp) / t_prefill / 1e12
+
+    # decode: W warm-up steps, then exactly K timed steps (device events on the library stream, bracketed by syncs)
+    gpu.generate(max(W, 1))
+    T_start = gpu.seq_len()
+    wall0 = time.perf_counter()
+    ids, ms = gpu.generate(K)
+    wall = time.perf_counter() - wall0
+    T_end = gpu.seq_len()
+    ms_per_step = ms / K
+    tok_s = B * K / (ms / 1e3)
+    wbytes, _ = gpu.step_bytes(B)
+    d = cfg["hidden"] // cfg["n_heads"]
+    es = 2 if cfg["dtype"] == "f16" else 4
+    kv_per_pos = es * cfg["n_layers"] * B * cfg["n_kv_heads"] * d * 2
+    step_bytes = wbytes + kv_per_pos * (T_start + T_end + 1) / 2.0
+    step_gbs = step_bytes / (ms_per_step / 1e3) / 1e9
+
+    # per-kernel device times of single decode steps -> roofline of the dominant kernel
+    nxt = gpu.sample()
+    acc = {}
+    n_prof = 5
+    for _ in range(n_prof):
+        for name, t in gpu.profile_decode(nxt):
+            acc.setdefault(name, []).append(t)
+    dom = "gemm_ffn13" if "gemm_ffn13" in acc else max(acc, key=lambda k: sum(acc[k]))
+    dom_ms = float(np.mean(acc[dom]))
+    nW13 = 2 if cfg["act"] in (3, 4) else 1
+    dom_bytes = float(cfg["hidden"]) * cfg["ffn_dim"] * nW13 * es      # the weights one launch streams, once
+    dom_gbs = dom_bytes / (dom_ms / 1e3) / 1e9
+    kernel_ms = {k: round(float(np.sum(v)) / n_prof, 4) for k, v in acc.items()}
+
+    out = {
+        "metric": "decode tokens/s on 1 GPU (1B GQA fp16, batch 32)" if args.config == "cfg2_1b_gqa_f16" else "decode tokens/s on 1 GPU",
+        "value": round(tok_s, 1), "unit": "tokens/s", "n_gpus": 1, "steps": K, "warmup": W,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": cfg["dtype"], "data": "synthetic",
+        "config": {"workload": args.config, "batch": B, "prompt_len": Tp, "kv_len_start": T_start, "kv_len_end": T_end,
+                   "sampling": "greedy", "rope_base": cfg["rope_base"]},
+        "roofline": {"bound": "hbm", "achieved": round(dom_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(dom_gbs / HBM_PEAK_GBS, 4), "traffic": None,
+                     "kernel": "skinny_gemm_f16_kernel<%d, EPI_ACT16> (%s)" % (1 if B <= 32 else 2 if B <= 64 else 4, dom),
+                     "bytes_per_launch": dom_bytes, "avg_launch_ms": round(dom_ms, 5)},
+        "whole_step": {"algorithmic_bytes": round(step_bytes), "achieved_GBps": round(step_gbs, 1),
+                       "frac_of_hbm_peak": round(step_gbs / HBM_PEAK_GBS, 4), "host_wall_ms_per_step": round(wall / K * 1e3, 4)},
+        "prefill": {"tokens_per_s": round(prefill_tok_s, 1), "seconds": round(t_prefill, 4),
+                    "algorithmic_TFLOPs": round(prefill_tflops, 2),
+                    "frac_of_fp16_mfma_peak": round(prefill_tflops / MFMA_FP16_PEAK_TFLOPS, 4) if cfg["dtype"] == "f16" else None},
+        "kernel_ms_per_step": kernel_ms,
+        "load_seconds": round(t_load, 1),
+    }
+    if not args.no_topp:
+        u = synth.make_uniforms(7, B, K)
+        _, ms_p = gpu.generate(K, mode=TOPP, top_p=0.9, temperature=1.0, uniforms=u)
+        out["topp"] = {"top_p": 0.9, "tokens_per_s": round(B * K / (ms_p / 1e3), 1), "ms_per_step": round(ms_p / K, 4)}
+    if not args.no_cpu_baseline:
+        nxt = gpu.sample()
+        base, lg = cpu_baseline(cfg, gpu, weights, nxt, "cache from the GPU prefill")
+        gpu.decode(nxt)
+        out["cpu_baseline"] = base
+        out["parity_full_size"] = {"max_abs_logit_diff_vs_cpu": float(np.abs(gpu.logits() - lg).max()),
+                                   "top1_agree": float((gpu.logits().argmax(1) == lg.argmax(1)).mean())}
+    else:
+        out["cpu_baseline"] = None
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -117,11 +117,13 @@ static void launch(TSHipGpt* m, const char* name, void (*kernel)(KArgs...), dim3
     TSHIP_CHECK_HIP(hipGetLastError());
 }
 
-static int pick_ks_f16(int NT, int KT) {
-    int target = 2 * std::max(n_compute_units(), 64);
-    int ks = std::max(1, target / std::max(NT, 1));
-    ks = std::min(ks, std::max(1, KT / 8));
-    return std::min(ks, 16);
+// decode GEMM split-K: a block has NW wavefronts of 8 k-tiles each in flight; split K across blocks until one
+// pass covers the block's range (keeps partial-sum traffic small: K = 2048 needs no split at batch <= 32)
+static int pick_ks_f16(int NT, int KT, int BT) {
+    (void)NT;
+    const int NW = BT <= 2 ? 8 : 4;
+    int ks = (int)ceil_div(KT, NW * 8);
+    return std::max(1, std::min(ks, 16));
 }
 static int pick_ks_f32(int N, int K) {
     int target = 2 * std::max(n_compute_units(), 64);
@@ -143,7 +145,7 @@ static void gemmw_alloc(TSHipGpt* m, GemmW& w, int K, int N) {
     if (m->f16) {
         w.KT = (int)ceil_div(K, 16); w.NT = (int)ceil_div(N, 32);
         w.buf.alloc((size_t)w.KT * w.NT * 512 * sizeof(half_t));
-        w.KS = pick_ks_f16(w.NT, w.KT);
+        w.KS = pick_ks_f16(w.NT, w.KT, m->BT);
     } else {
         w.ld = N;
         w.buf.alloc((size_t)K * N * sizeof(float));
@@ -297,8 +299,12 @@ static void set_weight(TSHipGpt* m, const std::string& name, const float* host, 
 // kernel dispatch helpers
 // ------------------------------------------------------------------------------------------------
 static void run_resid_norm(TSHipGpt* m, const char* name, int rows, ResidNormArgs a) {
-    if (m->f16) launch(m, name, resid_norm_kernel<half_t>, dim3(rows), dim3(256), a);
-    else launch(m, name, resid_norm_kernel<float>, dim3(rows), dim3(256), a);
+    const int h = m->c.hidden;
+#define TSHIP_RN(NPT)                                                                         \
+    if (m->f16) launch(m, name, resid_norm_kernel<half_t, NPT>, dim3(rows), dim3(256), a);   \
+    else launch(m, name, resid_norm_kernel<float, NPT>, dim3(rows), dim3(256), a);
+    if (h <= 1024) { TSHIP_RN(4) } else if (h <= 2048) { TSHIP_RN(8) } else if (h <= 4096) { TSHIP_RN(16) } else { TSHIP_RN(32) }
+#undef TSHIP_RN
 }
 
 // Y = X * W for <= 128 rows.  fp16: MFMA kernel; epilogue per `epi`.  fp32: tiled GEMM into partials.
@@ -306,13 +312,13 @@ static void run_skinny(TSHipGpt* m, const char* name, const GemmW& w, const void
     TSHIP_REQUIRE(m->f16, "internal: run_skinny is the fp16 path");
     e.W = w.buf.as<half_t>(); e.KT = w.KT; e.NT = w.NT; e.X = (const half_t*)X; e.ldx = (int)ldx;
     e.KS = (epi == EPI_PARTIAL) ? w.KS : 1; e.rows_valid = rows;
-    dim3 grid(w.NT * e.KS), block(256);
+    dim3 grid(w.NT * e.KS);
     const int BT = m->BT;
-#define TSHIP_SK(BTV)                                                                                       \
-    if (epi == EPI_PARTIAL) launch(m, name, skinny_gemm_f16_kernel<BTV, EPI_PARTIAL>, grid, block, e);      \
-    else if (epi == EPI_F32_BIAS) launch(m, name, skinny_gemm_f16_kernel<BTV, EPI_F32_BIAS>, grid, block, e); \
-    else launch(m, name, skinny_gemm_f16_kernel<BTV, EPI_ACT16>, grid, block, e);
-    if (BT == 1) { TSHIP_SK(1) } else if (BT == 2) { TSHIP_SK(2) } else { TSHIP_SK(4) }
+#define TSHIP_SK(BTV, NWV)                                                                                                  \
+    if (epi == EPI_PARTIAL) launch(m, name, skinny_gemm_f16_kernel<BTV, EPI_PARTIAL, NWV>, grid, dim3(NWV * 64), e);        \
+    else if (epi == EPI_F32_BIAS) launch(m, name, skinny_gemm_f16_kernel<BTV, EPI_F32_BIAS, NWV>, grid, dim3(NWV * 64), e); \
+    else launch(m, name, skinny_gemm_f16_kernel<BTV, EPI_ACT16, NWV>, grid, dim3(NWV * 64), e);
+    if (BT == 1) { TSHIP_SK(1, 8) } else if (BT == 2) { TSHIP_SK(2, 8) } else { TSHIP_SK(4, 4) }
 #undef TSHIP_SK
 }
 
@@ -388,7 +394,7 @@ static void decode_step(TSHipGpt* m, const int* d_ids, int B) {
     const long hp = round_up(h, 32), qp = round_up(m->Nqkv, 32);
     ResidNormArgs rn; std::memset(&rn, 0, sizeof(rn));
     rn.x = m->x.as<float>(); rn.ldx = h; rn.h = h; rn.eps = c.norm_eps; rn.norm_type = c.norm_type;
-    rn.xn = m->xn.p; rn.ldxn = m->ldh;
+    rn.xn = m->xn.p; rn.ldxn = m->ldh; rn.xn_kt = m->f16 ? (int)(m->ldh / 16) : 0;
 
     // embedding gather * sqrt(h) and the first layer's attention norm
     {
@@ -412,8 +418,8 @@ static void decode_step(TSHipGpt* m, const int* d_ids, int B) {
         {
             AttnArgs a = attn_args(m, L);
             a.qkv = m->part_qkv.as<float>(); a.KS = L.qkv.KS; a.split_stride = qstride; a.ldq = qp;
-            a.out = m->o.p; a.ld_out = m->ldh;
-            launch(m, "attn_decode", pick_attn(m, false), dim3(c.n_kv_heads, B), dim3(256), a);
+            a.out = m->o.p; a.ld_out = m->ldh; a.out_kt = m->f16 ? (int)(m->ldh / 16) : 0;
+            launch(m, "attn_decode", pick_attn(m, false), dim3(c.n_kv_heads, B), dim3(1024), a);
         }
         // output projection -> partials
         long hstride = (long)m->Bpad * hp;
@@ -445,7 +451,7 @@ static void decode_step(TSHipGpt* m, const int* d_ids, int B) {
         if (m->f16) {
             SkinnyArgs e; std::memset(&e, 0, sizeof(e));
             e.bias = L.b1.as<float>(); e.bias2 = L.b3.as<float>(); e.out16 = m->a.as<half_t>(); e.ld16 = (int)m->ldF;
-            e.act = c.act; e.gated = m->gated; e.n_valid = F;
+            e.act = c.act; e.gated = m->gated; e.n_valid = F; e.out16_kt = L.w2.KT;
             run_skinny(m, "gemm_ffn13", L.w13, m->xn.p, m->ldh, B, EPI_ACT16, e);
         } else {
             long fp = m->F13, fstride = (long)m->Bpad * fp;
@@ -574,7 +580,7 @@ static void prefill(TSHipGpt* m, const int32_t* host_ids, int B, int Tp) {
     TSHIP_CHECK_HIP(hipMemcpyAsync(rowmap.p, map.data(), B * sizeof(int), hipMemcpyHostToDevice, stream()));
     {
         ResidNormArgs a = rn;
-        a.row_map = rowmap.as<int>(); a.xn = m->xn.p; a.ldxn = m->ldh;
+        a.row_map = rowmap.as<int>(); a.xn = m->xn.p; a.ldxn = m->ldh; a.xn_kt = m->f16 ? (int)(m->ldh / 16) : 0;
         a.gamma = m->fn_g.as<float>(); a.beta = m->fn_b.as<float>();
         run_resid_norm(m, "p_final_norm", B, a);
     }
@@ -819,9 +825,13 @@ TSHIP_API int TSHip_GptGetHidden(TSHipGpt* m, float* host_out) {
     const int B = m->cur_batch, h = m->c.hidden;
     TSHIP_CHECK_HIP(hipStreamSynchronize(stream()));
     if (m->f16) {
-        std::vector<half_t> tmp((size_t)B * m->ldh);
+        std::vector<half_t> tmp((size_t)m->Bpad * m->ldh);
         TSHIP_CHECK_HIP(hipMemcpy(tmp.data(), m->xn.p, tmp.size() * sizeof(half_t), hipMemcpyDeviceToHost));
-        for (int b = 0; b < B; ++b) for (int i = 0; i < h; ++i) host_out[(size_t)b * h + i] = (float)tmp[(size_t)b * m->ldh + i];
+        const int KT = (int)(m->ldh / 16);
+        for (int b = 0; b < B; ++b) for (int i = 0; i < h; ++i) {
+            size_t idx = ((((size_t)(b >> 5) * KT + (i >> 4)) * 64) + (b & 31) + 32 * ((i >> 3) & 1)) * 8 + (i & 7);   // fragment packed
+            host_out[(size_t)b * h + i] = (float)tmp[idx];
+        }
     } else {
         TSHIP_CHECK_HIP(hipMemcpy2D(host_out, (size_t)h * sizeof(float), m->xn.p, (size_t)m->ldh * sizeof(float), (size_t)h * sizeof(float), B, hipMemcpyDeviceToHost));
     }

@@ -65,7 +65,7 @@ static void run_moe_ffn(TSHipGpt* m, LayerW& L, int rows, const ResidNormArgs& p
     if (m->f16) {
         half_t* xg = (half_t*)(base + o.xg); half_t* mid = (half_t*)(base + o.mid);
         launch(m, "moe_gather", moe_gather_kernel<half_t>, dim3(rows, E), dim3(256), (const float*)xn32, h, (const int*)counts, (const int*)lists, Bp, xg,
-               m->ldh, xg_stride);
+               m->ldh, xg_stride, (int)(m->ldh / 16));
         // pointer tables are written once per layer object (weights never move)
         std::vector<const half_t*> t1(E), t2(E);
         for (int e = 0; e < E; ++e) { t1[e] = L.e1[e]->buf.as<half_t>(); t2[e] = L.e2[e]->buf.as<half_t>(); }
@@ -74,7 +74,7 @@ static void run_moe_ffn(TSHipGpt* m, LayerW& L, int rows, const ResidNormArgs& p
         TSHIP_CHECK_HIP(hipStreamSynchronize(stream()));
         SkinnyArgs e1; std::memset(&e1, 0, sizeof(e1));
         e1.W = t1[0]; e1.KT = L.e1[0]->KT; e1.NT = L.e1[0]->NT; e1.X = xg; e1.ldx = (int)m->ldh; e1.KS = 1;
-        e1.bias = zero; e1.out16 = mid; e1.ld16 = (int)o.ld4h; e1.act = c.act; e1.gated = 0; e1.n_valid = 4 * h;
+        e1.bias = zero; e1.out16 = mid; e1.ld16 = (int)o.ld4h; e1.out16_kt = L.e2[0]->KT; e1.act = c.act; e1.gated = 0; e1.n_valid = 4 * h;
         e1.Wtab = (const half_t* const*)(base + o.wtab1); e1.x_estride = xg_stride; e1.out16_estride = mid_stride; e1.rows_tab = counts;
         SkinnyArgs e2; std::memset(&e2, 0, sizeof(e2));
         e2.W = t2[0]; e2.KT = L.e2[0]->KT; e2.NT = L.e2[0]->NT; e2.X = mid; e2.ldx = (int)o.ld4h; e2.KS = 1;
@@ -82,19 +82,19 @@ static void run_moe_ffn(TSHipGpt* m, LayerW& L, int rows, const ResidNormArgs& p
         e2.Wtab = (const half_t* const*)(base + o.wtab2); e2.x_estride = mid_stride; e2.out_estride = y_stride; e2.rows_tab = counts;
         dim3 g1(e1.NT, E), g2(e2.NT, E);
         if (m->BT == 1) {
-            launch(m, "moe_gemm1", skinny_gemm_f16_kernel<1, EPI_ACT16>, g1, dim3(256), e1);
-            launch(m, "moe_gemm2", skinny_gemm_f16_kernel<1, EPI_F32_BIAS>, g2, dim3(256), e2);
+            launch(m, "moe_gemm1", skinny_gemm_f16_kernel<1, EPI_ACT16, 8>, g1, dim3(512), e1);
+            launch(m, "moe_gemm2", skinny_gemm_f16_kernel<1, EPI_F32_BIAS, 8>, g2, dim3(512), e2);
         } else if (m->BT == 2) {
-            launch(m, "moe_gemm1", skinny_gemm_f16_kernel<2, EPI_ACT16>, g1, dim3(256), e1);
-            launch(m, "moe_gemm2", skinny_gemm_f16_kernel<2, EPI_F32_BIAS>, g2, dim3(256), e2);
+            launch(m, "moe_gemm1", skinny_gemm_f16_kernel<2, EPI_ACT16, 8>, g1, dim3(512), e1);
+            launch(m, "moe_gemm2", skinny_gemm_f16_kernel<2, EPI_F32_BIAS, 8>, g2, dim3(512), e2);
         } else {
-            launch(m, "moe_gemm1", skinny_gemm_f16_kernel<4, EPI_ACT16>, g1, dim3(256), e1);
-            launch(m, "moe_gemm2", skinny_gemm_f16_kernel<4, EPI_F32_BIAS>, g2, dim3(256), e2);
+            launch(m, "moe_gemm1", skinny_gemm_f16_kernel<4, EPI_ACT16, 4>, g1, dim3(256), e1);
+            launch(m, "moe_gemm2", skinny_gemm_f16_kernel<4, EPI_F32_BIAS, 4>, g2, dim3(256), e2);
         }
     } else {
         float* xg = (float*)(base + o.xg); float* mid = (float*)(base + o.mid);
         launch(m, "moe_gather", moe_gather_kernel<float>, dim3(rows, E), dim3(256), (const float*)xn32, h, (const int*)counts, (const int*)lists, Bp, xg,
-               m->ldh, xg_stride);
+               m->ldh, xg_stride, 0);
         for (int e = 0; e < E; ++e) {
             // fp32 models: every expert runs on `rows` rows; rows past the expert's count hold stale finite data
             // and are never read back

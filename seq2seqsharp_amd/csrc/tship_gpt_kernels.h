@@ -26,6 +26,13 @@ __device__ __forceinline__ float act_apply(int act, float w) {
     return w;
 }
 
+// GEMM inputs of the fp16 decode path are stored "fragment packed": for every k-tile of 16 the 32 rows form the
+// 1 KiB B-operand fragment of v_mfma_f32_32x32x16_f16 (lane l holds row l%32, k = kt*16 + 8*(l/32) .. +7), so a
+// wavefront fetches it with one coalesced 16-byte load per lane.  Index of element (row b, column k):
+__device__ __forceinline__ long xpack_index(int b, int k, int KT) {
+    return ((((long)(b >> 5) * KT + (k >> 4)) * 64) + (b & 31) + 32 * ((k >> 3) & 1)) * 8 + (k & 7);
+}
+
 template <typename T> __device__ __forceinline__ float to_f32(T v) { return (float)v; }
 template <typename T> __device__ __forceinline__ T from_f32(float v) { return (T)v; }
 
@@ -80,16 +87,24 @@ struct SkinnyArgs {
     float* out; int ld_out; long split_stride;
     const float* bias; const float* bias2;
     half_t* out16; int ld16;
+    int out16_kt;          // > 0: out16 is fragment packed with this many k-tiles per row block; 0: row-major with ld16
     int act; int gated; int n_valid; int rows_valid;
     // optional batch of independent problems (MoE experts) on blockIdx.y: weights from a pointer table,
     // activations / outputs at a fixed stride, row counts read on the device
     const half_t* const* Wtab; long x_estride; long out_estride; long out16_estride; const int* rows_tab;
 };
 
-template <int BT, int EPI>
-__global__ __launch_bounds__(256) void skinny_gemm_f16_kernel(SkinnyArgs a) {
+// NW wavefronts per block work on the same 32-column tile and split the block's k range; every wavefront keeps
+// 8 weight fragments and 8 activation fragments (16 KiB) in flight.  Accumulators are added pairwise through LDS
+// (a fixed tree, so the sum order never changes); the last two are transposed through LDS so that the epilogue
+// writes coalesced rows.  X is fragment packed (xpack_index).
+template <int BT, int EPI, int NW>
+__global__ __launch_bounds__(NW * 64) void skinny_gemm_f16_kernel(SkinnyArgs a) {
     constexpr int U = 8;
-    __shared__ float red[4][BT * 32][33];
+    constexpr int RED = (NW / 2) * BT * 16 * 64, FIN = 2 * BT * 32 * 33;
+    __shared__ float smem[RED > FIN ? RED : FIN];      // the tree buffers are dead when the transpose buffer is written
+    float (*red)[BT][16][64] = (float (*)[BT][16][64])smem;
+    float (*fin)[BT * 32][33] = (float (*)[BT * 32][33])smem;
     if (a.Wtab) {
         const int e = blockIdx.y;
         a.rows_valid = a.rows_tab[e];
@@ -98,11 +113,11 @@ __global__ __launch_bounds__(256) void skinny_gemm_f16_kernel(SkinnyArgs a) {
         if (a.out) a.out += e * a.out_estride;
         if (a.out16) a.out16 += e * a.out16_estride;
     }
-    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63, w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int nt = blockIdx.x / a.KS, ks = blockIdx.x % a.KS;
     const int per = (a.KT + a.KS - 1) / a.KS;
     const int k0 = ks * per, k1 = min(a.KT, k0 + per);
-    const int pw = (max(k1 - k0, 0) + 3) / 4;
+    const int pw = (max(k1 - k0, 0) + NW - 1) / NW;
     const int wk0 = k0 + w * pw, wk1 = min(k1, wk0 + pw);
 
     floatx16 acc[BT];
@@ -112,7 +127,7 @@ __global__ __launch_bounds__(256) void skinny_gemm_f16_kernel(SkinnyArgs a) {
         for (int v = 0; v < 16; ++v) acc[bt][v] = 0.0f;
 
     const half_t* wp = a.W + ((long)nt * a.KT * 64 + lane) * 8;
-    const half_t* xp = a.X + (long)(lane & 31) * a.ldx + (lane >> 5) * 8;
+    const half_t* xp = a.X + lane * 8;
     for (int kt = wk0; kt < wk1; kt += U) {
         half8 wf[U];
         half8 xf[U][BT];
@@ -121,7 +136,7 @@ __global__ __launch_bounds__(256) void skinny_gemm_f16_kernel(SkinnyArgs a) {
             if (kt + u < wk1) {
                 wf[u] = *(const half8*)(wp + (long)(kt + u) * 512);
 #pragma unroll
-                for (int bt = 0; bt < BT; ++bt) xf[u][bt] = *(const half8*)(xp + (long)bt * 32 * a.ldx + (kt + u) * 16);
+                for (int bt = 0; bt < BT; ++bt) xf[u][bt] = *(const half8*)(xp + ((long)bt * a.KT + kt + u) * 512);
             }
         }
 #pragma unroll
@@ -132,32 +147,54 @@ __global__ __launch_bounds__(256) void skinny_gemm_f16_kernel(SkinnyArgs a) {
             }
         }
     }
-    // accumulator lane l, register v holds column nt*32 + 8*(v/4) + 4*(l/32) + v%4 of batch row bt*32 + l%32
+    // pairwise tree over wavefronts down to two: in each round the upper half stores, the lower half adds
 #pragma unroll
-    for (int bt = 0; bt < BT; ++bt)
+    for (int half = NW / 2; half >= 2; half >>= 1) {
+        if (w >= half && w < 2 * half) {
 #pragma unroll
-        for (int v = 0; v < 16; ++v) red[w][bt * 32 + (lane & 31)][8 * (v / 4) + 4 * (lane >> 5) + (v % 4)] = acc[bt][v];
+            for (int bt = 0; bt < BT; ++bt)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) red[w - half][bt][v][lane] = acc[bt][v];
+        }
+        __syncthreads();
+        if (w < half) {
+#pragma unroll
+            for (int bt = 0; bt < BT; ++bt)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) acc[bt][v] += red[w][bt][v][lane];
+        }
+        __syncthreads();
+    }
+    // accumulator lane l, register v: column nt*32 + 8*(v/4) + 4*(l/32) + v%4 of batch row bt*32 + l%32
+    if (w < 2) {
+#pragma unroll
+        for (int bt = 0; bt < BT; ++bt)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) fin[w][bt * 32 + (lane & 31)][8 * (v / 4) + 4 * (lane >> 5) + (v % 4)] = acc[bt][v];
+    }
     __syncthreads();
-
-    const int n = threadIdx.x & 31, bq = threadIdx.x >> 5;
-    for (int b = bq; b < BT * 32; b += 8) {
-        if (b >= a.rows_valid) break;
-        float s = (red[0][b][n] + red[1][b][n]) + (red[2][b][n] + red[3][b][n]);
+    for (int idx = threadIdx.x; idx < BT * 1024; idx += NW * 64) {
+        const int n = idx & 31, b = idx >> 5;
+        if (b >= a.rows_valid) continue;
+        const float s = NW >= 2 ? fin[0][b][n] + fin[1][b][n] : fin[0][b][n];
         if (EPI == EPI_PARTIAL) {
             a.out[ks * a.split_stride + (long)b * a.ld_out + nt * 32 + n] = s;
         } else if (EPI == EPI_F32_BIAS) {
-            int col = nt * 32 + n;
+            const int col = nt * 32 + n;
             if (col < a.n_valid) a.out[(long)b * a.ld_out + col] = s + a.bias[col];
         } else {
+            float val; int f; bool ok;
             if (a.gated) {
-                if (n < 16) {
-                    float c = (red[0][b][n + 16] + red[1][b][n + 16]) + (red[2][b][n + 16] + red[3][b][n + 16]);
-                    int f = nt * 16 + n;
-                    if (f < a.n_valid) a.out16[(long)b * a.ld16 + f] = (half_t)(act_apply(a.act, s + a.bias[f]) * (c + a.bias2[f]));
-                }
+                const float c = fin[0][b][(n & 15) + 16] + fin[1][b][(n & 15) + 16];
+                f = nt * 16 + n; ok = n < 16 && f < a.n_valid;
+                val = ok ? act_apply(a.act, s + a.bias[f]) * (c + a.bias2[f]) : 0.0f;
             } else {
-                int f = nt * 32 + n;
-                if (f < a.n_valid) a.out16[(long)b * a.ld16 + f] = (half_t)act_apply(a.act, s + a.bias[f]);
+                f = nt * 32 + n; ok = f < a.n_valid;
+                val = ok ? act_apply(a.act, s + a.bias[f]) : 0.0f;
+            }
+            if (ok) {
+                if (a.out16_kt > 0) a.out16[xpack_index(b, f, a.out16_kt)] = (half_t)val;
+                else a.out16[(long)b * a.ld16 + f] = (half_t)val;
             }
         }
     }
@@ -316,39 +353,79 @@ struct ResidNormArgs {
     const float* part; int KS; long split_stride; long ld_part; const float* bias;
     const float* gamma; const float* beta; float eps; int norm_type;
     void* xn; long ldxn;
+    int xn_kt;              // > 0 (fp16 only): xn is fragment packed with this many k-tiles; 0: row-major with ldxn
     const int* row_map;     // optional: block r works on row row_map[r] of x and writes row r of xn
     int* advance_pos;       // optional: block 0 increments this device counter (end of a decode step)
 };
 
-template <typename AT>
+template <typename AT, int NPT>   // NPT * 256 >= hidden
 __global__ __launch_bounds__(256) void resid_norm_kernel(ResidNormArgs a) {
-    constexpr int NPT = 32;   // hidden <= 8192
     __shared__ float sred[4];
     const int r = blockIdx.x, t = threadIdx.x;
     const long xr = a.row_map ? a.row_map[r] : r;
+    const float* __restrict__ part = a.part;
+    const float* __restrict__ xin = a.x + xr * a.ldx;
     float v[NPT];
-    float sum = 0.0f, sq = 0.0f;
     long erow = a.ids ? (long)a.ids[r] : 0;
+    // all loads first (independent), then the arithmetic, then the stores
 #pragma unroll
     for (int i = 0; i < NPT; ++i) {
         int c = t + i * 256;
-        float val = 0.0f;
+        v[i] = 0.0f;
         if (c < a.h) {
             if (a.ids) {
                 float e = a.emb_f16 ? (float)((const half_t*)a.emb)[erow * a.h + c] : ((const float*)a.emb)[erow * a.h + c];
-                val = e * a.emb_scale;
+                v[i] = e * a.emb_scale;
             } else {
-                val = a.x[xr * a.ldx + c];
+                v[i] = xin[c];
             }
-            if (a.part) {
-                float s = a.part[(long)r * a.ld_part + c];
-                for (int k = 1; k < a.KS; ++k) s += a.part[k * a.split_stride + (long)r * a.ld_part + c];
-                val = (s + a.bias[c]) + val;
-            }
-            if (a.ids || a.part) a.x[xr * a.ldx + c] = val;
-            sum += val; sq += val * val;
         }
-        v[i] = val;
+    }
+    if (part) {
+        float s[NPT];
+#pragma unroll
+        for (int i = 0; i < NPT; ++i) {
+            int c = t + i * 256;
+            s[i] = (c < a.h) ? part[(long)r * a.ld_part + c] : 0.0f;
+        }
+        // splits are added in index order; four at a time so that their loads are in flight together
+        int k = 1;
+        for (; k + 3 < a.KS; k += 4) {
+            float p0[NPT], p1[NPT], p2[NPT], p3[NPT];
+#pragma unroll
+            for (int i = 0; i < NPT; ++i) {
+                int c = t + i * 256;
+                const float* q = part + (long)r * a.ld_part + c;
+                bool ok = c < a.h;
+                p0[i] = ok ? q[k * a.split_stride] : 0.0f;
+                p1[i] = ok ? q[(k + 1) * a.split_stride] : 0.0f;
+                p2[i] = ok ? q[(k + 2) * a.split_stride] : 0.0f;
+                p3[i] = ok ? q[(k + 3) * a.split_stride] : 0.0f;
+            }
+#pragma unroll
+            for (int i = 0; i < NPT; ++i) s[i] = (((s[i] + p0[i]) + p1[i]) + p2[i]) + p3[i];
+        }
+        for (; k < a.KS; ++k) {
+#pragma unroll
+            for (int i = 0; i < NPT; ++i) {
+                int c = t + i * 256;
+                if (c < a.h) s[i] += part[k * a.split_stride + (long)r * a.ld_part + c];
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < NPT; ++i) {
+            int c = t + i * 256;
+            if (c < a.h) v[i] = (s[i] + a.bias[c]) + v[i];
+        }
+    }
+    float sum = 0.0f, sq = 0.0f;
+#pragma unroll
+    for (int i = 0; i < NPT; ++i) {
+        int c = t + i * 256;
+        if (c < a.h) {
+            if (a.ids || part) a.x[xr * a.ldx + c] = v[i];
+            sum += v[i]; sq += v[i] * v[i];
+        }
     }
     if (a.advance_pos && r == 0 && t == 0) *a.advance_pos += 1;
     if (!a.xn) return;
@@ -362,7 +439,7 @@ __global__ __launch_bounds__(256) void resid_norm_kernel(ResidNormArgs a) {
             if (c < a.h) {
                 float y = a.gamma[c] * (v[i] / rms);
                 if (a.beta) y += a.beta[c];
-                out[c] = (AT)y;
+                if (a.xn_kt > 0) ((AT*)a.xn)[xpack_index(r, c, a.xn_kt)] = (AT)y; else out[c] = (AT)y;
             }
         }
     } else {
@@ -380,7 +457,7 @@ __global__ __launch_bounds__(256) void resid_norm_kernel(ResidNormArgs a) {
             if (c < a.h) {
                 float y = a.gamma[c] * ((v[i] - mean) / sigma);
                 if (a.beta) y += a.beta[c];
-                out[c] = (AT)y;
+                if (a.xn_kt > 0) ((AT*)a.xn)[xpack_index(r, c, a.xn_kt)] = (AT)y; else out[c] = (AT)y;
             }
         }
     }
@@ -399,6 +476,7 @@ struct AttnArgs {
     int pos0;                                      // prefill: cache offset of the first query row
     int Tq;                                        // prefill: query rows per sequence
     void* out; long ld_out;                        // [rows][H*D] in the activation type
+    int out_kt;                                    // > 0: out is fragment packed with this many k-tiles
     float scale;
 };
 
@@ -411,27 +489,41 @@ __device__ __forceinline__ void rope_pair(float x0, float x1, float c, float s, 
 }
 
 // Single-query attention of G query heads that share one KV head over T cached positions.
-// Lanes are grouped LPR to a cache row (16-byte loads, head_dim contiguous); every lane group keeps its own
-// online-softmax state over the rows it visits; the groups of all 4 wavefronts are merged at the end.
+// Lanes are grouped LPR to a cache row (16-byte loads, head_dim contiguous); a wavefront covers RPW rows per
+// load and keeps UR loads of keys and of values in flight, refilling each register as soon as it is consumed.
+// Every lane group keeps its own online-softmax state over the rows it visits; the groups of a wavefront are
+// merged with lane shuffles and the NW wavefronts through LDS.
 // sQ: LDS [G][D] queries, already rotated and scaled.  Result (fp32) is written to sOut [G][D] in LDS.
-template <typename CT, int D, int G>
-__device__ __forceinline__ void attn_core(const float* sQ, const CT* Kb, const CT* Vb, int T, float* sM,
-                                          float* sL, float* sAcc, float* sOut) {
+template <typename CT, int D, int G, int NW>
+__device__ __forceinline__ void attn_core(const float* sQ, const CT* Kb, const CT* Vb, int T, float* sM, float* sL, float* sAcc,
+                                          float* sOut) {
     constexpr int EPL = 16 / (int)sizeof(CT);
     constexpr int LPR = D / EPL;
     constexpr int RPW = 64 / LPR;
-    constexpr int NW = 4;
-    constexpr int NG = NW * RPW;
     constexpr int UR = 4;
+    constexpr int SWEEP = NW * RPW * UR;
     typedef CT vec_t __attribute__((ext_vector_type(EPL)));
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int sub = lane % LPR, rg = lane / LPR;
 
-    float q[G][EPL];
+    // fp16 cache: queries are kept as packed halves and the dot product uses v_dot2_f32_f16 (fp32 accumulate);
+    // fp32 cache: plain fp32 multiply-add
+    constexpr bool H16 = sizeof(CT) == 2;
+    float q[H16 ? 1 : G][H16 ? 1 : EPL];
+    half2v q2[H16 ? G : 1][H16 ? EPL / 2 : 1];
 #pragma unroll
-    for (int g = 0; g < G; ++g)
+    for (int g = 0; g < G; ++g) {
+        if constexpr (H16) {
 #pragma unroll
-        for (int e = 0; e < EPL; ++e) q[g][e] = sQ[g * D + sub * EPL + e];
+            for (int e = 0; e < EPL / 2; ++e) {
+                q2[g][e][0] = (half_t)sQ[g * D + sub * EPL + 2 * e];
+                q2[g][e][1] = (half_t)sQ[g * D + sub * EPL + 2 * e + 1];
+            }
+        } else {
+#pragma unroll
+            for (int e = 0; e < EPL; ++e) q[g][e] = sQ[g * D + sub * EPL + e];
+        }
+    }
     float m[G], l[G], acc[G][EPL];
 #pragma unroll
     for (int g = 0; g < G; ++g) {
@@ -439,34 +531,50 @@ __device__ __forceinline__ void attn_core(const float* sQ, const CT* Kb, const C
 #pragma unroll
         for (int e = 0; e < EPL; ++e) acc[g][e] = 0.0f;
     }
-    for (int base = wave * RPW; base < T; base += NW * RPW * UR) {
-        vec_t kv[UR], vv[UR];
-        bool ok[UR];
+    vec_t kv[UR], vv[UR];
+    int tt[UR];
 #pragma unroll
-        for (int u = 0; u < UR; ++u) {
-            int t = base + u * NW * RPW + rg;
-            ok[u] = t < T;
-            if (ok[u]) {
-                kv[u] = *(const vec_t*)(Kb + (long)t * D + sub * EPL);
-                vv[u] = *(const vec_t*)(Vb + (long)t * D + sub * EPL);
-            } else {
+    for (int u = 0; u < UR; ++u) {
+        tt[u] = (u * NW + wave) * RPW + rg;
 #pragma unroll
-                for (int e = 0; e < EPL; ++e) { kv[u][e] = (CT)0.0f; vv[u][e] = (CT)0.0f; }
-            }
+        for (int e = 0; e < EPL; ++e) { kv[u][e] = (CT)0.0f; vv[u][e] = (CT)0.0f; }
+        if (tt[u] < T) {
+            kv[u] = *(const vec_t*)(Kb + (long)tt[u] * D + sub * EPL);
+            vv[u] = *(const vec_t*)(Vb + (long)tt[u] * D + sub * EPL);
         }
+    }
+    for (int base = 0; base < T; base += SWEEP) {
 #pragma unroll
         for (int u = 0; u < UR; ++u) {
+            const bool ok = tt[u] < T;
+            const vec_t kc = kv[u];
+            float vf[EPL];
+#pragma unroll
+            for (int e = 0; e < EPL; ++e) vf[e] = (float)vv[u][e];
+            tt[u] += SWEEP;
+            if (tt[u] < T) {
+                kv[u] = *(const vec_t*)(Kb + (long)tt[u] * D + sub * EPL);
+                vv[u] = *(const vec_t*)(Vb + (long)tt[u] * D + sub * EPL);
+            }
             float s[G];
 #pragma unroll
             for (int g = 0; g < G; ++g) {
                 float d = 0.0f;
+                if constexpr (H16) {
 #pragma unroll
-                for (int e = 0; e < EPL; ++e) d = fmaf(q[g][e], (float)kv[u][e], d);
+                    for (int e = 0; e < EPL / 2; ++e) {
+                        half2v kp; kp[0] = (half_t)kc[2 * e]; kp[1] = (half_t)kc[2 * e + 1];
+                        d = __builtin_amdgcn_fdot2(q2[g][e], kp, d, false);
+                    }
+                } else {
+#pragma unroll
+                    for (int e = 0; e < EPL; ++e) d = fmaf(q[g][e], (float)kc[e], d);
+                }
 #pragma unroll
                 for (int o = LPR / 2; o > 0; o >>= 1) d += __shfl_xor(d, o, 64);
                 s[g] = d;
             }
-            if (ok[u]) {
+            if (ok) {
 #pragma unroll
                 for (int g = 0; g < G; ++g) {
                     float mn = fmaxf(m[g], s[g]);
@@ -474,27 +582,43 @@ __device__ __forceinline__ void attn_core(const float* sQ, const CT* Kb, const C
                     float p = __expf(s[g] - mn);
                     l[g] = l[g] * corr + p;
 #pragma unroll
-                    for (int e = 0; e < EPL; ++e) acc[g][e] = acc[g][e] * corr + p * (float)vv[u][e];
+                    for (int e = 0; e < EPL; ++e) acc[g][e] = acc[g][e] * corr + p * vf[e];
                     m[g] = mn;
                 }
             }
         }
     }
-    const int gi = wave * RPW + rg;
+    // merge the row groups of this wavefront
 #pragma unroll
-    for (int g = 0; g < G; ++g) {
-        if (sub == 0) { sM[gi * G + g] = m[g]; sL[gi * G + g] = l[g]; }
+    for (int o = LPR; o < 64; o <<= 1) {
 #pragma unroll
-        for (int e = 0; e < EPL; ++e) sAcc[(gi * G + g) * D + sub * EPL + e] = acc[g][e];
+        for (int g = 0; g < G; ++g) {
+            float m2 = __shfl_xor(m[g], o, 64), l2 = __shfl_xor(l[g], o, 64);
+            float M = fmaxf(m[g], m2);
+            float w1 = (m[g] == M) ? 1.0f : __expf(m[g] - M);
+            float w2 = (m2 == M) ? 1.0f : __expf(m2 - M);
+            l[g] = l[g] * w1 + l2 * w2;
+#pragma unroll
+            for (int e = 0; e < EPL; ++e) acc[g][e] = acc[g][e] * w1 + __shfl_xor(acc[g][e], o, 64) * w2;
+            m[g] = M;
+        }
+    }
+    if (rg == 0) {
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+            if (sub == 0) { sM[wave * G + g] = m[g]; sL[wave * G + g] = l[g]; }
+#pragma unroll
+            for (int e = 0; e < EPL; ++e) sAcc[(wave * G + g) * D + sub * EPL + e] = acc[g][e];
+        }
     }
     __syncthreads();
-    for (int idx = threadIdx.x; idx < G * D; idx += 256) {
+    for (int idx = threadIdx.x; idx < G * D; idx += NW * 64) {
         int g = idx / D, d = idx % D;
         float M = -INFINITY;
-        for (int i = 0; i < NG; ++i) M = fmaxf(M, sM[i * G + g]);
+        for (int i = 0; i < NW; ++i) M = fmaxf(M, sM[i * G + g]);
         float L = 0.0f, O = 0.0f;
-        for (int i = 0; i < NG; ++i) {
-            float wgt = __expf(sM[i * G + g] - M);    // groups that saw no row have m = -inf -> weight 0
+        for (int i = 0; i < NW; ++i) {
+            float wgt = __expf(sM[i * G + g] - M);    // wavefronts that saw no row have m = -inf -> weight 0
             L += sL[i * G + g] * wgt;
             O += sAcc[(i * G + g) * D + d] * wgt;
         }
@@ -503,15 +627,13 @@ __device__ __forceinline__ void attn_core(const float* sQ, const CT* Kb, const C
     __syncthreads();
 }
 
-template <typename CT, int D, int G>
+template <typename CT, int D, int G, int NW>
 struct AttnSmem {
-    static constexpr int EPL = 16 / (int)sizeof(CT);
-    static constexpr int NG = 4 * (64 / (D / EPL));
     float in[(G + 2) * D];
     float q[G * D];
-    float m[NG * G];
-    float l[NG * G];
-    float acc[NG * G * D];
+    float m[NW * G];
+    float l[NW * G];
+    float acc[NW * G * D];
     float out[G * D];
 };
 
@@ -520,12 +642,13 @@ struct AttnSmem {
 // Replaces: AsContiguous head split, RoPE, GQA Expand, Concate(cache), MulBatch, Softmax, MulBatch, transpose
 // (Seq2SeqSharp/Layers/GroupQueryAttention.cs:121-224, Layers/MultiHeadAttention.cs:133-230).
 template <typename CT, typename AT, int D, int G>
-__global__ __launch_bounds__(256) void attn_decode_kernel(AttnArgs a) {
-    __shared__ AttnSmem<CT, D, G> sm;
+__global__ __launch_bounds__(1024) void attn_decode_kernel(AttnArgs a) {
+    constexpr int NW = 16, NTH = NW * 64;
+    __shared__ AttnSmem<CT, D, G, NW> sm;
     const int kvh = blockIdx.x, b = blockIdx.y, t = threadIdx.x;
     const int pos = *a.d_pos;
     const int HD = a.H * D, GD = a.Hkv * D;
-    for (int idx = t; idx < (G + 2) * D; idx += 256) {
+    for (int idx = t; idx < (G + 2) * D; idx += NTH) {
         int col;
         if (idx < G * D) col = kvh * G * D + idx;
         else if (idx < (G + 1) * D) col = HD + kvh * D + (idx - G * D);
@@ -537,19 +660,23 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(AttnArgs a) {
     __syncthreads();
     CT* Kb = (CT*)a.kcache + ((long)b * a.Hkv + kvh) * a.max_len * D;
     CT* Vb = (CT*)a.vcache + ((long)b * a.Hkv + kvh) * a.max_len * D;
-    for (int p = t; p < (G + 1) * D / 2; p += 256) {
+    for (int p = t; p < (G + 1) * D / 2; p += NTH) {
         int vec = p / (D / 2), i = p % (D / 2);
         float x0 = sm.in[vec * D + 2 * i], x1 = sm.in[vec * D + 2 * i + 1], y0 = x0, y1 = x1;
         if (a.rope_cos) rope_pair(x0, x1, a.rope_cos[(long)pos * (D / 2) + i], a.rope_sin[(long)pos * (D / 2) + i], y0, y1);
         if (vec < G) { sm.q[vec * D + 2 * i] = a.scale * y0; sm.q[vec * D + 2 * i + 1] = a.scale * y1; }
         else { Kb[(long)pos * D + 2 * i] = (CT)y0; Kb[(long)pos * D + 2 * i + 1] = (CT)y1; }
     }
-    for (int d = t; d < D; d += 256) Vb[(long)pos * D + d] = (CT)sm.in[(G + 1) * D + d];
+    for (int d = t; d < D; d += NTH) Vb[(long)pos * D + d] = (CT)sm.in[(G + 1) * D + d];
     __threadfence_block();
     __syncthreads();
-    attn_core<CT, D, G>(sm.q, Kb, Vb, pos + 1, sm.m, sm.l, sm.acc, sm.out);
-    AT* out = (AT*)a.out + (long)b * a.ld_out + kvh * G * D;
-    for (int idx = t; idx < G * D; idx += 256) out[idx] = (AT)sm.out[idx];
+    attn_core<CT, D, G, NW>(sm.q, Kb, Vb, pos + 1, sm.m, sm.l, sm.acc, sm.out);
+    if (a.out_kt > 0) {
+        for (int idx = t; idx < G * D; idx += NTH) ((AT*)a.out)[xpack_index(b, kvh * G * D + idx, a.out_kt)] = (AT)sm.out[idx];
+    } else {
+        AT* out = (AT*)a.out + (long)b * a.ld_out + kvh * G * D;
+        for (int idx = t; idx < G * D; idx += NTH) out[idx] = (AT)sm.out[idx];
+    }
 }
 
 // prefill, step 1: grid (Tq, batch).  Rotates the keys of every position and writes keys and values into the cache.
@@ -581,7 +708,7 @@ __global__ __launch_bounds__(256) void kv_write_kernel(AttnArgs a) {
 // is exactly 0 in fp32, so leaving masked positions out gives the same sums.
 template <typename CT, typename AT, int D, int G>
 __global__ __launch_bounds__(256) void attn_prefill_kernel(AttnArgs a) {
-    __shared__ AttnSmem<CT, D, G> sm;
+    __shared__ AttnSmem<CT, D, G, 4> sm;
     const int tq = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z, t = threadIdx.x;
     const long row = (long)b * a.Tq + tq;
     const int pos = a.pos0 + tq;
@@ -595,7 +722,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(AttnArgs a) {
     __syncthreads();
     const CT* Kb = (const CT*)a.kcache + ((long)b * a.Hkv + kvh) * a.max_len * D;
     const CT* Vb = (const CT*)a.vcache + ((long)b * a.Hkv + kvh) * a.max_len * D;
-    attn_core<CT, D, G>(sm.q, Kb, Vb, pos + 1, sm.m, sm.l, sm.acc, sm.out);
+    attn_core<CT, D, G, 4>(sm.q, Kb, Vb, pos + 1, sm.m, sm.l, sm.acc, sm.out);
     AT* out = (AT*)a.out + row * a.ld_out + kvh * G * D;
     for (int idx = t; idx < G * D; idx += 256) out[idx] = (AT)sm.out[idx];
 }

@@ -9,7 +9,7 @@
 // (TensorApplyCPU.cs:1246), TopK by the reference's insertion rule (TensorApplyCPU.cs:1099-1146).
 #pragma once
 
-#include "tship_internal.h"
+#include "tship_gpt_kernels.h"
 
 namespace tship {
 
@@ -120,12 +120,16 @@ __global__ void moe_lists_kernel(const float* __restrict__ top_idx, int rows, in
 // IndexSelect(inputNorm, tokenIdx_e) for every expert (MoEFeedForward.cs:155): grid (max_rows, E)
 template <typename AT>
 __global__ __launch_bounds__(256) void moe_gather_kernel(const float* __restrict__ xn32, int h, const int* __restrict__ counts,
-                                                          const int* __restrict__ lists, int max_rows, AT* __restrict__ xg, long ld, long estride) {
+                                                          const int* __restrict__ lists, int max_rows, AT* __restrict__ xg, long ld, long estride,
+                                                          int packed_kt) {
     const int j = blockIdx.x, e = blockIdx.y;
     if (j >= counts[e]) return;
     const int tok = lists[e * max_rows + j];
-    AT* dst = xg + e * estride + (long)j * ld;
-    for (int c = threadIdx.x; c < h; c += 256) dst[c] = (AT)xn32[(long)tok * h + c];
+    AT* dst = xg + e * estride;
+    for (int c = threadIdx.x; c < h; c += 256) {
+        if (packed_kt > 0) dst[xpack_index(j, c, packed_kt)] = (AT)xn32[(long)tok * h + c];
+        else dst[(long)j * ld + c] = (AT)xn32[(long)tok * h + c];
+    }
 }
 
 // EltMul by the expert's probability, scatter-add in expert-major order into zeros, then input + result
