@@ -31,7 +31,7 @@ __device__ __forceinline__ float block_max_256(float v, float* s) {
     return fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3]));
 }
 
-__global__ __launch_bounds__(256) void topp_kernel(TopPArgs a) {
+static __global__ __launch_bounds__(256) void topp_kernel(TopPArgs a) {
     __shared__ float sred[4];
     __shared__ unsigned short cnt[16][256];
     __shared__ int s_total[17];
