@@ -94,6 +94,10 @@ struct TSHipGpt {
     // decode state
     DevBuf x, xn, o, a, part_qkv, part_h, part_f, logits, ids, d_pos, hidden;
     DevBuf moe_ws;
+    DevBuf ssq;                    // deferred-norm path: per-column-tile sums of squares [h/32][Bpad]
+    bool fused_norm = false;       // fp16 + RMSNorm + dense layers: residual/norm folded into the GEMM tails
+    bool vt = false;               // fp16 cache with head_dim 64/128: values stored transposed for the MFMA attention kernels
+    long ML = 0;                   // cache rows per (sequence, KV head): max_seq_len rounded up to 32
     int pos = 0;                   // host mirror of *d_pos
     int cur_batch = 0;
     Profiler* prof = nullptr;
@@ -317,6 +321,7 @@ static void run_skinny(TSHipGpt* m, const char* name, const GemmW& w, const void
 #define TSHIP_SK(BTV, NWV)                                                                                                  \
     if (epi == EPI_PARTIAL) launch(m, name, skinny_gemm_f16_kernel<BTV, EPI_PARTIAL, NWV>, grid, dim3(NWV * 64), e);        \
     else if (epi == EPI_F32_BIAS) launch(m, name, skinny_gemm_f16_kernel<BTV, EPI_F32_BIAS, NWV>, grid, dim3(NWV * 64), e); \
+    else if (epi == EPI_RESID_TAIL) launch(m, name, skinny_gemm_f16_kernel<BTV, EPI_RESID_TAIL, NWV>, grid, dim3(NWV * 64), e); \
     else launch(m, name, skinny_gemm_f16_kernel<BTV, EPI_ACT16, NWV>, grid, dim3(NWV * 64), e);
     if (BT == 1) { TSHIP_SK(1, 8) } else if (BT == 2) { TSHIP_SK(2, 8) } else { TSHIP_SK(4, 4) }
 #undef TSHIP_SK
@@ -352,7 +357,17 @@ static AttnKernel pick_attn_d(int D, int G, bool prefill) {
         default: throw Error("head_dim must be 16, 32, 64 or 128");
     }
 }
+template <int D>
+static AttnKernel pick_attn_mfma(int G, bool prefill) {
+    switch (G) {
+        case 1: return prefill ? attn_mfma_kernel<D, 1, true> : attn_mfma_kernel<D, 1, false>;
+        case 2: return prefill ? attn_mfma_kernel<D, 2, true> : attn_mfma_kernel<D, 2, false>;
+        case 4: return prefill ? attn_mfma_kernel<D, 4, true> : attn_mfma_kernel<D, 4, false>;
+        default: throw Error("query heads per KV head must be 1, 2 or 4");
+    }
+}
 static AttnKernel pick_attn(TSHipGpt* m, bool prefill) {
+    if (m->vt) return m->D == 64 ? pick_attn_mfma<64>(m->G, prefill) : pick_attn_mfma<128>(m->G, prefill);
     return m->f16 ? pick_attn_d<half_t, half_t>(m->D, m->G, prefill) : pick_attn_d<float, float>(m->D, m->G, prefill);
 }
 template <typename CT>
@@ -370,7 +385,7 @@ static AttnKernel pick_kvw(TSHipGpt* m) { return m->f16 ? pick_kvw_t<half_t>(m->
 static AttnArgs attn_args(TSHipGpt* m, LayerW& L) {
     AttnArgs a; std::memset(&a, 0, sizeof(a));
     a.bias = L.bqkv.as<float>(); a.H = m->c.n_heads; a.Hkv = m->c.n_kv_heads;
-    a.kcache = L.kc.p; a.vcache = L.vc.p; a.max_len = m->c.max_seq_len;
+    a.kcache = L.kc.p; a.vcache = L.vc.p; a.max_len = m->ML; a.vt = m->vt ? 1 : 0;
     if (m->c.use_rope) { a.rope_cos = m->rope_cos.as<float>(); a.rope_sin = m->rope_sin.as<float>(); }
     a.d_pos = m->d_pos.as<int>();
     a.scale = 1.0f / (float)std::sqrt((double)m->D);   // GroupQueryAttention.cs:193
@@ -386,9 +401,83 @@ static void moe_get_routing(TSHipGpt* m, int layer, float* top_idx, float* top_v
 static void sample_tokens(TSHipGpt* m, int mode, float top_p, float temperature, const float* host_uniforms, const float* dev_uniforms, int B, int* gen_out);
 
 // ------------------------------------------------------------------------------------------------
+// decode step, deferred-norm form (fp16 weights, RMSNorm, dense feed-forward): 5 launches per layer.
+//   gemm_qkv   : X = half(gamma1 * x) packed -> split-K partials
+//   attn_decode: (sum partials) * rinv + bias, RoPE, cache append, attention
+//   gemm_wo    : tail adds partials + b0 + x -> x, half(gamma2 * x), tile sums of squares
+//   gemm_ffn13 : act((X W1) * rinv + b1) * ((X W3) * rinv + b3) -> packed fp16
+//   gemm_ffn2  : tail as gemm_wo, with the next layer's (or the final) gamma
+// rinv = 1 / sqrt(mean(x^2) + eps) is rebuilt by every consumer from the tile sums, so no launch exists only to
+// normalise (RMSNormalization.Norm, Seq2SeqSharp/Layers/RMSNormalization.cs:33-37, folded into its neighbours).
+// ------------------------------------------------------------------------------------------------
+static void decode_step_fn(TSHipGpt* m, const int* d_ids, int B) {
+    auto& c = m->c;
+    const int h = c.hidden, F = c.ffn_dim;
+    const long hp = round_up(h, 32), qp = round_up(m->Nqkv, 32), Vp = round_up(c.vocab, 32);
+    const int NTh = (int)(hp / 32), xkt = (int)(m->ldh / 16);
+    float* ssq = m->ssq.as<float>();
+    auto with_ssq = [&](SkinnyArgs& e) { e.ssq = ssq; e.ssq_nt = NTh; e.ssq_ld = m->Bpad; e.inv_h = 1.0f / (float)h; e.eps = c.norm_eps; };
+    auto tail = [&](SkinnyArgs& e, const float* bias, const float* gamma) {
+        e.out = m->part_h.as<float>(); e.ld_out = (int)hp; e.split_stride = (long)m->Bpad * hp;
+        e.bias = bias; e.n_valid = h; e.x = m->x.as<float>(); e.ldx_res = h; e.gamma = gamma;
+        e.xg16 = m->xn.as<half_t>(); e.xg_kt = xkt; e.ssq_out = ssq; e.ssq_out_ld = m->Bpad;
+    };
+    {
+        FnPrepArgs a; std::memset(&a, 0, sizeof(a));
+        a.x = m->x.as<float>(); a.ldx = h; a.h = h; a.ids = d_ids; a.emb = m->emb.p; a.emb_f16 = 1; a.emb_scale = (float)std::sqrt((double)h);
+        a.gamma = m->L[0]->n1_g.as<float>(); a.xg16 = m->xn.as<half_t>(); a.xg_kt = xkt; a.ssq_out = ssq; a.ssq_ld = m->Bpad;
+        if (h <= 2048) launch(m, "embed_prepare", fn_prepare_kernel<8>, dim3(B), dim3(256), a);
+        else if (h <= 4096) launch(m, "embed_prepare", fn_prepare_kernel<16>, dim3(B), dim3(256), a);
+        else launch(m, "embed_prepare", fn_prepare_kernel<32>, dim3(B), dim3(256), a);
+    }
+    for (int l = 0; l < c.n_layers; ++l) {
+        LayerW& L = *m->L[l];
+        const long qstride = (long)m->Bpad * qp;
+        {
+            SkinnyArgs e; std::memset(&e, 0, sizeof(e));
+            e.out = m->part_qkv.as<float>(); e.ld_out = (int)qp; e.split_stride = qstride;
+            run_skinny(m, "gemm_qkv", L.qkv, m->xn.p, m->ldh, B, EPI_PARTIAL, e);
+        }
+        {
+            AttnArgs a = attn_args(m, L);
+            a.qkv = m->part_qkv.as<float>(); a.KS = L.qkv.KS; a.split_stride = qstride; a.ldq = qp;
+            a.out = m->o.p; a.ld_out = m->ldh; a.out_kt = xkt;
+            a.ssq = ssq; a.ssq_nt = NTh; a.ssq_ld = m->Bpad; a.inv_h = 1.0f / (float)h; a.eps = c.norm_eps;
+            launch(m, "attn_decode", pick_attn(m, false), dim3(c.n_kv_heads, B), dim3(m->vt ? (m->D == 128 ? 256 : 512) : 1024), a);
+        }
+        {
+            SkinnyArgs e; std::memset(&e, 0, sizeof(e));
+            tail(e, L.bo.as<float>(), L.n2_g.as<float>());
+            run_skinny(m, "gemm_wo", L.wo, m->o.p, m->ldh, B, EPI_RESID_TAIL, e);
+        }
+        {
+            SkinnyArgs e; std::memset(&e, 0, sizeof(e));
+            e.bias = L.b1.as<float>(); e.bias2 = L.b3.as<float>(); e.out16 = m->a.as<half_t>(); e.ld16 = (int)m->ldF;
+            e.act = c.act; e.gated = m->gated; e.n_valid = F; e.out16_kt = L.w2.KT;
+            with_ssq(e);
+            run_skinny(m, "gemm_ffn13", L.w13, m->xn.p, m->ldh, B, EPI_ACT16, e);
+        }
+        {
+            SkinnyArgs e; std::memset(&e, 0, sizeof(e));
+            tail(e, L.b2.as<float>(), l + 1 < c.n_layers ? m->L[l + 1]->n1_g.as<float>() : m->fn_g.as<float>());
+            run_skinny(m, "gemm_ffn2", L.w2, m->a.p, m->ldF, B, EPI_RESID_TAIL, e);
+        }
+    }
+    {
+        SkinnyArgs e; std::memset(&e, 0, sizeof(e));
+        e.out = m->logits.as<float>(); e.ld_out = (int)Vp; e.bias = m->head_b.as<float>(); e.n_valid = c.vocab;
+        with_ssq(e);
+        e.advance_pos = m->d_pos.as<int>();
+        run_skinny(m, "gemm_head", m->head, m->xn.p, m->ldh, B, EPI_F32_BIAS, e);
+    }
+    m->pos += 1;
+}
+
+// ------------------------------------------------------------------------------------------------
 // decode step: tokens (device int32 [batch]) -> logits (device fp32 [batch][vocab])
 // ------------------------------------------------------------------------------------------------
 static void decode_step(TSHipGpt* m, const int* d_ids, int B) {
+    if (m->fused_norm) { decode_step_fn(m, d_ids, B); return; }
     auto& c = m->c;
     const int h = c.hidden, F = c.ffn_dim;
     const long hp = round_up(h, 32), qp = round_up(m->Nqkv, 32);
@@ -419,7 +508,7 @@ static void decode_step(TSHipGpt* m, const int* d_ids, int B) {
             AttnArgs a = attn_args(m, L);
             a.qkv = m->part_qkv.as<float>(); a.KS = L.qkv.KS; a.split_stride = qstride; a.ldq = qp;
             a.out = m->o.p; a.ld_out = m->ldh; a.out_kt = m->f16 ? (int)(m->ldh / 16) : 0;
-            launch(m, "attn_decode", pick_attn(m, false), dim3(c.n_kv_heads, B), dim3(1024), a);
+            launch(m, "attn_decode", pick_attn(m, false), dim3(c.n_kv_heads, B), dim3(m->vt ? (m->D == 128 ? 256 : 512) : 1024), a);
         }
         // output projection -> partials
         long hstride = (long)m->Bpad * hp;
@@ -539,7 +628,8 @@ static void prefill(TSHipGpt* m, const int32_t* host_ids, int B, int Tp) {
             run_gemm_f32(m, "p_gemm_qkv", L.qkv, pxn.as<float>(), m->ldh, (int)R, pqkv.as<float>(), qp, 0, 1);
         }
         launch(m, "p_kv_write", pick_kvw(m), dim3(Tp, B), dim3(256), aa);
-        launch(m, "p_attn", pick_attn(m, true), dim3(Tp, c.n_kv_heads, B), dim3(256), aa);
+        if (m->vt) { const int QB = 16 / m->G; launch(m, "p_attn", pick_attn(m, true), dim3((unsigned)ceil_div(Tp, QB), c.n_kv_heads, B), dim3(m->D == 128 ? 256 : 512), aa); }
+        else launch(m, "p_attn", pick_attn(m, true), dim3(Tp, c.n_kv_heads, B), dim3(256), aa);
         ResidNormArgs a2 = rn;
         a2.gamma = L.n2_g.as<float>(); a2.beta = L.n2_b.as<float>();
         if (m->f16) {
@@ -578,7 +668,14 @@ static void prefill(TSHipGpt* m, const int32_t* host_ids, int B, int Tp) {
     for (int b = 0; b < B; ++b) map[b] = Tp * (b + 1) - 1;
     rowmap.alloc(B * sizeof(int));
     TSHIP_CHECK_HIP(hipMemcpyAsync(rowmap.p, map.data(), B * sizeof(int), hipMemcpyHostToDevice, stream()));
-    {
+    if (m->fused_norm) {
+        FnPrepArgs a; std::memset(&a, 0, sizeof(a));
+        a.x = m->x.as<float>(); a.ldx = h; a.h = h; a.src = px.as<float>(); a.ld_src = h; a.row_map = rowmap.as<int>();
+        a.gamma = m->fn_g.as<float>(); a.xg16 = m->xn.as<half_t>(); a.xg_kt = (int)(m->ldh / 16); a.ssq_out = m->ssq.as<float>(); a.ssq_ld = m->Bpad;
+        if (h <= 2048) launch(m, "p_final_prepare", fn_prepare_kernel<8>, dim3(B), dim3(256), a);
+        else if (h <= 4096) launch(m, "p_final_prepare", fn_prepare_kernel<16>, dim3(B), dim3(256), a);
+        else launch(m, "p_final_prepare", fn_prepare_kernel<32>, dim3(B), dim3(256), a);
+    } else {
         ResidNormArgs a = rn;
         a.row_map = rowmap.as<int>(); a.xn = m->xn.p; a.ldxn = m->ldh; a.xn_kt = m->f16 ? (int)(m->ldh / 16) : 0;
         a.gamma = m->fn_g.as<float>(); a.beta = m->fn_b.as<float>();
@@ -588,6 +685,7 @@ static void prefill(TSHipGpt* m, const int32_t* host_ids, int B, int Tp) {
     if (m->f16) {
         SkinnyArgs e; std::memset(&e, 0, sizeof(e));
         e.out = m->logits.as<float>(); e.ld_out = (int)Vp; e.bias = m->head_b.as<float>(); e.n_valid = c.vocab;
+        if (m->fused_norm) { e.ssq = m->ssq.as<float>(); e.ssq_nt = (int)(round_up(h, 32) / 32); e.ssq_ld = m->Bpad; e.inv_h = 1.0f / (float)h; e.eps = c.norm_eps; }
         run_skinny(m, "gemm_head", m->head, m->xn.p, m->ldh, B, EPI_F32_BIAS, e);
     } else {
         run_gemm_f32(m, "gemm_head", m->head, m->xn.as<float>(), m->ldh, B, m->logits.as<float>(), Vp, 0, 1, m->head_b.as<float>());
@@ -639,6 +737,8 @@ TSHIP_API int TSHip_GptCreate(const TSHipGptConfig* cfg, TSHipGpt** out) {
         TSHIP_REQUIRE(!m->gated, "TSHip_GptCreate: the reference's MoE experts are two-matrix MLPs; a gated activation has no third matrix");
     }
     const long h4 = 4L * c.hidden;
+    m->ML = round_up(c.max_seq_len, 32);
+    m->vt = m->f16 && (m->D == 64 || m->D == 128);
     m->ldh = round_up(c.hidden, 16);
     m->ldF = round_up(std::max<long>(c.ffn_dim, c.n_experts > 1 ? h4 : 0), 16);
     const int h = c.hidden;
@@ -647,7 +747,7 @@ TSHIP_API int TSHip_GptCreate(const TSHipGptConfig* cfg, TSHipGpt** out) {
         LayerW& L = *m->L.back();
         L.moe = c.n_experts > 1 && i > 1;      // Networks/GPTDecoder.cs:114-124
         if (L.moe) for (int e = 0; e < c.n_experts; ++e) { L.e1.emplace_back(new GemmW()); L.e2.emplace_back(new GemmW()); }
-        size_t cache_bytes = (size_t)c.max_batch * c.n_kv_heads * c.max_seq_len * m->D * m->esz();
+        size_t cache_bytes = (size_t)c.max_batch * c.n_kv_heads * m->ML * m->D * m->esz();
         L.kc.alloc(cache_bytes); L.vc.alloc(cache_bytes);
     }
     build_expected(m.get());
@@ -681,6 +781,10 @@ TSHIP_API int TSHip_GptCreate(const TSHipGptConfig* cfg, TSHipGpt** out) {
     m->d_pos.alloc(sizeof(int));
     m->hidden.alloc((size_t)m->Bpad * h * sizeof(float));
     if (c.n_experts > 1) moe_alloc(m.get());
+    m->fused_norm = m->f16 && c.norm_type == 0 && c.n_experts <= 1;
+    if (m->fused_norm) {
+        m->ssq.alloc((size_t)(hp / 32) * m->Bpad * sizeof(float));
+    }
     TSHIP_CHECK_HIP(hipStreamSynchronize(stream()));
     *out = m.release();
     TSHIP_END
@@ -824,7 +928,18 @@ TSHIP_API int TSHip_GptGetHidden(TSHipGpt* m, float* host_out) {
     TSHIP_REQUIRE(m->cur_batch > 0, "TSHip_GptGetHidden: nothing computed yet");
     const int B = m->cur_batch, h = m->c.hidden;
     TSHIP_CHECK_HIP(hipStreamSynchronize(stream()));
-    if (m->f16) {
+    if (m->fused_norm) {
+        // the normalised hidden state is never materialised on this path: rebuild it from the residual stream
+        std::vector<float> xs((size_t)B * h), gm(h);
+        TSHIP_CHECK_HIP(hipMemcpy(xs.data(), m->x.p, xs.size() * sizeof(float), hipMemcpyDeviceToHost));
+        TSHIP_CHECK_HIP(hipMemcpy(gm.data(), m->fn_g.p, gm.size() * sizeof(float), hipMemcpyDeviceToHost));
+        for (int b = 0; b < B; ++b) {
+            double sq = 0.0;
+            for (int i = 0; i < h; ++i) sq += (double)xs[(size_t)b * h + i] * xs[(size_t)b * h + i];
+            float rms = (float)std::sqrt(sq / h + m->c.norm_eps);
+            for (int i = 0; i < h; ++i) host_out[(size_t)b * h + i] = gm[i] * (xs[(size_t)b * h + i] / rms);
+        }
+    } else if (m->f16) {
         std::vector<half_t> tmp((size_t)m->Bpad * m->ldh);
         TSHIP_CHECK_HIP(hipMemcpy(tmp.data(), m->xn.p, tmp.size() * sizeof(half_t), hipMemcpyDeviceToHost));
         const int KT = (int)(m->ldh / 16);
@@ -853,15 +968,18 @@ TSHIP_API int TSHip_GptGetKV(TSHipGpt* m, int layer, int which, float* host_out)
     TSHIP_BEGIN
     TSHIP_REQUIRE(m && host_out, "TSHip_GptGetKV: null argument");
     TSHIP_REQUIRE(layer >= 0 && layer < m->c.n_layers && (which == 0 || which == 1), "TSHip_GptGetKV: bad layer or selector");
-    const int B = m->cur_batch, G = m->c.n_kv_heads, D = m->D, T = m->pos; const long ML = m->c.max_seq_len;
+    const int B = m->cur_batch, G = m->c.n_kv_heads, D = m->D, T = m->pos; const long ML = m->ML;
     TSHIP_CHECK_HIP(hipStreamSynchronize(stream()));
     const char* base = (const char*)(which ? m->L[layer]->vc.p : m->L[layer]->kc.p);
-    std::vector<char> tmp((size_t)T * D * m->esz());
+    const bool transposed = which == 1 && m->vt;          // values are kept [D][ML] for the MFMA attention kernels
+    std::vector<char> tmp((size_t)ML * D * m->esz());
     for (int b = 0; b < B; ++b) for (int g = 0; g < G; ++g) {
         TSHIP_CHECK_HIP(hipMemcpy(tmp.data(), base + ((size_t)b * G + g) * ML * D * m->esz(), tmp.size(), hipMemcpyDeviceToHost));
         float* dst = host_out + ((size_t)b * G + g) * T * D;
-        if (m->f16) { const half_t* s = (const half_t*)tmp.data(); for (long i = 0; i < (long)T * D; ++i) dst[i] = (float)s[i]; }
-        else std::memcpy(dst, tmp.data(), tmp.size());
+        for (long t = 0; t < T; ++t) for (int d = 0; d < D; ++d) {
+            size_t idx = transposed ? (size_t)d * ML + t : (size_t)t * D + d;
+            dst[t * D + d] = m->f16 ? (float)((const half_t*)tmp.data())[idx] : ((const float*)tmp.data())[idx];
+        }
     }
     TSHIP_END
 }
@@ -881,13 +999,16 @@ TSHIP_API int TSHip_GptSetKV(TSHipGpt* m, int layer, int which, const float* hos
     TSHIP_REQUIRE(m && host_in, "TSHip_GptSetKV: null argument");
     TSHIP_REQUIRE(layer >= 0 && layer < m->c.n_layers && (which == 0 || which == 1), "TSHip_GptSetKV: bad layer or selector");
     TSHIP_REQUIRE(batch >= 1 && batch <= m->c.max_batch && len >= 0 && len <= m->c.max_seq_len, "TSHip_GptSetKV: out of range");
-    const int G = m->c.n_kv_heads, D = m->D; const long ML = m->c.max_seq_len;
+    const int G = m->c.n_kv_heads, D = m->D; const long ML = m->ML;
     char* base = (char*)(which ? m->L[layer]->vc.p : m->L[layer]->kc.p);
-    std::vector<char> tmp((size_t)len * D * m->esz());
+    const bool transposed = which == 1 && m->vt;
+    std::vector<char> tmp((size_t)ML * D * m->esz(), 0);
     for (int b = 0; b < batch; ++b) for (int g = 0; g < G; ++g) {
         const float* src = host_in + ((size_t)b * G + g) * len * D;
-        if (m->f16) { half_t* d = (half_t*)tmp.data(); for (long i = 0; i < (long)len * D; ++i) d[i] = (half_t)src[i]; }
-        else std::memcpy(tmp.data(), src, tmp.size());
+        for (long t = 0; t < len; ++t) for (int d = 0; d < D; ++d) {
+            size_t idx = transposed ? (size_t)d * ML + t : (size_t)t * D + d;
+            if (m->f16) ((half_t*)tmp.data())[idx] = (half_t)src[t * D + d]; else ((float*)tmp.data())[idx] = src[t * D + d];
+        }
         TSHIP_CHECK_HIP(hipMemcpy(base + ((size_t)b * G + g) * ML * D * m->esz(), tmp.data(), tmp.size(), hipMemcpyHostToDevice));
     }
     TSHIP_END

@@ -115,7 +115,7 @@ static void sample_tokens(TSHipGpt* m, int mode, float top_p, float temperature,
                           int* gen_out) {
     const long Vp = round_up(m->c.vocab, 32);
     if (mode == TSHIP_GREEDY) {
-        launch(m, "greedy", greedy_kernel, dim3(B), dim3(256), (const float*)m->logits.as<float>(), Vp, m->c.vocab, m->ids.as<int>(), gen_out);
+        launch(m, "greedy", greedy_kernel, dim3(B), dim3(1024), (const float*)m->logits.as<float>(), Vp, m->c.vocab, m->ids.as<int>(), gen_out, (const int*)nullptr);
         return;
     }
     TSHIP_REQUIRE(mode == TSHIP_TOPP, "unknown sampling mode");

@@ -78,7 +78,7 @@ __global__ void copy_cols_kernel(const float* __restrict__ src, long ld_src, lon
 // A block owns one 32-column tile and one k-split; its 4 wavefronts split the k range again and are
 // reduced through LDS.  HBM-bound: every weight byte is read exactly once with 16-byte loads.
 // ------------------------------------------------------------------------------------------------
-enum { EPI_PARTIAL = 0, EPI_F32_BIAS = 1, EPI_ACT16 = 2 };
+enum { EPI_PARTIAL = 0, EPI_F32_BIAS = 1, EPI_ACT16 = 2, EPI_RESID_TAIL = 3 };
 
 struct SkinnyArgs {
     const half_t* W; int KT; int NT;
@@ -92,6 +92,13 @@ struct SkinnyArgs {
     // optional batch of independent problems (MoE experts) on blockIdx.y: weights from a pointer table,
     // activations / outputs at a fixed stride, row counts read on the device
     const half_t* const* Wtab; long x_estride; long out_estride; long out16_estride; const int* rows_tab;
+    // deferred RMSNorm: the input rows were stored as half(gamma * x); the epilogue multiplies row b by
+    // 1 / sqrt(sum_t ssq[t][b] / h + eps), the factor the norm would have applied (exact up to rounding)
+    const float* ssq; int ssq_nt; int ssq_ld; float inv_h; float eps;
+    // EPI_RESID_TAIL (KS == 1: the block holds the complete sums of its column tile): adds bias and residual, stores
+    // x, the next GEMM's packed input half(gamma * x) and the tile's per-row sum of squares
+    float* x; int ldx_res; const float* gamma; half_t* xg16; int xg_kt; float* ssq_out; int ssq_out_ld;
+    int* advance_pos;      // optional: one thread of the launch increments this device counter
 };
 
 // NW wavefronts per block work on the same 32-column tile and split the block's k range; every wavefront keeps
@@ -147,6 +154,25 @@ __global__ __launch_bounds__(NW * 64) void skinny_gemm_f16_kernel(SkinnyArgs a) 
             }
         }
     }
+    // rinv per row from the tile sums: NCH chunks of tiles are added in parallel, then the chunk sums in order
+    __shared__ float srinv[BT * 32];
+    constexpr int NCH = (NW * 64) / (BT * 32);
+    __shared__ float schunk[NCH][BT * 32];
+    if (a.ssq) {
+        const int b = threadIdx.x % (BT * 32), ch = threadIdx.x / (BT * 32);
+        const int per_ch = (a.ssq_nt + NCH - 1) / NCH;
+        float s = 0.0f;
+        for (int t = ch * per_ch; t < min(a.ssq_nt, (ch + 1) * per_ch); ++t) s += a.ssq[(long)t * a.ssq_ld + b];
+        schunk[ch][b] = s;
+        __syncthreads();
+        if (threadIdx.x < BT * 32) {
+            float tot = 0.0f;
+#pragma unroll
+            for (int c = 0; c < NCH; ++c) tot += schunk[c][threadIdx.x];
+            srinv[threadIdx.x] = 1.0f / sqrtf(tot * a.inv_h + a.eps);
+        }
+    }
+    if (a.advance_pos && blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) *a.advance_pos += 1;
     // pairwise tree over wavefronts down to two: in each round the upper half stores, the lower half adds
 #pragma unroll
     for (int half = NW / 2; half >= 2; half >>= 1) {
@@ -173,30 +199,57 @@ __global__ __launch_bounds__(NW * 64) void skinny_gemm_f16_kernel(SkinnyArgs a) 
             for (int v = 0; v < 16; ++v) fin[w][bt * 32 + (lane & 31)][8 * (v / 4) + 4 * (lane >> 5) + (v % 4)] = acc[bt][v];
     }
     __syncthreads();
-    for (int idx = threadIdx.x; idx < BT * 1024; idx += NW * 64) {
+    constexpr int ITER = BT * 1024 / (NW * 64);
+    float keep[ITER];
+#pragma unroll
+    for (int it = 0; it < ITER; ++it) {
+        const int idx = threadIdx.x + it * NW * 64;
         const int n = idx & 31, b = idx >> 5;
+        keep[it] = 0.0f;
         if (b >= a.rows_valid) continue;
-        const float s = NW >= 2 ? fin[0][b][n] + fin[1][b][n] : fin[0][b][n];
+        float s = fin[0][b][n] + fin[1][b][n];
+        const float rinv = a.ssq ? srinv[b] : 1.0f;
         if (EPI == EPI_PARTIAL) {
             a.out[ks * a.split_stride + (long)b * a.ld_out + nt * 32 + n] = s;
+        } else if (EPI == EPI_RESID_TAIL) {
+            keep[it] = s;
         } else if (EPI == EPI_F32_BIAS) {
             const int col = nt * 32 + n;
-            if (col < a.n_valid) a.out[(long)b * a.ld_out + col] = s + a.bias[col];
+            if (col < a.n_valid) a.out[(long)b * a.ld_out + col] = s * rinv + a.bias[col];
         } else {
             float val; int f; bool ok;
             if (a.gated) {
                 const float c = fin[0][b][(n & 15) + 16] + fin[1][b][(n & 15) + 16];
                 f = nt * 16 + n; ok = n < 16 && f < a.n_valid;
-                val = ok ? act_apply(a.act, s + a.bias[f]) * (c + a.bias2[f]) : 0.0f;
+                val = ok ? act_apply(a.act, s * rinv + a.bias[f]) * (c * rinv + a.bias2[f]) : 0.0f;
             } else {
                 f = nt * 32 + n; ok = f < a.n_valid;
-                val = ok ? act_apply(a.act, s + a.bias[f]) : 0.0f;
+                val = ok ? act_apply(a.act, s * rinv + a.bias[f]) : 0.0f;
             }
             if (ok) {
                 if (a.out16_kt > 0) a.out16[xpack_index(b, f, a.out16_kt)] = (half_t)val;
                 else a.out16[(long)b * a.ld16 + f] = (half_t)val;
             }
         }
+    }
+    if (EPI != EPI_RESID_TAIL) return;
+#pragma unroll
+    for (int it = 0; it < ITER; ++it) {
+        const int idx = threadIdx.x + it * NW * 64;
+        const int n = idx & 31, b = idx >> 5;
+        if (b >= a.rows_valid) continue;                      // uniform over the 32 lanes that share a row
+        const int col = nt * 32 + n;
+        float v = keep[it];
+        float q = 0.0f;
+        if (col < a.n_valid) {
+            v = (v + a.bias[col]) + a.x[(long)b * a.ldx_res + col];
+            a.x[(long)b * a.ldx_res + col] = v;
+            a.xg16[xpack_index(b, col, a.xg_kt)] = (half_t)(a.gamma[col] * v);
+            q = v * v;
+        }
+#pragma unroll
+        for (int o = 16; o > 0; o >>= 1) q += __shfl_xor(q, o, 64);
+        if (n == 0) a.ssq_out[(long)nt * a.ssq_out_ld + b] = q;
     }
 }
 
@@ -463,6 +516,38 @@ __global__ __launch_bounds__(256) void resid_norm_kernel(ResidNormArgs a) {
     }
 }
 
+// Deferred-norm entry: x = E[id] * scale (or x = row row_map[r] of an existing stream) -> the next GEMM's packed
+// input half(gamma * x) and the per-column-tile sums of squares.  One block per row.
+struct FnPrepArgs {
+    float* x; long ldx; int h;
+    const int* ids; const void* emb; int emb_f16; float emb_scale;
+    const float* src; long ld_src; const int* row_map;
+    const float* gamma; half_t* xg16; int xg_kt; float* ssq_out; int ssq_ld;
+};
+template <int NPT>
+__global__ __launch_bounds__(256) void fn_prepare_kernel(FnPrepArgs a) {
+    const int r = blockIdx.x, t = threadIdx.x;
+    const long erow = a.ids ? (long)a.ids[r] : 0;
+    const long srow = a.row_map ? a.row_map[r] : r;
+#pragma unroll
+    for (int i = 0; i < NPT; ++i) {
+        const int c = t + i * 256;
+        float v = 0.0f;
+        if (c < a.h) {
+            if (a.ids) {
+                float e = a.emb_f16 ? (float)((const half_t*)a.emb)[erow * a.h + c] : ((const float*)a.emb)[erow * a.h + c];
+                v = e * a.emb_scale;
+            } else v = a.src[srow * a.ld_src + c];
+            a.x[(long)r * a.ldx + c] = v;
+            a.xg16[xpack_index(r, c, a.xg_kt)] = (half_t)(a.gamma[c] * v);
+        }
+        float q = v * v;
+#pragma unroll
+        for (int o = 16; o > 0; o >>= 1) q += __shfl_xor(q, o, 64);
+        if ((t & 31) == 0 && c < a.h) a.ssq_out[(long)(c >> 5) * a.ssq_ld + r] = q;
+    }
+}
+
 // ------------------------------------------------------------------------------------------------
 // attention
 // ------------------------------------------------------------------------------------------------
@@ -478,6 +563,8 @@ struct AttnArgs {
     void* out; long ld_out;                        // [rows][H*D] in the activation type
     int out_kt;                                    // > 0: out is fragment packed with this many k-tiles
     float scale;
+    const float* ssq; int ssq_nt; int ssq_ld; float inv_h; float eps;   // deferred RMSNorm of the projection input (see SkinnyArgs)
+    int vt;      // 1: the value cache is stored transposed, [batch][kv_head][D][max_len] (MFMA attention kernels)
 };
 
 // rotary embedding of one (even, odd) pair, two roundings per output like the reference's C# expression
@@ -648,6 +735,13 @@ __global__ __launch_bounds__(1024) void attn_decode_kernel(AttnArgs a) {
     const int kvh = blockIdx.x, b = blockIdx.y, t = threadIdx.x;
     const int pos = *a.d_pos;
     const int HD = a.H * D, GD = a.Hkv * D;
+    float rinv = 1.0f;
+    if (a.ssq) {
+        float s = 0.0f;
+        for (int tt = (t & 63); tt < a.ssq_nt; tt += 64) s += a.ssq[(long)tt * a.ssq_ld + b];
+        s = wave_sum(s);                                   // same butterfly in every wavefront: identical result
+        rinv = 1.0f / sqrtf(s * a.inv_h + a.eps);
+    }
     for (int idx = t; idx < (G + 2) * D; idx += NTH) {
         int col;
         if (idx < G * D) col = kvh * G * D + idx;
@@ -655,7 +749,7 @@ __global__ __launch_bounds__(1024) void attn_decode_kernel(AttnArgs a) {
         else col = HD + GD + kvh * D + (idx - (G + 1) * D);
         float s = a.qkv[(long)b * a.ldq + col];
         for (int k = 1; k < a.KS; ++k) s += a.qkv[k * a.split_stride + (long)b * a.ldq + col];
-        sm.in[idx] = s + a.bias[col];
+        sm.in[idx] = s * rinv + a.bias[col];
     }
     __syncthreads();
     CT* Kb = (CT*)a.kcache + ((long)b * a.Hkv + kvh) * a.max_len * D;
@@ -699,7 +793,9 @@ __global__ __launch_bounds__(256) void kv_write_kernel(AttnArgs a) {
     for (int p = t; p < GD; p += 256) {
         int kvh = p / D, d = p % D;
         int col = HD + GD + p;
-        Vb[((long)kvh * a.max_len + pos) * D + d] = (CT)(a.qkv[row * a.ldq + col] + a.bias[col]);
+        const float val = a.qkv[row * a.ldq + col] + a.bias[col];
+        if (a.vt) Vb[((long)kvh * D + d) * a.max_len + pos] = (CT)val;
+        else Vb[((long)kvh * a.max_len + pos) * D + d] = (CT)val;
     }
 }
 
@@ -727,21 +823,203 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(AttnArgs a) {
     for (int idx = t; idx < G * D; idx += 256) out[idx] = (AT)sm.out[idx];
 }
 
+
+// ------------------------------------------------------------------------------------------------
+// MFMA attention (fp16 cache, head_dim 64 or 128).  One block per (batch row, KV head) and QB query positions
+// (decode: 1, prefill: 16 / G); the 16 columns of v_mfma_f32_16x16x32_f16 are (query position, query head of the
+// group).  Keys are row-major [T][D]; values are stored TRANSPOSED [D][max_len] so that both products read
+// 16-byte runs:
+//   S[32 t][16 col]   = K tile (two 16-row A operands, rows permuted so that lane group q ends up with
+//                       t = t0 + 8q .. 8q+7)  x  Q (B operand, kept in registers)
+//   O^T[D][16 col]   += V^T tile (A operand: 16 d-rows x 32 t)  x  P (B operand: the lane's own 8 probabilities)
+// Online softmax per column with one running maximum per wavefront; wavefronts take 32-row chunks round robin and
+// are merged through LDS.  All arithmetic on scores, probabilities' sums and outputs is fp32.
+// ------------------------------------------------------------------------------------------------
+template <int D, int G, bool PREFILL>
+__global__ __launch_bounds__(D == 128 ? 256 : 512) void attn_mfma_kernel(AttnArgs a) {
+    constexpr int NW = D == 128 ? 4 : 8, NTH = NW * 64;
+    constexpr int QB = PREFILL ? 16 / G : 1, NCOL = QB * G;
+    constexpr int KD = D / 32, DT = D / 16;
+    __shared__ float sIn[(G + 2) * D];
+    __shared__ float sQ[16][D];
+    __shared__ float sM[NW][16];
+    __shared__ float sL[NW][16];
+    __shared__ float sO[NW][D][16];
+    const int t = threadIdx.x, lane = t & 63, w = __builtin_amdgcn_readfirstlane(t >> 6);
+    const int r16 = lane & 15, q = lane >> 4;
+    const int HD = a.H * D, GD = a.Hkv * D;
+    int kvh, b, tq0 = 0, pos_base, T;
+    if (PREFILL) { kvh = blockIdx.y; b = blockIdx.z; tq0 = blockIdx.x * QB; pos_base = a.pos0 + tq0; T = min(pos_base + QB, a.pos0 + a.Tq); }
+    else { kvh = blockIdx.x; b = blockIdx.y; pos_base = *a.d_pos; T = pos_base + 1; }
+    half_t* Kb = (half_t*)a.kcache + ((long)b * a.Hkv + kvh) * a.max_len * D;
+    half_t* Vt = (half_t*)a.vcache + ((long)b * a.Hkv + kvh) * (long)D * a.max_len;
+
+    for (int i = t; i < 16 * D; i += NTH) (&sQ[0][0])[i] = 0.0f;
+    if (!PREFILL) {
+        float rinv = 1.0f;
+        if (a.ssq) {
+            float s = 0.0f;
+            for (int tt = lane; tt < a.ssq_nt; tt += 64) s += a.ssq[(long)tt * a.ssq_ld + b];
+            s = wave_sum(s);
+            rinv = 1.0f / sqrtf(s * a.inv_h + a.eps);
+        }
+        for (int idx = t; idx < (G + 2) * D; idx += NTH) {
+            int col;
+            if (idx < G * D) col = kvh * G * D + idx;
+            else if (idx < (G + 1) * D) col = HD + kvh * D + (idx - G * D);
+            else col = HD + GD + kvh * D + (idx - (G + 1) * D);
+            float s = a.qkv[(long)b * a.ldq + col];
+            for (int k = 1; k < a.KS; ++k) s += a.qkv[k * a.split_stride + (long)b * a.ldq + col];
+            sIn[idx] = s * rinv + a.bias[col];
+        }
+        __syncthreads();
+        const int pos = pos_base;
+        for (int p = t; p < (G + 1) * D / 2; p += NTH) {
+            int vec = p / (D / 2), i = p % (D / 2);
+            float x0 = sIn[vec * D + 2 * i], x1 = sIn[vec * D + 2 * i + 1], y0 = x0, y1 = x1;
+            if (a.rope_cos) rope_pair(x0, x1, a.rope_cos[(long)pos * (D / 2) + i], a.rope_sin[(long)pos * (D / 2) + i], y0, y1);
+            if (vec < G) { sQ[vec][2 * i] = a.scale * y0; sQ[vec][2 * i + 1] = a.scale * y1; }
+            else { Kb[(long)pos * D + 2 * i] = (half_t)y0; Kb[(long)pos * D + 2 * i + 1] = (half_t)y1; }
+        }
+        for (int d = t; d < D; d += NTH) Vt[(long)d * a.max_len + pos] = (half_t)sIn[(G + 1) * D + d];
+        __threadfence_block();
+    } else {
+        __syncthreads();
+        for (int p = t; p < NCOL * D / 2; p += NTH) {
+            int col = p / (D / 2), i = p % (D / 2);
+            int qi = col / G, g = col % G;
+            if (tq0 + qi >= a.Tq) continue;
+            long row = (long)b * a.Tq + tq0 + qi;
+            int pos = pos_base + qi;
+            int c0 = (kvh * G + g) * D + 2 * i;
+            float x0 = a.qkv[row * a.ldq + c0] + a.bias[c0], x1 = a.qkv[row * a.ldq + c0 + 1] + a.bias[c0 + 1], y0 = x0, y1 = x1;
+            if (a.rope_cos) rope_pair(x0, x1, a.rope_cos[(long)pos * (D / 2) + i], a.rope_sin[(long)pos * (D / 2) + i], y0, y1);
+            sQ[col][2 * i] = a.scale * y0; sQ[col][2 * i + 1] = a.scale * y1;
+        }
+    }
+    __syncthreads();
+
+    // B operand of the score product: lane (col = r16, q) holds Q[col][kd*32 + 8q .. +7]
+    half8 qf[KD];
+#pragma unroll
+    for (int kd = 0; kd < KD; ++kd)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) qf[kd][j] = (half_t)sQ[r16][kd * 32 + 8 * q + j];
+    // last position this lane's column may attend to
+    const int qi_lane = PREFILL ? r16 / G : 0;
+    const int tmax = PREFILL ? pos_base + qi_lane : T - 1;
+    const bool col_ok = r16 < NCOL;
+
+    float m_run = -INFINITY, l_run = 0.0f;
+    floatx4 acc_o[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) acc_o[dt] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+
+    const int nchunks = (T + 31) / 32;
+    // row of the key tile this lane loads: tile 0 rows -> t0 + 8*(r/4) + r%4, tile 1 rows -> + 4
+    const int krow = 8 * (r16 >> 2) + (r16 & 3);
+    for (int c = w; c < nchunks; c += NW) {
+        const int t0 = c * 32;
+        half8 kf[2][KD], vf[DT];
+#pragma unroll
+        for (int tile = 0; tile < 2; ++tile)
+#pragma unroll
+            for (int kd = 0; kd < KD; ++kd) kf[tile][kd] = *(const half8*)(Kb + (long)(t0 + krow + 4 * tile) * D + kd * 32 + 8 * q);
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) vf[dt] = *(const half8*)(Vt + (long)(dt * 16 + r16) * a.max_len + t0 + 8 * q);
+        floatx4 sA = floatx4{0.0f, 0.0f, 0.0f, 0.0f}, sB = sA;
+#pragma unroll
+        for (int kd = 0; kd < KD; ++kd) {
+            sA = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf[0][kd], qf[kd], sA, 0, 0, 0);
+            sB = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf[1][kd], qf[kd], sB, 0, 0, 0);
+        }
+        // this lane: column r16, positions t0 + 8q + j  (j < 4 from sA, j >= 4 from sB)
+        float s[8];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) { s[j] = sA[j]; s[4 + j] = sB[j]; }
+        float cm = -INFINITY;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const int tj = t0 + 8 * q + j;
+            if (col_ok && tj > tmax) s[j] = -INFINITY;
+            if (!col_ok) s[j] = 0.0f;
+            cm = fmaxf(cm, s[j]);
+        }
+        cm = fmaxf(cm, __shfl_xor(cm, 16, 64));
+        cm = fmaxf(cm, __shfl_xor(cm, 32, 64));
+        const float m_new = fmaxf(m_run, cm);
+        const float corr = (m_new == -INFINITY) ? 1.0f : __expf(m_run - m_new);     // m_run = -inf -> 0, and the sums are still 0
+        half8 pf;
+        float psum = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const float p = (s[j] == -INFINITY) ? 0.0f : __expf(s[j] - m_new);
+            psum += p;
+            pf[j] = (half_t)p;
+        }
+        l_run = l_run * corr + psum;
+        m_run = m_new;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc_o[dt][i] *= corr;
+            acc_o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vf[dt], pf, acc_o[dt], 0, 0, 0);
+        }
+    }
+    // the four lane groups of a column saw different positions: add their sums (the maximum is already common)
+    l_run += __shfl_xor(l_run, 16, 64);
+    l_run += __shfl_xor(l_run, 32, 64);
+    if (q == 0) { sM[w][r16] = m_run; sL[w][r16] = l_run; }
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) sO[w][dt * 16 + 4 * q + i][r16] = acc_o[dt][i];
+    __syncthreads();
+    for (int idx = t; idx < NCOL * D; idx += NTH) {
+        const int col = idx % NCOL, d = idx / NCOL;
+        float M = -INFINITY;
+#pragma unroll
+        for (int i = 0; i < NW; ++i) M = fmaxf(M, sM[i][col]);
+        float L = 0.0f, O = 0.0f;
+#pragma unroll
+        for (int i = 0; i < NW; ++i) {
+            const float wgt = (sM[i][col] == -INFINITY) ? 0.0f : __expf(sM[i][col] - M);
+            L += sL[i][col] * wgt;
+            O += sO[i][d][col] * wgt;
+        }
+        const float o = O / L;
+        const int qi = col / G, g = col % G;
+        if (PREFILL) {
+            if (tq0 + qi < a.Tq) {
+                half_t* out = (half_t*)a.out + ((long)b * a.Tq + tq0 + qi) * a.ld_out + (kvh * G + g) * D;
+                out[d] = (half_t)o;
+            }
+        } else {
+            const int kcol = (kvh * G + g) * D + d;
+            if (a.out_kt > 0) ((half_t*)a.out)[xpack_index(b, kcol, a.out_kt)] = (half_t)o;
+            else ((half_t*)a.out)[(long)b * a.ld_out + kcol] = (half_t)o;
+        }
+    }
+}
+
 // ------------------------------------------------------------------------------------------------
 // sampling on the device
 // ------------------------------------------------------------------------------------------------
 // Greedy: argmax over a row of logits, lowest index among equal maxima (TensorApplyCPU.cs:339-360 applied to the
 // softmax output; softmax is monotone, so the winner is the same up to ties created by rounding of the division).
-__global__ __launch_bounds__(256) void greedy_kernel(const float* __restrict__ logits, long ld, int V, int* __restrict__ next_ids,
-                                                     int* __restrict__ gen_out) {
-    __shared__ float sv[4];
-    __shared__ int si[4];
+__global__ __launch_bounds__(1024) void greedy_kernel(const float* __restrict__ logits, long ld, int V, int* __restrict__ next_ids,
+                                                      int* __restrict__ gen_out, const int* __restrict__ d_step) {
+    __shared__ float sv[16];
+    __shared__ int si[16];
     const int b = blockIdx.x, t = threadIdx.x;
     const float* row = logits + (long)b * ld;
     float best = -INFINITY; int bi = 0x7fffffff;
-    for (int i = t; i < V; i += 256) {
-        float v = row[i];
-        if (v > best || (v == best && i < bi)) { best = v; bi = i; }
+    for (int i0 = t; i0 < V; i0 += 1024 * 8) {
+        float v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) { int i = i0 + u * 1024; v[u] = i < V ? row[i] : -INFINITY; }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) { int i = i0 + u * 1024; if (i < V && (v[u] > best || (v[u] == best && i < bi))) { best = v[u]; bi = i; } }
     }
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) {
@@ -751,10 +1029,10 @@ __global__ __launch_bounds__(256) void greedy_kernel(const float* __restrict__ l
     if ((t & 63) == 0) { sv[t >> 6] = best; si[t >> 6] = bi; }
     __syncthreads();
     if (t == 0) {
-        for (int w = 1; w < 4; ++w) if (sv[w] > best || (sv[w] == best && si[w] < bi)) { best = sv[w]; bi = si[w]; }
+        for (int w = 1; w < 16; ++w) if (sv[w] > best || (sv[w] == best && si[w] < bi)) { best = sv[w]; bi = si[w]; }
         if (bi == 0x7fffffff) bi = 0;   // a row of NaNs: the reference's scan never moves off index 0
         next_ids[b] = bi;
-        if (gen_out) gen_out[b] = bi;
+        if (gen_out) gen_out[(d_step ? (long)*d_step * gridDim.x : 0) + b] = bi;
     }
 }
 
