@@ -69,6 +69,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-topp", action="store_true")
     ap.add_argument("--prompt", type=int, default=0, help="override the prompt length")
+    ap.add_argument("--no-copy-calibration", action="store_true",
+                    help="skip the 256 MiB plain copy that gives rocprofv3 counter runs a kernel of known traffic")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build drives one GPU per process and measures one GPU; --gpus %d is not supported "
@@ -127,6 +129,22 @@ def main():
     dom_gbs = dom_bytes / (dom_ms / 1e3) / 1e9
     kernel_ms = {k: round(float(np.sum(v)) / n_prof, 4) for k, v in acc.items()}
 
+    # a plain copy of known size: the reference point for scaling FETCH_SIZE / WRITE_SIZE in counter runs
+    if not args.no_copy_calibration:
+        from seq2seqsharp_amd import ops
+        from seq2seqsharp_amd.tensor import HipTensor
+        src = ops.fill(HipTensor([64 * 1024 * 1024]), 1.0)        # 256 MiB of float32
+        dst = HipTensor([64 * 1024 * 1024])
+        ops.copy(dst, src)
+        ops.copy(dst, src)
+        src.dispose()
+        dst.dispose()
+
+    traffic = None
+    tpath = os.path.join(ROOT, "profiles", "decode_%s_ffn13_traffic.json" % args.config)
+    if os.path.exists(tpath):
+        traffic = json.load(open(tpath)).get("traffic_bytes_per_launch")
+
     out = {
         "metric": "decode tokens/s on 1 GPU (1B GQA fp16, batch 32)" if args.config == "cfg2_1b_gqa_f16" else "decode tokens/s on 1 GPU",
         "value": round(tok_s, 1), "unit": "tokens/s", "n_gpus": 1, "steps": K, "warmup": W,
@@ -135,7 +153,7 @@ def main():
         "config": {"workload": args.config, "batch": B, "prompt_len": Tp, "kv_len_start": T_start, "kv_len_end": T_end,
                    "sampling": "greedy", "rope_base": cfg["rope_base"]},
         "roofline": {"bound": "hbm", "achieved": round(dom_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(dom_gbs / HBM_PEAK_GBS, 4), "traffic": None,
+                     "frac": round(dom_gbs / HBM_PEAK_GBS, 4), "traffic": traffic,
                      "kernel": "skinny_gemm_f16_kernel<%d, EPI_ACT16> (%s)" % (1 if B <= 32 else 2 if B <= 64 else 4, dom),
                      "bytes_per_launch": dom_bytes, "avg_launch_ms": round(dom_ms, 5)},
         "whole_step": {"algorithmic_bytes": round(step_bytes), "achieved_GBps": round(step_gbs, 1),

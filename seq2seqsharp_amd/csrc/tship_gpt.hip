@@ -14,6 +14,7 @@
 #include "tship_sample_kernels.h"
 
 #include <cmath>
+#include <cstdlib>
 #include <cstring>
 #include <map>
 #include <memory>
@@ -93,11 +94,15 @@ struct TSHipGpt {
 
     // decode state
     DevBuf x, xn, o, a, part_qkv, part_h, part_f, logits, ids, d_pos, hidden;
-    DevBuf moe_ws;
+    DevBuf moe_ws, topp_scratch, topp_uni, gen_buf, uni_buf;
     DevBuf ssq;                    // deferred-norm path: per-column-tile sums of squares [h/32][Bpad]
     bool fused_norm = false;       // fp16 + RMSNorm + dense layers: residual/norm folded into the GEMM tails
     bool vt = false;               // fp16 cache with head_dim 64/128: values stored transposed for the MFMA attention kernels
     long ML = 0;                   // cache rows per (sequence, KV head): max_seq_len rounded up to 32
+    // one decode step (sample + decode) captured as a HIP graph; valid for one (batch, sampling mode) at a time
+    hipGraphExec_t step_graph = nullptr;
+    int graph_batch = 0, graph_mode = -1; float graph_top_p = 0.0f, graph_temp = 0.0f;
+    const float* graph_uniforms = nullptr; int* graph_gen = nullptr;
     int pos = 0;                   // host mirror of *d_pos
     int cur_batch = 0;
     Profiler* prof = nullptr;
@@ -117,7 +122,8 @@ static void launch(TSHipGpt* m, const char* name, void (*kernel)(KArgs...), dim3
         m->prof->ev0.push_back(e0);
         m->prof->ev1.push_back(e1);
     }
-    hipExtLaunchKernelGGL(kernel, grid, block, 0, stream(), e0, e1, 0, args...);
+    if (e0) hipExtLaunchKernelGGL(kernel, grid, block, 0, stream(), e0, e1, 0, args...);
+    else hipLaunchKernelGGL(kernel, grid, block, 0, stream(), args...);
     TSHIP_CHECK_HIP(hipGetLastError());
 }
 
@@ -398,7 +404,7 @@ static AttnArgs attn_args(TSHipGpt* m, LayerW& L) {
 static void run_moe_ffn(TSHipGpt* m, LayerW& L, int rows, const ResidNormArgs& pre);
 static void moe_alloc(TSHipGpt* m);
 static void moe_get_routing(TSHipGpt* m, int layer, float* top_idx, float* top_val, float* probs);
-static void sample_tokens(TSHipGpt* m, int mode, float top_p, float temperature, const float* host_uniforms, const float* dev_uniforms, int B, int* gen_out);
+static void sample_tokens(TSHipGpt* m, int mode, float top_p, float temperature, const float* host_uniforms, const float* dev_uniforms, int B, int* gen_out, const int* d_step);
 
 // ------------------------------------------------------------------------------------------------
 // decode step, deferred-norm form (fp16 weights, RMSNorm, dense feed-forward): 5 launches per layer.
@@ -778,7 +784,7 @@ TSHIP_API int TSHip_GptCreate(const TSHipGptConfig* cfg, TSHipGpt** out) {
     if (!m->f16) m->part_f.alloc((size_t)16 * m->Bpad * m->F13 * sizeof(float));
     m->logits.alloc((size_t)m->Bpad * Vp * sizeof(float));
     m->ids.alloc((size_t)m->Bpad * sizeof(int));
-    m->d_pos.alloc(sizeof(int));
+    m->d_pos.alloc(2 * sizeof(int));      // [0] cached positions, [1] step counter of the running generate call
     m->hidden.alloc((size_t)m->Bpad * h * sizeof(float));
     if (c.n_experts > 1) moe_alloc(m.get());
     m->fused_norm = m->f16 && c.norm_type == 0 && c.n_experts <= 1;
@@ -792,7 +798,11 @@ TSHIP_API int TSHip_GptCreate(const TSHipGptConfig* cfg, TSHipGpt** out) {
 
 TSHIP_API int TSHip_GptDestroy(TSHipGpt* m) {
     TSHIP_BEGIN
-    if (m) { (void)hipStreamSynchronize(stream()); delete m; }
+    if (m) {
+        (void)hipStreamSynchronize(stream());
+        if (m->step_graph) (void)hipGraphExecDestroy(m->step_graph);
+        delete m;
+    }
     TSHIP_END
 }
 
@@ -870,7 +880,7 @@ TSHIP_API int TSHip_GptSample(TSHipGpt* m, int mode, float top_p, float temperat
     TSHIP_REQUIRE(m && host_ids_out, "TSHip_GptSample: null argument");
     TSHIP_REQUIRE(m->cur_batch > 0, "TSHip_GptSample: no logits yet; prefill or decode first");
     const int B = m->cur_batch;
-    sample_tokens(m, mode, top_p, temperature, host_uniforms, nullptr, B, nullptr);
+    sample_tokens(m, mode, top_p, temperature, host_uniforms, nullptr, B, nullptr, nullptr);
     TSHIP_CHECK_HIP(hipMemcpyAsync(host_ids_out, m->ids.p, B * sizeof(int), hipMemcpyDeviceToHost, stream()));
     TSHIP_CHECK_HIP(hipStreamSynchronize(stream()));
     TSHIP_END
@@ -885,11 +895,49 @@ TSHIP_API int TSHip_GptGenerate(TSHipGpt* m, int n_steps, int mode, float top_p,
     TSHIP_REQUIRE(m->pos + n_steps <= m->c.max_seq_len, "TSHip_GptGenerate: KV cache too small for n_steps (max_seq_len)");
     TSHIP_REQUIRE(mode == TSHIP_GREEDY || (mode == TSHIP_TOPP && host_uniforms), "TSHip_GptGenerate: top-p needs the uniform stream");
     const int B = m->cur_batch;
-    DevBuf gen, uni;
-    gen.alloc((size_t)n_steps * B * sizeof(int));
+    // token and uniform buffers live in the model so that the captured step graph stays valid across calls
+    DevBuf& gen = m->gen_buf; DevBuf& uni = m->uni_buf;
+    if (gen.bytes < (size_t)n_steps * B * sizeof(int)) gen.alloc((size_t)std::max(n_steps, 256) * m->Bpad * sizeof(int));
     if (mode == TSHIP_TOPP) {
-        uni.alloc((size_t)n_steps * B * sizeof(float));
+        if (uni.bytes < (size_t)n_steps * B * sizeof(float)) uni.alloc((size_t)std::max(n_steps, 256) * m->Bpad * sizeof(float));
         TSHIP_CHECK_HIP(hipMemcpyAsync(uni.p, host_uniforms, (size_t)n_steps * B * sizeof(float), hipMemcpyHostToDevice, stream()));
+        TSHIP_CHECK_HIP(hipStreamSynchronize(stream()));
+    }
+    // the step counter that indexes gen/uniforms on the device starts at zero for every call
+    TSHIP_CHECK_HIP(hipMemsetAsync(m->d_pos.as<int>() + 1, 0, sizeof(int), stream()));
+    const int* d_step = m->d_pos.as<int>() + 1;
+    const float* uni_base = mode == TSHIP_TOPP ? uni.as<float>() : nullptr;
+    bool any_moe = false; for (auto& L : m->L) any_moe = any_moe || L->moe;
+    const bool use_graph = !any_moe && std::getenv("TSHIP_NO_GRAPH") == nullptr;
+    if (mode == TSHIP_TOPP) {      // scratch must exist before capture (no allocation inside a graph)
+        const long Vs = round_up(m->c.vocab, 64);
+        size_t need = (size_t)m->Bpad * Vs * 5 * 4;
+        if (m->topp_scratch.bytes < need) m->topp_scratch.alloc(need);
+    }
+    if (use_graph) {
+        // (sample -> decode) of one step is captured once; every replay reads the position, the step counter and the
+        // token ids from device memory, so identical launches walk through the sequence
+        if (m->step_graph && (m->graph_batch != B || m->graph_mode != mode || m->graph_top_p != top_p || m->graph_temp != temperature ||
+                              m->graph_uniforms != uni_base || m->graph_gen != gen.as<int>())) {
+            (void)hipGraphExecDestroy(m->step_graph); m->step_graph = nullptr;
+        }
+        if (!m->step_graph) {
+            hipGraph_t graph = nullptr;
+            TSHIP_CHECK_HIP(hipStreamSynchronize(stream()));
+            TSHIP_CHECK_HIP(hipStreamBeginCapture(stream(), hipStreamCaptureModeThreadLocal));
+            const int saved_pos = m->pos;
+            try {
+                sample_tokens(m, mode, top_p, temperature, nullptr, uni_base, B, gen.as<int>(), d_step);
+                decode_step(m, m->ids.as<int>(), B);
+            } catch (...) { hipGraph_t g2 = nullptr; (void)hipStreamEndCapture(stream(), &g2); if (g2) (void)hipGraphDestroy(g2); m->pos = saved_pos; throw; }
+            m->pos = saved_pos;                    // capturing launched nothing
+            TSHIP_CHECK_HIP(hipStreamEndCapture(stream(), &graph));
+            hipError_t ge = hipGraphInstantiate(&m->step_graph, graph, nullptr, nullptr, 0);
+            (void)hipGraphDestroy(graph);
+            TSHIP_CHECK_HIP(ge);
+            m->graph_batch = B; m->graph_mode = mode; m->graph_top_p = top_p; m->graph_temp = temperature;
+            m->graph_uniforms = uni_base; m->graph_gen = gen.as<int>();
+        }
     }
     hipEvent_t e0, e1;
     TSHIP_CHECK_HIP(hipEventCreate(&e0));
@@ -897,9 +945,11 @@ TSHIP_API int TSHip_GptGenerate(TSHipGpt* m, int n_steps, int mode, float top_p,
     TSHIP_CHECK_HIP(hipStreamSynchronize(stream()));
     TSHIP_CHECK_HIP(hipEventRecord(e0, stream()));
     for (int s = 0; s < n_steps; ++s) {
-        sample_tokens(m, mode, top_p, temperature, nullptr, mode == TSHIP_TOPP ? uni.as<float>() + (size_t)s * B : nullptr, B,
-                      gen.as<int>() + (size_t)s * B);
-        decode_step(m, m->ids.as<int>(), B);
+        if (use_graph) { TSHIP_CHECK_HIP(hipGraphLaunch(m->step_graph, stream())); m->pos += 1; }
+        else {
+            sample_tokens(m, mode, top_p, temperature, nullptr, uni_base, B, gen.as<int>(), d_step);
+            decode_step(m, m->ids.as<int>(), B);
+        }
     }
     TSHIP_CHECK_HIP(hipEventRecord(e1, stream()));
     TSHIP_CHECK_HIP(hipStreamSynchronize(stream()));

@@ -110,33 +110,33 @@ static void run_moe_ffn(TSHipGpt* m, LayerW& L, int rows, const ResidNormArgs& p
            (const float*)top_idx, (const int*)slot, k, E);
 }
 
-// next tokens from the logits on the device -> m->ids (and gen_out); greedy or top-p
+// next tokens from the logits on the device -> m->ids (and gen_out); greedy or top-p.
+// With d_step set, gen_out and dev_uniforms are bases indexed by the device step counter (graph replays).
 static void sample_tokens(TSHipGpt* m, int mode, float top_p, float temperature, const float* host_uniforms, const float* dev_uniforms, int B,
-                          int* gen_out) {
+                          int* gen_out, const int* d_step = nullptr) {
     const long Vp = round_up(m->c.vocab, 32);
     if (mode == TSHIP_GREEDY) {
-        launch(m, "greedy", greedy_kernel, dim3(B), dim3(1024), (const float*)m->logits.as<float>(), Vp, m->c.vocab, m->ids.as<int>(), gen_out, (const int*)nullptr);
+        launch(m, "greedy", greedy_kernel, dim3(B), dim3(1024), (const float*)m->logits.as<float>(), Vp, m->c.vocab, m->ids.as<int>(), gen_out, d_step);
         return;
     }
     TSHIP_REQUIRE(mode == TSHIP_TOPP, "unknown sampling mode");
     TSHIP_REQUIRE(m->c.vocab <= 65535, "top-p sampling supports vocabularies up to 65535");
     TSHIP_REQUIRE(temperature > 0.0f, "temperature must be positive");
     const long Vs = round_up(m->c.vocab, 64);
-    static thread_local DevBuf scratch, uni;
     size_t need = (size_t)m->Bpad * Vs * 5 * 4;
-    if (scratch.bytes < need) scratch.alloc(need);
+    if (m->topp_scratch.bytes < need) m->topp_scratch.alloc(need);
     if (!dev_uniforms) {
         TSHIP_REQUIRE(host_uniforms, "top-p sampling needs one uniform draw per row");
-        if (uni.bytes < (size_t)B * 4) uni.alloc((size_t)m->Bpad * 4);
-        TSHIP_CHECK_HIP(hipMemcpyAsync(uni.p, host_uniforms, (size_t)B * 4, hipMemcpyHostToDevice, stream()));
-        dev_uniforms = uni.as<float>();
+        if (m->topp_uni.bytes < (size_t)m->Bpad * 4) m->topp_uni.alloc((size_t)m->Bpad * 4);
+        TSHIP_CHECK_HIP(hipMemcpyAsync(m->topp_uni.p, host_uniforms, (size_t)B * 4, hipMemcpyHostToDevice, stream()));
+        dev_uniforms = m->topp_uni.as<float>();
     }
     TopPArgs a; std::memset(&a, 0, sizeof(a));
     a.in = m->logits.as<float>(); a.ld = Vp; a.V = m->c.vocab; a.in_is_logits = 1;
     a.uniforms = dev_uniforms; a.top_p = top_p; a.Vs = Vs;
-    char* s = (char*)scratch.p; size_t one = (size_t)m->Bpad * Vs * 4;
+    char* s = (char*)m->topp_scratch.p; size_t one = (size_t)m->Bpad * Vs * 4;
     a.keysA = (unsigned*)s; a.keysB = (unsigned*)(s + one); a.idxA = (int*)(s + 2 * one); a.idxB = (int*)(s + 3 * one); a.accp = (float*)(s + 4 * one);
-    a.next_ids = m->ids.as<int>(); a.gen_out = gen_out;
+    a.next_ids = m->ids.as<int>(); a.gen_out = gen_out; a.d_step = d_step;
     // Decoder.cs:720-723 divides the logits by the temperature (fp32 division) before the softmax
     a.temperature = temperature;
     launch(m, "topp", topp_kernel, dim3(B), dim3(256), a);

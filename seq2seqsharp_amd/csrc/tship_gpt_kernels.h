@@ -172,7 +172,7 @@ __global__ __launch_bounds__(NW * 64) void skinny_gemm_f16_kernel(SkinnyArgs a) 
             srinv[threadIdx.x] = 1.0f / sqrtf(tot * a.inv_h + a.eps);
         }
     }
-    if (a.advance_pos && blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) *a.advance_pos += 1;
+    if (a.advance_pos && blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) { a.advance_pos[0] += 1; a.advance_pos[1] += 1; }
     // pairwise tree over wavefronts down to two: in each round the upper half stores, the lower half adds
 #pragma unroll
     for (int half = NW / 2; half >= 2; half >>= 1) {
@@ -480,7 +480,7 @@ __global__ __launch_bounds__(256) void resid_norm_kernel(ResidNormArgs a) {
             sum += v[i]; sq += v[i] * v[i];
         }
     }
-    if (a.advance_pos && r == 0 && t == 0) *a.advance_pos += 1;
+    if (a.advance_pos && r == 0 && t == 0) { a.advance_pos[0] += 1; a.advance_pos[1] += 1; }
     if (!a.xn) return;
     AT* out = (AT*)a.xn + (long)r * a.ldxn;
     if (a.norm_type == 0) {

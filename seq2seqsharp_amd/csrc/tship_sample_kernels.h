@@ -20,6 +20,7 @@ struct TopPArgs {
     unsigned* keysA; unsigned* keysB; int* idxA; int* idxB; float* accp;   // scratch, each [rows][Vs]
     long Vs;
     int* next_ids; int* gen_out; float* out_f32;   // any of them may be null
+    const int* d_step;                             // optional: uniforms and gen_out are indexed by *d_step * rows + row
 };
 
 __device__ __forceinline__ float block_max_256(float v, float* s) {
@@ -125,7 +126,8 @@ static __global__ __launch_bounds__(256) void topp_kernel(TopPArgs a) {
         if (t == 0) { s_n = n; s_acc = acc; s_pick = 0x7fffffff; }
     }
     __syncthreads();
-    const int n = s_n; const float acc = s_acc, u = a.uniforms[r];
+    const long slot = (a.d_step ? (long)*a.d_step * gridDim.x : 0) + r;
+    const int n = s_n; const float acc = s_acc, u = a.uniforms[slot];
     int best = 0x7fffffff;
     for (int k = t; k < n; k += 256) if (accp[k] / acc >= u) { best = k; break; }
     atomicMin(&s_pick, best);
@@ -133,7 +135,7 @@ static __global__ __launch_bounds__(256) void topp_kernel(TopPArgs a) {
     if (t == 0) {
         int id = s_pick == 0x7fffffff ? 0 : iA[s_pick];
         if (a.next_ids) a.next_ids[r] = id;
-        if (a.gen_out) a.gen_out[r] = id;
+        if (a.gen_out) a.gen_out[slot] = id;
         if (a.out_f32) a.out_f32[r] = (float)id;
     }
 }

@@ -8,7 +8,33 @@ import statistics
 import sys
 
 
+def _avg(db_path, counter, like):
+    cur = sqlite3.connect(db_path).cursor()
+    r = list(cur.execute("select count(*), avg(counter_value) from pmc_events where counter_name = ? and name like ?", (counter, like)))
+    return (r[0][0], r[0][1]) if r and r[0][0] else (0, None)
+
+
+def traffic(fetch_db, write_db, kernel_like, copy_like, copy_bytes, out_json):
+    """HBM bytes per launch of one kernel from a FETCH_SIZE run and a WRITE_SIZE run (KiB per dispatch), each scaled by
+    what the same counter reads for a plain copy kernel that reads and writes `copy_bytes`."""
+    import json
+    nf, f = _avg(fetch_db, "FETCH_SIZE", kernel_like)
+    nw, w = _avg(write_db, "WRITE_SIZE", kernel_like)
+    _, cf = _avg(fetch_db, "FETCH_SIZE", copy_like)
+    _, cw = _avg(write_db, "WRITE_SIZE", copy_like)
+    fs, ws = copy_bytes / (cf * 1024.0), copy_bytes / (cw * 1024.0)
+    out = {"kernel_like": kernel_like, "dispatches": nf, "fetch_kib_per_dispatch": f, "write_kib_per_dispatch": w,
+           "copy_kernel_like": copy_like, "copy_bytes": copy_bytes, "copy_fetch_kib": cf, "copy_write_kib": cw,
+           "fetch_scale": fs, "write_scale": ws,
+           "traffic_bytes_per_launch": round((f * fs + (w or 0.0) * ws) * 1024.0)}
+    json.dump(out, open(out_json, "w"), indent=1)
+    print(json.dumps(out, indent=1))
+
+
 def main():
+    if sys.argv[1] == "--traffic":
+        traffic(sys.argv[2], sys.argv[3], sys.argv[4], sys.argv[5], int(sys.argv[6]), sys.argv[7])
+        return
     db_path, cmd = sys.argv[1], (sys.argv[2] if len(sys.argv) > 2 else "")
     cur = sqlite3.connect(db_path).cursor()
     print("command:", cmd)

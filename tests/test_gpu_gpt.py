@@ -146,6 +146,29 @@ def test_generate_matches_stepwise_and_is_deterministic(G):
     gpu.prefill(seqs)
     ids2, _ = gpu.generate(12)
     assert np.array_equal(ids, ids2)                       # split-K partials are summed in a fixed order
+    # the captured step graph replayed in pieces, with eager steps and synchronisations in between
+    gpu.reset()
+    gpu.prefill(seqs)
+    a, _ = gpu.generate(5)
+    t = gpu.sample()
+    gpu.decode(t)
+    b, _ = gpu.generate(3)
+    t2 = gpu.sample()
+    gpu.decode(t2)
+    c, _ = gpu.generate(2)
+    assert np.array_equal(np.concatenate([a, t[None], b, t2[None], c]), ids)
+    u = synth.make_uniforms(3, 4, 6)
+    gpu.reset()
+    gpu.prefill(seqs)
+    p1, _ = gpu.generate(6, mode=G.TOPP, top_p=0.8, uniforms=u)
+    gpu.reset()
+    gpu.prefill(seqs)
+    p2 = []
+    for s in range(6):
+        t = gpu.sample(mode=G.TOPP, top_p=0.8, uniforms=u[s])
+        p2.append(t)
+        gpu.decode(t)
+    assert np.array_equal(p1, np.stack(p2))
     gpu.close()
 
 
