@@ -463,10 +463,23 @@ static void decode_step_fn(TSHipGpt* m, const int* d_ids, int B) {
             with_ssq(e);
             run_skinny(m, "gemm_ffn13", L.w13, m->xn.p, m->ldh, B, EPI_ACT16, e);
         }
-        {
+        const float* next_gamma = l + 1 < c.n_layers ? m->L[l + 1]->n1_g.as<float>() : m->fn_g.as<float>();
+        if (L.w2.KS == 1) {
             SkinnyArgs e; std::memset(&e, 0, sizeof(e));
-            tail(e, L.b2.as<float>(), l + 1 < c.n_layers ? m->L[l + 1]->n1_g.as<float>() : m->fn_g.as<float>());
+            tail(e, L.b2.as<float>(), next_gamma);
             run_skinny(m, "gemm_ffn2", L.w2, m->a.p, m->ldF, B, EPI_RESID_TAIL, e);
+        } else {
+            // long K: split across blocks so that every CU streams weights, then a small tail kernel
+            SkinnyArgs e; std::memset(&e, 0, sizeof(e));
+            e.out = m->part_h.as<float>(); e.ld_out = (int)hp; e.split_stride = (long)m->Bpad * hp;
+            run_skinny(m, "gemm_ffn2", L.w2, m->a.p, m->ldF, B, EPI_PARTIAL, e);
+            ResidTailArgs r; std::memset(&r, 0, sizeof(r));
+            r.x = m->x.as<float>(); r.ldx = h; r.h = h; r.rows = B;
+            r.part = m->part_h.as<float>(); r.KS = L.w2.KS; r.split_stride = (long)m->Bpad * hp; r.ld_part = hp; r.bias = L.b2.as<float>();
+            r.gamma = next_gamma; r.xg16 = m->xn.as<half_t>(); r.xg_kt = xkt; r.ssq_out = ssq; r.ssq_ld = m->Bpad;
+            if (m->BT == 1) launch(m, "resid_tail", resid_tail_kernel<4>, dim3(NTh), dim3(256), r);
+            else if (m->BT == 2) launch(m, "resid_tail", resid_tail_kernel<8>, dim3(NTh), dim3(256), r);
+            else launch(m, "resid_tail", resid_tail_kernel<16>, dim3(NTh), dim3(256), r);
         }
     }
     {
@@ -820,6 +833,14 @@ TSHIP_API int TSHip_GptFinalize(TSHipGpt* m) {
     for (auto& n : m->expected)
         if (!m->seen.count(n)) throw Error("TSHip_GptFinalize: weight '" + n + "' was never set");
     // RMSNorm has no beta (Layers/RMSNormalization.cs:33-37): keep null pointers there
+    if (m->fused_norm) {
+        // deferred-norm path: the output projection runs unsplit with the residual tail in its epilogue; the FFN down
+        // projection keeps its K split only when K is long enough to need more than two passes per wavefront
+        for (auto& L : m->L) {
+            L->wo.KS = 1;
+            if (L->w2.KS <= 2) L->w2.KS = 1;
+        }
+    }
     m->finalized = true;
     TSHIP_END
 }

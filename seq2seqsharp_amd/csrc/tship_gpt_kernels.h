@@ -516,6 +516,50 @@ __global__ __launch_bounds__(256) void resid_norm_kernel(ResidNormArgs a) {
     }
 }
 
+// Residual tail for a split-K projection on the deferred-norm path: one block per 32-column tile.
+// x[:, tile] += sum of the split-K partials (in split order) + bias; stores x, the next GEMM's packed input
+// half(gamma * x) and the tile's per-row sum of squares.  All loads of a thread are issued before the first use.
+struct ResidTailArgs {
+    float* x; long ldx; int h; int rows;
+    const float* part; int KS; long split_stride; long ld_part; const float* bias;
+    const float* gamma; half_t* xg16; int xg_kt; float* ssq_out; int ssq_ld;
+};
+template <int RPT>      // rows per thread: 256 threads cover 8 rows x 32 columns per pass
+__global__ __launch_bounds__(256) void resid_tail_kernel(ResidTailArgs a) {
+    const int nt = blockIdx.x, t = threadIdx.x, n = t & 31, b0 = t >> 5;
+    const int col = nt * 32 + n;
+    const bool okc = col < a.h;
+    float p[RPT][8], xv[RPT];
+    const float bias = okc ? a.bias[col] : 0.0f, gm = okc ? a.gamma[col] : 0.0f;
+#pragma unroll
+    for (int i = 0; i < RPT; ++i) {
+        const int b = b0 + 8 * i;
+        const bool ok = okc && b < a.rows;
+        xv[i] = ok ? a.x[(long)b * a.ldx + col] : 0.0f;
+#pragma unroll
+        for (int k = 0; k < 8; ++k) p[i][k] = (ok && k < a.KS) ? a.part[k * a.split_stride + (long)b * a.ld_part + col] : 0.0f;
+    }
+#pragma unroll
+    for (int i = 0; i < RPT; ++i) {
+        const int b = b0 + 8 * i;
+        if (b >= a.rows) continue;                       // uniform over the 32 lanes that share a row
+        float s = p[i][0];
+#pragma unroll
+        for (int k = 1; k < 8; ++k) if (k < a.KS) s += p[i][k];
+        for (int k = 8; k < a.KS; ++k) s += a.part[k * a.split_stride + (long)b * a.ld_part + col];
+        float v = 0.0f;
+        if (okc) {
+            v = (s + bias) + xv[i];
+            a.x[(long)b * a.ldx + col] = v;
+            a.xg16[xpack_index(b, col, a.xg_kt)] = (half_t)(gm * v);
+        }
+        float q = v * v;
+#pragma unroll
+        for (int o = 16; o > 0; o >>= 1) q += __shfl_xor(q, o, 64);
+        if (n == 0) a.ssq_out[(long)nt * a.ssq_ld + b] = q;
+    }
+}
+
 // Deferred-norm entry: x = E[id] * scale (or x = row row_map[r] of an existing stream) -> the next GEMM's packed
 // input half(gamma * x) and the per-column-tile sums of squares.  One block per row.
 struct FnPrepArgs {
@@ -854,32 +898,78 @@ __global__ __launch_bounds__(D == 128 ? 256 : 512) void attn_mfma_kernel(AttnArg
     half_t* Kb = (half_t*)a.kcache + ((long)b * a.Hkv + kvh) * a.max_len * D;
     half_t* Vt = (half_t*)a.vcache + ((long)b * a.Hkv + kvh) * (long)D * a.max_len;
 
+    // geometry needed by the early loads
+    const int nchunks = (T + 31) / 32;
+    const int krow = 8 * (r16 >> 2) + (r16 & 3);      // key-tile row of this lane: tile 0 -> t0 + krow, tile 1 -> + 4
+    half8 kfA[2][KD], vfA[DT], kfB[2][KD], vfB[DT];
+    auto load_chunk = [&](int c, half8 (&kf)[2][KD], half8 (&vf)[DT]) {
+        const int t0 = c * 32;
+#pragma unroll
+        for (int tile = 0; tile < 2; ++tile)
+#pragma unroll
+            for (int kd = 0; kd < KD; ++kd) kf[tile][kd] = *(const half8*)(Kb + (long)(t0 + krow + 4 * tile) * D + kd * 32 + 8 * q);
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) vf[dt] = *(const half8*)(Vt + (long)(dt * 16 + r16) * a.max_len + t0 + 8 * q);
+    };
+    // the first chunk of this wavefront does not depend on the prologue unless it holds the row being appended
+    const bool early = !PREFILL && w < nchunks - 1;
+    if (early) load_chunk(w, kfA, vfA);
+
     for (int i = t; i < 16 * D; i += NTH) (&sQ[0][0])[i] = 0.0f;
     if (!PREFILL) {
-        float rinv = 1.0f;
-        if (a.ssq) {
-            float s = 0.0f;
-            for (int tt = lane; tt < a.ssq_nt; tt += 64) s += a.ssq[(long)tt * a.ssq_ld + b];
-            s = wave_sum(s);
-            rinv = 1.0f / sqrtf(s * a.inv_h + a.eps);
+        constexpr int CPT = ((G + 2) * D + NTH - 1) / NTH;        // projection columns per thread
+        constexpr int PPT = ((G + 1) * D / 2 + NTH - 1) / NTH;    // rotary pairs per thread
+        const int pos = pos_base;
+        // every global load of the prologue is issued before the first use
+        float ssq_part = 0.0f;
+        if (a.ssq) for (int tt = lane; tt < a.ssq_nt; tt += 64) ssq_part += a.ssq[(long)tt * a.ssq_ld + b];
+        float part[CPT][8], bias[CPT];
+#pragma unroll
+        for (int ci = 0; ci < CPT; ++ci) {
+            const int idx = t + ci * NTH;
+            bias[ci] = 0.0f;
+#pragma unroll
+            for (int k = 0; k < 8; ++k) part[ci][k] = 0.0f;
+            if (idx < (G + 2) * D) {
+                int col;
+                if (idx < G * D) col = kvh * G * D + idx;
+                else if (idx < (G + 1) * D) col = HD + kvh * D + (idx - G * D);
+                else col = HD + GD + kvh * D + (idx - (G + 1) * D);
+#pragma unroll
+                for (int k = 0; k < 8; ++k) if (k < a.KS) part[ci][k] = a.qkv[k * a.split_stride + (long)b * a.ldq + col];
+                bias[ci] = a.bias[col];
+            }
         }
-        for (int idx = t; idx < (G + 2) * D; idx += NTH) {
-            int col;
-            if (idx < G * D) col = kvh * G * D + idx;
-            else if (idx < (G + 1) * D) col = HD + kvh * D + (idx - G * D);
-            else col = HD + GD + kvh * D + (idx - (G + 1) * D);
-            float s = a.qkv[(long)b * a.ldq + col];
-            for (int k = 1; k < a.KS; ++k) s += a.qkv[k * a.split_stride + (long)b * a.ldq + col];
-            sIn[idx] = s * rinv + a.bias[col];
+        float rc[PPT], rs[PPT];
+#pragma unroll
+        for (int pi = 0; pi < PPT; ++pi) {
+            const int p = t + pi * NTH;
+            rc[pi] = 1.0f; rs[pi] = 0.0f;
+            if (p < (G + 1) * D / 2 && a.rope_cos) { rc[pi] = a.rope_cos[(long)pos * (D / 2) + p % (D / 2)]; rs[pi] = a.rope_sin[(long)pos * (D / 2) + p % (D / 2)]; }
+        }
+        float rinv = 1.0f;
+        if (a.ssq) rinv = 1.0f / sqrtf(wave_sum(ssq_part) * a.inv_h + a.eps);
+#pragma unroll
+        for (int ci = 0; ci < CPT; ++ci) {
+            const int idx = t + ci * NTH;
+            if (idx < (G + 2) * D) {
+                float s = part[ci][0];
+#pragma unroll
+                for (int k = 1; k < 8; ++k) if (k < a.KS) s += part[ci][k];
+                sIn[idx] = s * rinv + bias[ci];
+            }
         }
         __syncthreads();
-        const int pos = pos_base;
-        for (int p = t; p < (G + 1) * D / 2; p += NTH) {
-            int vec = p / (D / 2), i = p % (D / 2);
-            float x0 = sIn[vec * D + 2 * i], x1 = sIn[vec * D + 2 * i + 1], y0 = x0, y1 = x1;
-            if (a.rope_cos) rope_pair(x0, x1, a.rope_cos[(long)pos * (D / 2) + i], a.rope_sin[(long)pos * (D / 2) + i], y0, y1);
-            if (vec < G) { sQ[vec][2 * i] = a.scale * y0; sQ[vec][2 * i + 1] = a.scale * y1; }
-            else { Kb[(long)pos * D + 2 * i] = (half_t)y0; Kb[(long)pos * D + 2 * i + 1] = (half_t)y1; }
+#pragma unroll
+        for (int pi = 0; pi < PPT; ++pi) {
+            const int p = t + pi * NTH;
+            if (p < (G + 1) * D / 2) {
+                const int vec = p / (D / 2), i = p % (D / 2);
+                float x0 = sIn[vec * D + 2 * i], x1 = sIn[vec * D + 2 * i + 1], y0 = x0, y1 = x1;
+                if (a.rope_cos) rope_pair(x0, x1, rc[pi], rs[pi], y0, y1);
+                if (vec < G) { sQ[vec][2 * i] = a.scale * y0; sQ[vec][2 * i + 1] = a.scale * y1; }
+                else { Kb[(long)pos * D + 2 * i] = (half_t)y0; Kb[(long)pos * D + 2 * i + 1] = (half_t)y1; }
+            }
         }
         for (int d = t; d < D; d += NTH) Vt[(long)d * a.max_len + pos] = (half_t)sIn[(G + 1) * D + d];
         __threadfence_block();
@@ -915,18 +1005,9 @@ __global__ __launch_bounds__(D == 128 ? 256 : 512) void attn_mfma_kernel(AttnArg
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) acc_o[dt] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
 
-    const int nchunks = (T + 31) / 32;
-    // row of the key tile this lane loads: tile 0 rows -> t0 + 8*(r/4) + r%4, tile 1 rows -> + 4
-    const int krow = 8 * (r16 >> 2) + (r16 & 3);
-    for (int c = w; c < nchunks; c += NW) {
+    // two register sets: the next chunk's keys and values are in flight while the current chunk is processed
+    auto do_chunk = [&](int c, half8 (&kf)[2][KD], half8 (&vf)[DT]) {
         const int t0 = c * 32;
-        half8 kf[2][KD], vf[DT];
-#pragma unroll
-        for (int tile = 0; tile < 2; ++tile)
-#pragma unroll
-            for (int kd = 0; kd < KD; ++kd) kf[tile][kd] = *(const half8*)(Kb + (long)(t0 + krow + 4 * tile) * D + kd * 32 + 8 * q);
-#pragma unroll
-        for (int dt = 0; dt < DT; ++dt) vf[dt] = *(const half8*)(Vt + (long)(dt * 16 + r16) * a.max_len + t0 + 8 * q);
         floatx4 sA = floatx4{0.0f, 0.0f, 0.0f, 0.0f}, sB = sA;
 #pragma unroll
         for (int kd = 0; kd < KD; ++kd) {
@@ -964,6 +1045,20 @@ __global__ __launch_bounds__(D == 128 ? 256 : 512) void attn_mfma_kernel(AttnArg
 #pragma unroll
             for (int i = 0; i < 4; ++i) acc_o[dt][i] *= corr;
             acc_o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vf[dt], pf, acc_o[dt], 0, 0, 0);
+        }
+    };
+    {
+        int c = w;
+        if (c < nchunks) {
+            if (!early) load_chunk(c, kfA, vfA);
+            while (true) {
+                if (c + NW < nchunks) load_chunk(c + NW, kfB, vfB);
+                do_chunk(c, kfA, vfA);
+                c += NW; if (c >= nchunks) break;
+                if (c + NW < nchunks) load_chunk(c + NW, kfA, vfA);
+                do_chunk(c, kfB, vfB);
+                c += NW; if (c >= nchunks) break;
+            }
         }
     }
     // the four lane groups of a column saw different positions: add their sums (the maximum is already common)
