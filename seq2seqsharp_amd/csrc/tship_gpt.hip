@@ -97,7 +97,7 @@ struct TSHipGpt {
     DevBuf moe_ws, topp_scratch, topp_uni, gen_buf, uni_buf;
     DevBuf ssq;                    // deferred-norm path: per-column-tile sums of squares [h/32][Bpad]
     bool fused_norm = false;       // fp16 + RMSNorm + dense layers: residual/norm folded into the GEMM tails
-    bool vt = false;               // fp16 cache with head_dim 64/128: values stored transposed for the MFMA attention kernels
+    bool vt = false;               // fp16 cache with head_dim 64/128: keys and values stored fragment-major for the MFMA attention kernels
     long ML = 0;                   // cache rows per (sequence, KV head): max_seq_len rounded up to 32
     // one decode step (sample + decode) captured as a HIP graph; valid for one (batch, sampling mode) at a time
     hipGraphExec_t step_graph = nullptr;
@@ -1042,13 +1042,13 @@ TSHIP_API int TSHip_GptGetKV(TSHipGpt* m, int layer, int which, float* host_out)
     const int B = m->cur_batch, G = m->c.n_kv_heads, D = m->D, T = m->pos; const long ML = m->ML;
     TSHIP_CHECK_HIP(hipStreamSynchronize(stream()));
     const char* base = (const char*)(which ? m->L[layer]->vc.p : m->L[layer]->kc.p);
-    const bool transposed = which == 1 && m->vt;          // values are kept [D][ML] for the MFMA attention kernels
+    const bool frag = m->vt;                               // fragment-major cache of the MFMA attention kernels
     std::vector<char> tmp((size_t)ML * D * m->esz());
     for (int b = 0; b < B; ++b) for (int g = 0; g < G; ++g) {
         TSHIP_CHECK_HIP(hipMemcpy(tmp.data(), base + ((size_t)b * G + g) * ML * D * m->esz(), tmp.size(), hipMemcpyDeviceToHost));
         float* dst = host_out + ((size_t)b * G + g) * T * D;
         for (long t = 0; t < T; ++t) for (int d = 0; d < D; ++d) {
-            size_t idx = transposed ? (size_t)d * ML + t : (size_t)t * D + d;
+            size_t idx = frag ? (size_t)(which ? vfrag_index((int)t, d, D) : kfrag_index((int)t, d, D)) : (size_t)t * D + d;
             dst[t * D + d] = m->f16 ? (float)((const half_t*)tmp.data())[idx] : ((const float*)tmp.data())[idx];
         }
     }
@@ -1072,12 +1072,12 @@ TSHIP_API int TSHip_GptSetKV(TSHipGpt* m, int layer, int which, const float* hos
     TSHIP_REQUIRE(batch >= 1 && batch <= m->c.max_batch && len >= 0 && len <= m->c.max_seq_len, "TSHip_GptSetKV: out of range");
     const int G = m->c.n_kv_heads, D = m->D; const long ML = m->ML;
     char* base = (char*)(which ? m->L[layer]->vc.p : m->L[layer]->kc.p);
-    const bool transposed = which == 1 && m->vt;
+    const bool frag = m->vt;
     std::vector<char> tmp((size_t)ML * D * m->esz(), 0);
     for (int b = 0; b < batch; ++b) for (int g = 0; g < G; ++g) {
         const float* src = host_in + ((size_t)b * G + g) * len * D;
         for (long t = 0; t < len; ++t) for (int d = 0; d < D; ++d) {
-            size_t idx = transposed ? (size_t)d * ML + t : (size_t)t * D + d;
+            size_t idx = frag ? (size_t)(which ? vfrag_index((int)t, d, D) : kfrag_index((int)t, d, D)) : (size_t)t * D + d;
             if (m->f16) ((half_t*)tmp.data())[idx] = (half_t)src[t * D + d]; else ((float*)tmp.data())[idx] = src[t * D + d];
         }
         TSHIP_CHECK_HIP(hipMemcpy(base + ((size_t)b * G + g) * ML * D * m->esz(), tmp.data(), tmp.size(), hipMemcpyHostToDevice));

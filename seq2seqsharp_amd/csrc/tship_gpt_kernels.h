@@ -608,7 +608,7 @@ struct AttnArgs {
     int out_kt;                                    // > 0: out is fragment packed with this many k-tiles
     float scale;
     const float* ssq; int ssq_nt; int ssq_ld; float inv_h; float eps;   // deferred RMSNorm of the projection input (see SkinnyArgs)
-    int vt;      // 1: the value cache is stored transposed, [batch][kv_head][D][max_len] (MFMA attention kernels)
+    int vt;      // 1: keys and values are stored fragment-major (kfrag_index / vfrag_index) for the MFMA attention kernels
 };
 
 // rotary embedding of one (even, odd) pair, two roundings per output like the reference's C# expression
@@ -817,6 +817,21 @@ __global__ __launch_bounds__(1024) void attn_decode_kernel(AttnArgs a) {
     }
 }
 
+// Fragment-major KV cache of the MFMA attention kernels (fp16, head_dim 64 or 128).  Positions are grouped in chunks
+// of 32; within a chunk every 1 KiB block is exactly one A operand of v_mfma_f32_16x16x32_f16 (64 lanes x 8 halfs),
+// so a wavefront's load instruction reads 1 KiB contiguous.
+//   keys:   block (chunk, tile, kd), lane r + 16 qq holds K[t = 32 chunk + 8 (r / 4) + 4 tile + r % 4][d = 32 kd + 8 qq + j]
+//   values: block (chunk, dt),       lane r + 16 qq holds V[t = 32 chunk + 8 qq + j][d = 16 dt + r]
+__host__ __device__ inline long kfrag_index(int t, int d, int D) {
+    const int c = t >> 5, tin = t & 31, q8 = tin >> 3, rem = tin & 7, tile = rem >> 2, r = 4 * q8 + (rem & 3);
+    const int kd = d >> 5, qq = (d & 31) >> 3, j = d & 7;
+    return ((((long)c * 2 + tile) * (D / 32) + kd) * 64 + r + 16 * qq) * 8 + j;
+}
+__host__ __device__ inline long vfrag_index(int t, int d, int D) {
+    const int c = t >> 5, qq = (t & 31) >> 3, j = t & 7;
+    return (((long)c * (D / 16) + (d >> 4)) * 64 + (d & 15) + 16 * qq) * 8 + j;
+}
+
 // prefill, step 1: grid (Tq, batch).  Rotates the keys of every position and writes keys and values into the cache.
 template <typename CT, int D>
 __global__ __launch_bounds__(256) void kv_write_kernel(AttnArgs a) {
@@ -831,14 +846,15 @@ __global__ __launch_bounds__(256) void kv_write_kernel(AttnArgs a) {
         int col = HD + kvh * D + 2 * i;
         float x0 = a.qkv[row * a.ldq + col] + a.bias[col], x1 = a.qkv[row * a.ldq + col + 1] + a.bias[col + 1], y0 = x0, y1 = x1;
         if (a.rope_cos) rope_pair(x0, x1, a.rope_cos[(long)pos * (D / 2) + i], a.rope_sin[(long)pos * (D / 2) + i], y0, y1);
-        CT* dst = Kb + ((long)kvh * a.max_len + pos) * D + 2 * i;
-        dst[0] = (CT)y0; dst[1] = (CT)y1;
+        CT* Kh = Kb + (long)kvh * a.max_len * D;
+        if (a.vt) { Kh[kfrag_index(pos, 2 * i, D)] = (CT)y0; Kh[kfrag_index(pos, 2 * i + 1, D)] = (CT)y1; }
+        else { Kh[(long)pos * D + 2 * i] = (CT)y0; Kh[(long)pos * D + 2 * i + 1] = (CT)y1; }
     }
     for (int p = t; p < GD; p += 256) {
         int kvh = p / D, d = p % D;
         int col = HD + GD + p;
         const float val = a.qkv[row * a.ldq + col] + a.bias[col];
-        if (a.vt) Vb[((long)kvh * D + d) * a.max_len + pos] = (CT)val;
+        if (a.vt) Vb[(long)kvh * a.max_len * D + vfrag_index(pos, d, D)] = (CT)val;
         else Vb[((long)kvh * a.max_len + pos) * D + d] = (CT)val;
     }
 }
@@ -871,8 +887,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(AttnArgs a) {
 // ------------------------------------------------------------------------------------------------
 // MFMA attention (fp16 cache, head_dim 64 or 128).  One block per (batch row, KV head) and QB query positions
 // (decode: 1, prefill: 16 / G); the 16 columns of v_mfma_f32_16x16x32_f16 are (query position, query head of the
-// group).  Keys are row-major [T][D]; values are stored TRANSPOSED [D][max_len] so that both products read
-// 16-byte runs:
+// group).  Keys and values are kept fragment-major (kfrag_index / vfrag_index), so every load is 1 KiB contiguous:
 //   S[32 t][16 col]   = K tile (two 16-row A operands, rows permuted so that lane group q ends up with
 //                       t = t0 + 8q .. 8q+7)  x  Q (B operand, kept in registers)
 //   O^T[D][16 col]   += V^T tile (A operand: 16 d-rows x 32 t)  x  P (B operand: the lane's own 8 probabilities)
@@ -900,16 +915,16 @@ __global__ __launch_bounds__(D == 128 ? 256 : 512) void attn_mfma_kernel(AttnArg
 
     // geometry needed by the early loads
     const int nchunks = (T + 31) / 32;
-    const int krow = 8 * (r16 >> 2) + (r16 & 3);      // key-tile row of this lane: tile 0 -> t0 + krow, tile 1 -> + 4
     half8 kfA[2][KD], vfA[DT], kfB[2][KD], vfB[DT];
     auto load_chunk = [&](int c, half8 (&kf)[2][KD], half8 (&vf)[DT]) {
-        const int t0 = c * 32;
+        const half_t* kc = Kb + (long)c * (32 * D) + lane * 8;
+        const half_t* vc = Vt + (long)c * (32 * D) + lane * 8;
 #pragma unroll
         for (int tile = 0; tile < 2; ++tile)
 #pragma unroll
-            for (int kd = 0; kd < KD; ++kd) kf[tile][kd] = *(const half8*)(Kb + (long)(t0 + krow + 4 * tile) * D + kd * 32 + 8 * q);
+            for (int kd = 0; kd < KD; ++kd) kf[tile][kd] = *(const half8*)(kc + (tile * KD + kd) * 512);
 #pragma unroll
-        for (int dt = 0; dt < DT; ++dt) vf[dt] = *(const half8*)(Vt + (long)(dt * 16 + r16) * a.max_len + t0 + 8 * q);
+        for (int dt = 0; dt < DT; ++dt) vf[dt] = *(const half8*)(vc + dt * 512);
     };
     // the first chunk of this wavefront does not depend on the prologue unless it holds the row being appended
     const bool early = !PREFILL && w < nchunks - 1;
@@ -968,10 +983,10 @@ __global__ __launch_bounds__(D == 128 ? 256 : 512) void attn_mfma_kernel(AttnArg
                 float x0 = sIn[vec * D + 2 * i], x1 = sIn[vec * D + 2 * i + 1], y0 = x0, y1 = x1;
                 if (a.rope_cos) rope_pair(x0, x1, rc[pi], rs[pi], y0, y1);
                 if (vec < G) { sQ[vec][2 * i] = a.scale * y0; sQ[vec][2 * i + 1] = a.scale * y1; }
-                else { Kb[(long)pos * D + 2 * i] = (half_t)y0; Kb[(long)pos * D + 2 * i + 1] = (half_t)y1; }
+                else { Kb[kfrag_index(pos, 2 * i, D)] = (half_t)y0; Kb[kfrag_index(pos, 2 * i + 1, D)] = (half_t)y1; }
             }
         }
-        for (int d = t; d < D; d += NTH) Vt[(long)d * a.max_len + pos] = (half_t)sIn[(G + 1) * D + d];
+        for (int d = t; d < D; d += NTH) Vt[vfrag_index(pos, d, D)] = (half_t)sIn[(G + 1) * D + d];
         __threadfence_block();
     } else {
         __syncthreads();
