@@ -627,6 +627,13 @@ static void prefill(TSHipGpt* m, const int32_t* host_ids, int B, int Tp) {
     }
     auto big = [&](const char* name, const GemmW& w, const void* X, long ldx, int epi, BigArgs e) {
         e.W = w.buf.as<half_t>(); e.KT = w.KT; e.NT = w.NT; e.X = (const half_t*)X; e.ldx = (int)ldx; e.R = (int)R;
+        if (R >= 512) {       // LDS-tiled kernel, 256 x 256 block tile
+            dim3 grid((unsigned)ceil_div(w.NT, 8), (unsigned)ceil_div(R, 256));
+            if (epi == BEPI_F32_BIAS) launch(m, name, big_gemm2_f16_kernel<BEPI_F32_BIAS>, grid, dim3(256), e);
+            else if (epi == BEPI_RESID) launch(m, name, big_gemm2_f16_kernel<BEPI_RESID>, grid, dim3(256), e);
+            else launch(m, name, big_gemm2_f16_kernel<BEPI_ACT16>, grid, dim3(256), e);
+            return;
+        }
         dim3 grid((unsigned)ceil_div(w.NT, 4), (unsigned)(Rp / 128));
         if (epi == BEPI_F32_BIAS) launch(m, name, big_gemm_f16_kernel<BEPI_F32_BIAS>, grid, dim3(256), e);
         else if (epi == BEPI_RESID) launch(m, name, big_gemm_f16_kernel<BEPI_RESID>, grid, dim3(256), e);

@@ -316,6 +316,113 @@ __global__ __launch_bounds__(256) void big_gemm_f16_kernel(BigArgs a) {
     }
 }
 
+// LDS-tiled prefill GEMM.  Block tile 256 rows x 256 columns, 4 wavefronts, each owning 128 x 128 (4 x 4 MFMA
+// tiles of 32 x 32, 256 accumulator registers).  K advances in chunks of 32 (two k-tiles): per chunk the block
+// stages 16 weight fragments (already fragment-ordered in memory: straight 1 KiB copies) and 16 activation fragments
+// (row-major in memory, scattered into fragment order) in LDS, double buffered: the next chunk's global loads are in
+// flight in registers while the MFMAs of the current chunk run, one barrier per chunk.
+// Per k-tile a wavefront reads 8 fragments from LDS for 16 MFMAs.
+template <int EPI>
+__global__ __launch_bounds__(256) void big_gemm2_f16_kernel(BigArgs a) {
+    __shared__ __attribute__((aligned(16))) half_t sW[2][16 * 512];
+    __shared__ __attribute__((aligned(16))) half_t sX[2][16 * 512];
+    const int t = threadIdx.x, lane = t & 63, w = __builtin_amdgcn_readfirstlane(t >> 6);
+    const int wr = w >> 1, wn = w & 1;
+    const int nt0 = blockIdx.x * 8;
+    const long row0 = (long)blockIdx.y * 256;
+    floatx16 acc[4][4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[j][i][v] = 0.0f;
+
+    // this thread's share of a chunk: 4 x 16 bytes of weights, 4 x 16 bytes of activations
+    const half8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+    const half_t* wsrc[4]; bool wok[4]; int wdst[4];
+    const half_t* xsrc[4]; bool xok[4]; int xdst[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int f = i * 4 + (t >> 6);                 // fragment of the chunk: n-tile f / 2, k-tile f % 2
+        const int nt = nt0 + (f >> 1);
+        wok[i] = nt < a.NT;
+        wsrc[i] = a.W + (((long)nt * a.KT + (f & 1)) * 64 + lane) * 8;
+        wdst[i] = f * 512 + lane * 8;
+        const int row = i * 64 + (t >> 2), seg = t & 3;  // 64-byte row segment of the chunk in four 16-byte pieces
+        xok[i] = row0 + row < a.R;
+        xsrc[i] = a.X + (row0 + row) * (long)a.ldx + seg * 8;
+        xdst[i] = (((row >> 5) * 2 + (seg >> 1)) * 64 + (row & 31) + 32 * (seg & 1)) * 8;
+    }
+    const int NC = (a.KT + 1) / 2;
+    half8 gw[4], gx[4];
+    auto gload = [&](int c) {
+        const bool k1 = 2 * c + 1 < a.KT;              // odd KT: the last chunk has one k-tile
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int f = i * 4 + (t >> 6);
+            gw[i] = (wok[i] && ((f & 1) == 0 || k1)) ? *(const half8*)(wsrc[i] + (long)c * 1024) : zero8;
+            gx[i] = (xok[i] && ((t & 3) < 2 || k1)) ? *(const half8*)(xsrc[i] + c * 32) : zero8;
+        }
+    };
+    auto lstore = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) { *(half8*)(&sW[buf][wdst[i]]) = gw[i]; *(half8*)(&sX[buf][xdst[i]]) = gx[i]; }
+    };
+    gload(0);
+    lstore(0);
+    __syncthreads();
+    for (int c = 0; c < NC; ++c) {
+        const int buf = c & 1;
+        if (c + 1 < NC) gload(c + 1);
+#pragma unroll
+        for (int kt = 0; kt < 2; ++kt) {
+            half8 wf[4], xf[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) wf[j] = *(const half8*)(&sW[buf][((4 * wn + j) * 2 + kt) * 512 + lane * 8]);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) xf[i] = *(const half8*)(&sX[buf][((4 * wr + i) * 2 + kt) * 512 + lane * 8]);
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) acc[j][i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf[j], xf[i], acc[j][i], 0, 0, 0);
+        }
+        if (c + 1 < NC) lstore(buf ^ 1);
+        __syncthreads();
+    }
+    // accumulator (j, i), lane l, register v: column (nt0 + 4 wn + j) * 32 + 8 (v / 4) + 4 (l / 32) + v % 4,
+    // row row0 + 128 wr + 32 i + l % 32
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int nt = nt0 + 4 * wn + j;
+        if (nt >= a.NT) continue;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const long row = row0 + 128 * wr + 32 * i + (lane & 31);
+            if (row >= a.R) continue;
+            if (EPI == BEPI_ACT16 && a.gated) {
+#pragma unroll
+                for (int v = 0; v < 8; ++v) {
+                    const int nl = 8 * (v / 4) + 4 * (lane >> 5) + (v % 4);
+                    const int f = nt * 16 + nl;
+                    if (f < a.n_valid)
+                        a.out16[row * a.ld16 + f] = (half_t)(act_apply(a.act, acc[j][i][v] + a.bias[f]) * (acc[j][i][v + 8] + a.bias2[f]));
+                }
+            } else {
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    const int col = nt * 32 + 8 * (v / 4) + 4 * (lane >> 5) + (v % 4);
+                    if (col >= a.n_valid) continue;
+                    const float s = acc[j][i][v] + a.bias[col];
+                    if (EPI == BEPI_F32_BIAS) a.out[row * a.ld_out + col] = s;
+                    else if (EPI == BEPI_RESID) a.out[row * a.ld_out + col] = s + a.out[row * a.ld_out + col];
+                    else a.out16[row * a.ld16 + col] = (half_t)act_apply(a.act, s);
+                }
+            }
+        }
+    }
+}
+
 // ------------------------------------------------------------------------------------------------
 // fp32 GEMM (fp32 models: prefill and decode): C[ks][M][N] = A[M][K-range ks] * B[K-range][N], 64x64 tile,
 // k accumulated sequentially inside a split.

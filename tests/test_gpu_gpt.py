@@ -172,19 +172,21 @@ def test_generate_matches_stepwise_and_is_deterministic(G):
     gpu.close()
 
 
-def test_decode_equals_prefill_recompute(G):
-    """Size-independent property at the real head shape (GQA 32/8 heads of 64): prefill(P) + decode(tokens) must give
+@pytest.mark.parametrize("batch", [4, 8])
+def test_decode_equals_prefill_recompute(G, batch):
+    """(batch 8: 768 and 800 prompt rows, which takes the LDS-tiled prefill GEMM; batch 4 takes the direct one.)
+    Size-independent property at the real head shape (GQA 32/8 heads of 64): prefill(P) + decode(tokens) must give
     the logits of prefill(P + n).  It exercises cache positions, the RoPE offset and the decode GEMM against the
     prefill GEMM on a model wide enough to use full MFMA tiles."""
-    cfg = dict(synth.CONFIGS["cfg2_1b_gqa_f16"], n_layers=2, vocab=4096, batch=4, prompt=96)
+    cfg = dict(synth.CONFIGS["cfg2_1b_gqa_f16"], n_layers=2, vocab=4096, batch=batch, prompt=96)
     w = synth.make_weights(cfg, 9)
     seqs = synth.make_prompts(cfg, 10, length=100)
-    a = G.HipGpt(cfg, w, max_batch=4, max_seq_len=128)
+    a = G.HipGpt(cfg, w, max_batch=batch, max_seq_len=128)
     a.prefill(seqs[:, :96])
     for t in range(96, 100):
         a.decode(seqs[:, t])
     la = a.logits()
-    b = G.HipGpt(cfg, w, max_batch=4, max_seq_len=128)
+    b = G.HipGpt(cfg, w, max_batch=batch, max_seq_len=128)
     b.prefill(seqs)
     lb = b.logits()
     assert np.abs(la - lb).max() <= 2e-2
@@ -193,6 +195,31 @@ def test_decode_equals_prefill_recompute(G):
     assert np.abs(ka - kb).max() <= 2e-2
     a.close()
     b.close()
+
+
+@pytest.mark.parametrize("name", ["odd_sizes", "gqa_leaky_d32_g4", "mha_ln_relu"])
+def test_fp16_long_prompt_prefill_against_oracle(G, oracle, name):
+    """More than 512 prompt rows: the prefill projections run on the LDS-tiled GEMM (ragged row, column and k tiles
+    with these sizes).  Logits of the last position and the whole KV cache of the last layer against the oracle."""
+    cfg = synth.tiny_config(dtype="f16", **dict(TINY[name], batch=5, prompt=131))
+    w = synth.make_weights(cfg, 21, random_bias=True)
+    orc = oracle.OracleGpt(cfg, w)
+    gpu = G.HipGpt(cfg, w, max_batch=5, max_seq_len=140)
+    seqs = synth.make_prompts(cfg, 22)
+    _, lg = orc.step(seqs, use_cache=True)
+    gpu.prefill(seqs)
+    gl = gpu.logits()
+    assert np.abs(gl - lg).max() <= FP16_ABS
+    assert (gl.argmax(1) == lg.argmax(1)).mean() >= 0.8
+    H, Gk = cfg["n_heads"], cfg["n_kv_heads"]
+    d = cfg["hidden"] // H
+    last = cfg["n_layers"] - 1
+    kc, vc = orc.get_cache(last, 0), orc.get_cache(last, 1)
+    ko = kc.reshape(5, H, d, 131)[:, ::H // Gk].transpose(0, 1, 3, 2)       # reference keeps K as [B*H, d, T]
+    vo = vc.reshape(5, H, 131, d)[:, ::H // Gk]
+    assert np.abs(gpu.get_kv(last, 0) - ko).max() <= 2e-2
+    assert np.abs(gpu.get_kv(last, 1) - vo).max() <= 2e-2
+    gpu.close()
 
 
 def test_topp_stream_matches_oracle(G, oracle):
