@@ -127,6 +127,27 @@ static void launch(TSHipGpt* m, const char* name, void (*kernel)(KArgs...), dim3
     TSHIP_CHECK_HIP(hipGetLastError());
 }
 
+// launch with dynamic LDS beyond the 64 KiB default limit (the attribute is set once per kernel)
+template <typename... KArgs, typename... Args>
+static void launch_shm(TSHipGpt* m, const char* name, void (*kernel)(KArgs...), dim3 grid, dim3 block, unsigned shm, Args... args) {
+    static std::set<const void*> raised;
+    if (!raised.count((const void*)kernel)) {
+        TSHIP_CHECK_HIP(hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shm));
+        raised.insert((const void*)kernel);
+    }
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    if (m && m->prof) {
+        TSHIP_CHECK_HIP(hipEventCreate(&e0));
+        TSHIP_CHECK_HIP(hipEventCreate(&e1));
+        m->prof->names.push_back(name);
+        m->prof->ev0.push_back(e0);
+        m->prof->ev1.push_back(e1);
+    }
+    if (e0) hipExtLaunchKernelGGL(kernel, grid, block, shm, stream(), e0, e1, 0, args...);
+    else hipLaunchKernelGGL(kernel, grid, block, shm, stream(), args...);
+    TSHIP_CHECK_HIP(hipGetLastError());
+}
+
 // decode GEMM split-K: a block has NW wavefronts of 8 k-tiles each in flight; split K across blocks until one
 // pass covers the block's range (keeps partial-sum traffic small: K = 2048 needs no split at batch <= 32)
 static int pick_ks_f16(int NT, int KT, int BT) {
@@ -628,10 +649,12 @@ static void prefill(TSHipGpt* m, const int32_t* host_ids, int B, int Tp) {
     auto big = [&](const char* name, const GemmW& w, const void* X, long ldx, int epi, BigArgs e) {
         e.W = w.buf.as<half_t>(); e.KT = w.KT; e.NT = w.NT; e.X = (const half_t*)X; e.ldx = (int)ldx; e.R = (int)R;
         if (R >= 512) {       // LDS-tiled kernel, 256 x 256 block tile
+            constexpr int CK = 4;
+            const unsigned shm = 2u * 2u * 8u * CK * 1024u;
             dim3 grid((unsigned)ceil_div(w.NT, 8), (unsigned)ceil_div(R, 256));
-            if (epi == BEPI_F32_BIAS) launch(m, name, big_gemm2_f16_kernel<BEPI_F32_BIAS>, grid, dim3(256), e);
-            else if (epi == BEPI_RESID) launch(m, name, big_gemm2_f16_kernel<BEPI_RESID>, grid, dim3(256), e);
-            else launch(m, name, big_gemm2_f16_kernel<BEPI_ACT16>, grid, dim3(256), e);
+            if (epi == BEPI_F32_BIAS) launch_shm(m, name, big_gemm2_f16_kernel<BEPI_F32_BIAS, CK>, grid, dim3(256), shm, e);
+            else if (epi == BEPI_RESID) launch_shm(m, name, big_gemm2_f16_kernel<BEPI_RESID, CK>, grid, dim3(256), shm, e);
+            else launch_shm(m, name, big_gemm2_f16_kernel<BEPI_ACT16, CK>, grid, dim3(256), shm, e);
             return;
         }
         dim3 grid((unsigned)ceil_div(w.NT, 4), (unsigned)(Rp / 128));

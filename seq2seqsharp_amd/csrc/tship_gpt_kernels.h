@@ -14,6 +14,7 @@
 #pragma once
 
 #include "tship_internal.h"
+#include <type_traits>
 
 namespace tship {
 
@@ -317,15 +318,18 @@ __global__ __launch_bounds__(256) void big_gemm_f16_kernel(BigArgs a) {
 }
 
 // LDS-tiled prefill GEMM.  Block tile 256 rows x 256 columns, 4 wavefronts, each owning 128 x 128 (4 x 4 MFMA
-// tiles of 32 x 32, 256 accumulator registers).  K advances in chunks of 32 (two k-tiles): per chunk the block
-// stages 16 weight fragments (already fragment-ordered in memory: straight 1 KiB copies) and 16 activation fragments
-// (row-major in memory, scattered into fragment order) in LDS, double buffered: the next chunk's global loads are in
-// flight in registers while the MFMAs of the current chunk run, one barrier per chunk.
-// Per k-tile a wavefront reads 8 fragments from LDS for 16 MFMAs.
-template <int EPI>
+// tiles of 32 x 32, 256 accumulator registers).  K advances in chunks of CK k-tiles (16 CK columns): per chunk the
+// block stages 8 CK weight fragments (already fragment-ordered in memory: straight 1 KiB copies) and 8 CK activation
+// fragments (row-major in memory, scattered into fragment order) in LDS, double buffered: the next chunk's global
+// loads are in flight in registers while the MFMAs of the current chunk run, one barrier per chunk.
+// Per k-tile a wavefront reads 8 fragments from LDS for 16 MFMAs.  Dynamic LDS: 2 x 16 KiB x CK.
+template <int EPI, int CK>
 __global__ __launch_bounds__(256) void big_gemm2_f16_kernel(BigArgs a) {
-    __shared__ __attribute__((aligned(16))) half_t sW[2][16 * 512];
-    __shared__ __attribute__((aligned(16))) half_t sX[2][16 * 512];
+    extern __shared__ __attribute__((aligned(16))) half_t big_smem[];
+    constexpr int FR = 8 * CK;                       // fragments of one operand per chunk
+    constexpr int LPT = FR / 4;                      // 16-byte loads per thread per operand and chunk
+    half_t* sW = big_smem;                           // [2][FR * 512]
+    half_t* sX = big_smem + 2 * FR * 512;            // [2][FR * 512]
     const int t = threadIdx.x, lane = t & 63, w = __builtin_amdgcn_readfirstlane(t >> 6);
     const int wr = w >> 1, wn = w & 1;
     const int nt0 = blockIdx.x * 8;
@@ -338,36 +342,29 @@ __global__ __launch_bounds__(256) void big_gemm2_f16_kernel(BigArgs a) {
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[j][i][v] = 0.0f;
 
-    // this thread's share of a chunk: 4 x 16 bytes of weights, 4 x 16 bytes of activations
     const half8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
-    const half_t* wsrc[4]; bool wok[4]; int wdst[4];
-    const half_t* xsrc[4]; bool xok[4]; int xdst[4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int f = i * 4 + (t >> 6);                 // fragment of the chunk: n-tile f / 2, k-tile f % 2
-        const int nt = nt0 + (f >> 1);
-        wok[i] = nt < a.NT;
-        wsrc[i] = a.W + (((long)nt * a.KT + (f & 1)) * 64 + lane) * 8;
-        wdst[i] = f * 512 + lane * 8;
-        const int row = i * 64 + (t >> 2), seg = t & 3;  // 64-byte row segment of the chunk in four 16-byte pieces
-        xok[i] = row0 + row < a.R;
-        xsrc[i] = a.X + (row0 + row) * (long)a.ldx + seg * 8;
-        xdst[i] = (((row >> 5) * 2 + (seg >> 1)) * 64 + (row & 31) + 32 * (seg & 1)) * 8;
-    }
-    const int NC = (a.KT + 1) / 2;
-    half8 gw[4], gx[4];
+    const int NC = (a.KT + CK - 1) / CK;
+    half8 gw[LPT], gx[LPT];
+    // fragment f of the chunk = (n-tile or row tile f / CK, k-tile f % CK); thread t fills lane t % 64 of fragments
+    // t / 64 + 4 i of both operands, so every LDS store of a wavefront is one contiguous KiB (no bank conflicts); the
+    // activation rows are read 16 bytes per lane (the neighbouring pieces of a row follow in the next k-tiles)
     auto gload = [&](int c) {
-        const bool k1 = 2 * c + 1 < a.KT;              // odd KT: the last chunk has one k-tile
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
+        for (int i = 0; i < LPT; ++i) {
             const int f = i * 4 + (t >> 6);
-            gw[i] = (wok[i] && ((f & 1) == 0 || k1)) ? *(const half8*)(wsrc[i] + (long)c * 1024) : zero8;
-            gx[i] = (xok[i] && ((t & 3) < 2 || k1)) ? *(const half8*)(xsrc[i] + c * 32) : zero8;
+            const int nt = nt0 + f / CK, kt = c * CK + f % CK;
+            gw[i] = (nt < a.NT && kt < a.KT) ? *(const half8*)(a.W + (((long)nt * a.KT + kt) * 64 + lane) * 8) : zero8;
+            const int row = (f / CK) * 32 + (lane & 31), ktx = c * CK + f % CK;
+            gx[i] = (row0 + row < a.R && ktx < a.KT) ? *(const half8*)(a.X + (row0 + row) * (long)a.ldx + ktx * 16 + 8 * (lane >> 5)) : zero8;
         }
     };
     auto lstore = [&](int buf) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) { *(half8*)(&sW[buf][wdst[i]]) = gw[i]; *(half8*)(&sX[buf][xdst[i]]) = gx[i]; }
+        for (int i = 0; i < LPT; ++i) {
+            const int f = i * 4 + (t >> 6);
+            *(half8*)(sW + ((long)buf * FR + f) * 512 + lane * 8) = gw[i];
+            *(half8*)(sX + ((long)buf * FR + f) * 512 + lane * 8) = gx[i];
+        }
     };
     gload(0);
     lstore(0);
@@ -375,13 +372,15 @@ __global__ __launch_bounds__(256) void big_gemm2_f16_kernel(BigArgs a) {
     for (int c = 0; c < NC; ++c) {
         const int buf = c & 1;
         if (c + 1 < NC) gload(c + 1);
+        const half_t* bw = sW + (long)buf * FR * 512 + lane * 8;
+        const half_t* bx = sX + (long)buf * FR * 512 + lane * 8;
 #pragma unroll
-        for (int kt = 0; kt < 2; ++kt) {
+        for (int kt = 0; kt < CK; ++kt) {
             half8 wf[4], xf[4];
 #pragma unroll
-            for (int j = 0; j < 4; ++j) wf[j] = *(const half8*)(&sW[buf][((4 * wn + j) * 2 + kt) * 512 + lane * 8]);
+            for (int j = 0; j < 4; ++j) wf[j] = *(const half8*)(bw + ((4 * wn + j) * CK + kt) * 512);
 #pragma unroll
-            for (int i = 0; i < 4; ++i) xf[i] = *(const half8*)(&sX[buf][((4 * wr + i) * 2 + kt) * 512 + lane * 8]);
+            for (int i = 0; i < 4; ++i) xf[i] = *(const half8*)(bx + ((4 * wr + i) * CK + kt) * 512);
 #pragma unroll
             for (int j = 0; j < 4; ++j)
 #pragma unroll
@@ -390,37 +389,106 @@ __global__ __launch_bounds__(256) void big_gemm2_f16_kernel(BigArgs a) {
         if (c + 1 < NC) lstore(buf ^ 1);
         __syncthreads();
     }
-    // accumulator (j, i), lane l, register v: column (nt0 + 4 wn + j) * 32 + 8 (v / 4) + 4 (l / 32) + v % 4,
-    // row row0 + 128 wr + 32 i + l % 32
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
+    // accumulator (j, i), lane l, register v = 4 g + e: column (nt0 + 4 wn + j) * 32 + 8 g + 4 (l / 32) + e,
+    // row row0 + 128 wr + 32 i + l % 32.  Biases (and the residual) are fetched in batches before the first store
+    // of a column tile, and the four consecutive columns of a group go out as one 16-byte (fp32) or 8-byte (fp16) store.
+    const int lh = lane >> 5;
+    const bool vec_ok = (a.n_valid % 4 == 0) && ((EPI == BEPI_ACT16 ? a.ld16 : a.ld_out) % 4 == 0);
+    // one column tile per call with a compile-time tile number: the accumulators must only ever be indexed statically
+    auto tile_out = [&](auto J) {
+        constexpr int j = decltype(J)::value;
         const int nt = nt0 + 4 * wn + j;
-        if (nt >= a.NT) continue;
+        if (nt >= a.NT) return;
+        if (EPI == BEPI_ACT16 && a.gated) {
+            float b1[8], b2[8];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const long row = row0 + 128 * wr + 32 * i + (lane & 31);
-            if (row >= a.R) continue;
-            if (EPI == BEPI_ACT16 && a.gated) {
+            for (int v = 0; v < 8; ++v) {
+                const int f = nt * 16 + 8 * (v / 4) + 4 * lh + (v % 4);
+                b1[v] = f < a.n_valid ? a.bias[f] : 0.0f;
+                b2[v] = f < a.n_valid ? a.bias2[f] : 0.0f;
+            }
 #pragma unroll
-                for (int v = 0; v < 8; ++v) {
-                    const int nl = 8 * (v / 4) + 4 * (lane >> 5) + (v % 4);
-                    const int f = nt * 16 + nl;
-                    if (f < a.n_valid)
-                        a.out16[row * a.ld16 + f] = (half_t)(act_apply(a.act, acc[j][i][v] + a.bias[f]) * (acc[j][i][v + 8] + a.bias2[f]));
+            for (int i = 0; i < 4; ++i) {
+                const long row = row0 + 128 * wr + 32 * i + (lane & 31);
+                if (row >= a.R) continue;
+#pragma unroll
+                for (int g = 0; g < 2; ++g) {
+                    const int f0 = nt * 16 + 8 * g + 4 * lh;
+                    half4v o;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) o[e] = (half_t)(act_apply(a.act, acc[j][i][4 * g + e] + b1[4 * g + e]) * (acc[j][i][4 * g + e + 8] + b2[4 * g + e]));
+                    half_t* dst = a.out16 + row * a.ld16 + f0;
+                    if (vec_ok && f0 + 3 < a.n_valid) *(half4v*)dst = o;
+                    else {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) if (f0 + e < a.n_valid) dst[e] = o[e];
+                    }
                 }
-            } else {
+            }
+        } else {
+            float bb[16];
 #pragma unroll
-                for (int v = 0; v < 16; ++v) {
-                    const int col = nt * 32 + 8 * (v / 4) + 4 * (lane >> 5) + (v % 4);
-                    if (col >= a.n_valid) continue;
-                    const float s = acc[j][i][v] + a.bias[col];
-                    if (EPI == BEPI_F32_BIAS) a.out[row * a.ld_out + col] = s;
-                    else if (EPI == BEPI_RESID) a.out[row * a.ld_out + col] = s + a.out[row * a.ld_out + col];
-                    else a.out16[row * a.ld16 + col] = (half_t)act_apply(a.act, s);
+            for (int v = 0; v < 16; ++v) {
+                const int col = nt * 32 + 8 * (v / 4) + 4 * lh + (v % 4);
+                bb[v] = col < a.n_valid ? a.bias[col] : 0.0f;
+            }
+            floatx4 old[4][4];
+            if (EPI == BEPI_RESID) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const long row = row0 + 128 * wr + 32 * i + (lane & 31);
+#pragma unroll
+                    for (int g = 0; g < 4; ++g) {
+                        const int c0 = nt * 32 + 8 * g + 4 * lh;
+                        const float* src = a.out + row * a.ld_out + c0;
+                        if (row < a.R && vec_ok && c0 + 3 < a.n_valid) old[i][g] = *(const floatx4*)src;
+                        else {
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) old[i][g][e] = (row < a.R && c0 + e < a.n_valid) ? src[e] : 0.0f;
+                        }
+                    }
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const long row = row0 + 128 * wr + 32 * i + (lane & 31);
+                if (row >= a.R) continue;
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const int c0 = nt * 32 + 8 * g + 4 * lh;
+                    floatx4 s;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) s[e] = acc[j][i][4 * g + e] + bb[4 * g + e];
+                    if (EPI == BEPI_ACT16) {
+                        half4v o;
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) o[e] = (half_t)act_apply(a.act, s[e]);
+                        half_t* dst = a.out16 + row * a.ld16 + c0;
+                        if (vec_ok && c0 + 3 < a.n_valid) *(half4v*)dst = o;
+                        else {
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) if (c0 + e < a.n_valid) dst[e] = o[e];
+                        }
+                    } else {
+                        if (EPI == BEPI_RESID) {
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) s[e] = s[e] + old[i][g][e];
+                        }
+                        float* dst = a.out + row * a.ld_out + c0;
+                        if (vec_ok && c0 + 3 < a.n_valid) *(floatx4*)dst = s;
+                        else {
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) if (c0 + e < a.n_valid) dst[e] = s[e];
+                        }
+                    }
                 }
             }
         }
-    }
+    };
+    tile_out(std::integral_constant<int, 0>{});
+    tile_out(std::integral_constant<int, 1>{});
+    tile_out(std::integral_constant<int, 2>{});
+    tile_out(std::integral_constant<int, 3>{});
 }
 
 // ------------------------------------------------------------------------------------------------

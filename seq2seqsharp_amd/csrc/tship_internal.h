@@ -56,6 +56,7 @@ typedef _Float16 half_t;
 typedef half_t half8 __attribute__((ext_vector_type(8)));
 typedef half_t half4 __attribute__((ext_vector_type(4)));
 typedef half_t half2v __attribute__((ext_vector_type(2)));
+typedef half_t half4v __attribute__((ext_vector_type(4)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 
