@@ -33,6 +33,10 @@ def algorithmic_prefill_flops(cfg, B, Tp):
     return 2.0 * B * Tp * per_tok + 2.0 * B * h * V + L * B * H * d * float(Tp) * Tp * 2.0
 
 
+def _log(msg):
+    print("[bench] " + msg, file=sys.stderr, flush=True)
+
+
 def cpu_baseline(cfg, gpu, weights, next_ids, budget_note):
     """One decode step of the CPU oracle (kind "port": a restatement of the reference's CPU path), single
     thread, at the benchmark's shape, on the KV cache the GPU prefill produced.  Also returns the logit
@@ -85,12 +89,15 @@ def main():
         cfg["prompt"] = args.prompt
     B, Tp, K, W = cfg["batch"], cfg["prompt"], args.steps, args.warmup
     t0 = time.perf_counter()
+    _log("generating weights for %s" % args.config)
     weights = synth.make_weights(cfg, seed=0)
+    _log("uploading weights")
     gpu = HipGpt(cfg, weights, max_batch=B, max_seq_len=Tp + 2 * (W + K) + 8)
     t_load = time.perf_counter() - t0
     prompts = synth.make_prompts(cfg, seed=1)
 
     # prefill (timed separately)
+    _log("prefill of %d x %d tokens" % (B, Tp))
     gpu.prefill(prompts[:, :8])            # touch every kernel once
     gpu.reset()
     t0 = time.perf_counter()
@@ -100,6 +107,7 @@ def main():
     prefill_tflops = algorithmic_prefill_flops(cfg, B, Tp) / t_prefill / 1e12
 
     # decode: W warm-up steps, then exactly K timed steps (device events on the library stream, bracketed by syncs)
+    _log("decode: %d warm-up + %d timed steps" % (W, K))
     gpu.generate(max(W, 1))
     T_start = gpu.seq_len()
     wall0 = time.perf_counter()
@@ -165,10 +173,12 @@ def main():
         "load_seconds": round(t_load, 1),
     }
     if not args.no_topp:
+        _log("top-p decode")
         u = synth.make_uniforms(7, B, K)
         _, ms_p = gpu.generate(K, mode=TOPP, top_p=0.9, temperature=1.0, uniforms=u)
         out["topp"] = {"top_p": 0.9, "tokens_per_s": round(B * K / (ms_p / 1e3), 1), "ms_per_step": round(ms_p / K, 4)}
     if not args.no_cpu_baseline:
+        _log("CPU baseline (one decode step of the oracle, single thread)")
         nxt = gpu.sample()
         base, lg = cpu_baseline(cfg, gpu, weights, nxt, "cache from the GPU prefill")
         gpu.decode(nxt)

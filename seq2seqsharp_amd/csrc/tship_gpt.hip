@@ -130,10 +130,12 @@ static void launch(TSHipGpt* m, const char* name, void (*kernel)(KArgs...), dim3
 // launch with dynamic LDS beyond the 64 KiB default limit (the attribute is set once per kernel)
 template <typename... KArgs, typename... Args>
 static void launch_shm(TSHipGpt* m, const char* name, void (*kernel)(KArgs...), dim3 grid, dim3 block, unsigned shm, Args... args) {
-    static std::set<const void*> raised;
-    if (!raised.count((const void*)kernel)) {
+    static std::map<const void*, unsigned> raised;
+    unsigned& have = raised[(const void*)kernel];
+    if (shm > 65536u && shm > have) {
+        TSHIP_REQUIRE(shm <= 160u * 1024u, "dynamic LDS request exceeds the 160 KiB of a compute unit");
         TSHIP_CHECK_HIP(hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shm));
-        raised.insert((const void*)kernel);
+        have = shm;
     }
     hipEvent_t e0 = nullptr, e1 = nullptr;
     if (m && m->prof) {
@@ -961,8 +963,7 @@ TSHIP_API int TSHip_GptGenerate(TSHipGpt* m, int n_steps, int mode, float top_p,
     bool any_moe = false; for (auto& L : m->L) any_moe = any_moe || L->moe;
     const bool use_graph = !any_moe && std::getenv("TSHIP_NO_GRAPH") == nullptr;
     if (mode == TSHIP_TOPP) {      // scratch must exist before capture (no allocation inside a graph)
-        const long Vs = round_up(m->c.vocab, 64);
-        size_t need = (size_t)m->Bpad * Vs * 5 * 4;
+        const size_t need = topp_scratch_bytes(m->Bpad, m->c.vocab);
         if (m->topp_scratch.bytes < need) m->topp_scratch.alloc(need);
     }
     if (use_graph) {

@@ -59,8 +59,10 @@ static void run_moe_ffn(TSHipGpt* m, LayerW& L, int rows, const ResidNormArgs& p
     r.gamma = pre.gamma; r.beta = pre.beta; r.eps = pre.eps;
     r.router = L.router.as<float>(); r.router_b = L.router_b.as<float>(); r.E = E; r.k = k;
     r.xn32 = xn32; r.probs = probs; r.top_val = top_val; r.top_idx = top_idx;
-    launch(m, "moe_router", moe_router_kernel, dim3(rows), dim3(64), r);
-    launch(m, "moe_lists", moe_lists_kernel, dim3(1), dim3(64), (const float*)top_idx, rows, k, E, Bp, counts, lists, slot);
+    r.router_lds = ((long)E * h <= 16384) ? 1 : 0;
+    const unsigned router_shm = (unsigned)((2L * h + (r.router_lds ? (long)E * h : 0)) * sizeof(float));
+    launch_shm(m, "moe_router", moe_router_kernel, dim3(rows), dim3(256), router_shm, r);
+    launch_shm(m, "moe_lists", moe_lists_kernel, dim3(1), dim3(64), (unsigned)(rows * k * sizeof(int)), (const float*)top_idx, rows, k, E, Bp, counts, lists, slot);
     const long xg_stride = (long)Bp * m->ldh, mid_stride = (long)Bp * o.ld4h, y_stride = (long)Bp * o.ldy;
     if (m->f16) {
         half_t* xg = (half_t*)(base + o.xg); half_t* mid = (half_t*)(base + o.mid);
@@ -122,8 +124,7 @@ static void sample_tokens(TSHipGpt* m, int mode, float top_p, float temperature,
     TSHIP_REQUIRE(mode == TSHIP_TOPP, "unknown sampling mode");
     TSHIP_REQUIRE(m->c.vocab <= 65535, "top-p sampling supports vocabularies up to 65535");
     TSHIP_REQUIRE(temperature > 0.0f, "temperature must be positive");
-    const long Vs = round_up(m->c.vocab, 64);
-    size_t need = (size_t)m->Bpad * Vs * 5 * 4;
+    const size_t need = topp_scratch_bytes(m->Bpad, m->c.vocab);
     if (m->topp_scratch.bytes < need) m->topp_scratch.alloc(need);
     if (!dev_uniforms) {
         TSHIP_REQUIRE(host_uniforms, "top-p sampling needs one uniform draw per row");
@@ -133,13 +134,12 @@ static void sample_tokens(TSHipGpt* m, int mode, float top_p, float temperature,
     }
     TopPArgs a; std::memset(&a, 0, sizeof(a));
     a.in = m->logits.as<float>(); a.ld = Vp; a.V = m->c.vocab; a.in_is_logits = 1;
-    a.uniforms = dev_uniforms; a.top_p = top_p; a.Vs = Vs;
-    char* s = (char*)m->topp_scratch.p; size_t one = (size_t)m->Bpad * Vs * 4;
-    a.keysA = (unsigned*)s; a.keysB = (unsigned*)(s + one); a.idxA = (int*)(s + 2 * one); a.idxB = (int*)(s + 3 * one); a.accp = (float*)(s + 4 * one);
+    a.uniforms = dev_uniforms; a.top_p = top_p;
+    topp_carve(a, m->topp_scratch.p, m->Bpad, m->c.vocab);
     a.next_ids = m->ids.as<int>(); a.gen_out = gen_out; a.d_step = d_step;
     // Decoder.cs:720-723 divides the logits by the temperature (fp32 division) before the softmax
     a.temperature = temperature;
-    launch(m, "topp", topp_kernel, dim3(B), dim3(256), a);
+    topp_run(a, B, [&](const char* name, void (*kernel)(TopPArgs), dim3 grid, dim3 block, const TopPArgs& args) { launch(m, name, kernel, grid, block, args); });
 }
 
 }  // namespace tship

@@ -134,6 +134,16 @@ __global__ __launch_bounds__(NW * 64) void skinny_gemm_f16_kernel(SkinnyArgs a) 
 #pragma unroll
         for (int v = 0; v < 16; ++v) acc[bt][v] = 0.0f;
 
+    // deferred-norm inputs: this thread's share of the per-tile sums of squares, fetched before the weight stream
+    __shared__ float srinv[BT * 32];
+    constexpr int NCH = (NW * 64) / (BT * 32);
+    __shared__ float schunk[NCH][BT * 32];
+    float ssq_part = 0.0f;
+    if (a.ssq) {
+        const int b = threadIdx.x % (BT * 32), ch = threadIdx.x / (BT * 32);
+        const int per_ch = (a.ssq_nt + NCH - 1) / NCH;
+        for (int t = ch * per_ch; t < min(a.ssq_nt, (ch + 1) * per_ch); ++t) ssq_part += a.ssq[(long)t * a.ssq_ld + b];
+    }
     const half_t* wp = a.W + ((long)nt * a.KT * 64 + lane) * 8;
     const half_t* xp = a.X + lane * 8;
     for (int kt = wk0; kt < wk1; kt += U) {
@@ -155,16 +165,10 @@ __global__ __launch_bounds__(NW * 64) void skinny_gemm_f16_kernel(SkinnyArgs a) 
             }
         }
     }
-    // rinv per row from the tile sums: NCH chunks of tiles are added in parallel, then the chunk sums in order
-    __shared__ float srinv[BT * 32];
-    constexpr int NCH = (NW * 64) / (BT * 32);
-    __shared__ float schunk[NCH][BT * 32];
+    // rinv per row from the tile sums: NCH chunks of tiles are added in parallel (loads issued before the weight
+    // stream, see above), then the chunk sums in order
     if (a.ssq) {
-        const int b = threadIdx.x % (BT * 32), ch = threadIdx.x / (BT * 32);
-        const int per_ch = (a.ssq_nt + NCH - 1) / NCH;
-        float s = 0.0f;
-        for (int t = ch * per_ch; t < min(a.ssq_nt, (ch + 1) * per_ch); ++t) s += a.ssq[(long)t * a.ssq_ld + b];
-        schunk[ch][b] = s;
+        schunk[threadIdx.x / (BT * 32)][threadIdx.x % (BT * 32)] = ssq_part;
         __syncthreads();
         if (threadIdx.x < BT * 32) {
             float tot = 0.0f;
@@ -374,17 +378,34 @@ __global__ __launch_bounds__(256) void big_gemm2_f16_kernel(BigArgs a) {
         if (c + 1 < NC) gload(c + 1);
         const half_t* bw = sW + (long)buf * FR * 512 + lane * 8;
         const half_t* bx = sX + (long)buf * FR * 512 + lane * 8;
-#pragma unroll
-        for (int kt = 0; kt < CK; ++kt) {
-            half8 wf[4], xf[4];
+        // fragments of k-tile kt + 1 are read from LDS while the 16 MFMAs of k-tile kt run
+        half8 wfA[4], xfA[4], wfB[4], xfB[4];
+        auto lread = [&](int kt, half8 (&wf)[4], half8 (&xf)[4]) {
 #pragma unroll
             for (int j = 0; j < 4; ++j) wf[j] = *(const half8*)(bw + ((4 * wn + j) * CK + kt) * 512);
 #pragma unroll
             for (int i = 0; i < 4; ++i) xf[i] = *(const half8*)(bx + ((4 * wr + i) * CK + kt) * 512);
+        };
+        auto mma = [&](half8 (&wf)[4], half8 (&xf)[4]) {
 #pragma unroll
             for (int j = 0; j < 4; ++j)
 #pragma unroll
                 for (int i = 0; i < 4; ++i) acc[j][i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf[j], xf[i], acc[j][i], 0, 0, 0);
+        };
+        // (the scheduling barriers keep the compiler from sinking the reads back to their first use)
+        lread(0, wfA, xfA);
+#pragma unroll
+        for (int kt = 0; kt < CK; kt += 2) {
+            if (kt + 1 < CK) lread(kt + 1, wfB, xfB);
+            __builtin_amdgcn_sched_barrier(0);
+            mma(wfA, xfA);
+            __builtin_amdgcn_sched_barrier(0);
+            if (kt + 1 < CK) {
+                if (kt + 2 < CK) lread(kt + 2, wfA, xfA);
+                __builtin_amdgcn_sched_barrier(0);
+                mma(wfB, xfB);
+                __builtin_amdgcn_sched_barrier(0);
+            }
         }
         if (c + 1 < NC) lstore(buf ^ 1);
         __syncthreads();

@@ -19,6 +19,7 @@ struct MoeRouterArgs {
     const float* gamma; const float* beta; float eps;
     const float* router; const float* router_b; int E; int k;
     float* xn32; float* probs; float* top_val; float* top_idx;
+    int router_lds;      // 1: the launch reserved LDS for the router matrix
 };
 
 __device__ __forceinline__ float tree8(float v) {
@@ -29,14 +30,19 @@ __device__ __forceinline__ float tree8(float v) {
     return v;
 }
 
-__global__ __launch_bounds__(64) void moe_router_kernel(MoeRouterArgs a) {
+// One block of 256 threads per token row.  Dynamic LDS: x[h], xn[h], and the router matrix [h][E] when it fits
+// (a.router_lds != 0), so that the serial dot products read LDS only.
+__global__ __launch_bounds__(256) void moe_router_kernel(MoeRouterArgs a) {
 #pragma clang fp contract(off)
-    __shared__ float sx[4096];
-    __shared__ float sxn[4096];
+    extern __shared__ float moe_smem[];
     __shared__ float sr[64];
     __shared__ float s_stat[2];
-    const int r = blockIdx.x, t = threadIdx.x, h = a.h;
-    for (int c = t; c < h; c += 64) {
+    const int r = blockIdx.x, t = threadIdx.x, h = a.h, E = a.E;
+    float* sx = moe_smem;
+    float* sxn = moe_smem + h;
+    float* srt = moe_smem + 2 * h;
+    if (a.router_lds) for (int i = t; i < h * E; i += 256) srt[i] = a.router[i];
+    for (int c = t; c < h; c += 256) {
         float v = a.x[(long)r * a.ldx + c];
         if (a.part) {
             float s = a.part[(long)r * a.ld_part + c];
@@ -47,42 +53,67 @@ __global__ __launch_bounds__(64) void moe_router_kernel(MoeRouterArgs a) {
         sx[c] = v;
     }
     __syncthreads();
+    // LayerNorm statistics in the reference's order (TensorApplyCPU.cs:1381-1409): eight interleaved partial sums
+    // added as a tree, then the tail; for the variance every group of eight squared deviations is added as a tree and
+    // the group sums sequentially.  The group trees are independent, so all threads compute them; only the two short
+    // sequential chains run on one thread.
+    const int ng = h > 8 ? (h - 8 + 7) / 8 : 0;       // full groups handled by the interleaved loops
     if (t < 8) {
         float lane = 0.0f;
-        int i = 0;
-        for (; i < h - 8; i += 8) lane += sx[i + t];
+#pragma unroll 8
+        for (int j = 0; j < ng; ++j) lane += sx[8 * j + t];
         float sum = tree8(lane);
-        for (; i < h; ++i) sum += sx[i];
-        float mean = sum / (float)h;
-        float sq = 0.0f;
-        for (i = 0; i < h - 8; i += 8) {
-            float d = sx[i + t] - mean;
-            sq += tree8(d * d);
+        for (int i = 8 * ng; i < h; ++i) sum += sx[i];
+        if (t == 0) s_stat[0] = sum / (float)h;
+    }
+    __syncthreads();
+    {
+        const float mean0 = s_stat[0];
+        for (int j = t; j < ng; j += 256) {
+            float dd[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) { const float d = sx[8 * j + u] - mean0; dd[u] = d * d; }
+            sxn[j] = ((dd[0] + dd[1]) + (dd[2] + dd[3])) + ((dd[4] + dd[5]) + (dd[6] + dd[7]));
         }
-        for (; i < h; ++i) { float d = sx[i] - mean; sq += d * d; }
-        float sigma = sqrtf(a.eps + sq / (float)h);
-        if (t == 0) { s_stat[0] = mean; s_stat[1] = sigma; }
+    }
+    __syncthreads();
+    if (t == 0) {
+        const float mean0 = s_stat[0];
+        float sq = 0.0f;
+#pragma unroll 8
+        for (int j = 0; j < ng; ++j) sq += sxn[j];
+        for (int i = 8 * ng; i < h; ++i) { const float d = sx[i] - mean0; sq += d * d; }
+        s_stat[1] = sqrtf(a.eps + sq / (float)h);
     }
     __syncthreads();
     const float mean = s_stat[0], sigma = s_stat[1];
-    for (int c = t; c < h; c += 64) {
+    for (int c = t; c < h; c += 256) {
         float y = a.gamma[c] * ((sx[c] - mean) / sigma);
         y += a.beta[c];
         sxn[c] = y;
         a.xn32[(long)r * h + c] = y;
     }
     __syncthreads();
-    if (t < a.E) {
+    if (t < E) {
+        // serial over l, product and sum rounded separately, zero inputs skipped (SGEMM.cs:482-549)
         float acc = a.router_b[t];
-        for (int l = 0; l < h; ++l) {
-            float xv = sxn[l];
-            if (xv != 0.0f) acc += xv * a.router[(long)l * a.E + t];
-        }
+        auto dot = [&](auto rt) {          // rt: LDS or global pointer (kept apart so that LDS reads stay ds_read)
+            int l = 0;
+            for (; l + 8 <= h; l += 8) {
+                float xv[8], wv[8];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) { xv[u] = sxn[l + u]; wv[u] = rt[(long)(l + u) * E + t]; }
+#pragma unroll
+                for (int u = 0; u < 8; ++u) { const float s = acc + xv[u] * wv[u]; acc = xv[u] != 0.0f ? s : acc; }
+            }
+            for (; l < h; ++l) { const float xv = sxn[l]; if (xv != 0.0f) acc += xv * rt[(long)l * E + t]; }
+        };
+        if (a.router_lds) dot((const float*)srt); else dot(a.router);
         sr[t] = acc + (-65000.0f);
     }
     __syncthreads();
     if (t == 0) {
-        const int E = a.E, k = a.k;
+        const int k = a.k;
         float mx = sr[0];
         for (int e = 1; e < E; ++e) mx = fmaxf(mx, sr[e]);
         float sum = 0.0f;
@@ -106,14 +137,16 @@ __global__ __launch_bounds__(64) void moe_router_kernel(MoeRouterArgs a) {
 
 // per-expert token lists in ascending token order (MoEFeedForward.cs:92-105); slot[i*k+j] = position of token i in
 // the list of its j-th expert
-__global__ void moe_lists_kernel(const float* __restrict__ top_idx, int rows, int k, int E, int max_rows, int* __restrict__ counts,
-                                 int* __restrict__ lists, int* __restrict__ slot) {
+__global__ __launch_bounds__(64) void moe_lists_kernel(const float* __restrict__ top_idx, int rows, int k, int E, int max_rows, int* __restrict__ counts,
+                                                        int* __restrict__ lists, int* __restrict__ slot) {
+    extern __shared__ int s_idx[];
+    for (int i = threadIdx.x; i < rows * k; i += 64) s_idx[i] = (int)top_idx[i];
+    __syncthreads();
     int e = threadIdx.x;
     if (e >= E) return;
     int n = 0;
-    for (int i = 0; i < rows; ++i)
-        for (int j = 0; j < k; ++j)
-            if ((int)top_idx[i * k + j] == e) { lists[e * max_rows + n] = i; slot[i * k + j] = n; ++n; }
+    for (int i = 0; i < rows * k; ++i)
+        if (s_idx[i] == e) { lists[e * max_rows + n] = i / k; slot[i] = n; ++n; }
     counts[e] = n;
 }
 

@@ -636,16 +636,16 @@ TSHIP_API int TSHip_TopPSample(const TSHipTensor* result, const TSHipTensor* pro
     TSHIP_REQUIRE(count(r) == rows && r.dtype == TSHIP_F32 && is_contiguous(r), "TSHip_TopPSample: result must be a contiguous Float32 [rows,1] tensor");
     TSHIP_REQUIRE(count(u) == rows && u.dtype == TSHIP_F32 && is_contiguous(u), "TSHip_TopPSample: uniforms must be a contiguous Float32 [rows] tensor");
     if (rows == 0) return 1;
-    const long Vs = round_up(K, 64);
     void* scratch = nullptr;
-    TSHIP_CHECK_HIP(hipMalloc(&scratch, (size_t)rows * Vs * 5 * 4));
+    TSHIP_CHECK_HIP(hipMalloc(&scratch, topp_scratch_bytes(rows, K)));
     TopPArgs a; std::memset(&a, 0, sizeof(a));
     a.in = (const float*)p.p; a.ld = p.st[0]; a.V = (int)K; a.in_is_logits = 0; a.temperature = 1.0f;
-    a.uniforms = (const float*)u.p; a.top_p = top_p; a.Vs = Vs;
-    char* s = (char*)scratch; size_t one = (size_t)rows * Vs * 4;
-    a.keysA = (unsigned*)s; a.keysB = (unsigned*)(s + one); a.idxA = (int*)(s + 2 * one); a.idxB = (int*)(s + 3 * one); a.accp = (float*)(s + 4 * one);
+    a.uniforms = (const float*)u.p; a.top_p = top_p;
+    topp_carve(a, scratch, rows, K);
     a.out_f32 = (float*)r.p;
-    hipLaunchKernelGGL(topp_kernel, dim3((unsigned)rows), dim3(256), 0, stream(), a);
+    topp_run(a, (int)rows, [&](const char*, void (*kernel)(TopPArgs), dim3 grid, dim3 block, const TopPArgs& args) {
+        hipLaunchKernelGGL(kernel, grid, block, 0, stream(), args);
+    });
     hipError_t e = hipGetLastError();
     if (e == hipSuccess) e = hipStreamSynchronize(stream());
     (void)hipFree(scratch);

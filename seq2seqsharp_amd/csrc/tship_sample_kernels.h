@@ -1,16 +1,20 @@
-// Top-p sampling on the device: one block per row.
+// Top-p sampling on the device.
 // Semantics of ComputeGraphTensor.TopPSample (Seq2SeqSharp/Tools/ComputeGraphTensor.cs:2305-2403) with
 // repeatPenalty = 0 (pow(x, 0) = 1: no decay) and the per-row random draw supplied by the caller:
 //   keep p > 0; order by p descending, equal p by ascending index (SortedDictionary<float, List<int>> walked in
 //   reverse, each list in insertion order); running fp32 sum in that order, stop after the element that makes
 //   acc >= topP; pick the first k with accP[k] / acc >= u.
-// The order is produced by a stable least-significant-digit radix sort on the float bit pattern; the running
-// sum is taken serially in fp32, so for given probabilities the chosen index is the reference's, bit for bit.
+// The order is produced by a stable least-significant-digit radix sort on the float bit pattern (four passes of
+// eight bits, every pass = histogram, scan, scatter over segments of 1024 elements, so a row is sorted by many
+// blocks); the running sum is taken serially in fp32 by one wavefront, so for given probabilities the chosen index
+// is the reference's, bit for bit.
 #pragma once
 
 #include "tship_internal.h"
 
 namespace tship {
+
+constexpr int TOPP_SEG = 1024;            // elements per sort block: 4 wavefronts x 4 rounds x 64 lanes, in index order
 
 struct TopPArgs {
     const float* in; long ld; int V;       // logits (softmax applied here) or probabilities
@@ -19,9 +23,23 @@ struct TopPArgs {
     float top_p;
     unsigned* keysA; unsigned* keysB; int* idxA; int* idxB; float* accp;   // scratch, each [rows][Vs]
     long Vs;
+    int* hist; int nseg;                   // scratch [rows][nseg][256]
+    int shift;                             // digit of the current sort pass
     int* next_ids; int* gen_out; float* out_f32;   // any of them may be null
     const int* d_step;                             // optional: uniforms and gen_out are indexed by *d_step * rows + row
 };
+
+inline size_t topp_scratch_bytes(long rows, long V) {
+    const long Vs = round_up(V, 64), nseg = ceil_div(V, (long)TOPP_SEG);
+    return (size_t)rows * Vs * 5 * 4 + (size_t)rows * nseg * 256 * 4;
+}
+inline void topp_carve(TopPArgs& a, void* scratch, long rows, long V) {
+    const long Vs = round_up(V, 64);
+    char* s = (char*)scratch; const size_t one = (size_t)rows * Vs * 4;
+    a.Vs = Vs; a.nseg = (int)ceil_div(V, (long)TOPP_SEG);
+    a.keysA = (unsigned*)s; a.keysB = (unsigned*)(s + one); a.idxA = (int*)(s + 2 * one); a.idxB = (int*)(s + 3 * one);
+    a.accp = (float*)(s + 4 * one); a.hist = (int*)(s + 5 * one);
+}
 
 __device__ __forceinline__ float block_max_256(float v, float* s) {
 #pragma unroll
@@ -32,112 +50,212 @@ __device__ __forceinline__ float block_max_256(float v, float* s) {
     return fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3]));
 }
 
-static __global__ __launch_bounds__(256) void topp_kernel(TopPArgs a) {
-    __shared__ float sred[4];
-    __shared__ unsigned short cnt[16][256];
-    __shared__ int s_total[17];
-    __shared__ int s_n;
-    __shared__ float s_acc;
-    __shared__ int s_pick;
+__device__ __forceinline__ float block_max_1024(float v, float* s) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) s[threadIdx.x >> 6] = v;
+    __syncthreads();
+    float m = s[0];
+#pragma unroll
+    for (int i = 1; i < 16; ++i) m = fmaxf(m, s[i]);
+    return m;
+}
+
+// probabilities (TensorApplyCPU.Softmax, TensorApplyCPU.cs:1230-1268) written as sort keys: grid (rows), 1024 threads
+static __global__ __launch_bounds__(1024) void topp_keys_kernel(TopPArgs a) {
+    __shared__ float sred[16];
     const int r = blockIdx.x, t = threadIdx.x, V = a.V;
     const float* row = a.in + (long)r * a.ld;
-    unsigned* kA = a.keysA + (long)r * a.Vs; unsigned* kB = a.keysB + (long)r * a.Vs;
-    int* iA = a.idxA + (long)r * a.Vs; int* iB = a.idxB + (long)r * a.Vs;
-    float* accp = a.accp + (long)r * a.Vs;
-
-    // probabilities (TensorApplyCPU.Softmax, TensorApplyCPU.cs:1230-1268), written as sort keys
+    unsigned* kA = a.keysA + (long)r * a.Vs;
+    int* iA = a.idxA + (long)r * a.Vs;
     float sum = 1.0f, mx = 0.0f;
     if (a.in_is_logits) {
         float lm = -INFINITY;
-        for (int i = t; i < V; i += 256) lm = fmaxf(lm, row[i] / a.temperature);
-        mx = block_max_256(lm, sred);
+        for (int i = t; i < V; i += 1024) lm = fmaxf(lm, row[i] / a.temperature);
+        mx = block_max_1024(lm, sred);
         float ls = 0.0f;
-        for (int i = t; i < V; i += 256) ls += expf(row[i] / a.temperature - mx);
+        for (int i = t; i < V; i += 1024) ls += expf(row[i] / a.temperature - mx);
         ls = wave_sum(ls);
         __syncthreads();
         if ((t & 63) == 0) sred[t >> 6] = ls;
         __syncthreads();
-        sum = (sred[0] + sred[1]) + (sred[2] + sred[3]);
+        sum = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) sum += sred[i];
     }
-    // each thread owns a contiguous chunk so that the scatter below is stable
-    const int chunk = (V + 255) / 256, c0 = t * chunk, c1 = min(V, c0 + chunk);
-    for (int i = c0; i < c1; ++i) {
-        float p = a.in_is_logits ? expf(row[i] / a.temperature - mx) / sum : row[i];
+    for (int i = t; i < V; i += 1024) {
+        const float p = a.in_is_logits ? expf(row[i] / a.temperature - mx) / sum : row[i];
         // p > 0: positive floats order like their bit patterns; descending order = ascending ~bits.
         // p <= 0 is dropped by the reference: give it the largest key so that it sorts behind every candidate.
         kA[i] = p > 0.0f ? ~__float_as_uint(p) : 0xffffffffu;
         iA[i] = i;
     }
+}
+
+// digit counts of one segment: grid (nseg, rows), 256 threads
+static __global__ __launch_bounds__(256) void topp_hist_kernel(TopPArgs a) {
+    __shared__ int h[256];
+    const int seg = blockIdx.x, r = blockIdx.y, t = threadIdx.x;
+    const unsigned* k = a.keysA + (long)r * a.Vs;
+    h[t] = 0;
     __syncthreads();
-    for (int pass = 0; pass < 8; ++pass) {
-        const int sh = pass * 4;
-        unsigned short c[16];
 #pragma unroll
-        for (int d = 0; d < 16; ++d) c[d] = 0;
-        for (int i = c0; i < c1; ++i) {
-            unsigned d = (kA[i] >> sh) & 15u;
-#pragma unroll
-            for (int q = 0; q < 16; ++q) c[q] += (d == (unsigned)q);
-        }
-#pragma unroll
-        for (int d = 0; d < 16; ++d) cnt[d][t] = c[d];
-        __syncthreads();
-        // exclusive scan over (digit major, thread minor): 16 threads scan one digit row each, then the digit totals
-        if (t < 16) {
-            int run = 0;
-            for (int j = 0; j < 256; ++j) { int v = cnt[t][j]; cnt[t][j] = (unsigned short)run; run += v; }
-            s_total[t] = run;
-        }
-        __syncthreads();
-        if (t == 0) { int run = 0; for (int d = 0; d < 16; ++d) { int v = s_total[d]; s_total[d] = run; run += v; } }
-        __syncthreads();
-        int off[16];
-#pragma unroll
-        for (int d = 0; d < 16; ++d) off[d] = s_total[d] + cnt[d][t];
-        for (int i = c0; i < c1; ++i) {
-            unsigned k = kA[i]; int id = iA[i];
-            unsigned d = (k >> sh) & 15u;
-            int dst = 0;
-#pragma unroll
-            for (int q = 0; q < 16; ++q) if (d == (unsigned)q) { dst = off[q]; off[q] += 1; }
-            kB[dst] = k; iB[dst] = id;
-        }
-        __syncthreads();
-        unsigned* tk = kA; kA = kB; kB = tk;
-        int* ti = iA; iA = iB; iB = ti;
-    }
-    // serial fp32 prefix in sorted order by the first wavefront; every lane keeps the same running value
-    if (t < 64) {
-        float acc = 0.0f; int n = 0; bool done = false;
-        for (int base = 0; base < V && !done; base += 64) {
-            int i = base + t;
-            unsigned k = i < V ? kA[i] : 0xffffffffu;
-            float p = k == 0xffffffffu ? 0.0f : __uint_as_float(~k);
-            float mine = 0.0f;
-            for (int j = 0; j < 64; ++j) {
-                float pj = __shfl(p, j, 64);
-                if (pj <= 0.0f) { done = true; break; }        // ran out of candidates
-                acc += pj; n += 1;
-                if (t == j) mine = acc;
-                if (acc >= a.top_p) { done = true; break; }
-            }
-            if (i < V) accp[i] = mine;
-        }
-        if (t == 0) { s_n = n; s_acc = acc; s_pick = 0x7fffffff; }
+    for (int it = 0; it < 4; ++it) {
+        const int e = seg * TOPP_SEG + it * 256 + t;
+        if (e < a.V) atomicAdd(&h[(k[e] >> a.shift) & 255u], 1);
     }
     __syncthreads();
+    a.hist[((long)r * a.nseg + seg) * 256 + t] = h[t];
+}
+
+// exclusive scan in (digit major, segment minor) order: grid (rows), 256 threads (one digit each)
+static __global__ __launch_bounds__(256) void topp_scan_kernel(TopPArgs a) {
+    __shared__ int tot[256];
+    const int r = blockIdx.x, d = threadIdx.x;
+    int* h = a.hist + (long)r * a.nseg * 256;
+    int run = 0;
+    for (int s = 0; s < a.nseg; ++s) { const int v = h[s * 256 + d]; h[s * 256 + d] = run; run += v; }
+    tot[d] = run;
+    __syncthreads();
+    if (d < 64) {       // one wavefront: 4 digits per lane, then a shuffle scan over the lane sums
+        const int v0 = tot[4 * d], v1 = tot[4 * d + 1], v2 = tot[4 * d + 2], v3 = tot[4 * d + 3];
+        const int mine = v0 + v1 + v2 + v3;
+        int inc = mine;
+#pragma unroll
+        for (int o = 1; o < 64; o <<= 1) { const int n = __shfl_up(inc, o, 64); if (d >= o) inc += n; }
+        const int base = inc - mine;
+        tot[4 * d] = base; tot[4 * d + 1] = base + v0; tot[4 * d + 2] = base + v0 + v1; tot[4 * d + 3] = base + v0 + v1 + v2;
+    }
+    __syncthreads();
+    const int base = tot[d];
+    for (int s = 0; s < a.nseg; ++s) h[s * 256 + d] += base;
+}
+
+// stable scatter of one segment: grid (nseg, rows), 256 threads.  Element order inside the segment is
+// (wavefront, round, lane); equal digits keep that order: rank inside a round from ballots, rounds and wavefronts
+// through a prefix over their digit counts.
+static __global__ __launch_bounds__(256) void topp_scatter_kernel(TopPArgs a) {
+    __shared__ int wh[16][256];
+    const int seg = blockIdx.x, r = blockIdx.y, t = threadIdx.x, lane = t & 63, w = t >> 6;
+    const unsigned* kin = a.keysA + (long)r * a.Vs; const int* iin = a.idxA + (long)r * a.Vs;
+    unsigned* kout = a.keysB + (long)r * a.Vs; int* iout = a.idxB + (long)r * a.Vs;
+    for (int i = t; i < 16 * 256; i += 256) (&wh[0][0])[i] = 0;
+    __syncthreads();
+    unsigned key[4]; int idx[4], rank[4]; bool valid[4];
+    const unsigned long long lt = (1ull << lane) - 1ull;
+#pragma unroll
+    for (int it = 0; it < 4; ++it) {
+        const int e = seg * TOPP_SEG + w * 256 + it * 64 + lane;
+        valid[it] = e < a.V;
+        key[it] = valid[it] ? kin[e] : 0u;
+        idx[it] = valid[it] ? iin[e] : 0;
+        const unsigned d = (key[it] >> a.shift) & 255u;
+        unsigned long long peers = __ballot(valid[it]);
+#pragma unroll
+        for (int b = 0; b < 8; ++b) {
+            const bool bit = (d >> b) & 1u;
+            const unsigned long long bal = __ballot(bit);
+            peers &= bit ? bal : ~bal;
+        }
+        rank[it] = __popcll(peers & lt);
+        if (valid[it] && rank[it] == 0) wh[w * 4 + it][d] = __popcll(peers);
+    }
+    __syncthreads();
+    {
+        int run = a.hist[((long)r * a.nseg + seg) * 256 + t];
+#pragma unroll
+        for (int s = 0; s < 16; ++s) { const int v = wh[s][t]; wh[s][t] = run; run += v; }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int it = 0; it < 4; ++it) {
+        if (!valid[it]) continue;
+        const unsigned d = (key[it] >> a.shift) & 255u;
+        const int dst = wh[w * 4 + it][d] + rank[it];
+        kout[dst] = key[it]; iout[dst] = idx[it];
+    }
+}
+
+// running sum and pick: grid (rows), one wavefront.  The sorted keys are in keysA / idxA.
+// Chunks of 64 probabilities are added strictly in order (every lane holds the same running value); the value
+// after each chunk is kept, so that the pick only has to replay one chunk.
+static __global__ __launch_bounds__(64) void topp_pick_kernel(TopPArgs a) {
+    const int r = blockIdx.x, lane = threadIdx.x, V = a.V;
+    const unsigned* keys = a.keysA + (long)r * a.Vs;
+    const int* idx = a.idxA + (long)r * a.Vs;
+    float* cp = a.accp + (long)r * a.Vs;              // cp[c]: running sum after chunk c
+    float acc = 0.0f; int n = 0, nch = 0;
+    for (int base = 0; base < V; base += 64) {
+        const int i = base + lane;
+        const unsigned k = i < V ? keys[i] : 0xffffffffu;
+        const float p = k == 0xffffffffu ? 0.0f : __uint_as_float(~k);
+        const bool has_end = __any(k == 0xffffffffu);
+        float trial = acc;
+#pragma unroll
+        for (int j = 0; j < 64; ++j) trial += __int_as_float(__builtin_amdgcn_readlane(__float_as_int(p), j));
+        if (!has_end && trial < a.top_p) {
+            acc = trial; n += 64;
+            if (lane == 0) cp[nch] = acc;
+            ++nch;
+            continue;
+        }
+        // the chunk that ends the walk: element by element
+        for (int j = 0; j < 64; ++j) {
+            const float pj = __shfl(p, j, 64);
+            if (pj <= 0.0f) break;                     // ran out of candidates
+            acc += pj; n += 1;
+            if (acc >= a.top_p) break;
+        }
+        if (lane == 0) cp[nch] = acc;
+        ++nch;
+        break;
+    }
+    __threadfence_block();
     const long slot = (a.d_step ? (long)*a.d_step * gridDim.x : 0) + r;
-    const int n = s_n; const float acc = s_acc, u = a.uniforms[slot];
-    int best = 0x7fffffff;
-    for (int k = t; k < n; k += 256) if (accp[k] / acc >= u) { best = k; break; }
-    atomicMin(&s_pick, best);
-    __syncthreads();
-    if (t == 0) {
-        int id = s_pick == 0x7fffffff ? 0 : iA[s_pick];
+    const float u = a.uniforms[slot];
+    int pick = 0x7fffffff;
+    if (n > 0) {
+        // first chunk whose final value passes the test holds the pick (the running sum never decreases)
+        int cstar = 0x7fffffff;
+        for (int c0 = 0; c0 < nch && cstar == 0x7fffffff; c0 += 64) {
+            const int c = c0 + lane;
+            const bool hit = c < nch && cp[c] / acc >= u;
+            const unsigned long long m = __ballot(hit);
+            if (m) cstar = c0 + (int)__ffsll((long long)m) - 1;
+        }
+        if (cstar != 0x7fffffff) {
+            float run = cstar > 0 ? cp[cstar - 1] : 0.0f;
+            const int i = cstar * 64 + lane;
+            const unsigned k = i < V ? keys[i] : 0xffffffffu;
+            const float p = k == 0xffffffffu ? 0.0f : __uint_as_float(~k);
+            for (int j = 0; j < 64 && cstar * 64 + j < n; ++j) {
+                run += __shfl(p, j, 64);
+                if (run / acc >= u) { pick = cstar * 64 + j; break; }
+            }
+        }
+    }
+    if (lane == 0) {
+        const int id = pick == 0x7fffffff ? 0 : idx[pick];
         if (a.next_ids) a.next_ids[r] = id;
         if (a.gen_out) a.gen_out[slot] = id;
         if (a.out_f32) a.out_f32[r] = (float)id;
     }
+}
+
+// the whole pipeline; `launch_fn(name, kernel, grid, block, args)` puts one kernel on the library stream
+template <typename LaunchFn>
+inline void topp_run(TopPArgs a, int rows, LaunchFn&& launch_fn) {
+    launch_fn("topp_keys", topp_keys_kernel, dim3((unsigned)rows), dim3(1024), a);
+    for (int pass = 0; pass < 4; ++pass) {
+        a.shift = pass * 8;
+        launch_fn("topp_hist", topp_hist_kernel, dim3((unsigned)a.nseg, (unsigned)rows), dim3(256), a);
+        launch_fn("topp_scan", topp_scan_kernel, dim3((unsigned)rows), dim3(256), a);
+        launch_fn("topp_scatter", topp_scatter_kernel, dim3((unsigned)a.nseg, (unsigned)rows), dim3(256), a);
+        unsigned* tk = a.keysA; a.keysA = a.keysB; a.keysB = tk;
+        int* ti = a.idxA; a.idxA = a.idxB; a.idxB = ti;
+    }
+    launch_fn("topp_pick", topp_pick_kernel, dim3((unsigned)rows), dim3(64), a);
 }
 
 }  // namespace tship
