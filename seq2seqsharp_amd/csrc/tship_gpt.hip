@@ -350,7 +350,7 @@ static void run_skinny(TSHipGpt* m, const char* name, const GemmW& w, const void
 #define TSHIP_SK(BTV, NWV)                                                                                                  \
     if (epi == EPI_PARTIAL) launch(m, name, skinny_gemm_f16_kernel<BTV, EPI_PARTIAL, NWV>, grid, dim3(NWV * 64), e);        \
     else if (epi == EPI_F32_BIAS) launch(m, name, skinny_gemm_f16_kernel<BTV, EPI_F32_BIAS, NWV>, grid, dim3(NWV * 64), e); \
-    else if (epi == EPI_RESID_TAIL) launch(m, name, skinny_gemm_f16_kernel<BTV, EPI_RESID_TAIL, NWV>, grid, dim3(NWV * 64), e); \
+    else if (epi == EPI_RESID_TAIL) launch(m, name, skinny_gemm_f16_kernel<BTV, EPI_RESID_TAIL, NWV, (BTV == 1 ? 16 : 8)>, grid, dim3(NWV * 64), e); \
     else launch(m, name, skinny_gemm_f16_kernel<BTV, EPI_ACT16, NWV>, grid, dim3(NWV * 64), e);
     if (BT == 1) { TSHIP_SK(1, 8) } else if (BT == 2) { TSHIP_SK(2, 8) } else { TSHIP_SK(4, 4) }
 #undef TSHIP_SK

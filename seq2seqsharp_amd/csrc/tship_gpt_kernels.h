@@ -106,10 +106,12 @@ struct SkinnyArgs {
 // 8 weight fragments and 8 activation fragments (16 KiB) in flight.  Accumulators are added pairwise through LDS
 // (a fixed tree, so the sum order never changes); the last two are transposed through LDS so that the epilogue
 // writes coalesced rows.  X is fragment packed (xpack_index).
-template <int BT, int EPI, int NW>
+template <int BT, int EPI, int NW, int U = 8>
 __global__ __launch_bounds__(NW * 64) void skinny_gemm_f16_kernel(SkinnyArgs a) {
-    constexpr int U = 8;
-    constexpr int RED = (NW / 2) * BT * 16 * 64, FIN = 2 * BT * 32 * 33;
+    // one batch tile and eight wavefronts: every wavefront stores its accumulator once and the epilogue adds the eight
+    // copies in wavefront order (one barrier); otherwise a pairwise tree followed by a transpose
+    constexpr bool ONE_ROUND = BT == 1 && NW == 8 && (EPI == EPI_ACT16 || EPI == EPI_RESID_TAIL);   // fp32 outputs keep the transpose: coalesced rows
+    constexpr int RED = (ONE_ROUND ? NW : NW / 2) * BT * 16 * 64, FIN = 2 * BT * 32 * 33;
     __shared__ float smem[RED > FIN ? RED : FIN];      // the tree buffers are dead when the transpose buffer is written
     float (*red)[BT][16][64] = (float (*)[BT][16][64])smem;
     float (*fin)[BT * 32][33] = (float (*)[BT * 32][33])smem;
@@ -143,6 +145,22 @@ __global__ __launch_bounds__(NW * 64) void skinny_gemm_f16_kernel(SkinnyArgs a) 
         const int b = threadIdx.x % (BT * 32), ch = threadIdx.x / (BT * 32);
         const int per_ch = (a.ssq_nt + NCH - 1) / NCH;
         for (int t = ch * per_ch; t < min(a.ssq_nt, (ch + 1) * per_ch); ++t) ssq_part += a.ssq[(long)t * a.ssq_ld + b];
+    }
+    // residual tail: the old residual, bias and gamma of this thread's outputs do not depend on the product
+    constexpr int ITER = BT * 1024 / (NW * 64);
+    float tail_x[ITER], tail_b[ITER], tail_g[ITER];
+    if (EPI == EPI_RESID_TAIL) {
+#pragma unroll
+        for (int it = 0; it < ITER; ++it) {
+            const int idx = threadIdx.x + it * NW * 64;
+            // (one-round epilogue: outputs (lane % 32, n1) and (lane % 32, n1 + 16); otherwise row-major over the tile)
+            const int col = nt * 32 + (ONE_ROUND ? 8 * (w >> 2) + 4 * (lane >> 5) + (w & 3) + 16 * it : (idx & 31));
+            const int b = ONE_ROUND ? (lane & 31) : (idx >> 5);
+            const bool ok = b < a.rows_valid && col < a.n_valid;
+            tail_x[it] = ok ? a.x[(long)b * a.ldx_res + col] : 0.0f;
+            tail_b[it] = ok ? a.bias[col] : 0.0f;
+            tail_g[it] = ok ? a.gamma[col] : 0.0f;
+        }
     }
     const half_t* wp = a.W + ((long)nt * a.KT * 64 + lane) * 8;
     const half_t* xp = a.X + lane * 8;
@@ -178,6 +196,71 @@ __global__ __launch_bounds__(NW * 64) void skinny_gemm_f16_kernel(SkinnyArgs a) 
         }
     }
     if (a.advance_pos && blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) { a.advance_pos[0] += 1; a.advance_pos[1] += 1; }
+    if constexpr (ONE_ROUND) {
+#pragma unroll
+        for (int v = 0; v < 16; ++v) red[w][0][v][lane] = acc[0][v];
+        __syncthreads();
+        // thread (wavefront w, lane): registers v = w and w + 8 of all eight copies -> batch row lane % 32, columns
+        // n1 = 8 (w / 4) + 4 (lane / 32) + w % 4 and n1 + 16 (the gate's two factors when the tile is interleaved)
+        float s1 = red[0][0][w][lane], s2 = red[0][0][w + 8][lane];
+#pragma unroll
+        for (int i = 1; i < NW; ++i) { s1 += red[i][0][w][lane]; s2 += red[i][0][w + 8][lane]; }
+        const int b = lane & 31, n1 = 8 * (w >> 2) + 4 * (lane >> 5) + (w & 3);
+        const bool rok = b < a.rows_valid;
+        const float rinv = a.ssq ? srinv[b] : 1.0f;
+        if (EPI == EPI_PARTIAL) {
+            if (rok) {
+                float* o = a.out + ks * a.split_stride + (long)b * a.ld_out + nt * 32 + n1;
+                o[0] = s1; o[16] = s2;
+            }
+        } else if (EPI == EPI_F32_BIAS) {
+            const int c1 = nt * 32 + n1, c2 = c1 + 16;
+            if (rok && c1 < a.n_valid) a.out[(long)b * a.ld_out + c1] = s1 * rinv + a.bias[c1];
+            if (rok && c2 < a.n_valid) a.out[(long)b * a.ld_out + c2] = s2 * rinv + a.bias[c2];
+        } else if (EPI == EPI_ACT16) {
+            if (a.gated) {
+                const int f = nt * 16 + n1;
+                if (rok && f < a.n_valid) {
+                    const float val = act_apply(a.act, s1 * rinv + a.bias[f]) * (s2 * rinv + a.bias2[f]);
+                    if (a.out16_kt > 0) a.out16[xpack_index(b, f, a.out16_kt)] = (half_t)val;
+                    else a.out16[(long)b * a.ld16 + f] = (half_t)val;
+                }
+            } else {
+#pragma unroll
+                for (int q = 0; q < 2; ++q) {
+                    const int f = nt * 32 + n1 + 16 * q;
+                    if (rok && f < a.n_valid) {
+                        const float val = act_apply(a.act, (q ? s2 : s1) * rinv + a.bias[f]);
+                        if (a.out16_kt > 0) a.out16[xpack_index(b, f, a.out16_kt)] = (half_t)val;
+                        else a.out16[(long)b * a.ld16 + f] = (half_t)val;
+                    }
+                }
+            }
+        } else {      // EPI_RESID_TAIL
+            __shared__ float sq[NW][32];
+            float q = 0.0f;
+#pragma unroll
+            for (int h2 = 0; h2 < 2; ++h2) {
+                const int col = nt * 32 + n1 + 16 * h2;
+                if (rok && col < a.n_valid) {
+                    const float v = ((h2 ? s2 : s1) + tail_b[h2]) + tail_x[h2];
+                    a.x[(long)b * a.ldx_res + col] = v;
+                    a.xg16[xpack_index(b, col, a.xg_kt)] = (half_t)(tail_g[h2] * v);
+                    q += v * v;
+                }
+            }
+            q += __shfl_xor(q, 32, 64);           // the two lane halves hold different columns of the same row
+            if (lane < 32) sq[w][lane] = q;
+            __syncthreads();
+            if (threadIdx.x < 32 && threadIdx.x < a.rows_valid) {
+                float tot = sq[0][threadIdx.x];
+#pragma unroll
+                for (int i = 1; i < NW; ++i) tot += sq[i][threadIdx.x];
+                a.ssq_out[(long)nt * a.ssq_out_ld + threadIdx.x] = tot;
+            }
+        }
+        return;
+    }
     // pairwise tree over wavefronts down to two: in each round the upper half stores, the lower half adds
 #pragma unroll
     for (int half = NW / 2; half >= 2; half >>= 1) {
@@ -204,7 +287,6 @@ __global__ __launch_bounds__(NW * 64) void skinny_gemm_f16_kernel(SkinnyArgs a) 
             for (int v = 0; v < 16; ++v) fin[w][bt * 32 + (lane & 31)][8 * (v / 4) + 4 * (lane >> 5) + (v % 4)] = acc[bt][v];
     }
     __syncthreads();
-    constexpr int ITER = BT * 1024 / (NW * 64);
     float keep[ITER];
 #pragma unroll
     for (int it = 0; it < ITER; ++it) {
@@ -247,9 +329,9 @@ __global__ __launch_bounds__(NW * 64) void skinny_gemm_f16_kernel(SkinnyArgs a) 
         float v = keep[it];
         float q = 0.0f;
         if (col < a.n_valid) {
-            v = (v + a.bias[col]) + a.x[(long)b * a.ldx_res + col];
+            v = (v + tail_b[it]) + tail_x[it];
             a.x[(long)b * a.ldx_res + col] = v;
-            a.xg16[xpack_index(b, col, a.xg_kt)] = (half_t)(a.gamma[col] * v);
+            a.xg16[xpack_index(b, col, a.xg_kt)] = (half_t)(tail_g[it] * v);
             q = v * v;
         }
 #pragma unroll
