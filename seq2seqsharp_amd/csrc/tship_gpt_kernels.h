@@ -418,8 +418,16 @@ __global__ __launch_bounds__(256) void big_gemm2_f16_kernel(BigArgs a) {
     half_t* sX = big_smem + 2 * FR * 512;            // [2][FR * 512]
     const int t = threadIdx.x, lane = t & 63, w = __builtin_amdgcn_readfirstlane(t >> 6);
     const int wr = w >> 1, wn = w & 1;
-    const int nt0 = blockIdx.x * 8;
-    const long row0 = (long)blockIdx.y * 256;
+    // Block -> tile: workgroups go to the 8 XCDs round robin (id % 8) and each XCD has its own L2, so the 32 blocks an
+    // XCD runs at a time are laid out as one patch of 8 row tiles x 4 column tiles (12 distinct operand tiles for 32
+    // blocks); consecutive patches go to different XCDs.
+    const int CT = (a.NT + 7) / 8, RT = (int)((a.R + 255) / 256), PC = (CT + 3) / 4;
+    const int xcd = blockIdx.x & 7, seq = blockIdx.x >> 3;
+    const int patch = (seq >> 5) * 8 + xcd, q = seq & 31;
+    const int ctile = (patch % PC) * 4 + (q & 3), rtile = (patch / PC) * 8 + (q >> 2);
+    if (ctile >= CT || rtile >= RT) return;
+    const int nt0 = ctile * 8;
+    const long row0 = (long)rtile * 256;
     floatx16 acc[4][4];
 #pragma unroll
     for (int j = 0; j < 4; ++j)

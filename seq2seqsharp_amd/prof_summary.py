@@ -55,15 +55,36 @@ def main():
         print("\nlast %d dispatches: busy %.1f %% of the span, mean gap between consecutive kernels %.2f us (median %.2f us)"
               % (len(sub), 100.0 * busy / span, sum(gaps) / len(gaps) / 1e3, statistics.median(gaps) / 1e3))
     try:
-        pmc = list(cur.execute("select name, counter_name, count(*), avg(counter_value), sum(counter_value) from pmc_events "
-                               "group by name, counter_name order by name, counter_name"))
+        # a counter has one row per hardware instance (XCD, shader engine ...) and dispatch: add the instances of a
+        # dispatch, then average over the dispatches of a kernel
+        pmc = list(cur.execute(
+            "select name, counter_name, count(*), avg(v), avg(d) from (select name, counter_name, dispatch_id, sum(counter_value) as v, "
+            "max(duration) as d from pmc_events group by name, counter_name, dispatch_id) group by name, counter_name order by name, counter_name"))
     except Exception:
         pmc = []
     if pmc:
-        print("\ncounters (per dispatch averages)")
-        print("%-78s %-18s %8s %16s" % ("kernel", "counter", "calls", "avg"))
-        for n, cn, c, a, s in pmc:
-            print("%-78s %-18s %8d %16.1f" % (re.sub(r"tship::", "", n)[:78], cn, c, a))
+        print("\ncounters (sum over hardware instances, average per dispatch)")
+        print("%-78s %-30s %8s %16s" % ("kernel", "counter", "calls", "per_dispatch"))
+        per = {}
+        top = set(r[0] for r in rows[:12])           # the twelve kernels with the largest total time
+        for n, cn, c, a, d in pmc:
+            if n in top:
+                print("%-78s %-30s %8d %16.1f" % (re.sub(r"tship::", "", n)[:78], cn, c, a))
+            per.setdefault(n, {})[cn] = (a, d)
+        # MFMA utilisation: busy cycles of the matrix pipes over (4 SIMDs x CUs x kernel cycles); SQ_BUSY_CYCLES counts
+        # the kernel's cycles once per shader engine (32 on MI355X), MFMA busy cycles once per SIMD
+        mrows = [(n, v) for n, v in per.items() if "SQ_VALU_MFMA_BUSY_CYCLES" in v and "SQ_BUSY_CYCLES" in v and v["SQ_BUSY_CYCLES"][0] > 0]
+        if mrows:
+            print("\nMFMA utilisation = SQ_VALU_MFMA_BUSY_CYCLES / (SQ_BUSY_CYCLES / 32 shader engines x 256 CUs x 4 SIMDs)")
+            for n, v in mrows:
+                cyc = v["SQ_BUSY_CYCLES"][0] / 32.0
+                util = v["SQ_VALU_MFMA_BUSY_CYCLES"][0] / (cyc * 256 * 4)
+                extra = ""
+                if "SQ_INSTS_VALU_MFMA_MOPS_F16" in v and v["SQ_BUSY_CYCLES"][1]:
+                    tflops = v["SQ_INSTS_VALU_MFMA_MOPS_F16"][0] * 512.0 / (v["SQ_BUSY_CYCLES"][1] * 1e-9) / 1e12
+                    extra = "  %.0f TFLOP/s issued" % tflops
+                if util > 0.001:
+                    print("%-78s %6.1f %%%s" % (re.sub(r"tship::", "", n)[:78], 100.0 * util, extra))
 
 
 if __name__ == "__main__":
