@@ -403,103 +403,9 @@ __global__ __launch_bounds__(256) void big_gemm_f16_kernel(BigArgs a) {
     }
 }
 
-// LDS-tiled prefill GEMM.  Block tile 256 rows x 256 columns, 4 wavefronts, each owning 128 x 128 (4 x 4 MFMA
-// tiles of 32 x 32, 256 accumulator registers).  K advances in chunks of CK k-tiles (16 CK columns): per chunk the
-// block stages 8 CK weight fragments (already fragment-ordered in memory: straight 1 KiB copies) and 8 CK activation
-// fragments (row-major in memory, scattered into fragment order) in LDS, double buffered: the next chunk's global
-// loads are in flight in registers while the MFMAs of the current chunk run, one barrier per chunk.
-// Per k-tile a wavefront reads 8 fragments from LDS for 16 MFMAs.  Dynamic LDS: 2 x 16 KiB x CK.
-template <int EPI, int CK>
-__global__ __launch_bounds__(256) void big_gemm2_f16_kernel(BigArgs a) {
-    extern __shared__ __attribute__((aligned(16))) half_t big_smem[];
-    constexpr int FR = 8 * CK;                       // fragments of one operand per chunk
-    constexpr int LPT = FR / 4;                      // 16-byte loads per thread per operand and chunk
-    half_t* sW = big_smem;                           // [2][FR * 512]
-    half_t* sX = big_smem + 2 * FR * 512;            // [2][FR * 512]
-    const int t = threadIdx.x, lane = t & 63, w = __builtin_amdgcn_readfirstlane(t >> 6);
-    const int wr = w >> 1, wn = w & 1;
-    // Block -> tile: workgroups go to the 8 XCDs round robin (id % 8) and each XCD has its own L2, so the 32 blocks an
-    // XCD runs at a time are laid out as one patch of 8 row tiles x 4 column tiles (12 distinct operand tiles for 32
-    // blocks); consecutive patches go to different XCDs.
-    const int CT = (a.NT + 7) / 8, RT = (int)((a.R + 255) / 256), PC = (CT + 3) / 4;
-    const int xcd = blockIdx.x & 7, seq = blockIdx.x >> 3;
-    const int patch = (seq >> 5) * 8 + xcd, q = seq & 31;
-    const int ctile = (patch % PC) * 4 + (q & 3), rtile = (patch / PC) * 8 + (q >> 2);
-    if (ctile >= CT || rtile >= RT) return;
-    const int nt0 = ctile * 8;
-    const long row0 = (long)rtile * 256;
-    floatx16 acc[4][4];
-#pragma unroll
-    for (int j = 0; j < 4; ++j)
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-#pragma unroll
-            for (int v = 0; v < 16; ++v) acc[j][i][v] = 0.0f;
-
-    const half8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
-    const int NC = (a.KT + CK - 1) / CK;
-    half8 gw[LPT], gx[LPT];
-    // fragment f of the chunk = (n-tile or row tile f / CK, k-tile f % CK); thread t fills lane t % 64 of fragments
-    // t / 64 + 4 i of both operands, so every LDS store of a wavefront is one contiguous KiB (no bank conflicts); the
-    // activation rows are read 16 bytes per lane (the neighbouring pieces of a row follow in the next k-tiles)
-    auto gload = [&](int c) {
-#pragma unroll
-        for (int i = 0; i < LPT; ++i) {
-            const int f = i * 4 + (t >> 6);
-            const int nt = nt0 + f / CK, kt = c * CK + f % CK;
-            gw[i] = (nt < a.NT && kt < a.KT) ? *(const half8*)(a.W + (((long)nt * a.KT + kt) * 64 + lane) * 8) : zero8;
-            const int row = (f / CK) * 32 + (lane & 31), ktx = c * CK + f % CK;
-            gx[i] = (row0 + row < a.R && ktx < a.KT) ? *(const half8*)(a.X + (row0 + row) * (long)a.ldx + ktx * 16 + 8 * (lane >> 5)) : zero8;
-        }
-    };
-    auto lstore = [&](int buf) {
-#pragma unroll
-        for (int i = 0; i < LPT; ++i) {
-            const int f = i * 4 + (t >> 6);
-            *(half8*)(sW + ((long)buf * FR + f) * 512 + lane * 8) = gw[i];
-            *(half8*)(sX + ((long)buf * FR + f) * 512 + lane * 8) = gx[i];
-        }
-    };
-    gload(0);
-    lstore(0);
-    __syncthreads();
-    for (int c = 0; c < NC; ++c) {
-        const int buf = c & 1;
-        if (c + 1 < NC) gload(c + 1);
-        const half_t* bw = sW + (long)buf * FR * 512 + lane * 8;
-        const half_t* bx = sX + (long)buf * FR * 512 + lane * 8;
-        // fragments of k-tile kt + 1 are read from LDS while the 16 MFMAs of k-tile kt run
-        half8 wfA[4], xfA[4], wfB[4], xfB[4];
-        auto lread = [&](int kt, half8 (&wf)[4], half8 (&xf)[4]) {
-#pragma unroll
-            for (int j = 0; j < 4; ++j) wf[j] = *(const half8*)(bw + ((4 * wn + j) * CK + kt) * 512);
-#pragma unroll
-            for (int i = 0; i < 4; ++i) xf[i] = *(const half8*)(bx + ((4 * wr + i) * CK + kt) * 512);
-        };
-        auto mma = [&](half8 (&wf)[4], half8 (&xf)[4]) {
-#pragma unroll
-            for (int j = 0; j < 4; ++j)
-#pragma unroll
-                for (int i = 0; i < 4; ++i) acc[j][i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf[j], xf[i], acc[j][i], 0, 0, 0);
-        };
-        // (the scheduling barriers keep the compiler from sinking the reads back to their first use)
-        lread(0, wfA, xfA);
-#pragma unroll
-        for (int kt = 0; kt < CK; kt += 2) {
-            if (kt + 1 < CK) lread(kt + 1, wfB, xfB);
-            __builtin_amdgcn_sched_barrier(0);
-            mma(wfA, xfA);
-            __builtin_amdgcn_sched_barrier(0);
-            if (kt + 1 < CK) {
-                if (kt + 2 < CK) lread(kt + 2, wfA, xfA);
-                __builtin_amdgcn_sched_barrier(0);
-                mma(wfB, xfB);
-                __builtin_amdgcn_sched_barrier(0);
-            }
-        }
-        if (c + 1 < NC) lstore(buf ^ 1);
-        __syncthreads();
-    }
+// Epilogue shared by the LDS-tiled prefill GEMMs.
+template <int EPI>
+__device__ __forceinline__ void big_gemm_store(const BigArgs& a, floatx16 (&acc)[4][4], int nt0, long row0, int wr, int wn, int lane) {
     // accumulator (j, i), lane l, register v = 4 g + e: column (nt0 + 4 wn + j) * 32 + 8 g + 4 (l / 32) + e,
     // row row0 + 128 wr + 32 i + l % 32.  Biases (and the residual) are fetched in batches before the first store
     // of a column tile, and the four consecutive columns of a group go out as one 16-byte (fp32) or 8-byte (fp16) store.
@@ -600,6 +506,211 @@ __global__ __launch_bounds__(256) void big_gemm2_f16_kernel(BigArgs a) {
     tile_out(std::integral_constant<int, 1>{});
     tile_out(std::integral_constant<int, 2>{});
     tile_out(std::integral_constant<int, 3>{});
+}
+
+// LDS-tiled prefill GEMM.  Block tile 256 rows x 256 columns, 4 wavefronts, each owning 128 x 128 (4 x 4 MFMA
+// tiles of 32 x 32, 256 accumulator registers).  K advances in chunks of CK k-tiles (16 CK columns): per chunk the
+// block stages 8 CK weight fragments (already fragment-ordered in memory: straight 1 KiB copies) and 8 CK activation
+// fragments (row-major in memory, scattered into fragment order) in LDS, double buffered: the next chunk's global
+// loads are in flight in registers while the MFMAs of the current chunk run, one barrier per chunk.
+// Per k-tile a wavefront reads 8 fragments from LDS for 16 MFMAs.  Dynamic LDS: 2 x 16 KiB x CK.
+template <int EPI, int CK>
+__global__ __launch_bounds__(256) void big_gemm2_f16_kernel(BigArgs a) {
+    extern __shared__ __attribute__((aligned(16))) half_t big_smem[];
+    constexpr int FR = 8 * CK;                       // fragments of one operand per chunk
+    constexpr int LPT = FR / 4;                      // 16-byte loads per thread per operand and chunk
+    half_t* sW = big_smem;                           // [2][FR * 512]
+    half_t* sX = big_smem + 2 * FR * 512;            // [2][FR * 512]
+    const int t = threadIdx.x, lane = t & 63, w = __builtin_amdgcn_readfirstlane(t >> 6);
+    const int wr = w >> 1, wn = w & 1;
+    // Block -> tile: workgroups go to the 8 XCDs round robin (id % 8) and each XCD has its own L2, so the 32 blocks an
+    // XCD runs at a time are laid out as one patch of 8 row tiles x 4 column tiles (12 distinct operand tiles for 32
+    // blocks); consecutive patches go to different XCDs.
+    const int CT = (a.NT + 7) / 8, RT = (int)((a.R + 255) / 256), PC = (CT + 3) / 4;
+    const int xcd = blockIdx.x & 7, seq = blockIdx.x >> 3;
+    const int patch = (seq >> 5) * 8 + xcd, q = seq & 31;
+    const int ctile = (patch % PC) * 4 + (q & 3), rtile = (patch / PC) * 8 + (q >> 2);
+    if (ctile >= CT || rtile >= RT) return;
+    const int nt0 = ctile * 8;
+    const long row0 = (long)rtile * 256;
+    floatx16 acc[4][4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[j][i][v] = 0.0f;
+
+    const half8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+    const int NC = (a.KT + CK - 1) / CK;
+    half8 gw[LPT], gx[LPT];
+    // fragment f of the chunk = (n-tile or row tile f / CK, k-tile f % CK); thread t fills lane t % 64 of fragments
+    // t / 64 + 4 i of both operands, so every LDS store of a wavefront is one contiguous KiB (no bank conflicts); the
+    // activation rows are read 16 bytes per lane (the neighbouring pieces of a row follow in the next k-tiles)
+    auto gload = [&](int c) {
+#pragma unroll
+        for (int i = 0; i < LPT; ++i) {
+            const int f = i * 4 + (t >> 6);
+            const int nt = nt0 + f / CK, kt = c * CK + f % CK;
+            gw[i] = (nt < a.NT && kt < a.KT) ? *(const half8*)(a.W + (((long)nt * a.KT + kt) * 64 + lane) * 8) : zero8;
+            const int row = (f / CK) * 32 + (lane & 31), ktx = c * CK + f % CK;
+            gx[i] = (row0 + row < a.R && ktx < a.KT) ? *(const half8*)(a.X + (row0 + row) * (long)a.ldx + ktx * 16 + 8 * (lane >> 5)) : zero8;
+        }
+    };
+    auto lstore = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < LPT; ++i) {
+            const int f = i * 4 + (t >> 6);
+            *(half8*)(sW + ((long)buf * FR + f) * 512 + lane * 8) = gw[i];
+            *(half8*)(sX + ((long)buf * FR + f) * 512 + lane * 8) = gx[i];
+        }
+    };
+    gload(0);
+    lstore(0);
+    __syncthreads();
+    for (int c = 0; c < NC; ++c) {
+        const int buf = c & 1;
+        if (c + 1 < NC) gload(c + 1);
+        const half_t* bw = sW + (long)buf * FR * 512 + lane * 8;
+        const half_t* bx = sX + (long)buf * FR * 512 + lane * 8;
+        // fragments of k-tile kt + 1 are read from LDS while the 16 MFMAs of k-tile kt run
+        half8 wfA[4], xfA[4], wfB[4], xfB[4];
+        auto lread = [&](int kt, half8 (&wf)[4], half8 (&xf)[4]) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) wf[j] = *(const half8*)(bw + ((4 * wn + j) * CK + kt) * 512);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) xf[i] = *(const half8*)(bx + ((4 * wr + i) * CK + kt) * 512);
+        };
+        auto mma = [&](half8 (&wf)[4], half8 (&xf)[4]) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) acc[j][i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf[j], xf[i], acc[j][i], 0, 0, 0);
+        };
+        // (the scheduling barriers keep the compiler from sinking the reads back to their first use)
+        lread(0, wfA, xfA);
+#pragma unroll
+        for (int kt = 0; kt < CK; kt += 2) {
+            if (kt + 1 < CK) lread(kt + 1, wfB, xfB);
+            __builtin_amdgcn_sched_barrier(0);
+            mma(wfA, xfA);
+            __builtin_amdgcn_sched_barrier(0);
+            if (kt + 1 < CK) {
+                if (kt + 2 < CK) lread(kt + 2, wfA, xfA);
+                __builtin_amdgcn_sched_barrier(0);
+                mma(wfB, xfB);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+        if (c + 1 < NC) lstore(buf ^ 1);
+        __syncthreads();
+    }
+    big_gemm_store<EPI>(a, acc, nt0, row0, wr, wn, lane);
+}
+
+// Same tiling with asynchronous staging: the operands go from global memory straight into LDS
+// (global_load_lds_dwordx4: 64 lanes x 16 bytes land lane-linear, which is exactly a fragment), four stages of two
+// k-tiles, so loads are issued three chunks ahead and need neither staging registers nor LDS stores.  The compiler
+// cannot tell which LDS bytes an in-flight load will write and would wait for all of them before any LDS read, so the
+// fragment reads and their waits are written out by hand.  Needs an even number of k-tiles; rows and column tiles
+// beyond the matrix are clamped to the last valid one on load and dropped on store.
+__device__ __forceinline__ void lds_read_frags(unsigned wa, unsigned xa, half8 (&wf)[4], half8 (&xf)[4]) {
+    asm volatile(
+        "ds_read_b128 %0, %8\n\t"
+        "ds_read_b128 %1, %8 offset:2048\n\t"
+        "ds_read_b128 %2, %8 offset:4096\n\t"
+        "ds_read_b128 %3, %8 offset:6144\n\t"
+        "ds_read_b128 %4, %9\n\t"
+        "ds_read_b128 %5, %9 offset:2048\n\t"
+        "ds_read_b128 %6, %9 offset:4096\n\t"
+        "ds_read_b128 %7, %9 offset:6144"
+        : "=&v"(wf[0]), "=&v"(wf[1]), "=&v"(wf[2]), "=&v"(wf[3]), "=&v"(xf[0]), "=&v"(xf[1]), "=&v"(xf[2]), "=&v"(xf[3])
+        : "v"(wa), "v"(xa)
+        : "memory");
+}
+template <int N>
+__device__ __forceinline__ void lds_wait_frags(half8 (&wf)[4], half8 (&xf)[4]) {
+    asm volatile("s_waitcnt lgkmcnt(%8)"
+                 : "+v"(wf[0]), "+v"(wf[1]), "+v"(wf[2]), "+v"(wf[3]), "+v"(xf[0]), "+v"(xf[1]), "+v"(xf[2]), "+v"(xf[3])
+                 : "n"(N)
+                 : "memory");
+}
+
+template <int EPI>
+__global__ __launch_bounds__(256) void big_gemm3_f16_kernel(BigArgs a) {
+    extern __shared__ __attribute__((aligned(16))) half_t big_smem[];
+    constexpr int CK = 2, NST = 4, FR = 8 * CK;          // k-tiles per stage, stages, fragments per operand and stage
+    constexpr int STAGE = 2 * FR * 512;                  // halfs per stage: weight fragments, then activation fragments
+    const int t = threadIdx.x, lane = t & 63, w = __builtin_amdgcn_readfirstlane(t >> 6);
+    const int wr = w >> 1, wn = w & 1;
+    const int CT = (a.NT + 7) / 8, RT = (int)((a.R + 255) / 256), PC = (CT + 3) / 4;
+    const int xcd = blockIdx.x & 7, seq = blockIdx.x >> 3;
+    const int patch = (seq >> 5) * 8 + xcd, q = seq & 31;
+    const int ctile = (patch % PC) * 4 + (q & 3), rtile = (patch / PC) * 8 + (q >> 2);
+    if (ctile >= CT || rtile >= RT) return;
+    const int nt0 = ctile * 8;
+    const long row0 = (long)rtile * 256;
+    floatx16 acc[4][4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[j][i][v] = 0.0f;
+
+    // wavefront w stages fragments f = 4 i + w (f / 2: n-tile or row tile, f % 2: k-tile) of both operands
+    const half_t* wsrc[4]; const half_t* xsrc[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int f = i * 4 + w, tl = f >> 1, ktl = f & 1;
+        const int nt = min(nt0 + tl, a.NT - 1);
+        wsrc[i] = a.W + (((long)nt * a.KT + ktl) * 64 + lane) * 8;
+        const long row = min(row0 + tl * 32 + (lane & 31), (long)a.R - 1);
+        xsrc[i] = a.X + row * (long)a.ldx + ktl * 16 + 8 * (lane >> 5);
+    }
+    typedef const void __attribute__((address_space(1)))* gptr_t;
+    typedef void __attribute__((address_space(3)))* lptr_t;
+    auto issue = [&](int c) {
+        half_t* st = big_smem + (c & (NST - 1)) * STAGE;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int f = i * 4 + w;
+            __builtin_amdgcn_global_load_lds((gptr_t)(wsrc[i] + (long)c * (CK * 512)), (lptr_t)(st + f * 512), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds((gptr_t)(xsrc[i] + (long)c * (CK * 16)), (lptr_t)(st + (FR + f) * 512), 16, 0, 0);
+        }
+    };
+    const int NC = a.KT / CK;
+    const unsigned lds0 = (unsigned)(size_t)(lptr_t)big_smem;
+    const unsigned woff = (unsigned)(((4 * wn) * CK) * 1024 + lane * 16);
+    const unsigned xoff = (unsigned)((FR + (4 * wr) * CK) * 1024 + lane * 16);
+    issue(0);
+    if (NC > 1) issue(1);
+    if (NC > 2) issue(2);
+    for (int c = 0; c < NC; ++c) {
+        // chunk c has landed once at most the loads of the chunks issued after it (8 per chunk) are outstanding
+        const int later = min(2, NC - 1 - c);
+        if (later == 2) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+        else if (later == 1) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+        else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __builtin_amdgcn_s_barrier();          // every wavefront's part of chunk c is in LDS, and chunk c - 1 is consumed
+        if (c + 3 < NC) issue(c + 3);           // into the stage chunk c - 1 used
+        const unsigned sb = lds0 + (unsigned)((c & (NST - 1)) * STAGE * 2);
+        half8 wfA[4], xfA[4], wfB[4], xfB[4];
+        lds_read_frags(sb + woff, sb + xoff, wfA, xfA);                     // k-tile 0: fragment (tile, 0) at tile * 2 KiB
+        lds_read_frags(sb + woff + 1024, sb + xoff + 1024, wfB, xfB);       // k-tile 1
+        lds_wait_frags<8>(wfA, xfA);
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc[j][i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wfA[j], xfA[i], acc[j][i], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);      // keep the second wait behind the first k-tile's MFMAs
+        lds_wait_frags<0>(wfB, xfB);
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc[j][i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wfB[j], xfB[i], acc[j][i], 0, 0, 0);
+    }
+    big_gemm_store<EPI>(a, acc, nt0, row0, wr, wn, lane);
 }
 
 // ------------------------------------------------------------------------------------------------
