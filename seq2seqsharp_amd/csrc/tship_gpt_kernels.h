@@ -665,8 +665,12 @@ __global__ __launch_bounds__(256) void big_gemm3_f16_kernel(BigArgs a) {
         const int f = i * 4 + w, tl = f >> 1, ktl = f & 1;
         const int nt = min(nt0 + tl, a.NT - 1);
         wsrc[i] = a.W + (((long)nt * a.KT + ktl) * 64 + lane) * 8;
-        const long row = min(row0 + tl * 32 + (lane & 31), (long)a.R - 1);
-        xsrc[i] = a.X + row * (long)a.ldx + ktl * 16 + 8 * (lane >> 5);
+        // activations: 1 KiB block f holds 16 rows x 64 bytes (both k-tiles of the chunk); lane l fetches 16-byte piece
+        // s = (l % 4) ^ ((row / 4) % 4) of row 16 f + l / 4, so that four lanes read one contiguous 64-byte run and the
+        // fragment reads below (32 rows x 2 pieces) spread evenly over the LDS banks
+        const int rl = f * 16 + (lane >> 2);
+        const long row = min(row0 + rl, (long)a.R - 1);
+        xsrc[i] = a.X + row * (long)a.ldx + 8 * ((lane & 3) ^ ((rl >> 2) & 3));
     }
     typedef const void __attribute__((address_space(1)))* gptr_t;
     typedef void __attribute__((address_space(3)))* lptr_t;
@@ -682,7 +686,12 @@ __global__ __launch_bounds__(256) void big_gemm3_f16_kernel(BigArgs a) {
     const int NC = a.KT / CK;
     const unsigned lds0 = (unsigned)(size_t)(lptr_t)big_smem;
     const unsigned woff = (unsigned)(((4 * wn) * CK) * 1024 + lane * 16);
-    const unsigned xoff = (unsigned)((FR + (4 * wr) * CK) * 1024 + lane * 16);
+    // B fragment (row tile i, k-tile kt), lane l: row r = 32 (4 wr + i) + l % 32, piece s = 2 kt + l / 32 at byte
+    // 64 r + 16 (s ^ ((r / 4) % 4)) of the activation area
+    const int xr = 128 * wr + (lane & 31);
+    const unsigned xsw = (unsigned)((xr >> 2) & 3);
+    const unsigned xoff0 = (unsigned)(FR * 1024 + xr * 64 + 16 * (((lane >> 5)) ^ xsw));          // k-tile 0: s = l / 32
+    const unsigned xoff1 = (unsigned)(FR * 1024 + xr * 64 + 16 * ((2 + (lane >> 5)) ^ xsw));      // k-tile 1: s = 2 + l / 32
     issue(0);
     if (NC > 1) issue(1);
     if (NC > 2) issue(2);
@@ -696,8 +705,8 @@ __global__ __launch_bounds__(256) void big_gemm3_f16_kernel(BigArgs a) {
         if (c + 3 < NC) issue(c + 3);           // into the stage chunk c - 1 used
         const unsigned sb = lds0 + (unsigned)((c & (NST - 1)) * STAGE * 2);
         half8 wfA[4], xfA[4], wfB[4], xfB[4];
-        lds_read_frags(sb + woff, sb + xoff, wfA, xfA);                     // k-tile 0: fragment (tile, 0) at tile * 2 KiB
-        lds_read_frags(sb + woff + 1024, sb + xoff + 1024, wfB, xfB);       // k-tile 1
+        lds_read_frags(sb + woff, sb + xoff0, wfA, xfA);                    // k-tile 0: weight fragment (tile, 0) at tile * 2 KiB
+        lds_read_frags(sb + woff + 1024, sb + xoff1, wfB, xfB);             // k-tile 1
         lds_wait_frags<8>(wfA, xfA);
 #pragma unroll
         for (int j = 0; j < 4; ++j)
