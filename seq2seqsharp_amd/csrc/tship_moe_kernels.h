@@ -34,23 +34,39 @@ __device__ __forceinline__ float tree8(float v) {
 // (a.router_lds != 0), so that the serial dot products read LDS only.
 __global__ __launch_bounds__(256) void moe_router_kernel(MoeRouterArgs a) {
 #pragma clang fp contract(off)
-    extern __shared__ float moe_smem[];
+    extern __shared__ __attribute__((aligned(16))) float moe_smem[];
     __shared__ float sr[64];
     __shared__ float s_stat[2];
     const int r = blockIdx.x, t = threadIdx.x, h = a.h, E = a.E;
     float* sx = moe_smem;
     float* sxn = moe_smem + h;
     float* srt = moe_smem + 2 * h;
-    if (a.router_lds) for (int i = t; i < h * E; i += 256) srt[i] = a.router[i];
-    for (int c = t; c < h; c += 256) {
-        float v = a.x[(long)r * a.ldx + c];
-        if (a.part) {
-            float s = a.part[(long)r * a.ld_part + c];
-            for (int k = 1; k < a.KS; ++k) s += a.part[k * a.split_stride + (long)r * a.ld_part + c];
-            v = (s + a.bias[c]) + v;
-            a.x[(long)r * a.ldx + c] = v;
+    for (int c0 = t; c0 < h; c0 += 256 * 4) {
+        float xv[4], pv[4][8], bv[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int c = c0 + u * 256;
+            const bool ok = c < h;
+            xv[u] = ok ? a.x[(long)r * a.ldx + c] : 0.0f;
+            bv[u] = (ok && a.part) ? a.bias[c] : 0.0f;
+#pragma unroll
+            for (int k = 0; k < 8; ++k) pv[u][k] = (ok && a.part && k < a.KS) ? a.part[k * a.split_stride + (long)r * a.ld_part + c] : 0.0f;
         }
-        sx[c] = v;
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int c = c0 + u * 256;
+            if (c >= h) continue;
+            float v = xv[u];
+            if (a.part) {
+                float s = pv[u][0];
+#pragma unroll
+                for (int k = 1; k < 8; ++k) if (k < a.KS) s += pv[u][k];
+                for (int k = 8; k < a.KS; ++k) s += a.part[k * a.split_stride + (long)r * a.ld_part + c];
+                v = (s + bv[u]) + v;
+                a.x[(long)r * a.ldx + c] = v;
+            }
+            sx[c] = v;
+        }
     }
     __syncthreads();
     // LayerNorm statistics in the reference's order (TensorApplyCPU.cs:1381-1409): eight interleaved partial sums
@@ -87,28 +103,63 @@ __global__ __launch_bounds__(256) void moe_router_kernel(MoeRouterArgs a) {
     }
     __syncthreads();
     const float mean = s_stat[0], sigma = s_stat[1];
-    for (int c = t; c < h; c += 256) {
-        float y = a.gamma[c] * ((sx[c] - mean) / sigma);
-        y += a.beta[c];
-        sxn[c] = y;
-        a.xn32[(long)r * h + c] = y;
+    for (int c0 = t; c0 < h; c0 += 256 * 4) {
+        float gv[4], bv[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) { const int c = c0 + u * 256; gv[u] = c < h ? a.gamma[c] : 0.0f; bv[u] = c < h ? a.beta[c] : 0.0f; }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int c = c0 + u * 256;
+            if (c >= h) continue;
+            float y = gv[u] * ((sx[c] - mean) / sigma);
+            y += bv[u];
+            sxn[c] = y;
+            a.xn32[(long)r * h + c] = y;
+        }
     }
     __syncthreads();
-    if (t < E) {
-        // serial over l, product and sum rounded separately, zero inputs skipped (SGEMM.cs:482-549)
-        float acc = a.router_b[t];
-        auto dot = [&](auto rt) {          // rt: LDS or global pointer (kept apart so that LDS reads stay ds_read)
-            int l = 0;
-            for (; l + 8 <= h; l += 8) {
-                float xv[8], wv[8];
+    // Router logits: sum over l of xn[l] * W[l][e], product and sum rounded separately, added strictly in order of l
+    // (SGEMM.cs:482-549; rows with xn[l] == 0 are skipped there, which equals adding a zero product).  The products
+    // are independent, so all threads form them (transposed into LDS: pt[e][l]); one thread per expert then adds its
+    // h products in order, reading them 16 bytes at a time.
+    if (a.router_lds) {
+        float* pt = srt;
+        const int n = h * E;
+        for (int i0 = t; i0 < n; i0 += 256 * 8) {
+            float wv[8];
 #pragma unroll
-                for (int u = 0; u < 8; ++u) { xv[u] = sxn[l + u]; wv[u] = rt[(long)(l + u) * E + t]; }
+            for (int u = 0; u < 8; ++u) { const int i = i0 + u * 256; wv[u] = i < n ? a.router[i] : 0.0f; }
 #pragma unroll
-                for (int u = 0; u < 8; ++u) { const float s = acc + xv[u] * wv[u]; acc = xv[u] != 0.0f ? s : acc; }
+            for (int u = 0; u < 8; ++u) {
+                const int i = i0 + u * 256;
+                if (i < n) { const int l = i / E, e = i - l * E; const float xv = sxn[l]; pt[e * h + l] = xv != 0.0f ? xv * wv[u] : 0.0f; }
             }
-            for (; l < h; ++l) { const float xv = sxn[l]; if (xv != 0.0f) acc += xv * rt[(long)l * E + t]; }
-        };
-        if (a.router_lds) dot((const float*)srt); else dot(a.router);
+        }
+        __syncthreads();
+    }
+    if (t < E) {
+        float acc = a.router_b[t];
+        if (a.router_lds) {
+            const float* p = srt + t * h;
+            int l = 0;
+            if ((h & 3) == 0) {
+                for (; l + 16 <= h; l += 16) {
+                    floatx4 q0 = *(const floatx4*)(p + l), q1 = *(const floatx4*)(p + l + 4), q2 = *(const floatx4*)(p + l + 8), q3 = *(const floatx4*)(p + l + 12);
+                    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) acc += q0[u];
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) acc += q1[u];
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) acc += q2[u];
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) acc += q3[u];
+                }
+            }
+            for (; l < h; ++l) acc += p[l];
+        } else {
+            for (int l = 0; l < h; ++l) { const float xv = sxn[l]; if (xv != 0.0f) acc += xv * a.router[(long)l * E + t]; }
+        }
         sr[t] = acc + (-65000.0f);
     }
     __syncthreads();
