@@ -197,6 +197,45 @@ def test_decode_equals_prefill_recompute(G, batch):
     b.close()
 
 
+def test_full_size_cfg2_properties(G):
+    """The benchmark configuration at its real size (16 layers, batch 32, prompt 1024), where the oracle would need
+    minutes: prefill(P) + two decode steps must reproduce prefill(P + 2); a KV cache read back and restored into a
+    second model agrees; generate() equals step-by-step greedy decoding on the same model, bit for bit."""
+    cfg = dict(synth.CONFIGS["cfg2_1b_gqa_f16"])
+    B, Tp = cfg["batch"], cfg["prompt"]
+    w = synth.make_weights(cfg, 0)
+    seqs = synth.make_prompts(cfg, 1, length=Tp + 2)
+    a = G.HipGpt(cfg, w, max_batch=B, max_seq_len=Tp + 16)
+    a.prefill(seqs[:, :Tp])
+    a.decode(seqs[:, Tp])
+    a.decode(seqs[:, Tp + 1])
+    la = a.logits()
+    b = G.HipGpt(cfg, w, max_batch=B, max_seq_len=Tp + 16)
+    b.prefill(seqs)
+    lb = b.logits()
+    assert np.abs(la - lb).max() <= FP16_ABS
+    assert (la.argmax(1) == lb.argmax(1)).mean() >= 0.99
+    # cache round trip through the host layout [batch, kv_head, len, head_dim]
+    for layer in (0, cfg["n_layers"] - 1):
+        for which in (0, 1):
+            kv = a.get_kv(layer, which)
+            assert kv.shape == (B, cfg["n_kv_heads"], Tp + 2, cfg["hidden"] // cfg["n_heads"])
+            assert np.abs(kv - b.get_kv(layer, which)).max() <= 2e-2
+    g1, _ = a.generate(4)
+    # rewind the same model to the end of the prompt and walk the same four steps one call at a time
+    a.set_seq_len(B, Tp + 1)
+    a.decode(seqs[:, Tp + 1])
+    assert np.array_equal(a.logits(), la)
+    steps = []
+    for _ in range(4):
+        nxt = a.sample()
+        steps.append(nxt)
+        a.decode(nxt)
+    assert np.array_equal(g1, np.stack(steps))
+    a.close()
+    b.close()
+
+
 @pytest.mark.parametrize("name", ["odd_sizes", "gqa_leaky_d32_g4", "mha_ln_relu"])
 def test_fp16_long_prompt_prefill_against_oracle(G, oracle, name):
     """More than 512 prompt rows: the prefill projections run on the LDS-tiled GEMM (ragged row, column and k tiles
