@@ -94,7 +94,7 @@ struct TSHipGpt {
 
     // decode state
     DevBuf x, xn, o, a, part_qkv, part_h, part_f, logits, ids, d_pos, hidden;
-    DevBuf moe_ws, topp_scratch, topp_uni, gen_buf, uni_buf;
+    DevBuf moe_ws, topp_scratch, topp_uni, gen_buf, uni_buf, tile_count;
     DevBuf ssq;                    // deferred-norm path: per-column-tile sums of squares [h/32][Bpad]
     bool fused_norm = false;       // fp16 + RMSNorm + dense layers: residual/norm folded into the GEMM tails
     bool vt = false;               // fp16 cache with head_dim 64/128: keys and values stored fragment-major for the MFMA attention kernels
@@ -344,13 +344,15 @@ static void run_resid_norm(TSHipGpt* m, const char* name, int rows, ResidNormArg
 static void run_skinny(TSHipGpt* m, const char* name, const GemmW& w, const void* X, long ldx, int rows, int epi, SkinnyArgs e) {
     TSHIP_REQUIRE(m->f16, "internal: run_skinny is the fp16 path");
     e.W = w.buf.as<half_t>(); e.KT = w.KT; e.NT = w.NT; e.X = (const half_t*)X; e.ldx = (int)ldx;
-    e.KS = (epi == EPI_PARTIAL) ? w.KS : 1; e.rows_valid = rows;
+    e.KS = (epi == EPI_PARTIAL || epi == EPI_SPLIT_TAIL) ? w.KS : 1; e.rows_valid = rows;
+    TSHIP_REQUIRE(epi != EPI_SPLIT_TAIL || (m->BT == 1 && e.tile_count), "internal: the split tail needs one batch tile and the tile counters");
     dim3 grid(w.NT * e.KS);
     const int BT = m->BT;
 #define TSHIP_SK(BTV, NWV)                                                                                                  \
     if (epi == EPI_PARTIAL) launch(m, name, skinny_gemm_f16_kernel<BTV, EPI_PARTIAL, NWV>, grid, dim3(NWV * 64), e);        \
     else if (epi == EPI_F32_BIAS) launch(m, name, skinny_gemm_f16_kernel<BTV, EPI_F32_BIAS, NWV>, grid, dim3(NWV * 64), e); \
     else if (epi == EPI_RESID_TAIL) launch(m, name, skinny_gemm_f16_kernel<BTV, EPI_RESID_TAIL, NWV, (BTV == 1 ? 16 : 8)>, grid, dim3(NWV * 64), e); \
+    else if (epi == EPI_SPLIT_TAIL) launch(m, name, skinny_gemm_f16_kernel<BTV, EPI_SPLIT_TAIL, NWV>, grid, dim3(NWV * 64), e); \
     else launch(m, name, skinny_gemm_f16_kernel<BTV, EPI_ACT16, NWV>, grid, dim3(NWV * 64), e);
     if (BT == 1) { TSHIP_SK(1, 8) } else if (BT == 2) { TSHIP_SK(2, 8) } else { TSHIP_SK(4, 4) }
 #undef TSHIP_SK
@@ -491,6 +493,14 @@ static void decode_step_fn(TSHipGpt* m, const int* d_ids, int B) {
             SkinnyArgs e; std::memset(&e, 0, sizeof(e));
             tail(e, L.b2.as<float>(), next_gamma);
             run_skinny(m, "gemm_ffn2", L.w2, m->a.p, m->ldF, B, EPI_RESID_TAIL, e);
+        } else if (m->BT == 1) {
+            // long K: split across blocks so that every CU streams weights; the block of a column tile that finishes
+            // last adds the partial sums and performs the tail
+            SkinnyArgs e; std::memset(&e, 0, sizeof(e));
+            tail(e, L.b2.as<float>(), next_gamma);
+            e.out = m->part_h.as<float>();       // exchange area [split][tile][1024]: 16 * Bpad * hp floats hold it for Bpad = 32
+            e.tile_count = m->tile_count.as<int>();
+            run_skinny(m, "gemm_ffn2", L.w2, m->a.p, m->ldF, B, EPI_SPLIT_TAIL, e);
         } else {
             // long K: split across blocks so that every CU streams weights, then a small tail kernel
             SkinnyArgs e; std::memset(&e, 0, sizeof(e));
@@ -656,7 +666,7 @@ static void prefill(TSHipGpt* m, const int32_t* host_ids, int B, int Tp) {
             // one-dimensional grid of 8-row x 4-column tile patches, 32 blocks each, rounded up to whole rounds of 8 patches
             const long CT = ceil_div(w.NT, 8), RT = ceil_div(R, 256), patches = ceil_div(CT, 4) * ceil_div(RT, 8);
             dim3 grid((unsigned)(round_up(patches, 8) * 32));
-            if (w.KT % 2 == 0 && std::getenv("TSHIP_GEMM2") == nullptr) {      // asynchronous staging: four stages of two k-tiles
+            if (w.KT % 2 == 0) {      // asynchronous staging: four stages of two k-tiles
                 if (epi == BEPI_F32_BIAS) launch_shm(m, name, big_gemm3_f16_kernel<BEPI_F32_BIAS>, grid, dim3(256), shm, e);
                 else if (epi == BEPI_RESID) launch_shm(m, name, big_gemm3_f16_kernel<BEPI_RESID>, grid, dim3(256), shm, e);
                 else launch_shm(m, name, big_gemm3_f16_kernel<BEPI_ACT16>, grid, dim3(256), shm, e);
@@ -843,6 +853,7 @@ TSHIP_API int TSHip_GptCreate(const TSHipGptConfig* cfg, TSHipGpt** out) {
     m->fused_norm = m->f16 && c.norm_type == 0 && c.n_experts <= 1;
     if (m->fused_norm) {
         m->ssq.alloc((size_t)(hp / 32) * m->Bpad * sizeof(float));
+        m->tile_count.alloc((size_t)(hp / 32) * sizeof(int));        // zero-filled; every use returns it to zero
     }
     TSHIP_CHECK_HIP(hipStreamSynchronize(stream()));
     *out = m.release();
@@ -890,6 +901,7 @@ TSHIP_API int TSHip_GptReset(TSHipGpt* m) {
     TSHIP_REQUIRE(m, "TSHip_GptReset: null model");
     m->pos = 0; m->cur_batch = 0;
     TSHIP_CHECK_HIP(hipMemsetAsync(m->d_pos.p, 0, sizeof(int), stream()));
+    if (m->tile_count.p) TSHIP_CHECK_HIP(hipMemsetAsync(m->tile_count.p, 0, m->tile_count.bytes, stream()));
     TSHIP_CHECK_HIP(hipStreamSynchronize(stream()));
     TSHIP_END
 }
