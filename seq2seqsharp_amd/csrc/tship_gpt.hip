@@ -479,7 +479,12 @@ static void decode_step_fn(TSHipGpt* m, const int* d_ids, int B) {
         {
             SkinnyArgs e; std::memset(&e, 0, sizeof(e));
             tail(e, L.bo.as<float>(), L.n2_g.as<float>());
-            run_skinny(m, "gemm_wo", L.wo, m->o.p, m->ldh, B, EPI_RESID_TAIL, e);
+            if (L.wo.KS > 1) {
+                e.out = m->part_h.as<float>(); e.tile_count = m->tile_count.as<int>();
+                run_skinny(m, "gemm_wo", L.wo, m->o.p, m->ldh, B, EPI_SPLIT_TAIL, e);
+            } else {
+                run_skinny(m, "gemm_wo", L.wo, m->o.p, m->ldh, B, EPI_RESID_TAIL, e);
+            }
         }
         {
             SkinnyArgs e; std::memset(&e, 0, sizeof(e));
@@ -888,8 +893,16 @@ TSHIP_API int TSHip_GptFinalize(TSHipGpt* m) {
         // deferred-norm path: the output projection runs unsplit with the residual tail in its epilogue; the FFN down
         // projection keeps its K split only when K is long enough to need more than two passes per wavefront
         for (auto& L : m->L) {
-            L->wo.KS = 1;
-            if (L->w2.KS <= 2) L->w2.KS = 1;
+            // residual-tail projections (N = hidden): split K so that the launch has about one block per compute unit
+            // (more blocks than that run in a second wave, which measured 2 us slower); BT > 1 keeps them unsplit
+            auto tail_ks = [&](const GemmW& w) {
+                if (m->BT != 1) return 1;
+                int ks = std::max(1, n_compute_units() / std::max(1, w.NT));
+                ks = std::min(ks, std::max(1, w.KT / 8));           // at least one k-tile per wavefront
+                return std::min(ks, 16);
+            };
+            L->wo.KS = tail_ks(L->wo);
+            L->w2.KS = m->BT == 1 ? tail_ks(L->w2) : (L->w2.KS <= 2 ? 1 : L->w2.KS);
         }
     }
     m->finalized = true;
