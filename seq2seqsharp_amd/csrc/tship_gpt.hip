@@ -344,15 +344,15 @@ static void run_resid_norm(TSHipGpt* m, const char* name, int rows, ResidNormArg
 static void run_skinny(TSHipGpt* m, const char* name, const GemmW& w, const void* X, long ldx, int rows, int epi, SkinnyArgs e) {
     TSHIP_REQUIRE(m->f16, "internal: run_skinny is the fp16 path");
     e.W = w.buf.as<half_t>(); e.KT = w.KT; e.NT = w.NT; e.X = (const half_t*)X; e.ldx = (int)ldx;
-    e.KS = (epi == EPI_PARTIAL || epi == EPI_SPLIT_TAIL || epi == EPI_SPLIT_ACT16) ? w.KS : 1; e.rows_valid = rows;
-    if (epi == EPI_SPLIT_TAIL || epi == EPI_SPLIT_ACT16) {
+    e.KS = (epi == EPI_PARTIAL || epi == EPI_SPLIT_TAIL) ? w.KS : 1; e.rows_valid = rows;
+    if (epi == EPI_SPLIT_TAIL) {
         // the exchange area holds [split][tile][1024] floats and one counter per tile
         TSHIP_REQUIRE(e.out == m->part_h.as<float>() && (size_t)e.KS * w.NT * 1024 * sizeof(float) <= m->part_h.bytes,
                       "internal: split-K exchange area too small");
         TSHIP_REQUIRE(e.tile_count == m->tile_count.as<int>() && (size_t)w.NT * sizeof(int) <= m->tile_count.bytes,
                       "internal: too few tile counters");
     }
-    TSHIP_REQUIRE((epi != EPI_SPLIT_TAIL && epi != EPI_SPLIT_ACT16) || (m->BT == 1 && e.tile_count), "internal: the split tail needs one batch tile and the tile counters");
+    TSHIP_REQUIRE(epi != EPI_SPLIT_TAIL || (m->BT == 1 && e.tile_count), "internal: the split tail needs one batch tile and the tile counters");
     dim3 grid(w.NT * e.KS);
     const int BT = m->BT;
 #define TSHIP_SK(BTV, NWV)                                                                                                  \
@@ -360,7 +360,6 @@ static void run_skinny(TSHipGpt* m, const char* name, const GemmW& w, const void
     else if (epi == EPI_F32_BIAS) launch(m, name, skinny_gemm_f16_kernel<BTV, EPI_F32_BIAS, NWV>, grid, dim3(NWV * 64), e); \
     else if (epi == EPI_RESID_TAIL) launch(m, name, skinny_gemm_f16_kernel<BTV, EPI_RESID_TAIL, NWV, (BTV == 1 ? 16 : 8)>, grid, dim3(NWV * 64), e); \
     else if (epi == EPI_SPLIT_TAIL) launch(m, name, skinny_gemm_f16_kernel<BTV, EPI_SPLIT_TAIL, NWV>, grid, dim3(NWV * 64), e); \
-    else if (epi == EPI_SPLIT_ACT16) launch(m, name, skinny_gemm_f16_kernel<BTV, EPI_SPLIT_ACT16, NWV>, grid, dim3(NWV * 64), e); \
     else launch(m, name, skinny_gemm_f16_kernel<BTV, EPI_ACT16, NWV>, grid, dim3(NWV * 64), e);
     if (BT == 1) { TSHIP_SK(1, 8) } else if (BT == 2) { TSHIP_SK(2, 8) } else { TSHIP_SK(4, 4) }
 #undef TSHIP_SK

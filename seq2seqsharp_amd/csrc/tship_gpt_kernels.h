@@ -79,7 +79,7 @@ __global__ void copy_cols_kernel(const float* __restrict__ src, long ld_src, lon
 // A block owns one 32-column tile and one k-split; its 4 wavefronts split the k range again and are
 // reduced through LDS.  HBM-bound: every weight byte is read exactly once with 16-byte loads.
 // ------------------------------------------------------------------------------------------------
-enum { EPI_PARTIAL = 0, EPI_F32_BIAS = 1, EPI_ACT16 = 2, EPI_RESID_TAIL = 3, EPI_SPLIT_TAIL = 4, EPI_SPLIT_ACT16 = 5 };
+enum { EPI_PARTIAL = 0, EPI_F32_BIAS = 1, EPI_ACT16 = 2, EPI_RESID_TAIL = 3, EPI_SPLIT_TAIL = 4 };
 
 struct SkinnyArgs {
     const half_t* W; int KT; int NT;
@@ -100,7 +100,7 @@ struct SkinnyArgs {
     // x, the next GEMM's packed input half(gamma * x) and the tile's per-row sum of squares
     float* x; int ldx_res; const float* gamma; half_t* xg16; int xg_kt; float* ssq_out; int ssq_out_ld;
     int* advance_pos;      // optional: one thread of the launch increments this device counter
-    // EPI_SPLIT_TAIL, EPI_SPLIT_ACT16 (KS > 1): the KS blocks of a column tile exchange their partial sums through `out` with
+    // EPI_SPLIT_TAIL (KS > 1): the KS blocks of a column tile exchange their partial sums through `out` with
     // agent-scope atomic stores and loads (they bypass the per-XCD L2, which is not coherent across XCDs for plain
     // accesses), count themselves in tile_count[nt], and the block that arrives last performs the epilogue
     int* tile_count;
@@ -114,7 +114,7 @@ template <int BT, int EPI, int NW, int U = 8>
 __global__ __launch_bounds__(NW * 64) void skinny_gemm_f16_kernel(SkinnyArgs a) {
     // one batch tile and eight wavefronts: every wavefront stores its accumulator once and the epilogue adds the eight
     // copies in wavefront order (one barrier); otherwise a pairwise tree followed by a transpose
-    constexpr bool ONE_ROUND = BT == 1 && NW == 8 && (EPI == EPI_ACT16 || EPI == EPI_RESID_TAIL || EPI == EPI_SPLIT_TAIL || EPI == EPI_SPLIT_ACT16);   // fp32 outputs keep the transpose: coalesced rows
+    constexpr bool ONE_ROUND = BT == 1 && NW == 8 && (EPI == EPI_ACT16 || EPI == EPI_RESID_TAIL || EPI == EPI_SPLIT_TAIL);   // fp32 outputs keep the transpose: coalesced rows
     constexpr int RED = (ONE_ROUND ? NW : NW / 2) * BT * 16 * 64, FIN = 2 * BT * 32 * 33;
     __shared__ float smem[RED > FIN ? RED : FIN];      // the tree buffers are dead when the transpose buffer is written
     float (*red)[BT][16][64] = (float (*)[BT][16][64])smem;
@@ -212,7 +212,7 @@ __global__ __launch_bounds__(NW * 64) void skinny_gemm_f16_kernel(SkinnyArgs a) 
         const int b = lane & 31, n1 = 8 * (w >> 2) + 4 * (lane >> 5) + (w & 3);
         const bool rok = b < a.rows_valid;
         const float rinv = a.ssq ? srinv[b] : 1.0f;
-        if (EPI == EPI_SPLIT_TAIL || EPI == EPI_SPLIT_ACT16) {
+        if (EPI == EPI_SPLIT_TAIL) {
             // publish this block's partial sums, then find out whether it is the last of its column tile
             __shared__ int s_last;
             // (exchange layout [split][tile][2][512 threads]: a wavefront's store is 256 contiguous bytes)
@@ -251,7 +251,7 @@ __global__ __launch_bounds__(NW * 64) void skinny_gemm_f16_kernel(SkinnyArgs a) 
             const int c1 = nt * 32 + n1, c2 = c1 + 16;
             if (rok && c1 < a.n_valid) a.out[(long)b * a.ld_out + c1] = s1 * rinv + a.bias[c1];
             if (rok && c2 < a.n_valid) a.out[(long)b * a.ld_out + c2] = s2 * rinv + a.bias[c2];
-        } else if (EPI == EPI_ACT16 || EPI == EPI_SPLIT_ACT16) {
+        } else if (EPI == EPI_ACT16) {
             if (a.gated) {
                 const int f = nt * 16 + n1;
                 if (rok && f < a.n_valid) {

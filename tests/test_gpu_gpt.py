@@ -373,6 +373,21 @@ def test_full_width_layer_against_oracle(G, oracle):
     gpu.close()
 
 
+@pytest.mark.parametrize("kv_heads,batch,prompt", [(1, 3, 40), (2, 8, 70)])
+def test_head_dim_128_against_oracle(G, oracle, kv_heads, batch, prompt):
+    """The 7B configuration's head shape (head_dim 128, 4 or 2 query heads per KV head) on a narrow model: prefill
+    (the second case has 560 prompt rows: LDS-tiled GEMM and MFMA prefill attention over several chunks) and decode
+    steps across a 32-position chunk boundary, fp16, against the oracle."""
+    cfg = synth.tiny_config(dtype="f16", hidden=512, n_heads=4, n_kv_heads=kv_heads, ffn_dim=1024, vocab=512, batch=batch, prompt=prompt)
+    orc, gpu, out, _ = _teacher_forced(G, oracle, cfg, 71, 4)
+    agree = []
+    for lg, gl in out:
+        assert np.abs(gl - lg).max() <= FP16_ABS
+        agree.append((gl.argmax(1) == lg.argmax(1)).mean())
+    assert np.mean(agree) >= 0.95
+    gpu.close()
+
+
 def test_argument_errors(G):
     from seq2seqsharp_amd._lib import TSHipError
     cfg = synth.tiny_config()
