@@ -664,12 +664,36 @@ static void prefill(TSHipGpt* m, const int32_t* host_ids, int B, int Tp) {
     ResidNormArgs rn; std::memset(&rn, 0, sizeof(rn));
     rn.x = px.as<float>(); rn.ldx = h; rn.h = h; rn.eps = c.norm_eps; rn.norm_type = c.norm_type;
     rn.xn = pxn.p; rn.ldxn = m->ldh;
-    {
+    // Deferred RMSNorm (fp16 RMSNorm models, LDS-tiled GEMMs): no norm kernels.  The producer of the residual stream
+    // stores half(gamma * x) and per-(32-column tile, row) sums of squares, a one-thread-per-row kernel turns those into
+    // 1 / rms, and the consuming GEMMs scale their output rows by it.
+    const bool deferred = m->fused_norm && R >= 512;
+    const int NTh = (int)(round_up(h, 32) / 32);
+    DevBuf pssq, prinv;
+    auto make_rinv = [&](const char* name) {
+        launch(m, name, rinv_rows_kernel, dim3((unsigned)ceil_div(R, 256)), dim3(256), (const float*)pssq.as<float>(), NTh, R, 1.0f / (float)h,
+               c.norm_eps, prinv.as<float>(), R);
+    };
+    if (deferred) {
+        pssq.alloc((size_t)NTh * R * sizeof(float));
+        prinv.alloc((size_t)R * sizeof(float));
+        FnPrepArgs a; std::memset(&a, 0, sizeof(a));
+        a.x = px.as<float>(); a.ldx = h; a.h = h;
+        a.ids = ids.as<int>(); a.emb = m->emb.p; a.emb_f16 = m->f16; a.emb_scale = (float)std::sqrt((double)h);
+        a.gamma = m->L[0]->n1_g.as<float>(); a.xg16 = pxn.as<half_t>(); a.xg_kt = 0; a.xg_ld = m->ldh; a.ssq_out = pssq.as<float>(); a.ssq_ld = R;
+        if (h <= 2048) launch(m, "p_embed_prepare", fn_prepare_kernel<8>, dim3((unsigned)R), dim3(256), a);
+        else if (h <= 4096) launch(m, "p_embed_prepare", fn_prepare_kernel<16>, dim3((unsigned)R), dim3(256), a);
+        else launch(m, "p_embed_prepare", fn_prepare_kernel<32>, dim3((unsigned)R), dim3(256), a);
+        make_rinv("p_rinv_attn");
+    } else {
         ResidNormArgs a = rn;
         a.ids = ids.as<int>(); a.emb = m->emb.p; a.emb_f16 = m->f16; a.emb_scale = (float)std::sqrt((double)h);
         a.gamma = m->L[0]->n1_g.as<float>(); a.beta = m->L[0]->n1_b.as<float>();
         run_resid_norm(m, "p_embed_norm", (int)R, a);
     }
+    auto producer = [&](BigArgs& e, const float* gamma) {        // residual GEMM that also emits the next GEMM's input
+        e.xg16 = pxn.as<half_t>(); e.ld_xg = (int)m->ldh; e.gamma = gamma; e.ssq_out = pssq.as<float>(); e.ssq_ld = R;
+    };
     auto big = [&](const char* name, const GemmW& w, const void* X, long ldx, int epi, BigArgs e) {
         e.W = w.buf.as<half_t>(); e.KT = w.KT; e.NT = w.NT; e.X = (const half_t*)X; e.ldx = (int)ldx; e.R = (int)R;
         if (R >= 512) {       // LDS-tiled kernel, 256 x 256 block tile
@@ -703,6 +727,7 @@ static void prefill(TSHipGpt* m, const int32_t* host_ids, int B, int Tp) {
         if (m->f16) {
             BigArgs e; std::memset(&e, 0, sizeof(e));
             e.out = pqkv.as<float>(); e.ld_out = (int)qp; e.bias = L.bqkv.as<float>(); e.n_valid = m->Nqkv;
+            if (deferred) e.rinv = prinv.as<float>();
             big("p_gemm_qkv", L.qkv, pxn.p, m->ldh, BEPI_F32_BIAS, e);
             aa.bias = zero_bias.as<float>();      // bias already added by the GEMM epilogue
         } else {
@@ -716,13 +741,14 @@ static void prefill(TSHipGpt* m, const int32_t* host_ids, int B, int Tp) {
         if (m->f16) {
             BigArgs e; std::memset(&e, 0, sizeof(e));
             e.out = px.as<float>(); e.ld_out = h; e.bias = L.bo.as<float>(); e.n_valid = h;
+            if (deferred) producer(e, L.n2_g.as<float>());
             big("p_gemm_wo", L.wo, po.p, m->ldh, BEPI_RESID, e);
         } else {
             run_gemm_f32(m, "p_gemm_wo", L.wo, po.as<float>(), m->ldh, (int)R, pqkv.as<float>(), qp, 0, 1);
             a2.part = pqkv.as<float>(); a2.KS = 1; a2.ld_part = qp; a2.bias = L.bo.as<float>();
         }
         if (L.moe) throw Error("TSHip_GptPrefill: MoE layers are prefilled token by token; use TSHip_GptDecode");
-        run_resid_norm(m, "p_norm_ffn", (int)R, a2);
+        if (deferred) make_rinv("p_rinv_ffn"); else run_resid_norm(m, "p_norm_ffn", (int)R, a2);
         ResidNormArgs a3 = rn;
         if (l + 1 < c.n_layers) { a3.gamma = m->L[l + 1]->n1_g.as<float>(); a3.beta = m->L[l + 1]->n1_b.as<float>(); }
         else a3.xn = nullptr;
@@ -730,9 +756,11 @@ static void prefill(TSHipGpt* m, const int32_t* host_ids, int B, int Tp) {
             BigArgs e; std::memset(&e, 0, sizeof(e));
             e.bias = L.b1.as<float>(); e.bias2 = L.b3.as<float>(); e.out16 = pa.as<half_t>(); e.ld16 = (int)m->ldF;
             e.act = c.act; e.gated = m->gated; e.n_valid = F;
+            if (deferred) e.rinv = prinv.as<float>();
             big("p_gemm_ffn13", L.w13, pxn.p, m->ldh, BEPI_ACT16, e);
             BigArgs e2; std::memset(&e2, 0, sizeof(e2));
             e2.out = px.as<float>(); e2.ld_out = h; e2.bias = L.b2.as<float>(); e2.n_valid = h;
+            if (deferred && l + 1 < c.n_layers) producer(e2, m->L[l + 1]->n1_g.as<float>());
             big("p_gemm_ffn2", L.w2, pa.p, m->ldF, BEPI_RESID, e2);
         } else {
             run_gemm_f32(m, "p_gemm_ffn13", L.w13, pxn.as<float>(), m->ldh, (int)R, pf.as<float>(), m->F13, 0, 1);
@@ -742,7 +770,8 @@ static void prefill(TSHipGpt* m, const int32_t* host_ids, int B, int Tp) {
             run_gemm_f32(m, "p_gemm_ffn2", L.w2, pa.as<float>(), m->ldF, (int)R, pqkv.as<float>(), qp, 0, 1);
             a3.part = pqkv.as<float>(); a3.KS = 1; a3.ld_part = qp; a3.bias = L.b2.as<float>();
         }
-        if (l + 1 < c.n_layers || !m->f16) run_resid_norm(m, "p_norm_attn", (int)R, a3);
+        if (deferred) { if (l + 1 < c.n_layers) make_rinv("p_rinv_attn"); }
+        else if (l + 1 < c.n_layers || !m->f16) run_resid_norm(m, "p_norm_attn", (int)R, a3);
     }
     // last position of every sequence (Decoder.cs:705-716) -> final norm -> vocabulary projection
     std::vector<int> map(B);

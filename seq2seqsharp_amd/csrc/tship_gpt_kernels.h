@@ -387,6 +387,11 @@ struct BigArgs {
     const float* bias; const float* bias2;
     half_t* out16; int ld16;
     int act; int gated; int n_valid;
+    // deferred RMSNorm (LDS-tiled kernels only).  Consumers: X holds half(gamma * x) and every output row is scaled by
+    // rinv[row] before the bias.  Producers (BEPI_RESID): besides the residual stream, store half(gamma * x) row-major
+    // into xg16 and the sum of squares of every (32-column tile, row) into ssq_out[tile * ssq_ld + row].
+    const float* rinv;
+    half_t* xg16; int ld_xg; const float* gamma; float* ssq_out; long ssq_ld;
 };
 
 template <int EPI>
@@ -445,6 +450,12 @@ __device__ __forceinline__ void big_gemm_store(const BigArgs& a, floatx16 (&acc)
     // of a column tile, and the four consecutive columns of a group go out as one 16-byte (fp32) or 8-byte (fp16) store.
     const int lh = lane >> 5;
     const bool vec_ok = (a.n_valid % 4 == 0) && ((EPI == BEPI_ACT16 ? a.ld16 : a.ld_out) % 4 == 0);
+    float rinv4[4];          // deferred norm: scale of this lane's four rows (1 when the input is already normalised)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const long row = row0 + 128 * wr + 32 * i + (lane & 31);
+        rinv4[i] = (a.rinv && row < a.R) ? a.rinv[row] : 1.0f;
+    }
     // one column tile per call with a compile-time tile number: the accumulators must only ever be indexed statically
     auto tile_out = [&](auto J) {
         constexpr int j = decltype(J)::value;
@@ -462,12 +473,13 @@ __device__ __forceinline__ void big_gemm_store(const BigArgs& a, floatx16 (&acc)
             for (int i = 0; i < 4; ++i) {
                 const long row = row0 + 128 * wr + 32 * i + (lane & 31);
                 if (row >= a.R) continue;
+                const float rv = rinv4[i];
 #pragma unroll
                 for (int g = 0; g < 2; ++g) {
                     const int f0 = nt * 16 + 8 * g + 4 * lh;
                     half4v o;
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) o[e] = (half_t)(act_apply(a.act, acc[j][i][4 * g + e] + b1[4 * g + e]) * (acc[j][i][4 * g + e + 8] + b2[4 * g + e]));
+                    for (int e = 0; e < 4; ++e) o[e] = (half_t)(act_apply(a.act, acc[j][i][4 * g + e] * rv + b1[4 * g + e]) * (acc[j][i][4 * g + e + 8] * rv + b2[4 * g + e]));
                     half_t* dst = a.out16 + row * a.ld16 + f0;
                     if (vec_ok && f0 + 3 < a.n_valid) *(half4v*)dst = o;
                     else {
@@ -482,6 +494,14 @@ __device__ __forceinline__ void big_gemm_store(const BigArgs& a, floatx16 (&acc)
             for (int v = 0; v < 16; ++v) {
                 const int col = nt * 32 + 8 * (v / 4) + 4 * lh + (v % 4);
                 bb[v] = col < a.n_valid ? a.bias[col] : 0.0f;
+            }
+            float gm[16], rowsq[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+            if (EPI == BEPI_RESID && a.xg16) {
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    const int col = nt * 32 + 8 * (v / 4) + 4 * lh + (v % 4);
+                    gm[v] = col < a.n_valid ? a.gamma[col] : 0.0f;
+                }
             }
             floatx4 old[4][4];
             if (EPI == BEPI_RESID) {
@@ -509,7 +529,7 @@ __device__ __forceinline__ void big_gemm_store(const BigArgs& a, floatx16 (&acc)
                     const int c0 = nt * 32 + 8 * g + 4 * lh;
                     floatx4 s;
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) s[e] = acc[j][i][4 * g + e] + bb[4 * g + e];
+                    for (int e = 0; e < 4; ++e) s[e] = acc[j][i][4 * g + e] * rinv4[i] + bb[4 * g + e];
                     if (EPI == BEPI_ACT16) {
                         half4v o;
 #pragma unroll
@@ -524,6 +544,21 @@ __device__ __forceinline__ void big_gemm_store(const BigArgs& a, floatx16 (&acc)
                         if (EPI == BEPI_RESID) {
 #pragma unroll
                             for (int e = 0; e < 4; ++e) s[e] = s[e] + old[i][g][e];
+                            if (a.xg16) {
+                                half4v xg;
+#pragma unroll
+                                for (int e = 0; e < 4; ++e) {
+                                    const bool ok = c0 + e < a.n_valid;
+                                    xg[e] = (half_t)(ok ? gm[4 * g + e] * s[e] : 0.0f);
+                                    rowsq[i] += ok ? s[e] * s[e] : 0.0f;
+                                }
+                                half_t* xd = a.xg16 + row * a.ld_xg + c0;
+                                if (vec_ok && (a.ld_xg & 3) == 0 && c0 + 3 < a.n_valid) *(half4v*)xd = xg;
+                                else {
+#pragma unroll
+                                    for (int e = 0; e < 4; ++e) if (c0 + e < a.n_valid) xd[e] = xg[e];
+                                }
+                            }
                         }
                         float* dst = a.out + row * a.ld_out + c0;
                         if (vec_ok && c0 + 3 < a.n_valid) *(floatx4*)dst = s;
@@ -532,6 +567,15 @@ __device__ __forceinline__ void big_gemm_store(const BigArgs& a, floatx16 (&acc)
                             for (int e = 0; e < 4; ++e) if (c0 + e < a.n_valid) dst[e] = s[e];
                         }
                     }
+                }
+            }
+            if (EPI == BEPI_RESID && a.xg16) {
+                // the two lane halves hold the two column halves of a row's tile
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const float q = rowsq[i] + __shfl_xor(rowsq[i], 32, 64);
+                    const long row = row0 + 128 * wr + 32 * i + (lane & 31);
+                    if (lane < 32 && row < a.R) a.ssq_out[(long)nt * a.ssq_ld + row] = q;
                 }
             }
         }
@@ -1000,13 +1044,30 @@ __global__ __launch_bounds__(256) void resid_tail_kernel(ResidTailArgs a) {
     }
 }
 
+// 1 / rms of every row from the per-tile sums of squares (deferred RMSNorm, prefill): one thread per row
+__global__ __launch_bounds__(256) void rinv_rows_kernel(const float* __restrict__ ssq, int ntiles, long ld, float inv_h, float eps,
+                                                        float* __restrict__ rinv, long rows) {
+    const long r = (long)blockIdx.x * 256 + threadIdx.x;
+    if (r >= rows) return;
+    float s = 0.0f;
+    for (int t0 = 0; t0 < ntiles; t0 += 8) {
+        float v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v[u] = t0 + u < ntiles ? ssq[(long)(t0 + u) * ld + r] : 0.0f;
+#pragma unroll
+        for (int u = 0; u < 8; ++u) s += v[u];
+    }
+    rinv[r] = 1.0f / sqrtf(s * inv_h + eps);
+}
+
 // Deferred-norm entry: x = E[id] * scale (or x = row row_map[r] of an existing stream) -> the next GEMM's packed
 // input half(gamma * x) and the per-column-tile sums of squares.  One block per row.
 struct FnPrepArgs {
     float* x; long ldx; int h;
     const int* ids; const void* emb; int emb_f16; float emb_scale;
     const float* src; long ld_src; const int* row_map;
-    const float* gamma; half_t* xg16; int xg_kt; float* ssq_out; int ssq_ld;
+    const float* gamma; half_t* xg16; int xg_kt; float* ssq_out; long ssq_ld;
+    long xg_ld;             // xg_kt == 0: xg16 is row-major with this leading dimension
 };
 template <int NPT>
 __global__ __launch_bounds__(256) void fn_prepare_kernel(FnPrepArgs a) {
@@ -1023,7 +1084,8 @@ __global__ __launch_bounds__(256) void fn_prepare_kernel(FnPrepArgs a) {
                 v = e * a.emb_scale;
             } else v = a.src[srow * a.ld_src + c];
             a.x[(long)r * a.ldx + c] = v;
-            a.xg16[xpack_index(r, c, a.xg_kt)] = (half_t)(a.gamma[c] * v);
+            if (a.xg_kt > 0) a.xg16[xpack_index(r, c, a.xg_kt)] = (half_t)(a.gamma[c] * v);
+            else a.xg16[(long)r * a.xg_ld + c] = (half_t)(a.gamma[c] * v);
         }
         float q = v * v;
 #pragma unroll
