@@ -398,9 +398,9 @@ static AttnKernel pick_attn_d(int D, int G, bool prefill) {
 template <int D>
 static AttnKernel pick_attn_mfma(int G, bool prefill) {
     switch (G) {
-        case 1: return prefill ? attn_mfma_kernel<D, 1, true> : attn_mfma_kernel<D, 1, false>;
-        case 2: return prefill ? attn_mfma_kernel<D, 2, true> : attn_mfma_kernel<D, 2, false>;
-        case 4: return prefill ? attn_mfma_kernel<D, 4, true> : attn_mfma_kernel<D, 4, false>;
+        case 1: return prefill ? attn_mfma_prefill_kernel<D, 1> : attn_mfma_kernel<D, 1>;
+        case 2: return prefill ? attn_mfma_prefill_kernel<D, 2> : attn_mfma_kernel<D, 2>;
+        case 4: return prefill ? attn_mfma_prefill_kernel<D, 4> : attn_mfma_kernel<D, 4>;
         default: throw Error("query heads per KV head must be 1, 2 or 4");
     }
 }
@@ -734,7 +734,10 @@ static void prefill(TSHipGpt* m, const int32_t* host_ids, int B, int Tp) {
             run_gemm_f32(m, "p_gemm_qkv", L.qkv, pxn.as<float>(), m->ldh, (int)R, pqkv.as<float>(), qp, 0, 1);
         }
         launch(m, "p_kv_write", pick_kvw(m), dim3(Tp, B), dim3(256), aa);
-        if (m->vt) { const int QB = 16 / m->G; launch(m, "p_attn", pick_attn(m, true), dim3((unsigned)ceil_div(Tp, QB), c.n_kv_heads, B), dim3(m->D == 128 ? 256 : 512), aa); }
+        if (m->vt) {      // a wavefront per 16 / G query positions, 8 (head_dim 64) or 4 (head_dim 128) wavefronts per block
+            const int per_block = (16 / m->G) * (m->D == 128 ? 4 : 8);
+            launch(m, "p_attn", pick_attn(m, true), dim3((unsigned)ceil_div(Tp, per_block), c.n_kv_heads, B), dim3(m->D == 128 ? 256 : 512), aa);
+        }
         else launch(m, "p_attn", pick_attn(m, true), dim3(Tp, c.n_kv_heads, B), dim3(256), aa);
         ResidNormArgs a2 = rn;
         a2.gamma = L.n2_g.as<float>(); a2.beta = L.n2_b.as<float>();

@@ -1387,19 +1387,18 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(AttnArgs a) {
 
 
 // ------------------------------------------------------------------------------------------------
-// MFMA attention (fp16 cache, head_dim 64 or 128).  One block per (batch row, KV head) and QB query positions
-// (decode: 1, prefill: 16 / G); the 16 columns of v_mfma_f32_16x16x32_f16 are (query position, query head of the
-// group).  Keys and values are kept fragment-major (kfrag_index / vfrag_index), so every load is 1 KiB contiguous:
+// MFMA attention (fp16 cache, head_dim 64 or 128), decode: one block per (batch row, KV head); the G query heads of
+// the group use G of the 16 columns of v_mfma_f32_16x16x32_f16.  Keys and values are kept fragment-major (kfrag_index / vfrag_index), so every load is 1 KiB contiguous:
 //   S[32 t][16 col]   = K tile (two 16-row A operands, rows permuted so that lane group q ends up with
 //                       t = t0 + 8q .. 8q+7)  x  Q (B operand, kept in registers)
 //   O^T[D][16 col]   += V^T tile (A operand: 16 d-rows x 32 t)  x  P (B operand: the lane's own 8 probabilities)
 // Online softmax per column with one running maximum per wavefront; wavefronts take 32-row chunks round robin and
 // are merged through LDS.  All arithmetic on scores, probabilities' sums and outputs is fp32.
 // ------------------------------------------------------------------------------------------------
-template <int D, int G, bool PREFILL>
+template <int D, int G>
 __global__ __launch_bounds__(D == 128 ? 256 : 512) void attn_mfma_kernel(AttnArgs a) {
     constexpr int NW = D == 128 ? 4 : 8, NTH = NW * 64;
-    constexpr int QB = PREFILL ? 16 / G : 1, NCOL = QB * G;
+    constexpr int NCOL = G;                   // MFMA columns in use: the G query heads of the group
     constexpr int KD = D / 32, DT = D / 16;
     __shared__ float sIn[(G + 2) * D];
     __shared__ float sQ[16][D];
@@ -1409,9 +1408,8 @@ __global__ __launch_bounds__(D == 128 ? 256 : 512) void attn_mfma_kernel(AttnArg
     const int t = threadIdx.x, lane = t & 63, w = __builtin_amdgcn_readfirstlane(t >> 6);
     const int r16 = lane & 15, q = lane >> 4;
     const int HD = a.H * D, GD = a.Hkv * D;
-    int kvh, b, tq0 = 0, pos_base, T;
-    if (PREFILL) { kvh = blockIdx.y; b = blockIdx.z; tq0 = blockIdx.x * QB; pos_base = a.pos0 + tq0; T = min(pos_base + QB, a.pos0 + a.Tq); }
-    else { kvh = blockIdx.x; b = blockIdx.y; pos_base = *a.d_pos; T = pos_base + 1; }
+    const int kvh = blockIdx.x, b = blockIdx.y;
+    const int pos_base = *a.d_pos, T = pos_base + 1;
     half_t* Kb = (half_t*)a.kcache + ((long)b * a.Hkv + kvh) * a.max_len * D;
     half_t* Vt = (half_t*)a.vcache + ((long)b * a.Hkv + kvh) * (long)D * a.max_len;
 
@@ -1429,11 +1427,11 @@ __global__ __launch_bounds__(D == 128 ? 256 : 512) void attn_mfma_kernel(AttnArg
         for (int dt = 0; dt < DT; ++dt) vf[dt] = *(const half8*)(vc + dt * 512);
     };
     // the first chunk of this wavefront does not depend on the prologue unless it holds the row being appended
-    const bool early = !PREFILL && w < nchunks - 1;
+    const bool early = w < nchunks - 1;
     if (early) load_chunk(w, kfA, vfA);
 
     for (int i = t; i < 16 * D; i += NTH) (&sQ[0][0])[i] = 0.0f;
-    if (!PREFILL) {
+    {
         constexpr int CPT = ((G + 2) * D + NTH - 1) / NTH;        // projection columns per thread
         constexpr int PPT = ((G + 1) * D / 2 + NTH - 1) / NTH;    // rotary pairs per thread
         const int pos = pos_base;
@@ -1490,19 +1488,6 @@ __global__ __launch_bounds__(D == 128 ? 256 : 512) void attn_mfma_kernel(AttnArg
         }
         for (int d = t; d < D; d += NTH) Vt[vfrag_index(pos, d, D)] = (half_t)sIn[(G + 1) * D + d];
         __threadfence_block();
-    } else {
-        __syncthreads();
-        for (int p = t; p < NCOL * D / 2; p += NTH) {
-            int col = p / (D / 2), i = p % (D / 2);
-            int qi = col / G, g = col % G;
-            if (tq0 + qi >= a.Tq) continue;
-            long row = (long)b * a.Tq + tq0 + qi;
-            int pos = pos_base + qi;
-            int c0 = (kvh * G + g) * D + 2 * i;
-            float x0 = a.qkv[row * a.ldq + c0] + a.bias[c0], x1 = a.qkv[row * a.ldq + c0 + 1] + a.bias[c0 + 1], y0 = x0, y1 = x1;
-            if (a.rope_cos) rope_pair(x0, x1, a.rope_cos[(long)pos * (D / 2) + i], a.rope_sin[(long)pos * (D / 2) + i], y0, y1);
-            sQ[col][2 * i] = a.scale * y0; sQ[col][2 * i + 1] = a.scale * y1;
-        }
     }
     __syncthreads();
 
@@ -1513,8 +1498,7 @@ __global__ __launch_bounds__(D == 128 ? 256 : 512) void attn_mfma_kernel(AttnArg
 #pragma unroll
         for (int j = 0; j < 8; ++j) qf[kd][j] = (half_t)sQ[r16][kd * 32 + 8 * q + j];
     // last position this lane's column may attend to
-    const int qi_lane = PREFILL ? r16 / G : 0;
-    const int tmax = PREFILL ? pos_base + qi_lane : T - 1;
+    const int tmax = T - 1;
     const bool col_ok = r16 < NCOL;
 
     float m_run = -INFINITY, l_run = 0.0f;
@@ -1600,17 +1584,133 @@ __global__ __launch_bounds__(D == 128 ? 256 : 512) void attn_mfma_kernel(AttnArg
             O += sO[i][d][col] * wgt;
         }
         const float o = O / L;
+        const int g = col;
+        const int kcol = (kvh * G + g) * D + d;
+        if (a.out_kt > 0) ((half_t*)a.out)[xpack_index(b, kcol, a.out_kt)] = (half_t)o;
+        else ((half_t*)a.out)[(long)b * a.ld_out + kcol] = (half_t)o;
+    }
+}
+
+// Prefill variant: a wavefront owns QB = 16 / G consecutive query positions (the 16 MFMA columns are its positions x
+// the G query heads of the group) and walks over every 32-position chunk of its own causal prefix, so there is no
+// merge across wavefronts.  The NW wavefronts of a block sit at neighbouring positions and fetch the same chunks at
+// about the same time: the block reads its prefix once from L2 and NW - 1 times from L1 (the variant with one such
+// group per block re-read the prefix from L2 for every four query positions).  grid (ceil(Tq / (QB NW)), Hkv, batch).
+template <int D, int G>
+__global__ __launch_bounds__(D == 128 ? 256 : 512) void attn_mfma_prefill_kernel(AttnArgs a) {
+    constexpr int NW = D == 128 ? 4 : 8;
+    constexpr int QB = 16 / G, KD = D / 32, DT = D / 16;
+    __shared__ float sbuf[NW][D * 16];       // per wavefront: Q staging [16 columns][D], later the outputs [D][16 columns]
+    __shared__ float sl[NW][16];
+    const int lane = threadIdx.x & 63, w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int r16 = lane & 15, q = lane >> 4;
+    const int kvh = blockIdx.y, b = blockIdx.z;
+    const int tq0 = (blockIdx.x * NW + w) * QB;
+    if (tq0 >= a.Tq) return;                  // no block-wide barrier below
+    const int pos_base = a.pos0 + tq0, T = min(pos_base + QB, a.pos0 + a.Tq);
+    const int nchunks = (T + 31) / 32;
+    const half_t* Kb = (const half_t*)a.kcache + ((long)b * a.Hkv + kvh) * a.max_len * D;
+    const half_t* Vt = (const half_t*)a.vcache + ((long)b * a.Hkv + kvh) * (long)D * a.max_len;
+    half8 kfA[2][KD], vfA[DT], kfB[2][KD], vfB[DT];
+    auto load_chunk = [&](int c, half8 (&kf)[2][KD], half8 (&vf)[DT]) {
+        const half_t* kc = Kb + (long)c * (32 * D) + lane * 8;
+        const half_t* vc = Vt + (long)c * (32 * D) + lane * 8;
+#pragma unroll
+        for (int tile = 0; tile < 2; ++tile)
+#pragma unroll
+            for (int kd = 0; kd < KD; ++kd) kf[tile][kd] = *(const half8*)(kc + (tile * KD + kd) * 512);
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) vf[dt] = *(const half8*)(vc + dt * 512);
+    };
+    load_chunk(0, kfA, vfA);                  // chunk 0 is complete or ends at this wavefront's own positions (written by kv_write)
+
+    // queries: projection + bias, rotary embedding, 1 / sqrt(d); columns beyond the prompt stay zero
+    float* sq = sbuf[w];
+    for (int i = lane; i < 16 * D; i += 64) sq[i] = 0.0f;
+    for (int p = lane; p < 16 * D / 2; p += 64) {
+        const int col = p / (D / 2), i = p % (D / 2);
         const int qi = col / G, g = col % G;
-        if (PREFILL) {
-            if (tq0 + qi < a.Tq) {
-                half_t* out = (half_t*)a.out + ((long)b * a.Tq + tq0 + qi) * a.ld_out + (kvh * G + g) * D;
-                out[d] = (half_t)o;
-            }
-        } else {
-            const int kcol = (kvh * G + g) * D + d;
-            if (a.out_kt > 0) ((half_t*)a.out)[xpack_index(b, kcol, a.out_kt)] = (half_t)o;
-            else ((half_t*)a.out)[(long)b * a.ld_out + kcol] = (half_t)o;
+        if (tq0 + qi >= a.Tq) continue;
+        const long row = (long)b * a.Tq + tq0 + qi;
+        const int pos = pos_base + qi;
+        const int c0 = (kvh * G + g) * D + 2 * i;
+        float x0 = a.qkv[row * a.ldq + c0] + a.bias[c0], x1 = a.qkv[row * a.ldq + c0 + 1] + a.bias[c0 + 1], y0 = x0, y1 = x1;
+        if (a.rope_cos) rope_pair(x0, x1, a.rope_cos[(long)pos * (D / 2) + i], a.rope_sin[(long)pos * (D / 2) + i], y0, y1);
+        sq[col * D + 2 * i] = a.scale * y0; sq[col * D + 2 * i + 1] = a.scale * y1;
+    }
+    __builtin_amdgcn_wave_barrier();
+    half8 qf[KD];
+#pragma unroll
+    for (int kd = 0; kd < KD; ++kd)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) qf[kd][j] = (half_t)sq[r16 * D + kd * 32 + 8 * q + j];
+    const int tmax = pos_base + r16 / G;      // last position this lane's column may attend to
+
+    float m_run = -INFINITY, l_run = 0.0f;
+    floatx4 acc_o[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) acc_o[dt] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+    auto do_chunk = [&](int c, half8 (&kf)[2][KD], half8 (&vf)[DT]) {
+        const int t0 = c * 32;
+        floatx4 sA = floatx4{0.0f, 0.0f, 0.0f, 0.0f}, sB = sA;
+#pragma unroll
+        for (int kd = 0; kd < KD; ++kd) {
+            sA = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf[0][kd], qf[kd], sA, 0, 0, 0);
+            sB = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf[1][kd], qf[kd], sB, 0, 0, 0);
         }
+        float s[8];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) { s[j] = sA[j]; s[4 + j] = sB[j]; }
+        float cm = -INFINITY;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            if (t0 + 8 * q + j > tmax) s[j] = -INFINITY;       // causal mask (adding -30000 gives exactly 0 after exp in fp32 too)
+            cm = fmaxf(cm, s[j]);
+        }
+        cm = fmaxf(cm, __shfl_xor(cm, 16, 64));
+        cm = fmaxf(cm, __shfl_xor(cm, 32, 64));
+        const float m_new = fmaxf(m_run, cm);
+        const float corr = (m_new == -INFINITY) ? 1.0f : __expf(m_run - m_new);
+        half8 pf;
+        float psum = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const float p = (s[j] == -INFINITY) ? 0.0f : __expf(s[j] - m_new);
+            psum += p;
+            pf[j] = (half_t)p;
+        }
+        l_run = l_run * corr + psum;
+        m_run = m_new;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc_o[dt][i] *= corr;
+            acc_o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vf[dt], pf, acc_o[dt], 0, 0, 0);
+        }
+    };
+    for (int c = 0; c < nchunks; c += 2) {
+        if (c + 1 < nchunks) load_chunk(c + 1, kfB, vfB);
+        do_chunk(c, kfA, vfA);
+        if (c + 1 >= nchunks) break;
+        if (c + 2 < nchunks) load_chunk(c + 2, kfA, vfA);
+        do_chunk(c + 1, kfB, vfB);
+    }
+    l_run += __shfl_xor(l_run, 16, 64);
+    l_run += __shfl_xor(l_run, 32, 64);
+    // outputs through this wavefront's LDS slice so that rows go out contiguously: O^T[d][col] -> out[row(col)][d]
+    __builtin_amdgcn_wave_barrier();          // the Q staging has been consumed
+    if (q == 0) sl[w][r16] = l_run;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) sq[(dt * 16 + 4 * q + i) * 16 + r16] = acc_o[dt][i];
+    __builtin_amdgcn_wave_barrier();
+    for (int col = 0; col < 16; ++col) {
+        const int qi = col / G, g = col % G;
+        if (tq0 + qi >= a.Tq) break;
+        half_t* out = (half_t*)a.out + ((long)b * a.Tq + tq0 + qi) * a.ld_out + (kvh * G + g) * D;
+        const float inv = 1.0f / sl[w][col];
+        for (int d = lane; d < D; d += 64) out[d] = (half_t)(sq[d * 16 + col] * inv);
     }
 }
 
