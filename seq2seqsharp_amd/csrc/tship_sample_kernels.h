@@ -178,60 +178,85 @@ static __global__ __launch_bounds__(256) void topp_scatter_kernel(TopPArgs a) {
 }
 
 // running sum and pick: grid (rows), one wavefront.  The sorted keys are in keysA / idxA.
-// Chunks of 64 probabilities are added strictly in order (every lane holds the same running value); the value
-// after each chunk is kept, so that the pick only has to replay one chunk.
+// The running sum is one dependent chain of fp32 additions (that is what fixes its value), so the cost per element is
+// what matters: the keys are fetched with scalar loads, 32 at a time and one unit ahead, and every addition is a single
+// v_add_f32 with a scalar operand.  The value after each unit of 32 is kept, so that the pick only replays one unit.
+typedef unsigned uint16s __attribute__((ext_vector_type(16)));
+__device__ __forceinline__ void topp_sload(uint16s& d, const unsigned* p) {
+    asm volatile("s_load_dwordx16 %0, %1, 0x0" : "=s"(d) : "s"(p) : "memory");
+}
+__device__ __forceinline__ void topp_swait(uint16s& a, uint16s& b) {
+    asm volatile("s_waitcnt lgkmcnt(0)" : "+s"(a), "+s"(b) : : "memory");
+}
+
 static __global__ __launch_bounds__(64) void topp_pick_kernel(TopPArgs a) {
     const int r = blockIdx.x, lane = threadIdx.x, V = a.V;
-    const unsigned* keys = a.keysA + (long)r * a.Vs;
+    const unsigned* keys = a.keysA + (long)r * a.Vs;       // Vs is a multiple of 64: whole units can be read
     const int* idx = a.idxA + (long)r * a.Vs;
-    float* cp = a.accp + (long)r * a.Vs;              // cp[c]: running sum after chunk c
-    float acc = 0.0f; int n = 0, nch = 0;
-    for (int base = 0; base < V; base += 64) {
-        const int i = base + lane;
-        const unsigned k = i < V ? keys[i] : 0xffffffffu;
-        const float p = k == 0xffffffffu ? 0.0f : __uint_as_float(~k);
-        const bool has_end = __any(k == 0xffffffffu);
-        float trial = acc;
+    float* cp = a.accp + (long)r * a.Vs;                   // cp[u]: running sum after unit u
+    float acc = 0.0f; int n = 0, nun = 0;
+    // two register sets with fixed roles (no copies: a register that a load is still writing must not be moved)
+    uint16s a0, a1, b0, b1;
+    auto unit = [&](int base, uint16s& c0, uint16s& c1) -> bool {        // returns true when the walk is over
+        // ascending keys: candidates (p > 0) first, dropped entries (key 0xffffffff) last; p = bits of ~key
+        const bool whole = base + 32 <= V && c1[15] != 0xffffffffu;
+        bool done = !whole;
+        if (whole) {
+            float trial = acc;
 #pragma unroll
-        for (int j = 0; j < 64; ++j) trial += __int_as_float(__builtin_amdgcn_readlane(__float_as_int(p), j));
-        if (!has_end && trial < a.top_p) {
-            acc = trial; n += 64;
-            if (lane == 0) cp[nch] = acc;
-            ++nch;
-            continue;
+            for (int j = 0; j < 16; ++j) trial += __uint_as_float(~c0[j]);
+#pragma unroll
+            for (int j = 0; j < 16; ++j) trial += __uint_as_float(~c1[j]);
+            if (trial < a.top_p) { acc = trial; n += 32; }
+            else done = true;
         }
-        // the chunk that ends the walk: element by element
-        for (int j = 0; j < 64; ++j) {
-            const float pj = __shfl(p, j, 64);
-            if (pj <= 0.0f) break;                     // ran out of candidates
-            acc += pj; n += 1;
-            if (acc >= a.top_p) break;
+        if (done) {
+            // the unit that ends the walk: element by element
+            const int i = base + lane;
+            const unsigned k = (lane < 32 && i < V) ? keys[i] : 0xffffffffu;
+            const float p = k == 0xffffffffu ? 0.0f : __uint_as_float(~k);
+            for (int j = 0; j < 32; ++j) {
+                const float pj = __shfl(p, j, 64);
+                if (pj <= 0.0f) break;                     // ran out of candidates
+                acc += pj; n += 1;
+                if (acc >= a.top_p) break;
+            }
         }
-        if (lane == 0) cp[nch] = acc;
-        ++nch;
-        break;
+        if (lane == 0) cp[nun] = acc;
+        ++nun;
+        return done;
+    };
+    topp_sload(a0, keys); topp_sload(a1, keys + 16);
+    for (int base = 0; base < V; base += 64) {
+        topp_swait(a0, a1);
+        if (base + 32 < V) { topp_sload(b0, keys + base + 32); topp_sload(b1, keys + base + 48); }
+        if (unit(base, a0, a1)) break;
+        if (base + 32 >= V) break;
+        topp_swait(b0, b1);
+        if (base + 64 < V) { topp_sload(a0, keys + base + 64); topp_sload(a1, keys + base + 80); }
+        if (unit(base + 32, b0, b1)) break;
     }
     __threadfence_block();
     const long slot = (a.d_step ? (long)*a.d_step * gridDim.x : 0) + r;
     const float u = a.uniforms[slot];
     int pick = 0x7fffffff;
     if (n > 0) {
-        // first chunk whose final value passes the test holds the pick (the running sum never decreases)
-        int cstar = 0x7fffffff;
-        for (int c0 = 0; c0 < nch && cstar == 0x7fffffff; c0 += 64) {
-            const int c = c0 + lane;
-            const bool hit = c < nch && cp[c] / acc >= u;
+        // first unit whose final value passes the test holds the pick (the running sum never decreases)
+        int ustar = 0x7fffffff;
+        for (int u0 = 0; u0 < nun && ustar == 0x7fffffff; u0 += 64) {
+            const int c = u0 + lane;
+            const bool hit = c < nun && cp[c] / acc >= u;
             const unsigned long long m = __ballot(hit);
-            if (m) cstar = c0 + (int)__ffsll((long long)m) - 1;
+            if (m) ustar = u0 + (int)__ffsll((long long)m) - 1;
         }
-        if (cstar != 0x7fffffff) {
-            float run = cstar > 0 ? cp[cstar - 1] : 0.0f;
-            const int i = cstar * 64 + lane;
-            const unsigned k = i < V ? keys[i] : 0xffffffffu;
+        if (ustar != 0x7fffffff) {
+            float run = ustar > 0 ? cp[ustar - 1] : 0.0f;
+            const int i = ustar * 32 + lane;
+            const unsigned k = (lane < 32 && i < V) ? keys[i] : 0xffffffffu;
             const float p = k == 0xffffffffu ? 0.0f : __uint_as_float(~k);
-            for (int j = 0; j < 64 && cstar * 64 + j < n; ++j) {
+            for (int j = 0; j < 32 && ustar * 32 + j < n; ++j) {
                 run += __shfl(p, j, 64);
-                if (run / acc >= u) { pick = cstar * 64 + j; break; }
+                if (run / acc >= u) { pick = ustar * 32 + j; break; }
             }
         }
     }
