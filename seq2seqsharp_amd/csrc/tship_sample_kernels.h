@@ -114,8 +114,15 @@ static __global__ __launch_bounds__(256) void topp_scan_kernel(TopPArgs a) {
     __shared__ int tot[256];
     const int r = blockIdx.x, d = threadIdx.x;
     int* h = a.hist + (long)r * a.nseg * 256;
+    // (loads in batches of eight: a load-modify-store loop would wait for memory once per segment)
     int run = 0;
-    for (int s = 0; s < a.nseg; ++s) { const int v = h[s * 256 + d]; h[s * 256 + d] = run; run += v; }
+    for (int s0 = 0; s0 < a.nseg; s0 += 8) {
+        int v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v[u] = s0 + u < a.nseg ? h[(s0 + u) * 256 + d] : 0;
+#pragma unroll
+        for (int u = 0; u < 8; ++u) { if (s0 + u < a.nseg) h[(s0 + u) * 256 + d] = run; run += v[u]; }
+    }
     tot[d] = run;
     __syncthreads();
     if (d < 64) {       // one wavefront: 4 digits per lane, then a shuffle scan over the lane sums
@@ -129,7 +136,13 @@ static __global__ __launch_bounds__(256) void topp_scan_kernel(TopPArgs a) {
     }
     __syncthreads();
     const int base = tot[d];
-    for (int s = 0; s < a.nseg; ++s) h[s * 256 + d] += base;
+    for (int s0 = 0; s0 < a.nseg; s0 += 8) {
+        int v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v[u] = s0 + u < a.nseg ? h[(s0 + u) * 256 + d] : 0;
+#pragma unroll
+        for (int u = 0; u < 8; ++u) if (s0 + u < a.nseg) h[(s0 + u) * 256 + d] = v[u] + base;
+    }
 }
 
 // stable scatter of one segment: grid (nseg, rows), 256 threads.  Element order inside the segment is
@@ -173,68 +186,84 @@ static __global__ __launch_bounds__(256) void topp_scatter_kernel(TopPArgs a) {
         if (!valid[it]) continue;
         const unsigned d = (key[it] >> a.shift) & 255u;
         const int dst = wh[w * 4 + it][d] + rank[it];
-        kout[dst] = key[it]; iout[dst] = idx[it];
+        kout[dst] = a.shift == 24 ? ~key[it] : key[it];      // the last pass leaves the probabilities' own bit patterns
+        iout[dst] = idx[it];
     }
 }
 
-// running sum and pick: grid (rows), one wavefront.  The sorted keys are in keysA / idxA.
+// running sum and pick: grid (rows), one wavefront.  keysA holds the sorted probabilities (their bit patterns, 0 for
+// dropped entries), idxA the token ids in the same order.
 // The running sum is one dependent chain of fp32 additions (that is what fixes its value), so the cost per element is
-// what matters: the keys are fetched with scalar loads, 32 at a time and one unit ahead, and every addition is a single
-// v_add_f32 with a scalar operand.  The value after each unit of 32 is kept, so that the pick only replays one unit.
-typedef unsigned uint16s __attribute__((ext_vector_type(16)));
-__device__ __forceinline__ void topp_sload(uint16s& d, const unsigned* p) {
-    asm volatile("s_load_dwordx16 %0, %1, 0x0" : "=s"(d) : "s"(p) : "memory");
-}
-__device__ __forceinline__ void topp_swait(uint16s& a, uint16s& b) {
-    asm volatile("s_waitcnt lgkmcnt(0)" : "+s"(a), "+s"(b) : : "memory");
-}
-
+// what matters: the probabilities are staged through LDS in segments of 8192 (the next segment's loads are in flight
+// while the current one is walked), read back 16 bytes at a time with every lane at the same address, one unit of 32
+// ahead, and added with one v_add_f32 each.  The value after each unit is kept, so that the pick only replays one unit.
 static __global__ __launch_bounds__(64) void topp_pick_kernel(TopPArgs a) {
+    constexpr int SEG = 8192;
+    __shared__ __attribute__((aligned(16))) float sp[2][SEG];
     const int r = blockIdx.x, lane = threadIdx.x, V = a.V;
-    const unsigned* keys = a.keysA + (long)r * a.Vs;       // Vs is a multiple of 64: whole units can be read
+    const float* pk = (const float*)(a.keysA + (long)r * a.Vs);      // Vs is a multiple of 64
     const int* idx = a.idxA + (long)r * a.Vs;
-    float* cp = a.accp + (long)r * a.Vs;                   // cp[u]: running sum after unit u
+    float* cp = a.accp + (long)r * a.Vs;                               // cp[u]: running sum after unit u
     float acc = 0.0f; int n = 0, nun = 0;
-    // two register sets with fixed roles (no copies: a register that a load is still writing must not be moved)
-    uint16s a0, a1, b0, b1;
-    auto unit = [&](int base, uint16s& c0, uint16s& c1) -> bool {        // returns true when the walk is over
-        // ascending keys: candidates (p > 0) first, dropped entries (key 0xffffffff) last; p = bits of ~key
-        const bool whole = base + 32 <= V && c1[15] != 0xffffffffu;
-        bool done = !whole;
-        if (whole) {
-            float trial = acc;
+    const int nseg = (V + SEG - 1) / SEG;
+    floatx4 reg[SEG / 256];
+    auto seg_load = [&](int s) {
 #pragma unroll
-            for (int j = 0; j < 16; ++j) trial += __uint_as_float(~c0[j]);
+        for (int i = 0; i < SEG / 256; ++i) {
+            const int e = s * SEG + (i * 64 + lane) * 4;
+            floatx4 v = e < V ? *(const floatx4*)(pk + e) : floatx4{0.0f, 0.0f, 0.0f, 0.0f};      // e + 3 < Vs
 #pragma unroll
-            for (int j = 0; j < 16; ++j) trial += __uint_as_float(~c1[j]);
-            if (trial < a.top_p) { acc = trial; n += 32; }
-            else done = true;
+            for (int j = 0; j < 4; ++j) if (e + j >= V) v[j] = 0.0f;                                 // padding is not a candidate
+            reg[i] = v;
         }
-        if (done) {
-            // the unit that ends the walk: element by element
-            const int i = base + lane;
-            const unsigned k = (lane < 32 && i < V) ? keys[i] : 0xffffffffu;
-            const float p = k == 0xffffffffu ? 0.0f : __uint_as_float(~k);
-            for (int j = 0; j < 32; ++j) {
-                const float pj = __shfl(p, j, 64);
-                if (pj <= 0.0f) break;                     // ran out of candidates
-                acc += pj; n += 1;
-                if (acc >= a.top_p) break;
-            }
-        }
-        if (lane == 0) cp[nun] = acc;
-        ++nun;
-        return done;
     };
-    topp_sload(a0, keys); topp_sload(a1, keys + 16);
-    for (int base = 0; base < V; base += 64) {
-        topp_swait(a0, a1);
-        if (base + 32 < V) { topp_sload(b0, keys + base + 32); topp_sload(b1, keys + base + 48); }
-        if (unit(base, a0, a1)) break;
-        if (base + 32 >= V) break;
-        topp_swait(b0, b1);
-        if (base + 64 < V) { topp_sload(a0, keys + base + 64); topp_sload(a1, keys + base + 80); }
-        if (unit(base + 32, b0, b1)) break;
+    auto seg_store = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < SEG / 256; ++i) *(floatx4*)&sp[buf][(i * 64 + lane) * 4] = reg[i];
+    };
+    auto unit_read = [&](int buf, int u, floatx4 (&q)[8]) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) q[i] = *(const floatx4*)&sp[buf][u * 32 + 4 * i];
+    };
+    seg_load(0);
+    seg_store(0);
+    bool over = false;
+    for (int s = 0; s < nseg && !over; ++s) {
+        const int buf = s & 1;
+        if (s + 1 < nseg) seg_load(s + 1);
+        __builtin_amdgcn_wave_barrier();
+        const int units = min(SEG, V - s * SEG + 31) / 32;             // units of this segment that hold candidates or padding
+        floatx4 q[8], qn[8];
+        unit_read(buf, 0, q);
+        for (int u = 0; u < units; ++u) {
+            if (u + 1 < units) unit_read(buf, u + 1, qn);
+            // descending probabilities: candidates (p > 0) first, dropped entries and padding (0) last
+            bool done = q[7][3] == 0.0f;
+            if (!done) {
+                float trial = acc;
+#pragma unroll
+                for (int i = 0; i < 8; ++i)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) trial += q[i][j];
+                if (trial < a.top_p) { acc = trial; n += 32; }
+                else done = true;
+            }
+            if (done) {
+                // the unit that ends the walk: element by element
+                for (int j = 0; j < 32; ++j) {
+                    const float pj = sp[buf][u * 32 + j];
+                    if (pj <= 0.0f) break;                 // ran out of candidates
+                    acc += pj; n += 1;
+                    if (acc >= a.top_p) break;
+                }
+            }
+            if (lane == 0) cp[nun] = acc;
+            ++nun;
+            if (done) { over = true; break; }
+#pragma unroll
+            for (int i = 0; i < 8; ++i) q[i] = qn[i];
+        }
+        if (!over && s + 1 < nseg) { __builtin_amdgcn_wave_barrier(); seg_store(buf ^ 1); }
     }
     __threadfence_block();
     const long slot = (a.d_step ? (long)*a.d_step * gridDim.x : 0) + r;
@@ -252,8 +281,7 @@ static __global__ __launch_bounds__(64) void topp_pick_kernel(TopPArgs a) {
         if (ustar != 0x7fffffff) {
             float run = ustar > 0 ? cp[ustar - 1] : 0.0f;
             const int i = ustar * 32 + lane;
-            const unsigned k = (lane < 32 && i < V) ? keys[i] : 0xffffffffu;
-            const float p = k == 0xffffffffu ? 0.0f : __uint_as_float(~k);
+            const float p = (lane < 32 && i < V) ? pk[i] : 0.0f;
             for (int j = 0; j < 32 && ustar * 32 + j < n; ++j) {
                 run += __shfl(p, j, 64);
                 if (run / acc >= u) { pick = ustar * 32 + j; break; }
