@@ -40,6 +40,8 @@ struct DevBuf {
     void release() {
         if (p) { (void)hipStreamSynchronize(stream()); (void)hipFree(p); p = nullptr; bytes = 0; }
     }
+    // grow-only workspace: keeps the allocation (and its contents) when it is already large enough
+    void reserve(size_t b) { if (b > bytes) alloc(b); }
     ~DevBuf() { release(); }
     DevBuf() {}
     DevBuf(const DevBuf&) = delete;
@@ -95,6 +97,7 @@ struct TSHipGpt {
     // decode state
     DevBuf x, xn, o, a, part_qkv, part_h, part_f, logits, ids, d_pos, hidden;
     DevBuf moe_ws, topp_scratch, topp_uni, gen_buf, uni_buf, tile_count;
+    DevBuf pw_ids, pw_x, pw_xn, pw_qkv, pw_o, pw_a, pw_f, pw_rowmap, pw_ssq, pw_rinv, pw_zero_bias;     // prefill workspace
     DevBuf ssq;                    // deferred-norm path: per-column-tile sums of squares [h/32][Bpad]
     bool fused_norm = false;       // fp16 + RMSNorm + dense layers: residual/norm folded into the GEMM tails
     bool vt = false;               // fp16 cache with head_dim 64/128: keys and values stored fragment-major for the MFMA attention kernels
@@ -650,16 +653,17 @@ static void prefill(TSHipGpt* m, const int32_t* host_ids, int B, int Tp) {
     const long qp = round_up(m->Nqkv, 32);
     TSHIP_REQUIRE(m->pos == 0, "TSHip_GptPrefill: the cache is not empty; call TSHip_GptReset first");
     TSHIP_REQUIRE(Tp >= 1 && Tp < c.max_seq_len, "TSHip_GptPrefill: prompt length exceeds max_seq_len");
-    DevBuf ids, px, pxn, pqkv, po, pa, pf, rowmap;
-    ids.alloc(R * sizeof(int));
+    // prefill workspace: kept in the model and only ever grown, so that repeated prefills do not pay for allocation
+    DevBuf &ids = m->pw_ids, &px = m->pw_x, &pxn = m->pw_xn, &pqkv = m->pw_qkv, &po = m->pw_o, &pa = m->pw_a, &pf = m->pw_f, &rowmap = m->pw_rowmap;
+    ids.reserve(R * sizeof(int));
     TSHIP_CHECK_HIP(hipMemcpyAsync(ids.p, host_ids, R * sizeof(int), hipMemcpyHostToDevice, stream()));
-    px.alloc((size_t)Rp * h * sizeof(float));
-    pxn.alloc((size_t)Rp * m->ldh * m->esz());
-    pqkv.alloc((size_t)Rp * qp * sizeof(float));
-    po.alloc((size_t)Rp * m->ldh * m->esz());
+    px.reserve((size_t)Rp * h * sizeof(float));
+    pxn.reserve((size_t)Rp * m->ldh * m->esz());
+    pqkv.reserve((size_t)Rp * qp * sizeof(float));
+    po.reserve((size_t)Rp * m->ldh * m->esz());
     bool any_dense = false; for (auto& L : m->L) any_dense = any_dense || !L->moe;
-    if (any_dense) pa.alloc((size_t)Rp * m->ldF * m->esz());
-    if (!m->f16 && any_dense) pf.alloc((size_t)Rp * m->F13 * sizeof(float));
+    if (any_dense) pa.reserve((size_t)Rp * m->ldF * m->esz());
+    if (!m->f16 && any_dense) pf.reserve((size_t)Rp * m->F13 * sizeof(float));
 
     ResidNormArgs rn; std::memset(&rn, 0, sizeof(rn));
     rn.x = px.as<float>(); rn.ldx = h; rn.h = h; rn.eps = c.norm_eps; rn.norm_type = c.norm_type;
@@ -669,14 +673,14 @@ static void prefill(TSHipGpt* m, const int32_t* host_ids, int B, int Tp) {
     // 1 / rms, and the consuming GEMMs scale their output rows by it.
     const bool deferred = m->fused_norm && R >= 512;
     const int NTh = (int)(round_up(h, 32) / 32);
-    DevBuf pssq, prinv;
+    DevBuf &pssq = m->pw_ssq, &prinv = m->pw_rinv;
     auto make_rinv = [&](const char* name) {
         launch(m, name, rinv_rows_kernel, dim3((unsigned)ceil_div(R, 256)), dim3(256), (const float*)pssq.as<float>(), NTh, R, 1.0f / (float)h,
                c.norm_eps, prinv.as<float>(), R);
     };
     if (deferred) {
-        pssq.alloc((size_t)NTh * R * sizeof(float));
-        prinv.alloc((size_t)R * sizeof(float));
+        pssq.reserve((size_t)NTh * R * sizeof(float));
+        prinv.reserve((size_t)R * sizeof(float));
         FnPrepArgs a; std::memset(&a, 0, sizeof(a));
         a.x = px.as<float>(); a.ldx = h; a.h = h;
         a.ids = ids.as<int>(); a.emb = m->emb.p; a.emb_f16 = m->f16; a.emb_scale = (float)std::sqrt((double)h);
@@ -718,7 +722,7 @@ static void prefill(TSHipGpt* m, const int32_t* host_ids, int B, int Tp) {
         else if (epi == BEPI_RESID) launch(m, name, big_gemm_f16_kernel<BEPI_RESID>, grid, dim3(256), e);
         else launch(m, name, big_gemm_f16_kernel<BEPI_ACT16>, grid, dim3(256), e);
     };
-    DevBuf zero_bias; zero_bias.alloc((size_t)std::max<long>(std::max<long>(qp, m->F13), round_up(h, 32)) * sizeof(float));
+    DevBuf& zero_bias = m->pw_zero_bias; zero_bias.reserve((size_t)std::max<long>(std::max<long>(qp, m->F13), round_up(h, 32)) * sizeof(float));
     for (int l = 0; l < c.n_layers; ++l) {
         LayerW& L = *m->L[l];
         AttnArgs aa = attn_args(m, L);
@@ -779,7 +783,7 @@ static void prefill(TSHipGpt* m, const int32_t* host_ids, int B, int Tp) {
     // last position of every sequence (Decoder.cs:705-716) -> final norm -> vocabulary projection
     std::vector<int> map(B);
     for (int b = 0; b < B; ++b) map[b] = Tp * (b + 1) - 1;
-    rowmap.alloc(B * sizeof(int));
+    rowmap.reserve(B * sizeof(int));
     TSHIP_CHECK_HIP(hipMemcpyAsync(rowmap.p, map.data(), B * sizeof(int), hipMemcpyHostToDevice, stream()));
     if (m->fused_norm) {
         FnPrepArgs a; std::memset(&a, 0, sizeof(a));
