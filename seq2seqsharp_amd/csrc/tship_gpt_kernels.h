@@ -144,11 +144,33 @@ __global__ __launch_bounds__(NW * 64) void skinny_gemm_f16_kernel(SkinnyArgs a) 
     __shared__ float srinv[BT * 32];
     constexpr int NCH = (NW * 64) / (BT * 32);
     __shared__ float schunk[NCH][BT * 32];
-    float ssq_part = 0.0f;
+    // (a chunk's tail beyond four tiles is added here, one dependent load after the other; its first four sums stay in
+    // registers until the weight stream has been requested, so that their latency hides behind it)
+    float ssq_part = 0.0f, ssq_v[4] = {0.0f, 0.0f, 0.0f, 0.0f};
     if (a.ssq) {
         const int b = threadIdx.x % (BT * 32), ch = threadIdx.x / (BT * 32);
         const int per_ch = (a.ssq_nt + NCH - 1) / NCH;
-        for (int t = ch * per_ch; t < min(a.ssq_nt, (ch + 1) * per_ch); ++t) ssq_part += a.ssq[(long)t * a.ssq_ld + b];
+        const int t0 = ch * per_ch, t1 = min(a.ssq_nt, t0 + per_ch);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) if (t0 + i < t1) ssq_v[i] = a.ssq[(long)(t0 + i) * a.ssq_ld + b];
+        if (per_ch > 4) {
+            ssq_part = ((ssq_v[0] + ssq_v[1]) + ssq_v[2]) + ssq_v[3];
+            ssq_v[0] = ssq_v[1] = ssq_v[2] = ssq_v[3] = 0.0f;
+            for (int t = t0 + 4; t < t1; ++t) ssq_part += a.ssq[(long)t * a.ssq_ld + b];
+        }
+    }
+    // bias of this thread's outputs in the one-round activation epilogue
+    float eb1 = 0.0f, eb2 = 0.0f;
+    if (ONE_ROUND && EPI == EPI_ACT16) {
+        const int n1 = 8 * (w >> 2) + 4 * (lane >> 5) + (w & 3);
+        if (a.gated) {
+            const int f = nt * 16 + n1;
+            if (f < a.n_valid) { eb1 = a.bias[f]; eb2 = a.bias2[f]; }
+        } else {
+            const int f = nt * 32 + n1;
+            if (f < a.n_valid) eb1 = a.bias[f];
+            if (f + 16 < a.n_valid) eb2 = a.bias[f + 16];
+        }
     }
     // residual tail: the old residual, bias and gamma of this thread's outputs do not depend on the product
     constexpr int ITER = BT * 1024 / (NW * 64);
@@ -190,6 +212,7 @@ __global__ __launch_bounds__(NW * 64) void skinny_gemm_f16_kernel(SkinnyArgs a) 
     // rinv per row from the tile sums: NCH chunks of tiles are added in parallel (loads issued before the weight
     // stream, see above), then the chunk sums in order
     if (a.ssq) {
+        ssq_part = (((ssq_part + ssq_v[0]) + ssq_v[1]) + ssq_v[2]) + ssq_v[3];
         schunk[threadIdx.x / (BT * 32)][threadIdx.x % (BT * 32)] = ssq_part;
         __syncthreads();
         if (threadIdx.x < BT * 32) {
@@ -255,7 +278,7 @@ __global__ __launch_bounds__(NW * 64) void skinny_gemm_f16_kernel(SkinnyArgs a) 
             if (a.gated) {
                 const int f = nt * 16 + n1;
                 if (rok && f < a.n_valid) {
-                    const float val = act_apply(a.act, s1 * rinv + a.bias[f]) * (s2 * rinv + a.bias2[f]);
+                    const float val = act_apply(a.act, s1 * rinv + eb1) * (s2 * rinv + eb2);
                     if (a.out16_kt > 0) a.out16[xpack_index(b, f, a.out16_kt)] = (half_t)val;
                     else a.out16[(long)b * a.ld16 + f] = (half_t)val;
                 }
@@ -264,7 +287,7 @@ __global__ __launch_bounds__(NW * 64) void skinny_gemm_f16_kernel(SkinnyArgs a) 
                 for (int q = 0; q < 2; ++q) {
                     const int f = nt * 32 + n1 + 16 * q;
                     if (rok && f < a.n_valid) {
-                        const float val = act_apply(a.act, (q ? s2 : s1) * rinv + a.bias[f]);
+                        const float val = act_apply(a.act, (q ? s2 : s1) * rinv + (q ? eb2 : eb1));
                         if (a.out16_kt > 0) a.out16[xpack_index(b, f, a.out16_kt)] = (half_t)val;
                         else a.out16[(long)b * a.ld16 + f] = (half_t)val;
                     }
