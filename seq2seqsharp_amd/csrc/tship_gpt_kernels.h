@@ -190,7 +190,26 @@ __global__ __launch_bounds__(NW * 64) void skinny_gemm_f16_kernel(SkinnyArgs a) 
     }
     const half_t* wp = a.W + ((long)nt * a.KT * 64 + lane) * 8;
     const half_t* xp = a.X + lane * 8;
-    for (int kt = wk0; kt < wk1; kt += U) {
+    // Full batches of U k-tiles run without conditions: a request under a condition of its own would make every
+    // later wait cover all requests, and the products could not start while the batch is still arriving.
+    int kt = wk0;
+    for (; kt + U <= wk1; kt += U) {
+        half8 wf[U];
+        half8 xf[U][BT];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            wf[u] = *(const half8*)(wp + (long)(kt + u) * 512);
+#pragma unroll
+            for (int bt = 0; bt < BT; ++bt) xf[u][bt] = *(const half8*)(xp + ((long)bt * a.KT + kt + u) * 512);
+        }
+        __builtin_amdgcn_sched_barrier(0);       // all requests of the batch go out before its first product
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+            for (int bt = 0; bt < BT; ++bt) acc[bt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf[u], xf[u][bt], acc[bt], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    if (kt < wk1) {
         half8 wf[U];
         half8 xf[U][BT];
 #pragma unroll
