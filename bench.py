@@ -98,6 +98,8 @@ def main():
 
     # prefill (timed separately)
     _log("prefill of %d x %d tokens" % (B, Tp))
+    if not args.no_topp:
+        gpu.set_repeat_penalty(2.0)        # DecodingOptions.RepeatPenalty's default; only the top-p leg below applies it
     gpu.prefill(prompts)                   # untimed: loads every kernel and sizes the prefill workspace
     gpu.reset()
     t0 = time.perf_counter()
@@ -176,7 +178,7 @@ def main():
         _log("top-p decode")
         u = synth.make_uniforms(7, B, K)
         _, ms_p = gpu.generate(K, mode=TOPP, top_p=0.9, temperature=1.0, uniforms=u)
-        out["topp"] = {"top_p": 0.9, "tokens_per_s": round(B * K / (ms_p / 1e3), 1), "ms_per_step": round(ms_p / K, 4)}
+        out["topp"] = {"top_p": 0.9, "repeat_penalty": 2.0, "tokens_per_s": round(B * K / (ms_p / 1e3), 1), "ms_per_step": round(ms_p / K, 4)}
     if not args.no_cpu_baseline:
         _log("CPU baseline (one decode step of the oracle, single thread)")
         nxt = gpu.sample()

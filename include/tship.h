@@ -107,9 +107,14 @@ TSHIP_API int TSHip_BuildSelfTriMask(const TSHipTensor* result, const TSHipTenso
 TSHIP_API int TSHip_IsCorrupted(const TSHipTensor* src, int* corrupted);
 
 /* Top-p sampling on the device, one row per sequence; semantics of ComputeGraphTensor.TopPSample
- * (Seq2SeqSharp/Tools/ComputeGraphTensor.cs:2305-2403) with repeatPenalty = 0 and the random draw of row i
- * replaced by uniforms[i].  probs [rows, K] f32, uniforms [rows] f32, result [rows,1] f32 (float indices). */
+ * (Seq2SeqSharp/Tools/ComputeGraphTensor.cs:2305-2403) with the random draw of row i replaced by uniforms[i].
+ * probs [rows, K] f32, uniforms [rows] f32, result [rows,1] f32 (float indices).
+ * TSHip_TopPSample: decodedSequences = null (no decay).
+ * TSHip_TopPSampleEx: decodedSequences given as host_seqs [rows][seq_ld] int32 with host_seq_lens [rows]; a token that
+ * occurs in its row's sequence is decayed by pow(dist / len, repeat_penalty) (:2320-2345; the reference's default is 2). */
 TSHIP_API int TSHip_TopPSample(const TSHipTensor* result, const TSHipTensor* probs, const TSHipTensor* uniforms, float top_p);
+TSHIP_API int TSHip_TopPSampleEx(const TSHipTensor* result, const TSHipTensor* probs, const TSHipTensor* uniforms, float top_p, float repeat_penalty,
+                                 const int32_t* host_seqs, const int32_t* host_seq_lens, int seq_ld);
 
 /* ---- fused GPTDecoder path: one object per model replica, preallocated compact KV cache, the whole
  *      token loop on the device (replaces GPT.RunForwardOnSingleDevice, Seq2SeqSharp/Applications/GPT.cs:212-335,
@@ -147,6 +152,11 @@ TSHIP_API int TSHip_GptReset(TSHipGpt* m);
 TSHIP_API int TSHip_GptPrefill(TSHipGpt* m, const int32_t* host_ids, int batch, int prompt_len);
 /* one decode step with the given tokens (Decoder.cs:661-678); leaves logits on the device */
 TSHIP_API int TSHip_GptDecode(TSHipGpt* m, const int32_t* host_ids, int batch);
+/* DecodingOptions.RepeatPenalty (Applications/DecodingOptions.cs:23, default 2.0 there; 0 here until set): top-p sampling
+ * decays tokens that already occur in the sequence, prompt included (Decoder.cs:761).  A non-zero value makes the model
+ * keep the last position of every token per sequence, from the next prompt on: set it before TSHip_GptPrefill (or after
+ * TSHip_GptReset).  TSHip_GptSetKV / TSHip_GptSetSeqLen do not reconstruct that history.  Greedy decoding ignores it. */
+TSHIP_API int TSHip_GptSetRepeatPenalty(TSHipGpt* m, float repeat_penalty);
 /* sampling modes */
 enum { TSHIP_GREEDY = 0, TSHIP_TOPP = 1 };
 /* choose next tokens from the logits on the device: softmax (after division by temperature when

@@ -107,6 +107,8 @@ struct TSHipGpt {
     int graph_batch = 0, graph_mode = -1; float graph_top_p = 0.0f, graph_temp = 0.0f;
     const float* graph_uniforms = nullptr; int* graph_gen = nullptr;
     int pos = 0;                   // host mirror of *d_pos
+    // repeat penalty of top-p sampling (DecodingOptions.RepeatPenalty): last sequence index of every token, per sequence
+    DevBuf last_pos; long last_ld = 0; float repeat_penalty = 0.0f; float graph_penalty = 0.0f;
     int cur_batch = 0;
     Profiler* prof = nullptr;
 
@@ -439,7 +441,15 @@ static AttnArgs attn_args(TSHipGpt* m, LayerW& L) {
 static void run_moe_ffn(TSHipGpt* m, LayerW& L, int rows, const ResidNormArgs& pre);
 static void moe_alloc(TSHipGpt* m);
 static void moe_get_routing(TSHipGpt* m, int layer, float* top_idx, float* top_val, float* probs);
-static void sample_tokens(TSHipGpt* m, int mode, float top_p, float temperature, const float* host_uniforms, const float* dev_uniforms, int B, int* gen_out, const int* d_step);
+static void sample_tokens(TSHipGpt* m, int mode, float top_p, float temperature, const float* host_uniforms, const float* dev_uniforms, int B, int* gen_out, const int* d_step, bool record);
+// tokens `d_ids` [rows][Tq] enter the sequences at indices pos0 ..: remember where each token occurred last
+static void record_history(TSHipGpt* m, const int* d_ids, int rows, int Tq, int pos0) {
+    if (!m->last_pos.p) return;
+    TSHIP_REQUIRE(rows <= m->c.max_batch && (size_t)rows * m->last_ld * sizeof(int) <= m->last_pos.bytes, "internal: token history table too small");
+    launch(m, "history", history_kernel, dim3((unsigned)ceil_div((long)rows * Tq, 256)), dim3(256), d_ids, rows, Tq, (long)Tq, pos0, (const int*)nullptr,
+           (int)m->c.vocab, m->last_pos.as<int>(), m->last_ld);
+}
+
 
 // ------------------------------------------------------------------------------------------------
 // decode step, deferred-norm form (fp16 weights, RMSNorm, dense feed-forward): 5 launches per layer.
@@ -657,6 +667,7 @@ static void prefill(TSHipGpt* m, const int32_t* host_ids, int B, int Tp) {
     DevBuf &ids = m->pw_ids, &px = m->pw_x, &pxn = m->pw_xn, &pqkv = m->pw_qkv, &po = m->pw_o, &pa = m->pw_a, &pf = m->pw_f, &rowmap = m->pw_rowmap;
     ids.reserve(R * sizeof(int));
     TSHIP_CHECK_HIP(hipMemcpyAsync(ids.p, host_ids, R * sizeof(int), hipMemcpyHostToDevice, stream()));
+    record_history(m, ids.as<int>(), B, Tp, 0);
     px.reserve((size_t)Rp * h * sizeof(float));
     pxn.reserve((size_t)Rp * m->ldh * m->esz());
     pqkv.reserve((size_t)Rp * qp * sizeof(float));
@@ -958,7 +969,23 @@ TSHIP_API int TSHip_GptReset(TSHipGpt* m) {
     m->pos = 0; m->cur_batch = 0;
     TSHIP_CHECK_HIP(hipMemsetAsync(m->d_pos.p, 0, sizeof(int), stream()));
     if (m->tile_count.p) TSHIP_CHECK_HIP(hipMemsetAsync(m->tile_count.p, 0, m->tile_count.bytes, stream()));
+    if (m->last_pos.p) TSHIP_CHECK_HIP(hipMemsetAsync(m->last_pos.p, 0xff, m->last_pos.bytes, stream()));      // -1: no token seen
     TSHIP_CHECK_HIP(hipStreamSynchronize(stream()));
+    TSHIP_END
+}
+
+TSHIP_API int TSHip_GptSetRepeatPenalty(TSHipGpt* m, float repeat_penalty) {
+    TSHIP_BEGIN
+    TSHIP_REQUIRE(m, "TSHip_GptSetRepeatPenalty: null model");
+    TSHIP_REQUIRE(std::isfinite(repeat_penalty), "TSHip_GptSetRepeatPenalty: the penalty must be finite");
+    if (repeat_penalty != 0.0f && !m->last_pos.p) {
+        TSHIP_REQUIRE(m->pos == 0, "TSHip_GptSetRepeatPenalty: sequences are under way; set the penalty before the prompt is fed or after TSHip_GptReset");
+        m->last_ld = round_up(m->c.vocab, 64);
+        m->last_pos.alloc((size_t)m->c.max_batch * m->last_ld * sizeof(int));
+        TSHIP_CHECK_HIP(hipMemsetAsync(m->last_pos.p, 0xff, m->last_pos.bytes, stream()));
+        TSHIP_CHECK_HIP(hipStreamSynchronize(stream()));
+    }
+    m->repeat_penalty = repeat_penalty;
     TSHIP_END
 }
 
@@ -978,6 +1005,7 @@ TSHIP_API int TSHip_GptPrefill(TSHipGpt* m, const int32_t* host_ids, int batch, 
             TSHIP_CHECK_HIP(hipMemcpyAsync(m->ids.p, col.data(), batch * sizeof(int), hipMemcpyHostToDevice, stream()));
             TSHIP_CHECK_HIP(hipStreamSynchronize(stream()));
             if (t == 0) TSHIP_REQUIRE(m->pos == 0, "TSHip_GptPrefill: the cache is not empty; call TSHip_GptReset first");
+            record_history(m, m->ids.as<int>(), batch, 1, m->pos);
             decode_step(m, m->ids.as<int>(), batch);
         }
         TSHIP_CHECK_HIP(hipStreamSynchronize(stream()));
@@ -998,6 +1026,7 @@ TSHIP_API int TSHip_GptDecode(TSHipGpt* m, const int32_t* host_ids, int batch) {
     for (int i = 0; i < batch; ++i) TSHIP_REQUIRE(host_ids[i] >= 0 && host_ids[i] < m->c.vocab, "TSHip_GptDecode: token id out of range");
     TSHIP_CHECK_HIP(hipMemcpyAsync(m->ids.p, host_ids, batch * sizeof(int), hipMemcpyHostToDevice, stream()));
     TSHIP_CHECK_HIP(hipStreamSynchronize(stream()));
+    record_history(m, m->ids.as<int>(), batch, 1, m->pos);
     decode_step(m, m->ids.as<int>(), batch);
     TSHIP_CHECK_HIP(hipStreamSynchronize(stream()));
     m->cur_batch = batch;
@@ -1009,7 +1038,7 @@ TSHIP_API int TSHip_GptSample(TSHipGpt* m, int mode, float top_p, float temperat
     TSHIP_REQUIRE(m && host_ids_out, "TSHip_GptSample: null argument");
     TSHIP_REQUIRE(m->cur_batch > 0, "TSHip_GptSample: no logits yet; prefill or decode first");
     const int B = m->cur_batch;
-    sample_tokens(m, mode, top_p, temperature, host_uniforms, nullptr, B, nullptr, nullptr);
+    sample_tokens(m, mode, top_p, temperature, host_uniforms, nullptr, B, nullptr, nullptr, false);
     TSHIP_CHECK_HIP(hipMemcpyAsync(host_ids_out, m->ids.p, B * sizeof(int), hipMemcpyDeviceToHost, stream()));
     TSHIP_CHECK_HIP(hipStreamSynchronize(stream()));
     TSHIP_END
@@ -1046,7 +1075,7 @@ TSHIP_API int TSHip_GptGenerate(TSHipGpt* m, int n_steps, int mode, float top_p,
         // (sample -> decode) of one step is captured once; every replay reads the position, the step counter and the
         // token ids from device memory, so identical launches walk through the sequence
         if (m->step_graph && (m->graph_batch != B || m->graph_mode != mode || m->graph_top_p != top_p || m->graph_temp != temperature ||
-                              m->graph_uniforms != uni_base || m->graph_gen != gen.as<int>())) {
+                              m->graph_uniforms != uni_base || m->graph_gen != gen.as<int>() || m->graph_penalty != m->repeat_penalty)) {
             (void)hipGraphExecDestroy(m->step_graph); m->step_graph = nullptr;
         }
         if (!m->step_graph) {
@@ -1055,7 +1084,7 @@ TSHIP_API int TSHip_GptGenerate(TSHipGpt* m, int n_steps, int mode, float top_p,
             TSHIP_CHECK_HIP(hipStreamBeginCapture(stream(), hipStreamCaptureModeThreadLocal));
             const int saved_pos = m->pos;
             try {
-                sample_tokens(m, mode, top_p, temperature, nullptr, uni_base, B, gen.as<int>(), d_step);
+                sample_tokens(m, mode, top_p, temperature, nullptr, uni_base, B, gen.as<int>(), d_step, true);
                 decode_step(m, m->ids.as<int>(), B);
             } catch (...) { hipGraph_t g2 = nullptr; (void)hipStreamEndCapture(stream(), &g2); if (g2) (void)hipGraphDestroy(g2); m->pos = saved_pos; throw; }
             m->pos = saved_pos;                    // capturing launched nothing
@@ -1064,7 +1093,7 @@ TSHIP_API int TSHip_GptGenerate(TSHipGpt* m, int n_steps, int mode, float top_p,
             (void)hipGraphDestroy(graph);
             TSHIP_CHECK_HIP(ge);
             m->graph_batch = B; m->graph_mode = mode; m->graph_top_p = top_p; m->graph_temp = temperature;
-            m->graph_uniforms = uni_base; m->graph_gen = gen.as<int>();
+            m->graph_uniforms = uni_base; m->graph_gen = gen.as<int>(); m->graph_penalty = m->repeat_penalty;
         }
     }
     hipEvent_t e0, e1;
@@ -1075,7 +1104,7 @@ TSHIP_API int TSHip_GptGenerate(TSHipGpt* m, int n_steps, int mode, float top_p,
     for (int s = 0; s < n_steps; ++s) {
         if (use_graph) { TSHIP_CHECK_HIP(hipGraphLaunch(m->step_graph, stream())); m->pos += 1; }
         else {
-            sample_tokens(m, mode, top_p, temperature, nullptr, uni_base, B, gen.as<int>(), d_step);
+            sample_tokens(m, mode, top_p, temperature, nullptr, uni_base, B, gen.as<int>(), d_step, true);
             decode_step(m, m->ids.as<int>(), B);
         }
     }
@@ -1209,6 +1238,7 @@ TSHIP_API int TSHip_GptProfileDecode(TSHipGpt* m, const int32_t* host_ids, int b
     TSHIP_CHECK_HIP(hipStreamSynchronize(stream()));
     Profiler prof;
     m->prof = &prof;
+    record_history(m, m->ids.as<int>(), batch, 1, m->pos);
     try { decode_step(m, m->ids.as<int>(), batch); } catch (...) { m->prof = nullptr; throw; }
     m->prof = nullptr;
     TSHIP_CHECK_HIP(hipStreamSynchronize(stream()));

@@ -114,11 +114,15 @@ static void run_moe_ffn(TSHipGpt* m, LayerW& L, int rows, const ResidNormArgs& p
 
 // next tokens from the logits on the device -> m->ids (and gen_out); greedy or top-p.
 // With d_step set, gen_out and dev_uniforms are bases indexed by the device step counter (graph replays).
+// record: the chosen tokens are about to be appended (generate loop), so their position enters the token history.
 static void sample_tokens(TSHipGpt* m, int mode, float top_p, float temperature, const float* host_uniforms, const float* dev_uniforms, int B,
-                          int* gen_out, const int* d_step = nullptr) {
+                          int* gen_out, const int* d_step, bool record) {
     const long Vp = round_up(m->c.vocab, 32);
+    int* last = m->last_pos.as<int>();           // null unless a repeat penalty was set
+    if (last) TSHIP_REQUIRE((size_t)B * m->last_ld * sizeof(int) <= m->last_pos.bytes && m->last_ld >= m->c.vocab, "internal: token history table too small");
     if (mode == TSHIP_GREEDY) {
-        launch(m, "greedy", greedy_kernel, dim3(B), dim3(1024), (const float*)m->logits.as<float>(), Vp, m->c.vocab, m->ids.as<int>(), gen_out, d_step);
+        launch(m, "greedy", greedy_kernel, dim3(B), dim3(1024), (const float*)m->logits.as<float>(), Vp, m->c.vocab, m->ids.as<int>(), gen_out, d_step,
+               record ? last : (int*)nullptr, m->last_ld, (const int*)m->d_pos.as<int>());
         return;
     }
     TSHIP_REQUIRE(mode == TSHIP_TOPP, "unknown sampling mode");
@@ -139,6 +143,9 @@ static void sample_tokens(TSHipGpt* m, int mode, float top_p, float temperature,
     a.next_ids = m->ids.as<int>(); a.gen_out = gen_out; a.d_step = d_step;
     // Decoder.cs:720-723 divides the logits by the temperature (fp32 division) before the softmax
     a.temperature = temperature;
+    // Decoder.cs:761: TopPSample(probs, TopP, RepeatPenalty, decodedSequences: tgtSeqs); the sequence length is the number
+    // of cached positions
+    a.repeat_penalty = m->repeat_penalty; a.last_pos = last; a.last_ld = m->last_ld; a.d_len = m->d_pos.as<int>(); a.record = record ? 1 : 0;
     topp_run(a, B, [&](const char* name, void (*kernel)(TopPArgs), dim3 grid, dim3 block, const TopPArgs& args) { launch(m, name, kernel, grid, block, args); });
 }
 

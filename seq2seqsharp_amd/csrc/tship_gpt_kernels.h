@@ -1795,8 +1795,11 @@ __global__ __launch_bounds__(D == 128 ? 256 : 512) void attn_mfma_prefill_kernel
 // ------------------------------------------------------------------------------------------------
 // Greedy: argmax over a row of logits, lowest index among equal maxima (TensorApplyCPU.cs:339-360 applied to the
 // softmax output; softmax is monotone, so the winner is the same up to ties created by rounding of the division).
+// last_pos (optional): table [rows][last_ld] of the last sequence index of every token; the chosen token is recorded
+// at index *d_len (the sequence length before it is appended).
 __global__ __launch_bounds__(1024) void greedy_kernel(const float* __restrict__ logits, long ld, int V, int* __restrict__ next_ids,
-                                                      int* __restrict__ gen_out, const int* __restrict__ d_step) {
+                                                      int* __restrict__ gen_out, const int* __restrict__ d_step,
+                                                      int* __restrict__ last_pos, long last_ld, const int* __restrict__ d_len) {
     __shared__ float sv[16];
     __shared__ int si[16];
     const int b = blockIdx.x, t = threadIdx.x;
@@ -1821,6 +1824,7 @@ __global__ __launch_bounds__(1024) void greedy_kernel(const float* __restrict__ 
         if (bi == 0x7fffffff) bi = 0;   // a row of NaNs: the reference's scan never moves off index 0
         next_ids[b] = bi;
         if (gen_out) gen_out[(d_step ? (long)*d_step * gridDim.x : 0) + b] = bi;
+        if (last_pos) last_pos[(long)b * last_ld + bi] = *d_len;
     }
 }
 

@@ -626,31 +626,69 @@ TSHIP_API int TSHip_IsCorrupted(const TSHipTensor* src, int* corrupted) {
     TSHIP_END
 }
 
-TSHIP_API int TSHip_TopPSample(const TSHipTensor* result, const TSHipTensor* probs, const TSHipTensor* uniforms, float top_p) {
+static int topp_sample_op(const char* who, const TSHipTensor* result, const TSHipTensor* probs, const TSHipTensor* uniforms, float top_p,
+                          float repeat_penalty, const int32_t* host_seqs, const int32_t* host_seq_lens, int seq_ld) {
     TSHIP_BEGIN
     ensure_init();
-    View r = make_view(result, "TSHip_TopPSample"), p = make_view(probs, "TSHip_TopPSample"), u = make_view(uniforms, "TSHip_TopPSample");
+    View r = make_view(result, who), p = make_view(probs, who), u = make_view(uniforms, who);
     TSHIP_REQUIRE(p.nd == 2 && p.dtype == TSHIP_F32 && p.st[1] == 1, "TSHip_TopPSample: probs must be a Float32 matrix with contiguous rows");
     const long rows = p.sz[0], K = p.sz[1];
     TSHIP_REQUIRE(K >= 1 && K <= 65535, "TSHip_TopPSample: between 1 and 65535 columns are supported");
     TSHIP_REQUIRE(count(r) == rows && r.dtype == TSHIP_F32 && is_contiguous(r), "TSHip_TopPSample: result must be a contiguous Float32 [rows,1] tensor");
     TSHIP_REQUIRE(count(u) == rows && u.dtype == TSHIP_F32 && is_contiguous(u), "TSHip_TopPSample: uniforms must be a contiguous Float32 [rows] tensor");
+    TSHIP_REQUIRE(std::isfinite(repeat_penalty), "TSHip_TopPSampleEx: the penalty must be finite");
     if (rows == 0) return 1;
-    void* scratch = nullptr;
-    TSHIP_CHECK_HIP(hipMalloc(&scratch, topp_scratch_bytes(rows, K)));
+    const bool decay = host_seqs != nullptr && repeat_penalty != 0.0f;
+    if (decay) {
+        TSHIP_REQUIRE(host_seq_lens && seq_ld >= 1, "TSHip_TopPSampleEx: sequences need their lengths and a row stride");
+        for (long i = 0; i < rows; ++i) TSHIP_REQUIRE(host_seq_lens[i] >= 0 && host_seq_lens[i] <= seq_ld, "TSHip_TopPSampleEx: sequence length out of range");
+    }
+    const long last_ld = round_up(K, 64);
+    const size_t sort_bytes = round_up((long)topp_scratch_bytes(rows, K), 256);
+    const size_t last_bytes = decay ? (size_t)rows * last_ld * sizeof(int) : 0;
+    const size_t seq_bytes = decay ? round_up((long)((size_t)rows * seq_ld * sizeof(int)), 256) : 0, len_bytes = decay ? round_up(rows * (long)sizeof(int), 256) : 0;
+    char* scratch = nullptr;
+    TSHIP_CHECK_HIP(hipMalloc((void**)&scratch, sort_bytes + last_bytes + seq_bytes + len_bytes));
     TopPArgs a; std::memset(&a, 0, sizeof(a));
     a.in = (const float*)p.p; a.ld = p.st[0]; a.V = (int)K; a.in_is_logits = 0; a.temperature = 1.0f;
     a.uniforms = (const float*)u.p; a.top_p = top_p;
     topp_carve(a, scratch, rows, K);
     a.out_f32 = (float*)r.p;
-    topp_run(a, (int)rows, [&](const char*, void (*kernel)(TopPArgs), dim3 grid, dim3 block, const TopPArgs& args) {
-        hipLaunchKernelGGL(kernel, grid, block, 0, stream(), args);
-    });
-    hipError_t e = hipGetLastError();
-    if (e == hipSuccess) e = hipStreamSynchronize(stream());
+    hipError_t e = hipSuccess;
+    if (decay) {
+        // tokens outside [0, K) can never be candidates; the history kernel skips them
+        int* last = (int*)(scratch + sort_bytes); int* d_seqs = (int*)(scratch + sort_bytes + last_bytes); int* d_lens = (int*)(scratch + sort_bytes + last_bytes + seq_bytes);
+        e = hipMemsetAsync(last, 0xff, last_bytes, stream());
+        if (e == hipSuccess) e = hipMemcpyAsync(d_seqs, host_seqs, (size_t)rows * seq_ld * sizeof(int), hipMemcpyHostToDevice, stream());
+        if (e == hipSuccess) e = hipMemcpyAsync(d_lens, host_seq_lens, (size_t)rows * sizeof(int), hipMemcpyHostToDevice, stream());
+        if (e == hipSuccess) {
+            hipLaunchKernelGGL(history_kernel, dim3((unsigned)ceil_div(rows * (long)seq_ld, 256)), dim3(256), 0, stream(), (const int*)d_seqs, (int)rows, seq_ld, (long)seq_ld, 0,
+                               (const int*)d_lens, (int)K, last, last_ld);
+            e = hipGetLastError();
+        }
+        a.repeat_penalty = repeat_penalty; a.last_pos = last; a.last_ld = last_ld; a.row_lens = d_lens;
+    }
+    if (e == hipSuccess) {
+        topp_run(a, (int)rows, [&](const char*, void (*kernel)(TopPArgs), dim3 grid, dim3 block, const TopPArgs& args) {
+            hipLaunchKernelGGL(kernel, grid, block, 0, stream(), args);
+        });
+        e = hipGetLastError();
+    }
+    // (the host arrays must stay valid until the copies are done: synchronise before returning in every case)
+    hipError_t es = hipStreamSynchronize(stream());
+    if (e == hipSuccess) e = es;
     (void)hipFree(scratch);
     TSHIP_CHECK_HIP(e);
     TSHIP_END
+}
+
+TSHIP_API int TSHip_TopPSample(const TSHipTensor* result, const TSHipTensor* probs, const TSHipTensor* uniforms, float top_p) {
+    return topp_sample_op("TSHip_TopPSample", result, probs, uniforms, top_p, 0.0f, nullptr, nullptr, 0);
+}
+
+TSHIP_API int TSHip_TopPSampleEx(const TSHipTensor* result, const TSHipTensor* probs, const TSHipTensor* uniforms, float top_p, float repeat_penalty,
+                                 const int32_t* host_seqs, const int32_t* host_seq_lens, int seq_ld) {
+    return topp_sample_op("TSHip_TopPSampleEx", result, probs, uniforms, top_p, repeat_penalty, host_seqs, host_seq_lens, seq_ld);
 }
 
 }  // extern "C"

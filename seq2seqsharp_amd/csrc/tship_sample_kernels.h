@@ -1,9 +1,13 @@
 // Top-p sampling on the device.
-// Semantics of ComputeGraphTensor.TopPSample (Seq2SeqSharp/Tools/ComputeGraphTensor.cs:2305-2403) with
-// repeatPenalty = 0 (pow(x, 0) = 1: no decay) and the per-row random draw supplied by the caller:
-//   keep p > 0; order by p descending, equal p by ascending index (SortedDictionary<float, List<int>> walked in
-//   reverse, each list in insertion order); running fp32 sum in that order, stop after the element that makes
-//   acc >= topP; pick the first k with accP[k] / acc >= u.
+// Semantics of ComputeGraphTensor.TopPSample (Seq2SeqSharp/Tools/ComputeGraphTensor.cs:2305-2403) with the per-row
+// random draw supplied by the caller:
+//   keep p > 0; a token that occurs in the row's sequence so far is decayed,
+//   p = (float)(p * (float)pow((float)dist / (float)len, repeatPenalty)), dist = len - (index of its last occurrence)
+//   (:2320-2345; the sequence is prompt + generated tokens, Decoder.cs:761); order by p descending, equal p by
+//   ascending index (SortedDictionary<float, List<int>> walked in reverse, each list in insertion order); running
+//   fp32 sum in that order, stop after the element that makes acc >= topP; pick the first k with accP[k] / acc >= u.
+// The last occurrence of every token is kept in a table [rows][vocabulary] (-1: not in the sequence) that the
+// caller maintains (history_kernel for given tokens; the pick and greedy kernels record the token they choose).
 // The order is produced by a stable least-significant-digit radix sort on the float bit pattern (four passes of
 // eight bits, every pass = histogram, scan, scatter over segments of 1024 elements, so a row is sorted by many
 // blocks); the running sum is taken serially in fp32 by one wavefront, so for given probabilities the chosen index
@@ -27,7 +31,24 @@ struct TopPArgs {
     int shift;                             // digit of the current sort pass
     int* next_ids; int* gen_out; float* out_f32;   // any of them may be null
     const int* d_step;                             // optional: uniforms and gen_out are indexed by *d_step * rows + row
+    // repeat penalty (0: none).  last_pos [rows][last_ld]; the row's sequence length is row_lens[row], else *d_len,
+    // else len.  record != 0: the pick kernel stores the chosen token's index (= that length) into the table.
+    float repeat_penalty; int* last_pos; long last_ld; const int* row_lens; const int* d_len; int len; int record;
 };
+
+__device__ __forceinline__ int topp_seq_len(const TopPArgs& a, int r) { return a.row_lens ? a.row_lens[r] : (a.d_len ? *a.d_len : a.len); }
+
+// last occurrence of every token of `ids` [rows][Tq] (sequence indices pos0 .. pos0 + Tq - 1, or fewer per row when
+// row_lens is given): grid (ceil(rows Tq / 256)), 256 threads
+static __global__ __launch_bounds__(256) void history_kernel(const int* __restrict__ ids, int rows, int Tq, long ld_ids, int pos0, const int* __restrict__ row_lens,
+                                                             int V, int* __restrict__ last_pos, long last_ld) {
+    const long idx = (long)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= (long)rows * Tq) return;
+    const int r = (int)(idx / Tq), j = (int)(idx % Tq);
+    if (row_lens && j >= row_lens[r]) return;
+    const int tok = ids[(long)r * ld_ids + j];
+    if (tok >= 0 && tok < V) atomicMax(&last_pos[(long)r * last_ld + tok], pos0 + j);
+}
 
 inline size_t topp_scratch_bytes(long rows, long V) {
     const long Vs = round_up(V, 64), nseg = ceil_div(V, (long)TOPP_SEG);
@@ -84,8 +105,20 @@ static __global__ __launch_bounds__(1024) void topp_keys_kernel(TopPArgs a) {
 #pragma unroll
         for (int i = 0; i < 16; ++i) sum += sred[i];
     }
+    const bool decay = a.last_pos && a.repeat_penalty != 0.0f;
+    const int len = decay ? topp_seq_len(a, r) : 0;
+    const int* last = decay ? a.last_pos + (long)r * a.last_ld : nullptr;
     for (int i = t; i < V; i += 1024) {
-        const float p = a.in_is_logits ? expf(row[i] / a.temperature - mx) / sum : row[i];
+        float p = a.in_is_logits ? expf(row[i] / a.temperature - mx) / sum : row[i];
+        if (decay && p > 0.0f) {
+            const int lp = last[i];
+            if (lp >= 0) {
+                // float division, double pow, one rounding to float, one fp32 multiply (ComputeGraphTensor.cs:2341-2342)
+                const float ratio = (float)(len - lp) / (float)len;
+                const float rp = (float)pow((double)ratio, (double)a.repeat_penalty);
+                p = p * rp;      // (a product that underflows to 0 stays a candidate of weight 0 there; it can never be picked)
+            }
+        }
         // p > 0: positive floats order like their bit patterns; descending order = ascending ~bits.
         // p <= 0 is dropped by the reference: give it the largest key so that it sorts behind every candidate.
         kA[i] = p > 0.0f ? ~__float_as_uint(p) : 0xffffffffu;
@@ -293,6 +326,7 @@ static __global__ __launch_bounds__(64) void topp_pick_kernel(TopPArgs a) {
         if (a.next_ids) a.next_ids[r] = id;
         if (a.gen_out) a.gen_out[slot] = id;
         if (a.out_f32) a.out_f32[r] = (float)id;
+        if (a.record && a.last_pos) a.last_pos[(long)r * a.last_ld + id] = topp_seq_len(a, r);     // the new token's index
     }
 }
 

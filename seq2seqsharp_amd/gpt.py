@@ -31,6 +31,7 @@ def _protos():
     L.TSHip_GptPrefill.argtypes = [vp, vp, C.c_int, C.c_int]
     L.TSHip_GptDecode.argtypes = [vp, vp, C.c_int]
     L.TSHip_GptSample.argtypes = [vp, C.c_int, C.c_float, C.c_float, vp, vp]
+    L.TSHip_GptSetRepeatPenalty.argtypes = [vp, C.c_float]
     L.TSHip_GptGenerate.argtypes = [vp, C.c_int, C.c_int, C.c_float, C.c_float, vp, vp, C.POINTER(C.c_float)]
     L.TSHip_GptGetLogits.argtypes = [vp, vp]
     L.TSHip_GptGetHidden.argtypes = [vp, vp]
@@ -102,6 +103,10 @@ class HipGpt:
         ids = np.ascontiguousarray(ids, dtype=np.int32).reshape(-1)
         check(lib().TSHip_GptDecode(self.h, _ptr(ids), ids.size))
         self.batch = ids.size
+
+    def set_repeat_penalty(self, repeat_penalty):
+        """DecodingOptions.RepeatPenalty for top-p sampling (the reference's default is 2.0); set before the prompt is fed."""
+        check(lib().TSHip_GptSetRepeatPenalty(self.h, float(repeat_penalty)))
 
     def sample(self, mode=GREEDY, top_p=0.0, temperature=1.0, uniforms=None):
         out = np.empty((self.batch,), np.int32)

@@ -44,6 +44,7 @@ def _p():
     L.TSHip_BuildSelfTriMask.argtypes = [T, T, C.c_int, C.c_float, C.c_float]
     L.TSHip_IsCorrupted.argtypes = [T, C.POINTER(C.c_int)]
     L.TSHip_TopPSample.argtypes = [T, T, T, C.c_float]
+    L.TSHip_TopPSampleEx.argtypes = [T, T, T, C.c_float, C.c_float, C.c_void_p, C.c_void_p, C.c_int]
     _ok = True
     return L
 
@@ -239,9 +240,17 @@ def iscorrupted(src):                                    # "iscorrupted"
     return bool(flag.value)
 
 
-def toppsample(result, probs, uniforms, top_p):
+def toppsample(result, probs, uniforms, top_p, repeat_penalty=0.0, seqs=None, seq_lens=None):
+    """ComputeGraphTensor.TopPSample (Seq2SeqSharp/Tools/ComputeGraphTensor.cs:2305-2403); `seqs` = decodedSequences as an
+    int32 array [rows, max_len] (with `seq_lens` [rows] when the rows differ in length), None = no decay."""
     r = _target(result, [probs.sizes[0], 1], F32)
-    check(_p().TSHip_TopPSample(_d(r), _d(probs), _d(uniforms), float(top_p)))
+    if seqs is None:
+        check(_p().TSHip_TopPSample(_d(r), _d(probs), _d(uniforms), float(top_p)))
+        return r
+    seqs = np.ascontiguousarray(seqs, dtype=np.int32)
+    lens = np.full((seqs.shape[0],), seqs.shape[1], np.int32) if seq_lens is None else np.ascontiguousarray(seq_lens, dtype=np.int32)
+    check(_p().TSHip_TopPSampleEx(_d(r), _d(probs), _d(uniforms), float(top_p), float(repeat_penalty),
+                                  seqs.ctypes.data_as(C.c_void_p), lens.ctypes.data_as(C.c_void_p), int(seqs.shape[1])))
     return r
 
 

@@ -289,6 +289,55 @@ def test_topp_stream_matches_oracle(G, oracle):
     gpu.close()
 
 
+@pytest.mark.parametrize("moe", [False, True])
+def test_topp_repeat_penalty_matches_oracle(G, oracle, moe):
+    """Decoder.cs:761 hands TopPSample the sequences so far (prompt + generated) and DecodingOptions.RepeatPenalty
+    (default 2): the device keeps the last position of every token and decays on the fly.  Graph loop, the stepwise
+    calls and the token-by-token prompt path of MoE models must all see the same history."""
+    from seq2seqsharp_amd._lib import TSHipError
+    kw = dict(n_layers=3, n_experts=4, experts_per_token=2, norm_type=synth.LAYERNORM, act=synth.RELU) if moe else {}
+    cfg = synth.tiny_config(vocab=300, batch=4, **kw)
+    w = synth.make_weights(cfg, 31, random_bias=True)
+    orc = oracle.OracleGpt(cfg, w)
+    gpu = G.HipGpt(cfg, w, max_batch=4, max_seq_len=64)
+    seqs = synth.make_prompts(cfg, 32)
+    seqs[:, 3] = seqs[:, 1]                                             # repeats inside the prompt
+    u = synth.make_uniforms(33, 4, 12)
+    gpu.set_repeat_penalty(2.0)
+    gpu.prefill(seqs)
+    late = G.HipGpt(cfg, w, max_batch=4, max_seq_len=64)
+    late.prefill(seqs)
+    with pytest.raises(TSHipError, match="under way"):                  # the history cannot start in the middle of a sequence
+        late.set_repeat_penalty(2.0)
+    late.close()
+    ids, _ = gpu.generate(8, mode=G.TOPP, top_p=0.95, temperature=1.0, uniforms=u[:8])
+    cur = seqs
+    want = []
+    for s in range(12):
+        p, _ = orc.step(cur, use_cache=True, sampling=True)
+        nxt = oracle.toppsample(p, 0.95, 2.0, cur, u[s]).astype(np.int32)
+        want.append(nxt)
+        cur = np.concatenate([cur, nxt[:, None]], 1)
+    want = np.stack(want)
+    assert np.array_equal(ids, want[:8])
+    # the penalty matters on this input
+    orc.reset()
+    p0, _ = orc.step(seqs, use_cache=True, sampling=True)
+    differs = any(not np.array_equal(oracle.toppsample(p0, 0.95, 2.0, seqs, u[s]), oracle.toppsample(p0, 0.95, 0.0, None, u[s])) for s in range(12))
+    assert differs
+    # stepwise continuation: sample (no recording) then decode with the caller's tokens (recorded)
+    for s in range(8, 12):
+        t = gpu.sample(mode=G.TOPP, top_p=0.95, uniforms=u[s])
+        assert np.array_equal(t, want[s])
+        gpu.decode(t)
+    # a new prompt after reset starts from an empty history
+    gpu.reset()
+    gpu.prefill(seqs)
+    ids2, _ = gpu.generate(8, mode=G.TOPP, top_p=0.95, temperature=1.0, uniforms=u[:8])
+    assert np.array_equal(ids2, want[:8])
+    gpu.close()
+
+
 @pytest.mark.parametrize("dtype,act", [("f32", synth.RELU), ("f32", synth.SILU), ("f16", synth.RELU)])
 def test_moe_model(G, oracle, dtype, act):
     """MoE layers (layers >= 2): routing indices bit-exact on the fp32 model, logits within the dtype's bar."""

@@ -213,6 +213,37 @@ def test_toppsample_bit_exact_given_probs(T, oracle):
     assert np.array_equal(got, oracle.argmax(small))                    # topP -> 0 is greedy
 
 
+def test_toppsample_repeat_penalty(T, oracle):
+    """decodedSequences given (ComputeGraphTensor.cs:2320-2345): tokens already in the row's sequence are decayed by
+    pow(dist / len, penalty) before the sort.  Penalty 2 (the reference's default) squares exactly in double; 1.5 and
+    0.5 go through pow proper."""
+    HT, ops = T
+    rng = np.random.default_rng(11)
+    rows, K, L = 8, 5000, 40
+    p = oracle.softmax((3.0 * rng.standard_normal((rows, K))).astype(np.float32))
+    seqs = rng.integers(0, K, size=(rows, L)).astype(np.int32)
+    top = np.argsort(-p, axis=1)[:, :12]
+    seqs[:, 5:17] = top                                                 # the likeliest tokens have been generated before
+    seqs[:, 30:34] = top[:, :4]                                         # some of them twice: the last occurrence counts
+    p[2, top[2, 0]] = p[2, top[2, 1]]                                   # a tie that the decay breaks or keeps
+    u = rng.random(rows).astype(np.float32)
+    for penalty in (2.0, 1.5, 0.5):
+        for top_p in (0.3, 0.9, 1.0):
+            got = ops.toppsample(None, HT.from_numpy(p), HT.from_numpy(u), top_p, penalty, seqs).numpy().reshape(-1)
+            assert np.array_equal(got, oracle.toppsample(p, top_p, penalty, seqs, u)), (penalty, top_p)
+    # the decay changes the outcome on this input (otherwise the test would pass without it)
+    assert not np.array_equal(oracle.toppsample(p, 0.9, 2.0, seqs, u), oracle.toppsample(p, 0.9, 0.0, None, u))
+    # rows of different lengths: every row against the oracle on its own sequence; an empty sequence decays nothing
+    lens = np.array([40, 1, 0, 17, 33, 40, 2, 9], np.int32)
+    got = ops.toppsample(None, HT.from_numpy(p), HT.from_numpy(u), 0.9, 2.0, seqs, lens).numpy().reshape(-1)
+    for i in range(rows):
+        want = oracle.toppsample(p[i:i + 1], 0.9, 2.0, seqs[i:i + 1, :lens[i]] if lens[i] else None, u[i:i + 1])
+        assert got[i] == want[0], i
+    # penalty 0 with sequences = no decay (pow(x, 0) = 1)
+    got = ops.toppsample(None, HT.from_numpy(p), HT.from_numpy(u), 0.9, 0.0, seqs).numpy().reshape(-1)
+    assert np.array_equal(got, oracle.toppsample(p, 0.9, 0.0, None, u))
+
+
 def test_error_paths(T):
     HT, ops = T
     from seq2seqsharp_amd._lib import TSHipError
