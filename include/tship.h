@@ -167,6 +167,12 @@ TSHIP_API int TSHip_GptSample(TSHipGpt* m, int mode, float top_p, float temperat
  * elapsed_ms (optional): device time of the loop measured with events on the library stream. */
 TSHIP_API int TSHip_GptGenerate(TSHipGpt* m, int n_steps, int mode, float top_p, float temperature,
                                 const float* host_uniforms, int32_t* host_ids_out, float* elapsed_ms);
+/* the same loop with the reference's stop rule (GPT.cs:299-302, Decoder.AreAllSentsCompleted, Decoder.cs:207-221): stops
+ * after the first step at which every sequence's new token is eos_id (the vocabulary's END tag, 0 in the reference).
+ * *steps_done steps were run; host_ids_out [max_steps, batch] holds that many rows.  The host looks at every step's
+ * tokens, which costs one small copy and one synchronisation per step. */
+TSHIP_API int TSHip_GptGenerateUntil(TSHipGpt* m, int max_steps, int eos_id, int mode, float top_p, float temperature,
+                                     const float* host_uniforms, int32_t* host_ids_out, int* steps_done, float* elapsed_ms);
 /* inspection for parity tests */
 TSHIP_API int TSHip_GptGetLogits(TSHipGpt* m, float* host_out /* [batch, vocab] */);
 TSHIP_API int TSHip_GptGetHidden(TSHipGpt* m, float* host_out /* [batch, hidden], after the final norm */);

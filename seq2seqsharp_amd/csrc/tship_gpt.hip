@@ -1044,8 +1044,10 @@ TSHIP_API int TSHip_GptSample(TSHipGpt* m, int mode, float top_p, float temperat
     TSHIP_END
 }
 
-TSHIP_API int TSHip_GptGenerate(TSHipGpt* m, int n_steps, int mode, float top_p, float temperature,
-                                const float* host_uniforms, int32_t* host_ids_out, float* elapsed_ms) {
+// the token loop; eos_id >= 0: the host looks at every step's tokens and stops after the first step whose tokens are
+// all eos_id (Decoder.AreAllSentsCompleted, Applications/Decoder.cs:207-221, as GPT.cs:299-302 uses it)
+static int generate_impl(TSHipGpt* m, int n_steps, int mode, float top_p, float temperature, const float* host_uniforms, int32_t* host_ids_out,
+                         float* elapsed_ms, int eos_id, int* steps_done) {
     TSHIP_BEGIN
     TSHIP_REQUIRE(m && host_ids_out, "TSHip_GptGenerate: null argument");
     TSHIP_REQUIRE(m->cur_batch > 0, "TSHip_GptGenerate: no logits yet; prefill first");
@@ -1101,11 +1103,21 @@ TSHIP_API int TSHip_GptGenerate(TSHipGpt* m, int n_steps, int mode, float top_p,
     TSHIP_CHECK_HIP(hipEventCreate(&e1));
     TSHIP_CHECK_HIP(hipStreamSynchronize(stream()));
     TSHIP_CHECK_HIP(hipEventRecord(e0, stream()));
+    int done = 0;
     for (int s = 0; s < n_steps; ++s) {
         if (use_graph) { TSHIP_CHECK_HIP(hipGraphLaunch(m->step_graph, stream())); m->pos += 1; }
         else {
             sample_tokens(m, mode, top_p, temperature, nullptr, uni_base, B, gen.as<int>(), d_step, true);
             decode_step(m, m->ids.as<int>(), B);
+        }
+        done = s + 1;
+        if (eos_id >= 0) {
+            // (one small copy and a synchronisation per step: the price of looking at the tokens on the host)
+            TSHIP_CHECK_HIP(hipMemcpyAsync(host_ids_out + (size_t)s * B, gen.as<int>() + (size_t)s * B, (size_t)B * sizeof(int), hipMemcpyDeviceToHost, stream()));
+            TSHIP_CHECK_HIP(hipStreamSynchronize(stream()));
+            bool all_eos = true;
+            for (int b = 0; b < B; ++b) all_eos = all_eos && host_ids_out[(size_t)s * B + b] == eos_id;
+            if (all_eos) break;
         }
     }
     TSHIP_CHECK_HIP(hipEventRecord(e1, stream()));
@@ -1114,8 +1126,21 @@ TSHIP_API int TSHip_GptGenerate(TSHipGpt* m, int n_steps, int mode, float top_p,
     TSHIP_CHECK_HIP(hipEventElapsedTime(&ms, e0, e1));
     (void)hipEventDestroy(e0); (void)hipEventDestroy(e1);
     if (elapsed_ms) *elapsed_ms = ms;
-    TSHIP_CHECK_HIP(hipMemcpy(host_ids_out, gen.p, (size_t)n_steps * B * sizeof(int), hipMemcpyDeviceToHost));
+    if (steps_done) *steps_done = done;
+    if (eos_id < 0) TSHIP_CHECK_HIP(hipMemcpy(host_ids_out, gen.p, (size_t)n_steps * B * sizeof(int), hipMemcpyDeviceToHost));
     TSHIP_END
+}
+
+TSHIP_API int TSHip_GptGenerate(TSHipGpt* m, int n_steps, int mode, float top_p, float temperature,
+                                const float* host_uniforms, int32_t* host_ids_out, float* elapsed_ms) {
+    return generate_impl(m, n_steps, mode, top_p, temperature, host_uniforms, host_ids_out, elapsed_ms, -1, nullptr);
+}
+
+TSHIP_API int TSHip_GptGenerateUntil(TSHipGpt* m, int max_steps, int eos_id, int mode, float top_p, float temperature,
+                                     const float* host_uniforms, int32_t* host_ids_out, int* steps_done, float* elapsed_ms) {
+    if (m && (eos_id < 0 || eos_id >= m->c.vocab)) { set_last_error("TSHip_GptGenerateUntil: eos_id out of range"); return 0; }
+    if (!steps_done) { set_last_error("TSHip_GptGenerateUntil: null argument"); return 0; }
+    return generate_impl(m, max_steps, mode, top_p, temperature, host_uniforms, host_ids_out, elapsed_ms, eos_id, steps_done);
 }
 
 TSHIP_API int TSHip_GptGetLogits(TSHipGpt* m, float* host_out) {

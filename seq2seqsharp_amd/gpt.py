@@ -32,6 +32,7 @@ def _protos():
     L.TSHip_GptDecode.argtypes = [vp, vp, C.c_int]
     L.TSHip_GptSample.argtypes = [vp, C.c_int, C.c_float, C.c_float, vp, vp]
     L.TSHip_GptSetRepeatPenalty.argtypes = [vp, C.c_float]
+    L.TSHip_GptGenerateUntil.argtypes = [vp, C.c_int, C.c_int, C.c_int, C.c_float, C.c_float, vp, vp, C.POINTER(C.c_int), C.POINTER(C.c_float)]
     L.TSHip_GptGenerate.argtypes = [vp, C.c_int, C.c_int, C.c_float, C.c_float, vp, vp, C.POINTER(C.c_float)]
     L.TSHip_GptGetLogits.argtypes = [vp, vp]
     L.TSHip_GptGetHidden.argtypes = [vp, vp]
@@ -121,6 +122,16 @@ class HipGpt:
         ms = C.c_float(0.0)
         check(lib().TSHip_GptGenerate(self.h, n_steps, mode, top_p, temperature, _ptr(u), _ptr(out), C.byref(ms)))
         return out, ms.value
+
+    def generate_until(self, max_steps, eos_id, mode=GREEDY, top_p=0.0, temperature=1.0, uniforms=None):
+        """The loop of GPT.RunForwardOnSingleDevice with its stop rule: ends after the first step at which every sequence's
+        new token is `eos_id` (Decoder.AreAllSentsCompleted).  Returns (ids [steps_done, batch], device milliseconds)."""
+        out = np.empty((max_steps, self.batch), np.int32)
+        u = None if uniforms is None else np.ascontiguousarray(uniforms, dtype=np.float32)
+        ms = C.c_float(0.0)
+        done = C.c_int(0)
+        check(lib().TSHip_GptGenerateUntil(self.h, max_steps, eos_id, mode, top_p, temperature, _ptr(u), _ptr(out), C.byref(done), C.byref(ms)))
+        return out[:done.value], ms.value
 
     def logits(self):
         out = np.empty((self.batch, self.cfg["vocab"]), np.float32)

@@ -437,6 +437,47 @@ def test_head_dim_128_against_oracle(G, oracle, kv_heads, batch, prompt):
     gpu.close()
 
 
+def test_generate_until_all_rows_emit_eos(G):
+    """GPT.cs:299-302: the loop ends after the first step at which every sequence's newest token is the END tag
+    (Decoder.cs:207-221); a row that ended earlier keeps generating until then."""
+    cfg = synth.tiny_config(batch=3, vocab=50)
+    w = synth.make_weights(cfg, 41)
+    gpu = G.HipGpt(cfg, w, max_batch=3, max_seq_len=48)
+    prompts = synth.make_prompts(cfg, 42)
+    prompts[1] = prompts[0]
+    prompts[2] = prompts[0]                                             # identical rows emit identical tokens
+    gpu.prefill(prompts)
+    full, _ = gpu.generate(20)
+    assert np.array_equal(full[:, 0], full[:, 1])
+    first = {}
+    for s, tok in enumerate(full[:, 0]):
+        first.setdefault(int(tok), s)
+    eos, stop = max(first.items(), key=lambda kv: kv[1])                # the token whose first occurrence comes last
+    assert stop >= 2
+    gpu.reset()
+    gpu.prefill(prompts)
+    got, _ = gpu.generate_until(20, eos)
+    assert got.shape[0] == stop + 1 and np.array_equal(got, full[:stop + 1])
+    assert gpu.seq_len() == prompts.shape[1] + stop + 1
+    rest, _ = gpu.generate(20 - stop - 1)                               # the state is that of the uninterrupted run
+    assert np.array_equal(rest, full[stop + 1:])
+    # rows that differ: one of them emitting the tag does not end the loop
+    gpu.reset()
+    prompts2 = synth.make_prompts(cfg, 43)
+    gpu.prefill(prompts2)
+    ref, _ = gpu.generate(12)
+    col = ref[:, 0]
+    others_differ = [s for s in range(12) if not (ref[s] == col[s]).all()]
+    assert others_differ
+    s0 = others_differ[0]
+    all_same = [s for s in range(12) if (ref[s] == col[s0]).all()]
+    gpu.reset()
+    gpu.prefill(prompts2)
+    got, _ = gpu.generate_until(12, int(col[s0]))
+    assert got.shape[0] == (all_same[0] + 1 if all_same else 12) and np.array_equal(got, ref[:got.shape[0]])
+    gpu.close()
+
+
 def test_argument_errors(G):
     from seq2seqsharp_amd._lib import TSHipError
     cfg = synth.tiny_config()
