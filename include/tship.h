@@ -157,6 +157,9 @@ TSHIP_API int TSHip_GptDecode(TSHipGpt* m, const int32_t* host_ids, int batch);
  * keep the last position of every token per sequence, from the next prompt on: set it before TSHip_GptPrefill (or after
  * TSHip_GptReset).  TSHip_GptSetKV / TSHip_GptSetSeqLen do not reconstruct that history.  Greedy decoding ignores it. */
 TSHIP_API int TSHip_GptSetRepeatPenalty(TSHipGpt* m, float repeat_penalty);
+/* DecodingOptions.BlockedTokens (Decoder.cs:745-753: -1 is added to their probabilities before the choice): the tokens
+ * are never chosen, by argmax or by top-p.  n = 0 clears the list. */
+TSHIP_API int TSHip_GptSetBlockedTokens(TSHipGpt* m, const int32_t* ids, int n);
 /* sampling modes */
 enum { TSHIP_GREEDY = 0, TSHIP_TOPP = 1 };
 /* choose next tokens from the logits on the device: softmax (after division by temperature when

@@ -109,6 +109,7 @@ struct TSHipGpt {
     int pos = 0;                   // host mirror of *d_pos
     // repeat penalty of top-p sampling (DecodingOptions.RepeatPenalty): last sequence index of every token, per sequence
     DevBuf last_pos; long last_ld = 0; float repeat_penalty = 0.0f; float graph_penalty = 0.0f;
+    DevBuf blocked;                // one byte per token, non-zero = DecodingOptions.BlockedTokens (allocated with the model: graphs keep its address)
     int cur_batch = 0;
     Profiler* prof = nullptr;
 
@@ -907,6 +908,8 @@ TSHIP_API int TSHip_GptCreate(const TSHipGptConfig* cfg, TSHipGpt** out) {
     m->logits.alloc((size_t)m->Bpad * Vp * sizeof(float));
     m->ids.alloc((size_t)m->Bpad * sizeof(int));
     m->d_pos.alloc(2 * sizeof(int));      // [0] cached positions, [1] step counter of the running generate call
+    m->blocked.alloc(round_up(c.vocab, 64));
+    TSHIP_CHECK_HIP(hipMemset(m->blocked.p, 0, m->blocked.bytes));
     m->hidden.alloc((size_t)m->Bpad * h * sizeof(float));
     if (c.n_experts > 1) moe_alloc(m.get());
     m->fused_norm = m->f16 && c.norm_type == 0 && c.n_experts <= 1;
@@ -971,6 +974,19 @@ TSHIP_API int TSHip_GptReset(TSHipGpt* m) {
     if (m->tile_count.p) TSHIP_CHECK_HIP(hipMemsetAsync(m->tile_count.p, 0, m->tile_count.bytes, stream()));
     if (m->last_pos.p) TSHIP_CHECK_HIP(hipMemsetAsync(m->last_pos.p, 0xff, m->last_pos.bytes, stream()));      // -1: no token seen
     TSHIP_CHECK_HIP(hipStreamSynchronize(stream()));
+    TSHIP_END
+}
+
+TSHIP_API int TSHip_GptSetBlockedTokens(TSHipGpt* m, const int32_t* ids, int n) {
+    TSHIP_BEGIN
+    TSHIP_REQUIRE(m && (ids || n == 0) && n >= 0, "TSHip_GptSetBlockedTokens: bad argument");
+    std::vector<unsigned char> mask(m->blocked.bytes, 0);
+    for (int i = 0; i < n; ++i) {
+        TSHIP_REQUIRE(ids[i] >= 0 && ids[i] < m->c.vocab, "TSHip_GptSetBlockedTokens: token id out of range");
+        mask[ids[i]] = 1;
+    }
+    TSHIP_CHECK_HIP(hipStreamSynchronize(stream()));
+    TSHIP_CHECK_HIP(hipMemcpy(m->blocked.p, mask.data(), mask.size(), hipMemcpyHostToDevice));
     TSHIP_END
 }
 

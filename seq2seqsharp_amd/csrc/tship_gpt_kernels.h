@@ -1797,9 +1797,13 @@ __global__ __launch_bounds__(D == 128 ? 256 : 512) void attn_mfma_prefill_kernel
 // softmax output; softmax is monotone, so the winner is the same up to ties created by rounding of the division).
 // last_pos (optional): table [rows][last_ld] of the last sequence index of every token; the chosen token is recorded
 // at index *d_len (the sequence length before it is appended).
+// blocked (optional): one byte per token; the reference adds -1 to the probabilities of blocked tokens
+// (Decoder.cs:745-753), which puts them below every other token: they are left out here.  (A blocked token could
+// only win there if every other probability had underflowed to zero.)
 __global__ __launch_bounds__(1024) void greedy_kernel(const float* __restrict__ logits, long ld, int V, int* __restrict__ next_ids,
                                                       int* __restrict__ gen_out, const int* __restrict__ d_step,
-                                                      int* __restrict__ last_pos, long last_ld, const int* __restrict__ d_len) {
+                                                      int* __restrict__ last_pos, long last_ld, const int* __restrict__ d_len,
+                                                      const unsigned char* __restrict__ blocked) {
     __shared__ float sv[16];
     __shared__ int si[16];
     const int b = blockIdx.x, t = threadIdx.x;
@@ -1808,7 +1812,7 @@ __global__ __launch_bounds__(1024) void greedy_kernel(const float* __restrict__ 
     for (int i0 = t; i0 < V; i0 += 1024 * 8) {
         float v[8];
 #pragma unroll
-        for (int u = 0; u < 8; ++u) { int i = i0 + u * 1024; v[u] = i < V ? row[i] : -INFINITY; }
+        for (int u = 0; u < 8; ++u) { int i = i0 + u * 1024; v[u] = (i < V && !(blocked && blocked[i])) ? row[i] : -INFINITY; }
 #pragma unroll
         for (int u = 0; u < 8; ++u) { int i = i0 + u * 1024; if (i < V && (v[u] > best || (v[u] == best && i < bi))) { best = v[u]; bi = i; } }
     }

@@ -34,6 +34,9 @@ struct TopPArgs {
     // repeat penalty (0: none).  last_pos [rows][last_ld]; the row's sequence length is row_lens[row], else *d_len,
     // else len.  record != 0: the pick kernel stores the chosen token's index (= that length) into the table.
     float repeat_penalty; int* last_pos; long last_ld; const int* row_lens; const int* d_len; int len; int record;
+    // one byte per token, non-zero = blocked: the reference adds -1 to such a probability (Decoder.cs:745-753), so it is
+    // <= 0 and never a candidate.  May be null.
+    const unsigned char* blocked;
 };
 
 __device__ __forceinline__ int topp_seq_len(const TopPArgs& a, int r) { return a.row_lens ? a.row_lens[r] : (a.d_len ? *a.d_len : a.len); }
@@ -121,7 +124,7 @@ static __global__ __launch_bounds__(1024) void topp_keys_kernel(TopPArgs a) {
         }
         // p > 0: positive floats order like their bit patterns; descending order = ascending ~bits.
         // p <= 0 is dropped by the reference: give it the largest key so that it sorts behind every candidate.
-        kA[i] = p > 0.0f ? ~__float_as_uint(p) : 0xffffffffu;
+        kA[i] = (p > 0.0f && !(a.blocked && a.blocked[i])) ? ~__float_as_uint(p) : 0xffffffffu;
         iA[i] = i;
     }
 }

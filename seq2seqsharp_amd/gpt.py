@@ -32,6 +32,7 @@ def _protos():
     L.TSHip_GptDecode.argtypes = [vp, vp, C.c_int]
     L.TSHip_GptSample.argtypes = [vp, C.c_int, C.c_float, C.c_float, vp, vp]
     L.TSHip_GptSetRepeatPenalty.argtypes = [vp, C.c_float]
+    L.TSHip_GptSetBlockedTokens.argtypes = [vp, vp, C.c_int]
     L.TSHip_GptGenerateUntil.argtypes = [vp, C.c_int, C.c_int, C.c_int, C.c_float, C.c_float, vp, vp, C.POINTER(C.c_int), C.POINTER(C.c_float)]
     L.TSHip_GptGenerate.argtypes = [vp, C.c_int, C.c_int, C.c_float, C.c_float, vp, vp, C.POINTER(C.c_float)]
     L.TSHip_GptGetLogits.argtypes = [vp, vp]
@@ -104,6 +105,11 @@ class HipGpt:
         ids = np.ascontiguousarray(ids, dtype=np.int32).reshape(-1)
         check(lib().TSHip_GptDecode(self.h, _ptr(ids), ids.size))
         self.batch = ids.size
+
+    def set_blocked_tokens(self, ids):
+        """DecodingOptions.BlockedTokens: tokens that are never chosen (Decoder.cs:745-753); an empty list clears them."""
+        ids = np.ascontiguousarray(ids, dtype=np.int32).reshape(-1)
+        check(lib().TSHip_GptSetBlockedTokens(self.h, _ptr(ids) if ids.size else None, int(ids.size)))
 
     def set_repeat_penalty(self, repeat_penalty):
         """DecodingOptions.RepeatPenalty for top-p sampling (the reference's default is 2.0); set before the prompt is fed."""

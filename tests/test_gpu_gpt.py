@@ -437,6 +437,34 @@ def test_head_dim_128_against_oracle(G, oracle, kv_heads, batch, prompt):
     gpu.close()
 
 
+def test_blocked_tokens(G, oracle):
+    """Decoder.cs:745-753: probs += scatter(-1 at the blocked ids) before argmax / TopPSample."""
+    cfg = synth.tiny_config(batch=4, vocab=120)
+    w = synth.make_weights(cfg, 51, random_bias=True)
+    orc = oracle.OracleGpt(cfg, w)
+    gpu = G.HipGpt(cfg, w, max_batch=4, max_seq_len=32)
+    seqs = synth.make_prompts(cfg, 52)
+    u = synth.make_uniforms(53, 4, 4)
+    p, _ = orc.step(seqs, use_cache=True, sampling=True)
+    blocked = np.unique(np.concatenate([oracle.argmax(p).astype(np.int32), np.argsort(-p[0])[:5].astype(np.int32)]))
+    pm = p.copy()
+    pm[:, blocked] = pm[:, blocked] + np.float32(-1.0)
+    gpu.prefill(seqs)
+    assert np.array_equal(gpu.sample(), oracle.argmax(p).astype(np.int32))
+    gpu.set_blocked_tokens(blocked)
+    got = gpu.sample()
+    assert np.array_equal(got, oracle.argmax(pm).astype(np.int32)) and not np.isin(got, blocked).any()
+    got = gpu.sample(mode=G.TOPP, top_p=0.9, uniforms=u[0])
+    assert np.array_equal(got, oracle.toppsample(pm, 0.9, 0.0, None, u[0]).astype(np.int32))
+    ids, _ = gpu.generate(4, mode=G.TOPP, top_p=0.9, uniforms=u)         # the graph loop sees the same list
+    assert np.array_equal(ids[0], got) and not np.isin(ids, blocked).any()
+    gpu.set_blocked_tokens([])
+    gpu.reset()
+    gpu.prefill(seqs)
+    assert np.array_equal(gpu.sample(), oracle.argmax(p).astype(np.int32))
+    gpu.close()
+
+
 def test_generate_until_all_rows_emit_eos(G):
     """GPT.cs:299-302: the loop ends after the first step at which every sequence's newest token is the END tag
     (Decoder.cs:207-221); a row that ended earlier keeps generating until then."""
