@@ -262,9 +262,24 @@ def test_float2half_matches_ieee_rne(oracle):
 
 
 # ---- top-p ----------------------------------------------------------------------------------------------------------
-def _topp_python(p, top_p, u):
-    """ComputeGraphTensor.TopPSample (ComputeGraphTensor.cs:2305-2403), repeatPenalty off, restated independently."""
-    items = [(float(w), j) for j, w in enumerate(p) if w > 0]
+def _topp_python(p, top_p, u, seq=None, penalty=0.0):
+    """ComputeGraphTensor.TopPSample (ComputeGraphTensor.cs:2305-2403) restated independently; `seq` = the row's
+    decodedSequence (tokens already in it are decayed by pow(dist / len, penalty), :2320-2345)."""
+    import math
+    last = {}
+    if seq is not None:
+        for j, tok in enumerate(seq):
+            last[int(tok)] = len(seq) - j                 # later occurrences overwrite: the last one counts
+    items = []
+    for j, w in enumerate(p):
+        if not w > 0:
+            continue
+        w = np.float32(w)
+        if j in last:
+            ratio = np.float32(np.float32(last[j]) / np.float32(len(seq)))
+            rp = np.float32(math.pow(float(ratio), float(np.float32(penalty))))
+            w = np.float32(w * rp)
+        items.append((float(w), j))
     items.sort(key=lambda t: (-t[0], t[1]))
     acc, cands, accp = np.float32(0), [], []
     for w, j in items:
@@ -293,6 +308,21 @@ def test_toppsample_bruteforce(oracle):
         tp = float(rng.choice([0.1, 0.5, 0.9, 1.0]))
         got = oracle.toppsample(p[None], tp, 0.0, None, np.array([u], np.float32))
         assert int(got[0]) == _topp_python(p, tp, u)
+
+
+def test_toppsample_repeat_penalty_bruteforce(oracle):
+    rng = np.random.default_rng(18)
+    for trial in range(40):
+        K = int(rng.integers(3, 40))
+        L = int(rng.integers(1, 30))
+        p = rng.random(K).astype(np.float32)
+        p = (p / p.sum()).astype(np.float32)
+        seq = rng.integers(0, K, L).astype(np.int32)
+        u = np.float32(rng.random())
+        tp = float(rng.choice([0.1, 0.5, 0.9, 1.0]))
+        pen = float(rng.choice([2.0, 1.0, 0.5, 1.5, 3.0]))
+        got = oracle.toppsample(p[None], tp, pen, seq[None], np.array([u], np.float32))
+        assert int(got[0]) == _topp_python(p, tp, u, seq, pen), trial
 
 
 def test_toppsample_small_p_is_argmax(oracle):
