@@ -122,7 +122,7 @@ static void sample_tokens(TSHipGpt* m, int mode, float top_p, float temperature,
     if (last) TSHIP_REQUIRE((size_t)B * m->last_ld * sizeof(int) <= m->last_pos.bytes && m->last_ld >= m->c.vocab, "internal: token history table too small");
     if (mode == TSHIP_GREEDY) {
         launch(m, "greedy", greedy_kernel, dim3(B), dim3(1024), (const float*)m->logits.as<float>(), Vp, m->c.vocab, m->ids.as<int>(), gen_out, d_step,
-               record ? last : (int*)nullptr, m->last_ld, (const int*)m->d_pos.as<int>(), (const unsigned char*)m->blocked.p);
+               record ? last : (int*)nullptr, m->last_ld, (const int*)m->d_pos.as<int>(), m->any_blocked ? (const unsigned char*)m->blocked.p : (const unsigned char*)nullptr);
         return;
     }
     TSHIP_REQUIRE(mode == TSHIP_TOPP, "unknown sampling mode");
@@ -145,7 +145,7 @@ static void sample_tokens(TSHipGpt* m, int mode, float top_p, float temperature,
     a.temperature = temperature;
     // Decoder.cs:761: TopPSample(probs, TopP, RepeatPenalty, decodedSequences: tgtSeqs); the sequence length is the number
     // of cached positions
-    a.blocked = (const unsigned char*)m->blocked.p;
+    a.blocked = m->any_blocked ? (const unsigned char*)m->blocked.p : nullptr;
     a.repeat_penalty = m->repeat_penalty; a.last_pos = last; a.last_ld = m->last_ld; a.d_len = m->d_pos.as<int>(); a.record = record ? 1 : 0;
     topp_run(a, B, [&](const char* name, void (*kernel)(TopPArgs), dim3 grid, dim3 block, const TopPArgs& args) { launch(m, name, kernel, grid, block, args); });
 }

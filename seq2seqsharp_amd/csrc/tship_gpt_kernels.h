@@ -1153,6 +1153,8 @@ struct AttnArgs {
     float scale;
     const float* ssq; int ssq_nt; int ssq_ld; float inv_h; float eps;   // deferred RMSNorm of the projection input (see SkinnyArgs)
     int vt;      // 1: keys and values are stored fragment-major (kfrag_index / vfrag_index) for the MFMA attention kernels
+    // decode with several blocks per (row, KV head): their number, the exchange area [pairs][S][G D + 2 G] floats and one counter per pair
+    int S; float* xchg; int* xcount;
 };
 
 // rotary embedding of one (even, odd) pair, two roundings per output like the reference's C# expression
@@ -1437,7 +1439,11 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(AttnArgs a) {
 // Online softmax per column with one running maximum per wavefront; wavefronts take 32-row chunks round robin and
 // are merged through LDS.  All arithmetic on scores, probabilities' sums and outputs is fp32.
 // ------------------------------------------------------------------------------------------------
-template <int D, int G>
+// SPLIT: a.S blocks (blockIdx.z) share one (batch row, KV head); chunks go round robin over all their wavefronts, every
+// block leaves its unnormalised sums in an exchange area and the block that arrives last merges them in block order
+// (same publication protocol as the split-K projections: agent-scope atomic stores, wait, counter; no spinning).
+// For launches with fewer (row, head) pairs than CUs.
+template <int D, int G, bool SPLIT>
 __global__ __launch_bounds__(D == 128 ? 256 : 512) void attn_mfma_kernel(AttnArgs a) {
     constexpr int NW = D == 128 ? 4 : 8, NTH = NW * 64;
     constexpr int NCOL = G;                   // MFMA columns in use: the G query heads of the group
@@ -1448,6 +1454,8 @@ __global__ __launch_bounds__(D == 128 ? 256 : 512) void attn_mfma_kernel(AttnArg
     __shared__ float sL[NW][16];
     __shared__ float sO[NW][D][16];
     const int t = threadIdx.x, lane = t & 63, w = __builtin_amdgcn_readfirstlane(t >> 6);
+    // wavefront slot among all wavefronts of the pair, and their number
+    const int gw = SPLIT ? (int)blockIdx.z * NW + w : w, GS = SPLIT ? a.S * NW : NW;
     const int r16 = lane & 15, q = lane >> 4;
     const int HD = a.H * D, GD = a.Hkv * D;
     const int kvh = blockIdx.x, b = blockIdx.y;
@@ -1468,14 +1476,14 @@ __global__ __launch_bounds__(D == 128 ? 256 : 512) void attn_mfma_kernel(AttnArg
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) vf[dt] = *(const half8*)(vc + dt * 512);
     };
-    // Chunks of this wavefront: w, w + NW, ...  A CU accepts about 64 KiB of outstanding loads; a wavefront that
+    // Chunks of this wavefront: gw, gw + GS, ...  A CU accepts about 64 KiB of outstanding loads; a wavefront that
     // requests more stalls at the request, and loads that hit in L2 come back behind the misses queued before them.
     // So: the prologue's operands are requested first and the first chunk (8 KiB per wavefront, 64 KiB per CU) right
     // behind them; every later chunk is requested right before the chunk ahead of it is processed.  The first request
     // is unconditional so that the waits below are counted exactly; a first chunk that holds the row being appended
     // is requested again after the prologue.
-    const int n_own = nchunks > w ? (nchunks - w + NW - 1) / NW : 0;
-    const bool validA = w < nchunks - 1;
+    const int n_own = nchunks > gw ? (nchunks - gw + GS - 1) / GS : 0;
+    const bool validA = gw < nchunks - 1;
 
     for (int i = t; i < 16 * D; i += NTH) (&sQ[0][0])[i] = 0.0f;
     {
@@ -1511,7 +1519,7 @@ __global__ __launch_bounds__(D == 128 ? 256 : 512) void attn_mfma_kernel(AttnArg
         }
         // the stream starts behind the prologue's own requests (its address does not depend on the position)
         __builtin_amdgcn_sched_barrier(0);
-        load_chunk(min(w, (int)(a.max_len >> 5) - 1), kfA, vfA);
+        load_chunk(min(gw, (int)(a.max_len >> 5) - 1), kfA, vfA);
         __builtin_amdgcn_sched_barrier(0);
         float rinv = 1.0f;
         if (a.ssq) rinv = 1.0f / sqrtf(wave_sum(ssq_part) * a.inv_h + a.eps);
@@ -1602,34 +1610,34 @@ __global__ __launch_bounds__(D == 128 ? 256 : 512) void attn_mfma_kernel(AttnArg
     // request never sits under a condition of its own (every later wait would have to cover it).  The first NFX chunks
     // form a chain of stages: a stage either requests the next chunk and processes its own, or processes the last
     // one; longer contexts continue in groups of NL chunks requested together.
-    if (n_own >= 1 && !validA) load_chunk(w, kfA, vfA);
+    if (n_own >= 1 && !validA) load_chunk(gw, kfA, vfA);
     constexpr int NFX = D == 128 ? 3 : 7, NL = D == 128 ? 2 : 4;
     auto group = [&](auto nc, int c0) {
         constexpr int N = decltype(nc)::value;
         half8 kr[N][2][KD], vr[N][DT];
 #pragma unroll
-        for (int g = 0; g < N; ++g) load_chunk(c0 + g * NW, kr[g], vr[g]);
+        for (int g = 0; g < N; ++g) load_chunk(c0 + g * GS, kr[g], vr[g]);
 #pragma unroll
-        for (int g = 0; g < N; ++g) do_chunk(c0 + g * NW, kr[g], vr[g]);
+        for (int g = 0; g < N; ++g) do_chunk(c0 + g * GS, kr[g], vr[g]);
     };
     auto chain = [&](auto self, auto gc, half8 (&kc)[2][KD], half8 (&vc)[DT]) -> void {
-        constexpr int g = decltype(gc)::value;           // kc, vc: chunk w + g NW, requested
-        const int cg = w + g * NW;
+        constexpr int g = decltype(gc)::value;           // kc, vc: chunk gw + g GS, requested
+        const int cg = gw + g * GS;
         if constexpr (g == NFX) {
             do_chunk(cg, kc, vc);
-            int c = cg + NW;
-            for (; c + (NL - 1) * NW < nchunks; c += NL * NW) group(std::integral_constant<int, NL>{}, c);
+            int c = cg + GS;
+            for (; c + (NL - 1) * GS < nchunks; c += NL * GS) group(std::integral_constant<int, NL>{}, c);
             if constexpr (NL == 4) {
-                if (c + 2 * NW < nchunks) group(std::integral_constant<int, 3>{}, c);
-                else if (c + NW < nchunks) group(std::integral_constant<int, 2>{}, c);
+                if (c + 2 * GS < nchunks) group(std::integral_constant<int, 3>{}, c);
+                else if (c + GS < nchunks) group(std::integral_constant<int, 2>{}, c);
                 else if (c < nchunks) group(std::integral_constant<int, 1>{}, c);
             } else {
                 if (c < nchunks) group(std::integral_constant<int, 1>{}, c);
             }
         } else {
-            if (cg + NW < nchunks) {
+            if (cg + GS < nchunks) {
                 half8 kn[2][KD], vn[DT];
-                load_chunk(cg + NW, kn, vn);
+                load_chunk(cg + GS, kn, vn);
                 do_chunk(cg, kc, vc);
                 self(self, std::integral_constant<int, g + 1>{}, kn, vn);
             } else {
@@ -1647,6 +1655,56 @@ __global__ __launch_bounds__(D == 128 ? 256 : 512) void attn_mfma_kernel(AttnArg
 #pragma unroll
         for (int i = 0; i < 4; ++i) sO[w][dt * 16 + 4 * q + i][r16] = acc_o[dt][i];
     __syncthreads();
+    if constexpr (SPLIT) {
+        // block sums relative to the block maximum -> exchange area [pair][block][NCOL D + 2 NCOL] floats
+        __shared__ int s_last;
+        const int pair = b * a.Hkv + kvh;
+        const long per = (long)NCOL * D + 2 * NCOL;
+        float* mine = a.xchg + ((long)pair * a.S + blockIdx.z) * per;
+        for (int idx = t; idx < NCOL * D; idx += NTH) {
+            const int col = idx % NCOL, d = idx / NCOL;
+            float M = -INFINITY;
+#pragma unroll
+            for (int i = 0; i < NW; ++i) M = fmaxf(M, sM[i][col]);
+            float L = 0.0f, O = 0.0f;
+#pragma unroll
+            for (int i = 0; i < NW; ++i) {
+                const float wgt = (sM[i][col] == -INFINITY) ? 0.0f : __expf(sM[i][col] - M);
+                L += sL[i][col] * wgt;
+                O += sO[i][d][col] * wgt;
+            }
+            __hip_atomic_store(mine + idx, O, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (d == 0) {
+                __hip_atomic_store(mine + NCOL * D + col, M, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __hip_atomic_store(mine + NCOL * D + NCOL + col, L, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");            // the stores have reached the point of coherence
+        __syncthreads();
+        if (t == 0) s_last = __hip_atomic_fetch_add(a.xcount + pair, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == a.S - 1;
+        __syncthreads();
+        if (!s_last) return;
+        // every block of the pair has published (its count came after its stores): merge in block order
+        const float* base = a.xchg + (long)pair * a.S * per;
+        for (int idx = t; idx < NCOL * D; idx += NTH) {
+            const int col = idx % NCOL, d = idx / NCOL;
+            float M = -INFINITY;
+            for (int s = 0; s < a.S; ++s) M = fmaxf(M, __hip_atomic_load(base + s * per + NCOL * D + col, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+            float L = 0.0f, O = 0.0f;
+            for (int s = 0; s < a.S; ++s) {
+                const float ms = __hip_atomic_load(base + s * per + NCOL * D + col, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                const float wgt = (ms == -INFINITY) ? 0.0f : __expf(ms - M);
+                L += __hip_atomic_load(base + s * per + NCOL * D + NCOL + col, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) * wgt;
+                O += __hip_atomic_load(base + s * per + idx, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) * wgt;
+            }
+            const float o = O / L;
+            const int kcol = (kvh * G + col) * D + d;
+            if (a.out_kt > 0) ((half_t*)a.out)[xpack_index(b, kcol, a.out_kt)] = (half_t)o;
+            else ((half_t*)a.out)[(long)b * a.ld_out + kcol] = (half_t)o;
+        }
+        if (t == 0) __hip_atomic_store(a.xcount + pair, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);       // ready for the next launch
+        return;
+    }
     for (int idx = t; idx < NCOL * D; idx += NTH) {
         const int col = idx % NCOL, d = idx / NCOL;
         float M = -INFINITY;

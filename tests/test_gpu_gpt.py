@@ -437,6 +437,27 @@ def test_head_dim_128_against_oracle(G, oracle, kv_heads, batch, prompt):
     gpu.close()
 
 
+@pytest.mark.parametrize("hidden,heads,kv_heads,batch,prompt,splits", [(256, 4, 2, 2, 300, 2), (512, 4, 1, 1, 200, 2), (256, 4, 4, 1, 530, 3),
+                                                                      (256, 4, 2, 3, 90, 16)])
+def test_decode_attention_split_over_blocks(G, oracle, monkeypatch, hidden, heads, kv_heads, batch, prompt, splits):
+    """Few (row, KV head) pairs and a long context: several blocks share a pair and the last one to arrive merges their
+    sums.  The library only splits at contexts of several thousand positions; the environment variable forces it here
+    (head_dim 64 and 128, two and three blocks, and sixteen blocks most of which have no chunk at all).  fp16, against
+    the oracle, with decode steps across a 32-position chunk boundary; then decode against the prefill path, which does
+    not split."""
+    monkeypatch.setenv("TSHIP_ATTN_SPLITS", str(splits))
+    cfg = synth.tiny_config(dtype="f16", hidden=hidden, n_heads=heads, n_kv_heads=kv_heads, ffn_dim=2 * hidden, vocab=300, batch=batch, prompt=prompt)
+    orc, gpu, out, cur = _teacher_forced(G, oracle, cfg, 81, 6)
+    for lg, gl in out:
+        assert np.abs(gl - lg).max() <= FP16_ABS
+    # the same sequences through prefill only (one block per query group there)
+    last = gpu.logits()
+    gpu.reset()
+    gpu.prefill(cur)
+    assert np.abs(gpu.logits() - last).max() <= 2e-2
+    gpu.close()
+
+
 def test_blocked_tokens(G, oracle):
     """Decoder.cs:745-753: probs += scatter(-1 at the blocked ids) before argmax / TopPSample."""
     cfg = synth.tiny_config(batch=4, vocab=120)
