@@ -10,8 +10,9 @@
 // caller maintains (history_kernel for given tokens; the pick and greedy kernels record the token they choose).
 // The order is produced by a stable least-significant-digit radix sort on the float bit pattern (four passes of
 // eight bits, every pass = histogram, scan, scatter over segments of 1024 elements, so a row is sorted by many
-// blocks); the running sum is taken serially in fp32 by one wavefront, so for given probabilities the chosen index
-// is the reference's, bit for bit.
+// blocks); the running sum has the values of the reference's one-by-one fp32 additions (computed with block-wide scans
+// in integer arithmetic, see topp_pick_scan_kernel), so for given probabilities the chosen index is the reference's,
+// bit for bit.
 #pragma once
 
 #include "tship_internal.h"
@@ -108,24 +109,47 @@ static __global__ __launch_bounds__(1024) void topp_keys_kernel(TopPArgs a) {
 #pragma unroll
         for (int i = 0; i < 16; ++i) sum += sred[i];
     }
+    // Repeat penalty: few tokens of the vocabulary occur in the sequence, but almost every wavefront holds one of them, and
+    // the double-precision pow would be paid by all 64 lanes.  So the pass over the vocabulary only notes those tokens
+    // (index and probability) in an LDS list, and the list is worked off densely afterwards.
+    constexpr int DECAY_CAP = 4096;
+    __shared__ int s_didx[DECAY_CAP];
+    __shared__ float s_dp[DECAY_CAP];
+    __shared__ int s_dn;
     const bool decay = a.last_pos && a.repeat_penalty != 0.0f;
     const int len = decay ? topp_seq_len(a, r) : 0;
     const int* last = decay ? a.last_pos + (long)r * a.last_ld : nullptr;
+    auto decayed = [&](float p, int lp) {
+        // float division, double pow, one rounding to float, one fp32 multiply (ComputeGraphTensor.cs:2341-2342)
+        const float ratio = (float)(len - lp) / (float)len;
+        const float rp = (float)pow((double)ratio, (double)a.repeat_penalty);
+        return p * rp;          // (a product that underflows to 0 stays a candidate of weight 0 there; it can never be picked)
+    };
+    // p > 0: positive floats order like their bit patterns; descending order = ascending ~bits.
+    // p <= 0 is dropped by the reference: give it the largest key so that it sorts behind every candidate.
+    auto key_of = [&](float p, int i) { return (p > 0.0f && !(a.blocked && a.blocked[i])) ? ~__float_as_uint(p) : 0xffffffffu; };
+    if (t == 0) s_dn = 0;
+    __syncthreads();
     for (int i = t; i < V; i += 1024) {
         float p = a.in_is_logits ? expf(row[i] / a.temperature - mx) / sum : row[i];
         if (decay && p > 0.0f) {
             const int lp = last[i];
             if (lp >= 0) {
-                // float division, double pow, one rounding to float, one fp32 multiply (ComputeGraphTensor.cs:2341-2342)
-                const float ratio = (float)(len - lp) / (float)len;
-                const float rp = (float)pow((double)ratio, (double)a.repeat_penalty);
-                p = p * rp;      // (a product that underflows to 0 stays a candidate of weight 0 there; it can never be picked)
+                const int slot = atomicAdd(&s_dn, 1);
+                if (slot < DECAY_CAP) { s_didx[slot] = i; s_dp[slot] = p; }
+                else p = decayed(p, lp);                             // list full (sequences longer than the list): in place
             }
         }
-        // p > 0: positive floats order like their bit patterns; descending order = ascending ~bits.
-        // p <= 0 is dropped by the reference: give it the largest key so that it sorts behind every candidate.
-        kA[i] = (p > 0.0f && !(a.blocked && a.blocked[i])) ? ~__float_as_uint(p) : 0xffffffffu;
+        kA[i] = key_of(p, i);
         iA[i] = i;
+    }
+    if (decay) {
+        __syncthreads();
+        const int nd = min(s_dn, DECAY_CAP);
+        for (int e = t; e < nd; e += 1024) {
+            const int i = s_didx[e];
+            kA[i] = key_of(decayed(s_dp[e], last[i]), i);
+        }
     }
 }
 
@@ -227,104 +251,252 @@ static __global__ __launch_bounds__(256) void topp_scatter_kernel(TopPArgs a) {
     }
 }
 
-// running sum and pick: grid (rows), one wavefront.  keysA holds the sorted probabilities (their bit patterns, 0 for
-// dropped entries), idxA the token ids in the same order.
-// The running sum is one dependent chain of fp32 additions (that is what fixes its value), so the cost per element is
-// what matters: the probabilities are staged through LDS in segments of 8192 (the next segment's loads are in flight
-// while the current one is walked), read back 16 bytes at a time with every lane at the same address, one unit of 32
-// ahead, and added with one v_add_f32 each.  The value after each unit is kept, so that the pick only replays one unit.
-static __global__ __launch_bounds__(64) void topp_pick_kernel(TopPArgs a) {
-    constexpr int SEG = 8192;
-    __shared__ __attribute__((aligned(16))) float sp[2][SEG];
-    const int r = blockIdx.x, lane = threadIdx.x, V = a.V;
-    const float* pk = (const float*)(a.keysA + (long)r * a.Vs);      // Vs is a multiple of 64
+// ------------------------------------------------------------------------------------------------
+// Running sum and pick, evaluated in parallel but with the values of the sequential fp32 sum, bit for bit.
+//
+// The reference adds the sorted probabilities one by one in fp32: acc_k = fl(acc_{k-1} + p_k).  While acc stays inside
+// one binade [2^e, 2^(e+1)) it is an integer multiple A of u = 2^(e-23), and (p_k <= acc, so p_k's exponent is not
+// larger) the rounded sum is A + d_k with d_k = floor(p_k / u) + 1 if the fraction of p_k / u is above 1/2, + 0 if below,
+// and on an exact tie whatever makes A + d_k even (round to nearest even).  floor and fraction come from shifting p_k's
+// 24-bit significand, so d_k is integer arithmetic; a tie makes d_k depend on the parity of the sum before it, and that
+// parity runs through the elements as a composition of maps "xor with a bit" / "constant 0", which is associative.  Two
+// block-wide scans (parity maps, then integers) therefore give every acc_k of a tile at once.  The element at which
+// the sum leaves the binade is added in floating point by itself, and the next tile starts behind it with the new u.
+// The first PICK_HEAD elements are added one by one by a single thread: the sum changes binade after 2, 4, 8 ...
+// elements of a flat distribution, and a peaked one (a trained model) reaches top_p within them, so the scans never start.
+// grid (rows), 512 threads; eight consecutive elements per thread and tile (256, 512 and 1024 threads measured the same
+// within 15 %: the kernel is bound by its instruction count on one CU, about 60 per element and pass).
+// ------------------------------------------------------------------------------------------------
+constexpr int PICK_E = 8, PICK_THREADS = 512, PICK_WAVES = PICK_THREADS / 64, PICK_TILE = PICK_E * PICK_THREADS;
+constexpr int PICK_HEAD = 512;                          // elements added one by one before the scans start
+constexpr unsigned PICK_CAP = 1u << 25;                  // sums saturate here: anything >= 2^24 has left the binade
+
+__device__ __forceinline__ unsigned pick_sat_add(unsigned a, unsigned b) { const unsigned s = a + b; return s > PICK_CAP ? PICK_CAP : s; }
+// parity maps in two bits: bit 1 = constant, bit 0 = the constant or the xor mask; `then(prev, cur)` = cur after prev
+__device__ __forceinline__ unsigned pick_map_then(unsigned prev, unsigned cur) { return (cur & 2u) ? cur : ((prev & 2u) | ((prev ^ cur) & 1u)); }
+__device__ __forceinline__ unsigned pick_map_apply(unsigned map, unsigned parity) { return (map & 2u) ? (map & 1u) : ((parity ^ map) & 1u); }
+
+// inclusive scan of saturating sums over the 64 lanes with data-parallel-primitive moves (no LDS): shifts by 1, 2, 4, 8
+// inside rows of 16 lanes, then the last lane of row 0 / 2 into rows 1 / 3 and of row 1 into rows 2 and 3
+__device__ __forceinline__ unsigned pick_wave_scan(unsigned x) {
+    x = pick_sat_add(x, (unsigned)__builtin_amdgcn_update_dpp(0, (int)x, 0x111, 0xf, 0xf, false));
+    x = pick_sat_add(x, (unsigned)__builtin_amdgcn_update_dpp(0, (int)x, 0x112, 0xf, 0xf, false));
+    x = pick_sat_add(x, (unsigned)__builtin_amdgcn_update_dpp(0, (int)x, 0x114, 0xf, 0xf, false));
+    x = pick_sat_add(x, (unsigned)__builtin_amdgcn_update_dpp(0, (int)x, 0x118, 0xf, 0xf, false));
+    x = pick_sat_add(x, (unsigned)__builtin_amdgcn_update_dpp(0, (int)x, 0x142, 0xa, 0xf, false));
+    x = pick_sat_add(x, (unsigned)__builtin_amdgcn_update_dpp(0, (int)x, 0x143, 0xc, 0xf, false));
+    return x;
+}
+// parity maps of the lanes below `lane`, composed, from two ballots (which lanes are constant, the lanes' low bits):
+// the last constant lane below fixes the value, the xor bits above it flip it
+__device__ __forceinline__ unsigned pick_map_below(unsigned long long isc, unsigned long long bit, int lane) {
+    const unsigned long long lower = (1ull << lane) - 1ull;
+    const unsigned long long c = isc & lower;
+    if (c == 0ull) return (unsigned)__popcll(bit & lower) & 1u;
+    const int q = 63 - __clzll((long long)c);
+    const unsigned long long above = lower & ~((2ull << q) - 1ull);
+    return 2u | ((((unsigned)(bit >> q)) ^ (unsigned)__popcll(bit & above)) & 1u);
+}
+
+// block barrier that orders LDS traffic only (outstanding global stores are not waited for)
+__device__ __forceinline__ void pick_lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
+static __global__ __launch_bounds__(PICK_THREADS) void topp_pick_scan_kernel(TopPArgs a) {
+    __shared__ unsigned s_wmap[PICK_WAVES], s_wsum[PICK_WAVES];
+    __shared__ int s_event[PICK_WAVES];
+    __shared__ float s_acc;
+    __shared__ int s_j0, s_n, s_state, s_pick[PICK_WAVES];
+    __shared__ float s_head[PICK_HEAD];                     // s_state: 0 = go on in this tile, 1 = next tile, 2 = finished
+    const int r = blockIdx.x, t = threadIdx.x, lane = t & 63, w = t >> 6, V = a.V;
+    const unsigned* pk = a.keysA + (long)r * a.Vs;                   // sorted probabilities as bit patterns, 0 = not a candidate
     const int* idx = a.idxA + (long)r * a.Vs;
-    float* cp = a.accp + (long)r * a.Vs;                               // cp[u]: running sum after unit u
-    float acc = 0.0f; int n = 0, nun = 0;
-    const int nseg = (V + SEG - 1) / SEG;
-    floatx4 reg[SEG / 256];
-    auto seg_load = [&](int s) {
+    float* accp = a.accp + (long)r * a.Vs;                           // accp[k]: running sum after element k
+    // a tile's bit patterns are fetched once (two 16-byte loads per thread: Vs is a multiple of 64 elements), the next
+    // tile's while this one is worked on
+    unsigned bits[PICK_E], nbits[PICK_E];
+    auto tile_load = [&](int kb, unsigned (&dst)[PICK_E]) {
+        const int k = kb + t * PICK_E;
+        uint4 lo = uint4{0u, 0u, 0u, 0u}, hi = lo;
+        if (k < a.Vs) { lo = *(const uint4*)(pk + k); hi = *(const uint4*)(pk + k + 4); }     // k + 7 < Vs
+        dst[0] = lo.x; dst[1] = lo.y; dst[2] = lo.z; dst[3] = lo.w; dst[4] = hi.x; dst[5] = hi.y; dst[6] = hi.z; dst[7] = hi.w;
 #pragma unroll
-        for (int i = 0; i < SEG / 256; ++i) {
-            const int e = s * SEG + (i * 64 + lane) * 4;
-            floatx4 v = e < V ? *(const floatx4*)(pk + e) : floatx4{0.0f, 0.0f, 0.0f, 0.0f};      // e + 3 < Vs
-#pragma unroll
-            for (int j = 0; j < 4; ++j) if (e + j >= V) v[j] = 0.0f;                                 // padding is not a candidate
-            reg[i] = v;
-        }
+        for (int i = 0; i < PICK_E; ++i) if (k + i >= V) dst[i] = 0u;                         // padding is not a candidate
     };
-    auto seg_store = [&](int buf) {
+    tile_load(0, bits);
+    // head of the row, one by one (starting from acc = 0 as the reference does).  Wavefront 0 holds these elements (lane L:
+    // 8 L .. 8 L + 7); they are broadcast lane by lane into scalar registers, so one element costs a read-lane and one add.
+    if (w == 0) {
+        float acc = 0.0f; int k = 0; bool stop = false;
+        for (int L = 0; L < PICK_HEAD / PICK_E && !stop; ++L) {
+            float pv[PICK_E];
 #pragma unroll
-        for (int i = 0; i < SEG / 256; ++i) *(floatx4*)&sp[buf][(i * 64 + lane) * 4] = reg[i];
-    };
-    auto unit_read = [&](int buf, int u, floatx4 (&q)[8]) {
+            for (int i = 0; i < PICK_E; ++i) pv[i] = __uint_as_float((unsigned)__builtin_amdgcn_readlane((int)bits[i], L));
 #pragma unroll
-        for (int i = 0; i < 8; ++i) q[i] = *(const floatx4*)&sp[buf][u * 32 + 4 * i];
-    };
-    seg_load(0);
-    seg_store(0);
-    bool over = false;
-    for (int s = 0; s < nseg && !over; ++s) {
-        const int buf = s & 1;
-        if (s + 1 < nseg) seg_load(s + 1);
-        __builtin_amdgcn_wave_barrier();
-        const int units = min(SEG, V - s * SEG + 31) / 32;             // units of this segment that hold candidates or padding
-        floatx4 q[8], qn[8];
-        unit_read(buf, 0, q);
-        for (int u = 0; u < units; ++u) {
-            if (u + 1 < units) unit_read(buf, u + 1, qn);
-            // descending probabilities: candidates (p > 0) first, dropped entries and padding (0) last
-            bool done = q[7][3] == 0.0f;
-            if (!done) {
-                float trial = acc;
-#pragma unroll
-                for (int i = 0; i < 8; ++i)
-#pragma unroll
-                    for (int j = 0; j < 4; ++j) trial += q[i][j];
-                if (trial < a.top_p) { acc = trial; n += 32; }
-                else done = true;
+            for (int i = 0; i < PICK_E; ++i) {
+                if (stop) break;
+                if (!(pv[i] > 0.0f)) { stop = true; break; }         // no more candidates (padding behind V is 0 as well)
+                acc += pv[i];
+                if (lane == 0) s_head[k] = acc;
+                ++k;
+                if (acc >= a.top_p) stop = true;
             }
-            if (done) {
-                // the unit that ends the walk: element by element
-                for (int j = 0; j < 32; ++j) {
-                    const float pj = sp[buf][u * 32 + j];
-                    if (pj <= 0.0f) break;                 // ran out of candidates
-                    acc += pj; n += 1;
-                    if (acc >= a.top_p) break;
+        }
+        if (lane == 0) { s_acc = acc; s_n = k; s_j0 = k; s_state = stop ? 2 : 0; }
+    }
+    __syncthreads();
+    for (int k = t; k < s_n && k < PICK_HEAD; k += PICK_THREADS) accp[k] = s_head[k];
+    for (int kb = 0; s_state != 2; kb += PICK_TILE) {
+        if (kb + PICK_TILE < V) tile_load(kb + PICK_TILE, nbits);
+        // work through this tile; every pass ends at an event: the sum leaves its binade (another pass), reaches top_p,
+        // runs out of candidates, or the tile ends
+        for (;;) {
+            const int j0 = s_j0;                                     // elements of the tile before j0 are done
+            const float acc0 = s_acc;
+            const unsigned abits = __float_as_uint(acc0);
+            const int aexp = (int)(abits >> 23);                     // biased; 0 = subnormal
+            pick_lds_barrier();                                         // everyone has read the state
+            if (j0 >= PICK_TILE) { if (t == 0) { s_state = 1; } pick_lds_barrier(); break; }
+            if (aexp <= 23) {
+                // a running sum below 2^-103, where 2^(e-23) is not a normal float (never after a softmax): one plain step
+                if (t == 0) {
+                    const int k = kb + j0;
+                    const float p = k < V ? __uint_as_float(pk[k]) : 0.0f;
+                    if (p > 0.0f) { const float v = acc0 + p; accp[k] = v; s_acc = v; s_j0 = j0 + 1; s_n = k + 1; if (v >= a.top_p) s_state = 2; }
+                    else s_state = 2;
                 }
+                pick_lds_barrier();
+                if (s_state == 2) break;
+                continue;
             }
-            if (lane == 0) cp[nun] = acc;
-            ++nun;
-            if (done) { over = true; break; }
+            const unsigned A0 = (abits & 0x7fffffu) | 0x800000u;
+            unsigned dfl[PICK_E], cls[PICK_E];                       // cls: 0 plain (d = dfl), 1 tie, 2 not a candidate, 3 already done
+            unsigned map = 0u;                                       // identity
 #pragma unroll
-            for (int i = 0; i < 8; ++i) q[i] = qn[i];
+            for (int i = 0; i < PICK_E; ++i) {
+                const unsigned b = bits[i];
+                dfl[i] = 0u;
+                if (t * PICK_E + i < j0) { cls[i] = 3u; continue; }
+                if (b == 0u) { cls[i] = 2u; continue; }              // (sorted: everything behind it is 0 as well)
+                const int pexp = (int)(b >> 23);
+                const unsigned m = pexp ? ((b & 0x7fffffu) | 0x800000u) : (b & 0x7fffffu);
+                const int sh = aexp - (pexp ? pexp : 1);             // >= 0: p <= acc
+                if (sh < 0) { dfl[i] = PICK_CAP; cls[i] = 0u; continue; }   // not sorted (NaN in the input): handled as leaving the binade
+                // m / 2^sh as 32.32 fixed point: integer part and the fraction, which the shift leaves exact (sh <= 32)
+                const unsigned long long x = sh <= 32 ? (((unsigned long long)m << 32) >> sh) : 0ull;      // sh > 32: below 1/2
+                const unsigned fl = (unsigned)(x >> 32), frac = (unsigned)x;
+                const bool gt = frac > 0x80000000u, tie = frac == 0x80000000u;
+                dfl[i] = fl + (gt ? 1u : 0u); cls[i] = tie ? 1u : 0u;
+                map = pick_map_then(map, tie ? 2u : (dfl[i] & 1u));
+            }
+            // exclusive scan of the parity maps over the block
+            const unsigned long long b_isc = __ballot((map & 2u) != 0u), b_bit = __ballot((map & 1u) != 0u);
+            if (lane == 63) s_wmap[w] = pick_map_then(pick_map_below(b_isc, b_bit, 63), map);        // the whole wavefront
+            pick_lds_barrier();
+            unsigned before = 0u;                                    // map of everything ahead of this thread
+            for (int i = 0; i < w; ++i) before = pick_map_then(before, s_wmap[i]);
+            before = pick_map_then(before, pick_map_below(b_isc, b_bit, lane));
+            unsigned parity = pick_map_apply(before, A0 & 1u);
+            // increments with the ties resolved, local prefix
+            unsigned loc[PICK_E], run = 0u;
+#pragma unroll
+            for (int i = 0; i < PICK_E; ++i) {
+                unsigned d = dfl[i];
+                if (cls[i] == 1u) d += (parity ^ d) & 1u;            // make the sum even
+                if (cls[i] >= 2u) d = 0u;
+                parity = (parity ^ d) & 1u;
+                run = pick_sat_add(run, d > PICK_CAP ? PICK_CAP : d);
+                loc[i] = run;
+            }
+            const unsigned sinc = pick_wave_scan(run);              // inclusive over the wavefront
+            if (lane == 63) s_wsum[w] = sinc;
+            pick_lds_barrier();
+            unsigned base = A0;
+            for (int i = 0; i < w; ++i) base = pick_sat_add(base, s_wsum[i]);
+            { const unsigned prev = __shfl_up(sinc, 1, 64); if (lane > 0) base = pick_sat_add(base, prev); }
+            // values, and the first event: 4 j + type, type 0 = leaves the binade, 1 = reaches top_p, 2 = no more candidates
+            // (val of an element at which the sum leaves the binade: the floating-point sum of the value before it and the
+            // element; it is only used if that element turns out to be the first event)
+            float val[PICK_E];
+            int event = 0x7fffffff;
+            const float scale = __uint_as_float((unsigned)(aexp - 23) << 23);      // 2^(e - 23) with e = aexp - 127: biased exponent aexp - 23 >= 1
+            unsigned Aprev = base;
+#pragma unroll
+            for (int i = 0; i < PICK_E; ++i) {
+                const int j = t * PICK_E + i;
+                const unsigned A = pick_sat_add(base, loc[i]);
+                val[i] = 0.0f;
+                int ev = 0x7fffffff;
+                if (cls[i] == 3u) ev = 0x7fffffff;
+                else if (cls[i] == 2u) ev = 4 * j + 2;
+                else if (A >= (1u << 24)) { ev = 4 * j + 0; val[i] = (float)Aprev * scale + __uint_as_float(bits[i]); }
+                else { val[i] = (float)A * scale; if (val[i] >= a.top_p) ev = 4 * j + 1; }
+                if (ev < event) event = ev;
+                Aprev = A;
+            }
+#pragma unroll
+            for (int o = 32; o > 0; o >>= 1) { const int other = __shfl_xor(event, o, 64); if (other < event) event = other; }
+            if (lane == 0) s_event[w] = event;
+            pick_lds_barrier();
+            event = s_event[0];
+#pragma unroll
+            for (int i = 1; i < PICK_WAVES; ++i) event = min(event, s_event[i]);
+            const int jstop = event == 0x7fffffff ? PICK_TILE : event >> 2, type = event == 0x7fffffff ? -1 : (event & 3);
+            // elements ahead of the event are final; so is an element that reaches top_p or at which the sum leaves its
+            // binade (one floating-point addition, done above)
+            const int jkeep = (type == 1 || type == 0) ? jstop + 1 : jstop;
+#pragma unroll
+            for (int i = 0; i < PICK_E; ++i) {
+                const int j = t * PICK_E + i;
+                if (j >= j0 && j < jkeep) { accp[kb + j] = val[i]; if (j == jkeep - 1) s_acc = val[i]; }      // the last final value is the running sum
+            }
+            pick_lds_barrier();              // (the stores to accp are not waited for here: they are read after the loop)
+            if (t == 0) {
+                if (jkeep > j0) s_n = kb + jkeep;
+                if (type == -1) { s_j0 = PICK_TILE; }
+                else if (type == 1 || type == 2) { s_state = 2; }
+                else { s_j0 = jstop + 1; if (s_acc >= a.top_p) s_state = 2; }
+            }
+            pick_lds_barrier();
+            if (s_state == 2) break;
         }
-        if (!over && s + 1 < nseg) { __builtin_amdgcn_wave_barrier(); seg_store(buf ^ 1); }
+        if (s_state == 2) break;
+        // next tile
+        pick_lds_barrier();
+        if (t == 0) { s_state = kb + PICK_TILE < V ? 0 : 2; s_j0 = 0; }
+#pragma unroll
+        for (int i = 0; i < PICK_E; ++i) bits[i] = nbits[i];
+        pick_lds_barrier();
     }
     __threadfence_block();
+    __syncthreads();
+    const int n = s_n;
+    const float acc = s_acc;
     const long slot = (a.d_step ? (long)*a.d_step * gridDim.x : 0) + r;
     const float u = a.uniforms[slot];
+    // first k < n with accp[k] / acc >= u.  The running sum never decreases, so the test is monotone in k: the last
+    // elements of 512 equal segments locate the segment, its (at most 128) elements the index: two loads per thread.
+    auto block_min = [&](int v) {
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) { const int other = __shfl_xor(v, o, 64); if (other < v) v = other; }
+        __syncthreads();
+        if (lane == 0) s_pick[w] = v;
+        __syncthreads();
+        int m = s_pick[0];
+#pragma unroll
+        for (int i = 1; i < PICK_WAVES; ++i) m = min(m, s_pick[i]);
+        return m;
+    };
     int pick = 0x7fffffff;
     if (n > 0) {
-        // first unit whose final value passes the test holds the pick (the running sum never decreases)
-        int ustar = 0x7fffffff;
-        for (int u0 = 0; u0 < nun && ustar == 0x7fffffff; u0 += 64) {
-            const int c = u0 + lane;
-            const bool hit = c < nun && cp[c] / acc >= u;
-            const unsigned long long m = __ballot(hit);
-            if (m) ustar = u0 + (int)__ffsll((long long)m) - 1;
-        }
-        if (ustar != 0x7fffffff) {
-            float run = ustar > 0 ? cp[ustar - 1] : 0.0f;
-            const int i = ustar * 32 + lane;
-            const float p = (lane < 32 && i < V) ? pk[i] : 0.0f;
-            for (int j = 0; j < 32 && ustar * 32 + j < n; ++j) {
-                run += __shfl(p, j, 64);
-                if (run / acc >= u) { pick = ustar * 32 + j; break; }
-            }
+        const int seg = (n + PICK_THREADS - 1) / PICK_THREADS;           // <= 128: vocabularies have at most 65535 entries
+        const int last = min(n, (t + 1) * seg) - 1;                      // last element of segment t (empty segments repeat n - 1)
+        const int hit_seg = block_min((t * seg < n && accp[last] / acc >= u) ? t : 0x7fffffff);
+        if (hit_seg != 0x7fffffff) {
+            const int k = hit_seg * seg + t;
+            pick = block_min((t < seg && k < n && accp[k] / acc >= u) ? k : 0x7fffffff);
         }
     }
-    if (lane == 0) {
+    if (t == 0) {
         const int id = pick == 0x7fffffff ? 0 : idx[pick];
         if (a.next_ids) a.next_ids[r] = id;
         if (a.gen_out) a.gen_out[slot] = id;
@@ -345,7 +517,7 @@ inline void topp_run(TopPArgs a, int rows, LaunchFn&& launch_fn) {
         unsigned* tk = a.keysA; a.keysA = a.keysB; a.keysB = tk;
         int* ti = a.idxA; a.idxA = a.idxB; a.idxB = ti;
     }
-    launch_fn("topp_pick", topp_pick_kernel, dim3((unsigned)rows), dim3(64), a);
+    launch_fn("topp_pick", topp_pick_scan_kernel, dim3((unsigned)rows), dim3(PICK_THREADS), a);
 }
 
 }  // namespace tship

@@ -1,6 +1,6 @@
 """Turn a rocprofv3 result database (--kernel-trace [--pmc ...]) into the short text summaries kept under profiles/.
 
-    python -m seq2seqsharp_amd.prof_summary gpurun_out/prof/decode_results.db "<command that produced it>" > profiles/<name>.txt
+    python -m seq2seqsharp_amd.prof_summary <rocprofv3 output dir>/decode_results.db "<command that produced it>" > <summary>.txt
 """
 import re
 import sqlite3

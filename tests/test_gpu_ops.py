@@ -213,6 +213,43 @@ def test_toppsample_bit_exact_given_probs(T, oracle):
     assert np.array_equal(got, oracle.argmax(small))                    # topP -> 0 is greedy
 
 
+def test_toppsample_running_sum_is_the_sequential_one(T, oracle):
+    """The device evaluates the running sum with block-wide scans in integer arithmetic; the values must be those of
+    the reference's one-by-one fp32 additions.  Inputs that stress it: flat rows walked to the end over many binades,
+    exact powers of two and equal values (ties of the rounding), sums that never reach top_p, tiny and subnormal
+    weights, one candidate, none."""
+    HT, ops = T
+    rng = np.random.default_rng(12)
+    rows = []
+    K = 32000
+    rows.append(np.full(K, 1.0 / K))                                    # flat
+    rows.append(rng.random(K) / K * 2)                                   # flat-ish, sum about 1
+    rows.append(2.0 ** rng.integers(-24, -10, K).astype(np.float64))     # powers of two only
+    rows.append(rng.integers(1, 4, K) * 2.0 ** -17)                      # few distinct values, many ties
+    rows.append(np.where(rng.random(K) < 0.5, 2.0 ** -16, 3 * 2.0 ** -17))
+    rows.append(rng.random(K) * 1e-9)                                    # never reaches top_p
+    rows.append(np.concatenate([[0.5, 0.25, 0.125], np.full(K - 3, 2.0 ** -30)]))
+    rows.append(np.concatenate([rng.random(50) * 1e-41, np.zeros(K - 50)]))          # subnormal weights only
+    rows.append(np.concatenate([[0.7], np.zeros(K - 1)]))                # one candidate
+    rows.append(np.zeros(K))                                             # none
+    rows.append(np.exp(rng.standard_normal(K) * 4) / 1e4)                # wide dynamic range
+    rows.append(np.concatenate([rng.random(2047) * 1e-3, [2.0 ** -9], rng.random(K - 2048) * 1e-4]))
+    p = np.stack(rows).astype(np.float32)
+    for seed in range(8):
+        u = np.random.default_rng(100 + seed).random(len(rows)).astype(np.float32)
+        for top_p in (0.5, 0.9, 1.0, 1e30):
+            got = ops.toppsample(None, HT.from_numpy(p), HT.from_numpy(u), top_p).numpy().reshape(-1)
+            want = oracle.toppsample(p, top_p, 0.0, None, u)
+            assert np.array_equal(got, want), (seed, top_p, np.nonzero(got != want)[0])
+    # small vocabularies: fewer elements than one tile, and an odd size
+    for K in (1, 2, 97, 2049, 4100):
+        q = oracle.softmax(rng.standard_normal((6, K)).astype(np.float32))
+        u = rng.random(6).astype(np.float32)
+        for top_p in (0.3, 1.0):
+            got = ops.toppsample(None, HT.from_numpy(q), HT.from_numpy(u), top_p).numpy().reshape(-1)
+            assert np.array_equal(got, oracle.toppsample(q, top_p, 0.0, None, u)), (K, top_p)
+
+
 def test_toppsample_repeat_penalty(T, oracle):
     """decodedSequences given (ComputeGraphTensor.cs:2320-2345): tokens already in the row's sequence are decayed by
     pow(dist / len, penalty) before the sort.  Penalty 2 (the reference's default) squares exactly in double; 1.5 and
