@@ -112,7 +112,7 @@ static __global__ __launch_bounds__(1024) void topp_keys_kernel(TopPArgs a) {
     // Repeat penalty: few tokens of the vocabulary occur in the sequence, but almost every wavefront holds one of them, and
     // the double-precision pow would be paid by all 64 lanes.  So the pass over the vocabulary only notes those tokens
     // (index and probability) in an LDS list, and the list is worked off densely afterwards.
-    constexpr int DECAY_CAP = 4096;
+    constexpr int DECAY_CAP = 8192;          // 64 KiB of LDS; more distinct tokens than this in a sequence are decayed in place
     __shared__ int s_didx[DECAY_CAP];
     __shared__ float s_dp[DECAY_CAP];
     __shared__ int s_dn;
