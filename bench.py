@@ -185,8 +185,14 @@ def main():
         base, lg = cpu_baseline(cfg, gpu, weights, nxt, "cache from the GPU prefill")
         gpu.decode(nxt)
         out["cpu_baseline"] = base
-        out["parity_full_size"] = {"max_abs_logit_diff_vs_cpu": float(np.abs(gpu.logits() - lg).max()),
-                                   "top1_agree": float((gpu.logits().argmax(1) == lg.argmax(1)).mean())}
+        gl = gpu.logits()
+        g1, c1 = gl.argmax(1), lg.argmax(1)
+        rows = np.nonzero(g1 != c1)[0]
+        out["parity_full_size"] = {"max_abs_logit_diff_vs_cpu": float(np.abs(gl - lg).max()),
+                                   "top1_agree": float((g1 == c1).mean()), "rows": int(gl.shape[0]),
+                                   # where the choices differ: how far apart the CPU's own logits of the two tokens are
+                                   # (a gap below the logit difference above is a tie at this precision)
+                                   "cpu_logit_gap_where_top1_differs": [float(lg[r, c1[r]] - lg[r, g1[r]]) for r in rows]}
     else:
         out["cpu_baseline"] = None
     print(json.dumps(out))
