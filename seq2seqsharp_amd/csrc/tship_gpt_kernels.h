@@ -1726,51 +1726,60 @@ __global__ __launch_bounds__(D == 128 ? 256 : 512) void attn_mfma_kernel(AttnArg
 }
 
 // Prefill variant: a wavefront owns QB = 16 / G consecutive query positions (the 16 MFMA columns are its positions x
-// the G query heads of the group) and walks over every 32-position chunk of its own causal prefix, so there is no
-// merge across wavefronts.  The NW wavefronts of a block sit at neighbouring positions and fetch the same chunks at
-// about the same time: the block reads its prefix once from L2 and NW - 1 times from L1 (the variant with one such
-// group per block re-read the prefix from L2 for every four query positions).  grid (ceil(Tq / (QB NW)), Hkv, batch).
+// the G query heads of the group), so there is no merge across wavefronts.  The NW wavefronts of a block sit at
+// neighbouring positions and need the same chunks: the block fetches every 32-position chunk of its causal prefix once,
+// straight into LDS (two stages; wavefront w brings fragments w, w + NW, ...), and all wavefronts read their MFMA
+// operands from there.  (With every wavefront streaming its own prefix the kernel was bound by L2: the L1 holds two
+// chunks and the wavefronts drift apart.)  grid (ceil(Tq / (QB NW)), Hkv, batch).
 template <int D, int G>
 __global__ __launch_bounds__(D == 128 ? 256 : 512) void attn_mfma_prefill_kernel(AttnArgs a) {
     constexpr int NW = D == 128 ? 4 : 8;
     constexpr int QB = 16 / G, KD = D / 32, DT = D / 16;
+    constexpr int NF = 2 * KD + DT;          // 1 KiB fragments per chunk: keys (tile, kd), then values (dt)
+    constexpr int FPW = NF / NW;             // fragments a wavefront brings per chunk
+    static_assert(NF % NW == 0, "fragments must divide among the wavefronts");
     __shared__ float sbuf[NW][D * 16];       // per wavefront: Q staging [16 columns][D], later the outputs [D][16 columns]
     __shared__ float sl[NW][16];
+    __shared__ __attribute__((aligned(16))) half_t schunk[2][NF * 512];
     const int lane = threadIdx.x & 63, w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int r16 = lane & 15, q = lane >> 4;
     const int kvh = blockIdx.y, b = blockIdx.z;
     const int tq0 = (blockIdx.x * NW + w) * QB;
-    if (tq0 >= a.Tq) return;                  // no block-wide barrier below
+    const bool active = tq0 < a.Tq;          // wavefronts beyond the prompt still fetch their share of every chunk
     const int pos_base = a.pos0 + tq0, T = min(pos_base + QB, a.pos0 + a.Tq);
-    const int nchunks = (T + 31) / 32;
+    // chunks of the block: up to the last position of its last active wavefront
+    const int tq_last = min(a.Tq, (int)(blockIdx.x + 1) * NW * QB);
+    const int nchunks = (a.pos0 + tq_last + 31) / 32;
     const half_t* Kb = (const half_t*)a.kcache + ((long)b * a.Hkv + kvh) * a.max_len * D;
     const half_t* Vt = (const half_t*)a.vcache + ((long)b * a.Hkv + kvh) * (long)D * a.max_len;
-    half8 kfA[2][KD], vfA[DT], kfB[2][KD], vfB[DT];
-    auto load_chunk = [&](int c, half8 (&kf)[2][KD], half8 (&vf)[DT]) {
-        const half_t* kc = Kb + (long)c * (32 * D) + lane * 8;
-        const half_t* vc = Vt + (long)c * (32 * D) + lane * 8;
+    typedef const void __attribute__((address_space(1)))* gptr_t;
+    typedef void __attribute__((address_space(3)))* lptr_t;
+    auto fetch = [&](int c) {                // this wavefront's fragments of chunk c -> stage c % 2
 #pragma unroll
-        for (int tile = 0; tile < 2; ++tile)
-#pragma unroll
-            for (int kd = 0; kd < KD; ++kd) kf[tile][kd] = *(const half8*)(kc + (tile * KD + kd) * 512);
-#pragma unroll
-        for (int dt = 0; dt < DT; ++dt) vf[dt] = *(const half8*)(vc + dt * 512);
+        for (int i = 0; i < FPW; ++i) {
+            const int f = w + i * NW;
+            const half_t* src = (f < 2 * KD ? Kb + (long)c * (32 * D) + f * 512 : Vt + (long)c * (32 * D) + (f - 2 * KD) * 512) + lane * 8;
+            __builtin_amdgcn_global_load_lds((gptr_t)src, (lptr_t)(&schunk[c & 1][f * 512]), 16, 0, 0);
+        }
     };
-    load_chunk(0, kfA, vfA);                  // chunk 0 is complete or ends at this wavefront's own positions (written by kv_write)
+    fetch(0);
 
     // queries: projection + bias, rotary embedding, 1 / sqrt(d); columns beyond the prompt stay zero
     float* sq = sbuf[w];
     for (int i = lane; i < 16 * D; i += 64) sq[i] = 0.0f;
-    for (int p = lane; p < 16 * D / 2; p += 64) {
-        const int col = p / (D / 2), i = p % (D / 2);
-        const int qi = col / G, g = col % G;
-        if (tq0 + qi >= a.Tq) continue;
-        const long row = (long)b * a.Tq + tq0 + qi;
-        const int pos = pos_base + qi;
-        const int c0 = (kvh * G + g) * D + 2 * i;
-        float x0 = a.qkv[row * a.ldq + c0] + a.bias[c0], x1 = a.qkv[row * a.ldq + c0 + 1] + a.bias[c0 + 1], y0 = x0, y1 = x1;
-        if (a.rope_cos) rope_pair(x0, x1, a.rope_cos[(long)pos * (D / 2) + i], a.rope_sin[(long)pos * (D / 2) + i], y0, y1);
-        sq[col * D + 2 * i] = a.scale * y0; sq[col * D + 2 * i + 1] = a.scale * y1;
+    if (active) {
+        for (int p = lane; p < 16 * D / 2; p += 64) {
+            const int col = p / (D / 2), i = p % (D / 2);
+            const int qi = col / G, g = col % G;
+            if (tq0 + qi >= a.Tq) continue;
+            const long row = (long)b * a.Tq + tq0 + qi;
+            const int pos = pos_base + qi;
+            const int c0 = (kvh * G + g) * D + 2 * i;
+            float x0 = a.qkv[row * a.ldq + c0] + a.bias[c0], x1 = a.qkv[row * a.ldq + c0 + 1] + a.bias[c0 + 1], y0 = x0, y1 = x1;
+            if (a.rope_cos) rope_pair(x0, x1, a.rope_cos[(long)pos * (D / 2) + i], a.rope_sin[(long)pos * (D / 2) + i], y0, y1);
+            // (scores are kept in units of log 2, so that the exponentials below are bare v_exp_f32)
+            sq[col * D + 2 * i] = (a.scale * 1.44269504f) * y0; sq[col * D + 2 * i + 1] = (a.scale * 1.44269504f) * y1;
+        }
     }
     __builtin_amdgcn_wave_barrier();
     half8 qf[KD];
@@ -1784,7 +1793,9 @@ __global__ __launch_bounds__(D == 128 ? 256 : 512) void attn_mfma_prefill_kernel
     floatx4 acc_o[DT];
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) acc_o[dt] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
-    auto do_chunk = [&](int c, half8 (&kf)[2][KD], half8 (&vf)[DT]) {
+    // masked = false: every position of the chunk is visible to every column (all chunks but the last one or two)
+    auto do_chunk = [&](auto masked_c, int c, half8 (&kf)[2][KD], half8 (&vf)[DT]) {
+        constexpr bool MASKED = decltype(masked_c)::value;
         const int t0 = c * 32;
         floatx4 sA = floatx4{0.0f, 0.0f, 0.0f, 0.0f}, sB = sA;
 #pragma unroll
@@ -1798,18 +1809,19 @@ __global__ __launch_bounds__(D == 128 ? 256 : 512) void attn_mfma_prefill_kernel
         float cm = -INFINITY;
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
-            if (t0 + 8 * q + j > tmax) s[j] = -INFINITY;       // causal mask (adding -30000 gives exactly 0 after exp in fp32 too)
+            if (MASKED && t0 + 8 * q + j > tmax) s[j] = -INFINITY;       // causal mask (adding -30000 gives exactly 0 after exp in fp32 too)
             cm = fmaxf(cm, s[j]);
         }
         cm = fmaxf(cm, __shfl_xor(cm, 16, 64));
         cm = fmaxf(cm, __shfl_xor(cm, 32, 64));
         const float m_new = fmaxf(m_run, cm);
-        const float corr = (m_new == -INFINITY) ? 1.0f : __expf(m_run - m_new);
+        // (unmasked chunks have finite scores, so m_new is finite and exp2(-inf - m_new) = 0 covers the first chunk)
+        const float corr = (MASKED && m_new == -INFINITY) ? 1.0f : __builtin_amdgcn_exp2f(m_run - m_new);
         half8 pf;
         float psum = 0.0f;
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
-            const float p = (s[j] == -INFINITY) ? 0.0f : __expf(s[j] - m_new);
+            const float p = (MASKED && s[j] == -INFINITY) ? 0.0f : __builtin_amdgcn_exp2f(s[j] - m_new);
             psum += p;
             pf[j] = (half_t)p;
         }
@@ -1822,12 +1834,29 @@ __global__ __launch_bounds__(D == 128 ? 256 : 512) void attn_mfma_prefill_kernel
             acc_o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vf[dt], pf, acc_o[dt], 0, 0, 0);
         }
     };
-    for (int c = 0; c < nchunks; c += 2) {
-        if (c + 1 < nchunks) load_chunk(c + 1, kfB, vfB);
-        do_chunk(c, kfA, vfA);
-        if (c + 1 >= nchunks) break;
-        if (c + 2 < nchunks) load_chunk(c + 2, kfA, vfA);
-        do_chunk(c + 1, kfB, vfB);
+    // Chunks [0, n_full) lie entirely at or below this wavefront's first query position; chunks from n_own on lie
+    // entirely behind its last one (the block's later wavefronts still need them).
+    const std::integral_constant<bool, false> plain; const std::integral_constant<bool, true> masked;
+    const int n_own = active ? (T + 31) / 32 : 0;
+    const int n_full = min(n_own, (pos_base + 1) / 32);
+    for (int c = 0; c < nchunks; ++c) {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");      // this wavefront's share of chunk c has landed
+        __syncthreads();                                      // ... and everybody's; chunk c - 1 is consumed
+        half8 kf[2][KD], vf[DT];
+        const half_t* st = schunk[c & 1] + lane * 8;
+#pragma unroll
+        for (int tile = 0; tile < 2; ++tile)
+#pragma unroll
+            for (int kd = 0; kd < KD; ++kd) kf[tile][kd] = *(const half8*)(st + (tile * KD + kd) * 512);
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) vf[dt] = *(const half8*)(st + (2 * KD + dt) * 512);
+        // the operands are in registers before the next chunk is requested into the other stage, so the wait the
+        // compiler puts ahead of LDS reads (they might alias the LDS destination of a load in flight) costs nothing
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        __builtin_amdgcn_sched_barrier(0);
+        if (c + 1 < nchunks) fetch(c + 1);
+        if (c < n_full) do_chunk(plain, c, kf, vf);
+        else if (c < n_own) do_chunk(masked, c, kf, vf);
     }
     l_run += __shfl_xor(l_run, 16, 64);
     l_run += __shfl_xor(l_run, 32, 64);
@@ -1839,6 +1868,7 @@ __global__ __launch_bounds__(D == 128 ? 256 : 512) void attn_mfma_prefill_kernel
 #pragma unroll
         for (int i = 0; i < 4; ++i) sq[(dt * 16 + 4 * q + i) * 16 + r16] = acc_o[dt][i];
     __builtin_amdgcn_wave_barrier();
+    if (!active) return;
     for (int col = 0; col < 16; ++col) {
         const int qi = col / G, g = col % G;
         if (tq0 + qi >= a.Tq) break;
