@@ -775,7 +775,14 @@ static void prefill(TSHipGpt* m, const int32_t* host_ids, int B, int Tp) {
         } else {
             run_gemm_f32(m, "p_gemm_qkv", L.qkv, pxn.as<float>(), m->ldh, (int)R, pqkv.as<float>(), qp, 0, 1);
         }
-        launch(m, "p_kv_write", pick_kvw(m), dim3(Tp, B), dim3(256), aa);
+        if (m->vt && aa.pos0 % 32 == 0) {      // whole fragments, one block per 32-position chunk
+            TSHIP_REQUIRE(qp % 4 == 0 && (long)round_up(aa.pos0 + Tp, 32) <= m->ML, "internal: cache chunk beyond the allocation");
+            dim3 grid((unsigned)ceil_div(Tp, 32), c.n_kv_heads, B);
+            if (m->D == 64) launch(m, "p_kv_write", kv_write_frag_kernel<64>, grid, dim3(256), aa);
+            else launch(m, "p_kv_write", kv_write_frag_kernel<128>, grid, dim3(512), aa);
+        } else {
+            launch(m, "p_kv_write", pick_kvw(m), dim3(Tp, B), dim3(256), aa);
+        }
         if (m->vt) {      // a wavefront per 16 / G query positions, 8 (head_dim 64) or 4 (head_dim 128) wavefronts per block
             const int per_block = (16 / m->G) * (m->D == 128 ? 4 : 8);
             launch(m, "p_attn", pick_attn(m, true), dim3((unsigned)ceil_div(Tp, per_block), c.n_kv_heads, B), dim3(m->D == 128 ? 256 : 512), aa);

@@ -1405,6 +1405,60 @@ __global__ __launch_bounds__(256) void kv_write_kernel(AttnArgs a) {
     }
 }
 
+// prefill, step 1 for the fragment-major fp16 cache when the first position starts a 32-position chunk: one block per
+// (chunk, KV head, batch row) writes the chunk's key and value fragments whole, 16 bytes per lane (the kernel above
+// scatters two-byte elements from one small block per position).  Wavefront w: key fragment w (tile w / KD, kd w % KD)
+// and value fragment w (dt = w).  grid (ceil(Tq / 32), Hkv, batch), D / 16 wavefronts.
+template <int D>
+__global__ __launch_bounds__(D * 4) void kv_write_frag_kernel(AttnArgs a) {
+    constexpr int KD = D / 32;
+    const int chunk = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    const int r = lane & 15, qq = lane >> 4;
+    const int HD = a.H * D, GD = a.Hkv * D;
+    const long cabs = (a.pos0 >> 5) + chunk;                     // chunk index in the cache (pos0 is a multiple of 32)
+    half_t* Kh = (half_t*)a.kcache + ((long)b * a.Hkv + kvh) * a.max_len * D + cabs * (32 * D);
+    half_t* Vh = (half_t*)a.vcache + ((long)b * a.Hkv + kvh) * (long)D * a.max_len + cabs * (32 * D);
+    {   // keys: lane (r, qq) of fragment (tile, kd) holds position 8 (r / 4) + 4 tile + r % 4, d = 32 kd + 8 qq .. + 7
+        const int tile = w / KD, kd = w % KD;
+        const int tq = chunk * 32 + 8 * (r >> 2) + 4 * tile + (r & 3);
+        const int d0 = 32 * kd + 8 * qq;
+        half8 o = half8{0, 0, 0, 0, 0, 0, 0, 0};
+        if (tq < a.Tq) {
+            const long row = (long)b * a.Tq + tq;
+            const int pos = a.pos0 + tq;
+            const int col = HD + kvh * D + d0;
+            const floatx4 x0 = *(const floatx4*)(a.qkv + row * a.ldq + col), x1 = *(const floatx4*)(a.qkv + row * a.ldq + col + 4);
+            const floatx4 b0 = *(const floatx4*)(a.bias + col), b1 = *(const floatx4*)(a.bias + col + 4);
+            float x[8];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) { x[j] = x0[j] + b0[j]; x[4 + j] = x1[j] + b1[j]; }
+#pragma unroll
+            for (int pr = 0; pr < 4; ++pr) {
+                float y0 = x[2 * pr], y1 = x[2 * pr + 1];
+                if (a.rope_cos) {
+                    const int i = d0 / 2 + pr;
+                    rope_pair(x[2 * pr], x[2 * pr + 1], a.rope_cos[(long)pos * (D / 2) + i], a.rope_sin[(long)pos * (D / 2) + i], y0, y1);
+                }
+                o[2 * pr] = (half_t)y0; o[2 * pr + 1] = (half_t)y1;
+            }
+        }
+        *(half8*)(Kh + (long)w * 512 + lane * 8) = o;
+    }
+    {   // values: lane (r, qq) of fragment dt holds d = 16 dt + r at positions 8 qq .. 8 qq + 7
+        const int d = 16 * w + r;
+        const int col = HD + GD + kvh * D + d;
+        const float bv = a.bias[col];
+        half8 o;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const int tq = chunk * 32 + 8 * qq + j;
+            o[j] = tq < a.Tq ? (half_t)(a.qkv[((long)b * a.Tq + tq) * a.ldq + col] + bv) : (half_t)0.0f;
+        }
+        *(half8*)(Vh + (long)w * 512 + lane * 8) = o;
+    }
+}
+
 // prefill, step 2: grid (Tq, Hkv, batch).  Causal attention of query row tq over cache positions 0..pos0+tq.
 // The reference adds -30000 to masked scores (TensorApplyCPU.cs:1016-1036, Decoder.cs:685-686); exp(-30000 - max)
 // is exactly 0 in fp32, so leaving masked positions out gives the same sums.
