@@ -147,8 +147,9 @@ TSHIP_API int TSHip_GptSetWeight(TSHipGpt* m, const char* name, const float* hos
 TSHIP_API int TSHip_GptFinalize(TSHipGpt* m);
 /* drop the KV cache contents (GPT.cs:236-247: a new dictionary per call) */
 TSHIP_API int TSHip_GptReset(TSHipGpt* m);
-/* prefill: ids [batch, prompt_len] int32 on the host, equal lengths; fills the cache and leaves the
- * last-position logits on the device (Decoder.cs:679-716) */
+/* prefill: ids [batch, prompt_len] int32 on the host, equal lengths; appends them to the cached sequences (the cache is
+ * empty after Create / Reset; a later call continues the same sequences, e.g. the next turn of a dialogue whose cache
+ * was kept, GPT.cs:236-247,312-328) and leaves the last-position logits on the device (Decoder.cs:679-716) */
 TSHIP_API int TSHip_GptPrefill(TSHipGpt* m, const int32_t* host_ids, int batch, int prompt_len);
 /* one decode step with the given tokens (Decoder.cs:661-678); leaves logits on the device */
 TSHIP_API int TSHip_GptDecode(TSHipGpt* m, const int32_t* host_ids, int batch);

@@ -688,13 +688,14 @@ static void prefill(TSHipGpt* m, const int32_t* host_ids, int B, int Tp) {
     const int h = c.hidden, F = c.ffn_dim;
     const long R = (long)B * Tp, Rp = round_up(R, 128);
     const long qp = round_up(m->Nqkv, 32);
-    TSHIP_REQUIRE(m->pos == 0, "TSHip_GptPrefill: the cache is not empty; call TSHip_GptReset first");
-    TSHIP_REQUIRE(Tp >= 1 && Tp < c.max_seq_len, "TSHip_GptPrefill: prompt length exceeds max_seq_len");
+    const int pos0 = m->pos;              // tokens are appended behind what the cache holds (nothing after Create / Reset)
+    TSHIP_REQUIRE(pos0 == 0 || m->cur_batch == B, "TSHip_GptPrefill: batch differs from the cached sequences; call TSHip_GptReset first");
+    TSHIP_REQUIRE(Tp >= 1 && pos0 + Tp < c.max_seq_len, "TSHip_GptPrefill: prompt length exceeds max_seq_len");
     // prefill workspace: kept in the model and only ever grown, so that repeated prefills do not pay for allocation
     DevBuf &ids = m->pw_ids, &px = m->pw_x, &pxn = m->pw_xn, &pqkv = m->pw_qkv, &po = m->pw_o, &pa = m->pw_a, &pf = m->pw_f, &rowmap = m->pw_rowmap;
     ids.reserve(R * sizeof(int));
     TSHIP_CHECK_HIP(hipMemcpyAsync(ids.p, host_ids, R * sizeof(int), hipMemcpyHostToDevice, stream()));
-    record_history(m, ids.as<int>(), B, Tp, 0);
+    record_history(m, ids.as<int>(), B, Tp, pos0);
     px.reserve((size_t)Rp * h * sizeof(float));
     pxn.reserve((size_t)Rp * m->ldh * m->esz());
     pqkv.reserve((size_t)Rp * qp * sizeof(float));
@@ -764,7 +765,7 @@ static void prefill(TSHipGpt* m, const int32_t* host_ids, int B, int Tp) {
     for (int l = 0; l < c.n_layers; ++l) {
         LayerW& L = *m->L[l];
         AttnArgs aa = attn_args(m, L);
-        aa.qkv = pqkv.as<float>(); aa.KS = 1; aa.split_stride = 0; aa.ldq = qp; aa.pos0 = 0; aa.Tq = Tp;
+        aa.qkv = pqkv.as<float>(); aa.KS = 1; aa.split_stride = 0; aa.ldq = qp; aa.pos0 = pos0; aa.Tq = Tp;
         aa.out = po.p; aa.ld_out = m->ldh;
         if (m->f16) {
             BigArgs e; std::memset(&e, 0, sizeof(e));
@@ -852,7 +853,7 @@ static void prefill(TSHipGpt* m, const int32_t* host_ids, int B, int Tp) {
     } else {
         run_gemm_f32(m, "gemm_head", m->head, m->xn.as<float>(), m->ldh, B, m->logits.as<float>(), Vp, 0, 1, m->head_b.as<float>());
     }
-    m->pos = Tp;
+    m->pos = pos0 + Tp;
     TSHIP_CHECK_HIP(hipMemcpyAsync(m->d_pos.p, &m->pos, sizeof(int), hipMemcpyHostToDevice, stream()));
     TSHIP_CHECK_HIP(hipStreamSynchronize(stream()));
     m->cur_batch = B;
@@ -1065,7 +1066,10 @@ TSHIP_API int TSHip_GptPrefill(TSHipGpt* m, const int32_t* host_ids, int batch, 
             for (int b = 0; b < batch; ++b) col[b] = host_ids[(long)b * prompt_len + t];
             TSHIP_CHECK_HIP(hipMemcpyAsync(m->ids.p, col.data(), batch * sizeof(int), hipMemcpyHostToDevice, stream()));
             TSHIP_CHECK_HIP(hipStreamSynchronize(stream()));
-            if (t == 0) TSHIP_REQUIRE(m->pos == 0, "TSHip_GptPrefill: the cache is not empty; call TSHip_GptReset first");
+            if (t == 0) {
+                TSHIP_REQUIRE(m->pos == 0 || m->cur_batch == batch, "TSHip_GptPrefill: batch differs from the cached sequences; call TSHip_GptReset first");
+                TSHIP_REQUIRE(m->pos + prompt_len < m->c.max_seq_len, "TSHip_GptPrefill: prompt length exceeds max_seq_len");
+            }
             record_history(m, m->ids.as<int>(), batch, 1, m->pos);
             decode_step(m, m->ids.as<int>(), batch);
         }

@@ -458,6 +458,37 @@ def test_decode_attention_split_over_blocks(G, oracle, monkeypatch, hidden, head
     gpu.close()
 
 
+@pytest.mark.parametrize("dtype,hidden,heads,kv_heads,first,second", [("f32", 64, 4, 2, 5, 7), ("f16", 256, 4, 2, 64, 40), ("f16", 256, 4, 2, 45, 530),
+                                                                    ("f16", 512, 4, 1, 32, 33)])
+def test_prefill_appends_to_cached_sequences(G, oracle, dtype, hidden, heads, kv_heads, first, second):
+    """A second prefill continues the cached sequences (the next turn of a dialogue whose cache was kept): the logits
+    and the cache are those of one prefill of the concatenation, and decoding goes on from there.  Covers a first part
+    that ends on a 32-position boundary (whole fragments written) and ones that do not, head_dim 64 and 128, and the
+    LDS-tiled GEMMs (530 x 2 rows)."""
+    cfg = synth.tiny_config(dtype=dtype, hidden=hidden, n_heads=heads, n_kv_heads=kv_heads, ffn_dim=2 * hidden, vocab=300, batch=2, prompt=first + second)
+    w = synth.make_weights(cfg, 91, random_bias=True)
+    orc = oracle.OracleGpt(cfg, w)
+    seqs = synth.make_prompts(cfg, 92)
+    gpu = G.HipGpt(cfg, w, max_batch=2, max_seq_len=first + second + 8)
+    gpu.prefill(seqs)
+    whole = gpu.logits()
+    k_whole = gpu.get_kv(cfg["n_layers"] - 1, 0)
+    gpu.reset()
+    gpu.prefill(seqs[:, :first])
+    gpu.prefill(seqs[:, first:])
+    assert gpu.seq_len() == first + second
+    tol = 1e-4 * float(np.abs(whole).max()) if dtype == "f32" else 2e-2
+    assert np.abs(gpu.logits() - whole).max() <= tol
+    assert np.abs(gpu.get_kv(cfg["n_layers"] - 1, 0) - k_whole).max() <= (1e-5 if dtype == "f32" else 2e-2)
+    p, lg = orc.step(seqs, use_cache=True)
+    assert np.abs(gpu.logits() - lg).max() <= (1e-4 * float(np.abs(lg).max()) if dtype == "f32" else FP16_ABS)
+    nxt = oracle.argmax(p).astype(np.int32)
+    p, lg = orc.step(np.concatenate([seqs, nxt[:, None]], 1), use_cache=True)
+    gpu.decode(nxt)
+    assert np.abs(gpu.logits() - lg).max() <= (1e-4 * float(np.abs(lg).max()) if dtype == "f32" else FP16_ABS)
+    gpu.close()
+
+
 def test_blocked_tokens(G, oracle):
     """Decoder.cs:745-753: probs += scatter(-1 at the blocked ids) before argmax / TopPSample."""
     cfg = synth.tiny_config(batch=4, vocab=120)
