@@ -364,6 +364,25 @@ static void run_skinny(TSHipGpt* m, const char* name, const GemmW& w, const void
     TSHIP_REQUIRE(epi != EPI_SPLIT_TAIL || (m->BT == 1 && e.tile_count), "internal: the split tail needs one batch tile and the tile counters");
     dim3 grid(w.NT * e.KS);
     const int BT = m->BT;
+    if (epi == EPI_ACT16 && BT == 1) {
+        // Column tiles per block.  A launch lasts as long as its busiest compute unit, and a unit's time goes with the
+        // bytes it requests: the block's weight tiles and one copy of the activations (as large as one tile).  Costs in
+        // half tiles: rounds of blocks over the units x (2 per tile + 2); 15 stands for a tile and a half per block.
+        const int ncu = n_compute_units();
+        int best = 10; long best_cost = ceil_div(w.NT, ncu) * 4;
+        const long hb = 2 * (w.NT / 3) + w.NT % 3, hcost = ceil_div(hb, ncu) * 5;
+        if (hcost < best_cost) { best = 15; best_cost = hcost; }
+        for (int nj = 2; nj <= 4; ++nj) {
+            const long cost = ceil_div(ceil_div(w.NT, nj), ncu) * (2 * nj + 2);
+            if (cost < best_cost) { best = 10 * nj; best_cost = cost; }
+        }
+        if (const char* v = std::getenv("TSHIP_FFN_TILES")) best = std::atoi(v);      // (tests: 10, 15, 20, 30 or 40)
+        if (best == 15) { launch(m, name, skinny_gemm_f16_kernel<1, EPI_ACT16, 8, 8, 2, true>, dim3((unsigned)hb), dim3(512), e); return; }
+        if (best == 20) { launch(m, name, skinny_gemm_f16_kernel<1, EPI_ACT16, 8, 8, 2>, dim3((unsigned)ceil_div(w.NT, 2)), dim3(512), e); return; }
+        if (best == 30) { launch(m, name, skinny_gemm_f16_kernel<1, EPI_ACT16, 8, 4, 3>, dim3((unsigned)ceil_div(w.NT, 3)), dim3(512), e); return; }
+        if (best == 40) { launch(m, name, skinny_gemm_f16_kernel<1, EPI_ACT16, 8, 4, 4>, dim3((unsigned)ceil_div(w.NT, 4)), dim3(512), e); return; }
+        TSHIP_REQUIRE(best == 10, "TSHIP_FFN_TILES: 10, 15, 20, 30 or 40");
+    }
 #define TSHIP_SK(BTV, NWV)                                                                                                  \
     if (epi == EPI_PARTIAL) launch(m, name, skinny_gemm_f16_kernel<BTV, EPI_PARTIAL, NWV>, grid, dim3(NWV * 64), e);        \
     else if (epi == EPI_F32_BIAS) launch(m, name, skinny_gemm_f16_kernel<BTV, EPI_F32_BIAS, NWV>, grid, dim3(NWV * 64), e); \

@@ -110,8 +110,19 @@ struct SkinnyArgs {
 // 8 weight fragments and 8 activation fragments (16 KiB) in flight.  Accumulators are added pairwise through LDS
 // (a fixed tree, so the sum order never changes); the last two are transposed through LDS so that the epilogue
 // writes coalesced rows.  X is fragment packed (xpack_index).
-template <int BT, int EPI, int NW, int U = 8>
+// NJ > 1 (activation epilogue only): the block works on NJ neighbouring column tiles with one copy of the activation
+// fragments.  A compute unit turns over a fixed number of requested bytes per microsecond, weights from HBM and
+// activations from L2 alike, and a launch lasts as long as its busiest unit; 352 tiles of 32 columns on 256 units
+// mean two tiles, twice 128 KiB of weights plus twice 128 KiB of activations, on the busiest ones.  176 blocks of two
+// tiles request 256 + 128 KiB each.  HALF: a block takes one tile and half of a neighbour (three blocks' worth of
+// tiles go to two blocks; 235 blocks of 192 + 128 KiB for 352 tiles).  A half tile is columns 0-7 and 16-23 of the
+// tile, or 8-15 and 24-31: whole 128-byte runs of a weight fragment, and both factors of a gated pair (n, n + 16).
+// The lanes of the other columns fetch their neighbours' bytes again (same cache lines, no further request) and
+// compute sums that are never stored.
+template <int BT, int EPI, int NW, int U = 8, int NJ = 1, bool HALF = false>
 __global__ __launch_bounds__(NW * 64) void skinny_gemm_f16_kernel(SkinnyArgs a) {
+    static_assert(!HALF || NJ == 2, "tile-and-a-half blocks are two-tile blocks with one tile half masked");
+    static_assert(NJ == 1 || (EPI == EPI_ACT16 && BT == 1 && NW == 8), "several column tiles per block: one-round activation epilogue only");
     // one batch tile and eight wavefronts: every wavefront stores its accumulator once and the epilogue adds the eight
     // copies in wavefront order (one barrier); otherwise a pairwise tree followed by a transpose
     constexpr bool ONE_ROUND = BT == 1 && NW == 8 && (EPI == EPI_ACT16 || EPI == EPI_RESID_TAIL || EPI == EPI_SPLIT_TAIL);   // fp32 outputs keep the transpose: coalesced rows
@@ -128,17 +139,35 @@ __global__ __launch_bounds__(NW * 64) void skinny_gemm_f16_kernel(SkinnyArgs a) 
         if (a.out16) a.out16 += e * a.out16_estride;
     }
     const int lane = threadIdx.x & 63, w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int nt = blockIdx.x / a.KS, ks = blockIdx.x % a.KS;
+    const int ks = blockIdx.x % a.KS;
+    // tile of slot j, and for a half tile which one: 0 whole, 1 columns 0-7 / 16-23, 2 columns 8-15 / 24-31
+    int tile_of[NJ], half_of[NJ];
+    if constexpr (HALF) {
+        const int grp = blockIdx.x >> 1, odd = blockIdx.x & 1, whole = (a.NT / 3) * 2;
+        if ((int)blockIdx.x < whole) {
+            tile_of[0] = 3 * grp + odd; half_of[0] = odd ? 2 : 0;
+            tile_of[1] = 3 * grp + 1 + odd; half_of[1] = odd ? 0 : 1;
+        } else {      // the one or two tiles left over: a block each
+            tile_of[0] = 3 * (a.NT / 3) + ((int)blockIdx.x - whole); half_of[0] = 0;
+            tile_of[1] = a.NT; half_of[1] = 0;
+        }
+    } else {
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) { tile_of[j] = (blockIdx.x / a.KS) * NJ + j; half_of[j] = 0; }
+    }
+    const int nt = tile_of[0];
     const int per = (a.KT + a.KS - 1) / a.KS;
     const int k0 = ks * per, k1 = min(a.KT, k0 + per);
     const int pw = (max(k1 - k0, 0) + NW - 1) / NW;
     const int wk0 = k0 + w * pw, wk1 = min(k1, wk0 + pw);
 
-    floatx16 acc[BT];
+    floatx16 acc[NJ][BT];
 #pragma unroll
-    for (int bt = 0; bt < BT; ++bt)
+    for (int j = 0; j < NJ; ++j)
 #pragma unroll
-        for (int v = 0; v < 16; ++v) acc[bt][v] = 0.0f;
+        for (int bt = 0; bt < BT; ++bt)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[j][bt][v] = 0.0f;
 
     // deferred-norm inputs: this thread's share of the per-tile sums of squares, fetched before the weight stream
     __shared__ float srinv[BT * 32];
@@ -160,16 +189,20 @@ __global__ __launch_bounds__(NW * 64) void skinny_gemm_f16_kernel(SkinnyArgs a) 
         }
     }
     // bias of this thread's outputs in the one-round activation epilogue
-    float eb1 = 0.0f, eb2 = 0.0f;
-    if (ONE_ROUND && EPI == EPI_ACT16) {
-        const int n1 = 8 * (w >> 2) + 4 * (lane >> 5) + (w & 3);
-        if (a.gated) {
-            const int f = nt * 16 + n1;
-            if (f < a.n_valid) { eb1 = a.bias[f]; eb2 = a.bias2[f]; }
-        } else {
-            const int f = nt * 32 + n1;
-            if (f < a.n_valid) eb1 = a.bias[f];
-            if (f + 16 < a.n_valid) eb2 = a.bias[f + 16];
+    float eb1[NJ], eb2[NJ];
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+        eb1[j] = 0.0f; eb2[j] = 0.0f;
+        if (ONE_ROUND && EPI == EPI_ACT16) {
+            const int n1 = 8 * (w >> 2) + 4 * (lane >> 5) + (w & 3);
+            if (a.gated) {
+                const int f = tile_of[j] * 16 + n1;
+                if (f < a.n_valid) { eb1[j] = a.bias[f]; eb2[j] = a.bias2[f]; }
+            } else {
+                const int f = tile_of[j] * 32 + n1;
+                if (f < a.n_valid) eb1[j] = a.bias[f];
+                if (f + 16 < a.n_valid) eb2[j] = a.bias[f + 16];
+            }
         }
     }
     // residual tail: the old residual, bias and gamma of this thread's outputs do not depend on the product
@@ -188,17 +221,25 @@ __global__ __launch_bounds__(NW * 64) void skinny_gemm_f16_kernel(SkinnyArgs a) 
             tail_g[it] = ok ? a.gamma[col] : 0.0f;
         }
     }
-    const half_t* wp = a.W + ((long)nt * a.KT * 64 + lane) * 8;
+    // (a tile beyond the last one reads the last one again; nothing of it is stored)
+    const half_t* wp[NJ];
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+        // lane l feeds column l % 32 of the tile; the lanes outside a half tile read what their neighbours 8 columns away read
+        const int src = half_of[j] == 1 ? (lane & ~8) : half_of[j] == 2 ? (lane | 8) : lane;
+        wp[j] = a.W + ((long)min(tile_of[j], a.NT - 1) * a.KT * 64 + src) * 8;
+    }
     const half_t* xp = a.X + lane * 8;
     // Full batches of U k-tiles run without conditions: a request under a condition of its own would make every
     // later wait cover all requests, and the products could not start while the batch is still arriving.
     int kt = wk0;
     for (; kt + U <= wk1; kt += U) {
-        half8 wf[U];
+        half8 wf[U][NJ];
         half8 xf[U][BT];
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            wf[u] = *(const half8*)(wp + (long)(kt + u) * 512);
+#pragma unroll
+            for (int j = 0; j < NJ; ++j) wf[u][j] = *(const half8*)(wp[j] + (long)(kt + u) * 512);
 #pragma unroll
             for (int bt = 0; bt < BT; ++bt) xf[u][bt] = *(const half8*)(xp + ((long)bt * a.KT + kt + u) * 512);
         }
@@ -206,16 +247,19 @@ __global__ __launch_bounds__(NW * 64) void skinny_gemm_f16_kernel(SkinnyArgs a) 
 #pragma unroll
         for (int u = 0; u < U; ++u)
 #pragma unroll
-            for (int bt = 0; bt < BT; ++bt) acc[bt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf[u], xf[u][bt], acc[bt], 0, 0, 0);
+            for (int j = 0; j < NJ; ++j)
+#pragma unroll
+                for (int bt = 0; bt < BT; ++bt) acc[j][bt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf[u][j], xf[u][bt], acc[j][bt], 0, 0, 0);
         __builtin_amdgcn_sched_barrier(0);
     }
     if (kt < wk1) {
-        half8 wf[U];
+        half8 wf[U][NJ];
         half8 xf[U][BT];
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             if (kt + u < wk1) {
-                wf[u] = *(const half8*)(wp + (long)(kt + u) * 512);
+#pragma unroll
+                for (int j = 0; j < NJ; ++j) wf[u][j] = *(const half8*)(wp[j] + (long)(kt + u) * 512);
 #pragma unroll
                 for (int bt = 0; bt < BT; ++bt) xf[u][bt] = *(const half8*)(xp + ((long)bt * a.KT + kt + u) * 512);
             }
@@ -224,7 +268,9 @@ __global__ __launch_bounds__(NW * 64) void skinny_gemm_f16_kernel(SkinnyArgs a) 
         for (int u = 0; u < U; ++u) {
             if (kt + u < wk1) {
 #pragma unroll
-                for (int bt = 0; bt < BT; ++bt) acc[bt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf[u], xf[u][bt], acc[bt], 0, 0, 0);
+                for (int j = 0; j < NJ; ++j)
+#pragma unroll
+                    for (int bt = 0; bt < BT; ++bt) acc[j][bt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf[u][j], xf[u][bt], acc[j][bt], 0, 0, 0);
             }
         }
     }
@@ -242,9 +288,46 @@ __global__ __launch_bounds__(NW * 64) void skinny_gemm_f16_kernel(SkinnyArgs a) 
         }
     }
     if (a.advance_pos && blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) { a.advance_pos[0] += 1; a.advance_pos[1] += 1; }
-    if constexpr (ONE_ROUND) {
+    if constexpr (ONE_ROUND && NJ > 1) {
+        // the column tiles one after the other through the same LDS buffer
+        const int b = lane & 31, n1 = 8 * (w >> 2) + 4 * (lane >> 5) + (w & 3);
+        const bool rok = b < a.rows_valid;
 #pragma unroll
-        for (int v = 0; v < 16; ++v) red[w][0][v][lane] = acc[0][v];
+        for (int j = 0; j < NJ; ++j) {
+            if (tile_of[j] >= a.NT) break;
+            if (j) __syncthreads();
+#pragma unroll
+            for (int v = 0; v < 16; ++v) red[w][0][v][lane] = acc[j][0][v];
+            __syncthreads();
+            float s1 = red[0][0][w][lane], s2 = red[0][0][w + 8][lane];
+#pragma unroll
+            for (int i = 1; i < NW; ++i) { s1 += red[i][0][w][lane]; s2 += red[i][0][w + 8][lane]; }
+            const float rinv = a.ssq ? srinv[b] : 1.0f;
+            // (outputs n1 and n1 + 16 belong to the first half of a tile when n1 < 8)
+            const bool mine = half_of[j] == 0 || (half_of[j] == 1) == (n1 < 8);
+            if (a.gated) {
+                const int f = tile_of[j] * 16 + n1;
+                if (rok && mine && f < a.n_valid) {
+                    const float val = act_apply(a.act, s1 * rinv + eb1[j]) * (s2 * rinv + eb2[j]);
+                    if (a.out16_kt > 0) a.out16[xpack_index(b, f, a.out16_kt)] = (half_t)val;
+                    else a.out16[(long)b * a.ld16 + f] = (half_t)val;
+                }
+            } else {
+#pragma unroll
+                for (int q = 0; q < 2; ++q) {
+                    const int f = tile_of[j] * 32 + n1 + 16 * q;
+                    if (rok && mine && f < a.n_valid) {
+                        const float val = act_apply(a.act, (q ? s2 : s1) * rinv + (q ? eb2[j] : eb1[j]));
+                        if (a.out16_kt > 0) a.out16[xpack_index(b, f, a.out16_kt)] = (half_t)val;
+                        else a.out16[(long)b * a.ld16 + f] = (half_t)val;
+                    }
+                }
+            }
+        }
+        return;
+    } else if constexpr (ONE_ROUND) {
+#pragma unroll
+        for (int v = 0; v < 16; ++v) red[w][0][v][lane] = acc[0][0][v];
         __syncthreads();
         // thread (wavefront w, lane): registers v = w and w + 8 of all eight copies -> batch row lane % 32, columns
         // n1 = 8 (w / 4) + 4 (lane / 32) + w % 4 and n1 + 16 (the gate's two factors when the tile is interleaved)
@@ -297,7 +380,7 @@ __global__ __launch_bounds__(NW * 64) void skinny_gemm_f16_kernel(SkinnyArgs a) 
             if (a.gated) {
                 const int f = nt * 16 + n1;
                 if (rok && f < a.n_valid) {
-                    const float val = act_apply(a.act, s1 * rinv + eb1) * (s2 * rinv + eb2);
+                    const float val = act_apply(a.act, s1 * rinv + eb1[0]) * (s2 * rinv + eb2[0]);
                     if (a.out16_kt > 0) a.out16[xpack_index(b, f, a.out16_kt)] = (half_t)val;
                     else a.out16[(long)b * a.ld16 + f] = (half_t)val;
                 }
@@ -306,7 +389,7 @@ __global__ __launch_bounds__(NW * 64) void skinny_gemm_f16_kernel(SkinnyArgs a) 
                 for (int q = 0; q < 2; ++q) {
                     const int f = nt * 32 + n1 + 16 * q;
                     if (rok && f < a.n_valid) {
-                        const float val = act_apply(a.act, (q ? s2 : s1) * rinv + (q ? eb2 : eb1));
+                        const float val = act_apply(a.act, (q ? s2 : s1) * rinv + (q ? eb2[0] : eb1[0]));
                         if (a.out16_kt > 0) a.out16[xpack_index(b, f, a.out16_kt)] = (half_t)val;
                         else a.out16[(long)b * a.ld16 + f] = (half_t)val;
                     }
@@ -344,14 +427,14 @@ __global__ __launch_bounds__(NW * 64) void skinny_gemm_f16_kernel(SkinnyArgs a) 
 #pragma unroll
             for (int bt = 0; bt < BT; ++bt)
 #pragma unroll
-                for (int v = 0; v < 16; ++v) red[w - half][bt][v][lane] = acc[bt][v];
+                for (int v = 0; v < 16; ++v) red[w - half][bt][v][lane] = acc[0][bt][v];
         }
         __syncthreads();
         if (w < half) {
 #pragma unroll
             for (int bt = 0; bt < BT; ++bt)
 #pragma unroll
-                for (int v = 0; v < 16; ++v) acc[bt][v] += red[w][bt][v][lane];
+                for (int v = 0; v < 16; ++v) acc[0][bt][v] += red[w][bt][v][lane];
         }
         __syncthreads();
     }
@@ -360,7 +443,7 @@ __global__ __launch_bounds__(NW * 64) void skinny_gemm_f16_kernel(SkinnyArgs a) 
 #pragma unroll
         for (int bt = 0; bt < BT; ++bt)
 #pragma unroll
-            for (int v = 0; v < 16; ++v) fin[w][bt * 32 + (lane & 31)][8 * (v / 4) + 4 * (lane >> 5) + (v % 4)] = acc[bt][v];
+            for (int v = 0; v < 16; ++v) fin[w][bt * 32 + (lane & 31)][8 * (v / 4) + 4 * (lane >> 5) + (v % 4)] = acc[0][bt][v];
     }
     __syncthreads();
     float keep[ITER];

@@ -458,6 +458,30 @@ def test_decode_attention_split_over_blocks(G, oracle, monkeypatch, hidden, head
     gpu.close()
 
 
+@pytest.mark.parametrize("name,tiles", [("gqa_rms_gate", 20), ("gqa_rms_gate", 30), ("gqa_rms_gate_silu", 40), ("mha_ln_relu", 20),
+                                        ("odd_sizes", 30), ("gqa_leaky_d32_g4", 40), ("gqa_rms_gate", 15), ("mha_ln_relu", 15),
+                                        ("odd_sizes", 15), ("gqa_leaky_d32_g4", 15), ("gqa_rms_gate_silu", 15)])
+def test_decode_ffn_up_projection_several_tiles_per_block(G, oracle, monkeypatch, name, tiles):
+    """Decode, FFN up projection: a block takes several neighbouring 32-column tiles with one copy of the activations
+    (the library does so when that shortens the busiest compute unit's work: more column tiles than compute units).  The
+    environment variable forces two, three and four tiles (20, 30, 40) and a tile and a half (15: one tile plus the
+    columns 0-7 / 16-23 or 8-15 / 24-31 of a neighbour) here: gated and plain activations, RMSNorm (deferred) and
+    LayerNorm, and tile counts that are no multiple of the tiles per block (the last blocks then have fewer)."""
+    monkeypatch.setenv("TSHIP_FFN_TILES", str(tiles))
+    cfg = synth.tiny_config(dtype="f16", **TINY[name])
+    orc, gpu, out, _ = _teacher_forced(G, oracle, cfg, 5, 5)
+    for lg, gl in out:
+        assert np.abs(gl - lg).max() <= FP16_ABS
+    forced = [gl for _, gl in out]
+    gpu.close()
+    # one tile per block computes the same sums in the same order: bit-equal logits
+    monkeypatch.setenv("TSHIP_FFN_TILES", "10")
+    _, gpu, out, _ = _teacher_forced(G, oracle, cfg, 5, 5)
+    for a, (_, b) in zip(forced, out):
+        assert np.array_equal(a, b)
+    gpu.close()
+
+
 @pytest.mark.parametrize("dtype,hidden,heads,kv_heads,first,second", [("f32", 64, 4, 2, 5, 7), ("f16", 256, 4, 2, 64, 40), ("f16", 256, 4, 2, 45, 530),
                                                                     ("f16", 512, 4, 1, 32, 33)])
 def test_prefill_appends_to_cached_sequences(G, oracle, dtype, hidden, heads, kv_heads, first, second):
