@@ -97,7 +97,7 @@ struct TSHipGpt {
     // decode state
     DevBuf x, xn, o, a, part_qkv, part_h, part_f, logits, ids, d_pos, hidden;
     DevBuf moe_ws, topp_scratch, topp_uni, gen_buf, uni_buf, tile_count;
-    DevBuf pw_ids, pw_x, pw_xn, pw_qkv, pw_o, pw_a, pw_f, pw_rowmap, pw_ssq, pw_rinv, pw_zero_bias;     // prefill workspace
+    DevBuf pw_ids, pw_x, pw_xn, pw_qkv, pw_o, pw_a, pw_f, pw_rowmap, pw_ssq, pw_rinv, pw_zero_bias, pw_moe;     // prefill workspace
     DevBuf ssq;                    // deferred-norm path: per-column-tile sums of squares [h/32][Bpad]
     bool fused_norm = false;       // fp16 + RMSNorm + dense layers: residual/norm folded into the GEMM tails
     bool vt = false;               // fp16 cache with head_dim 64/128: keys and values stored fragment-major for the MFMA attention kernels
@@ -403,6 +403,34 @@ static void run_gemm_f32(TSHipGpt* m, const char* name, const GemmW& w, const fl
     launch(m, name, gemm_f32_kernel, grid, dim3(256), g);
 }
 
+// Y = X * W for many rows (prefill), fp16: LDS-tiled MFMA kernels from 512 rows on, 128 x 128 tiles below.  X row-major
+// with at least round_up(R, 128) rows allocated (the small-tile kernel reads whole row tiles; rows from R on are never stored).
+static void run_big_gemm(TSHipGpt* m, const char* name, const GemmW& w, const void* X, long ldx, long R, int epi, BigArgs e) {
+    const long Rp = round_up(R, 128);
+    e.W = w.buf.as<half_t>(); e.KT = w.KT; e.NT = w.NT; e.X = (const half_t*)X; e.ldx = (int)ldx; e.R = (int)R;
+    if (R >= 512) {       // LDS-tiled kernel, 256 x 256 block tile
+        constexpr int CK = 4;
+        const unsigned shm = 2u * 2u * 8u * CK * 1024u;
+        // one-dimensional grid of 8-row x 4-column tile patches, 32 blocks each, rounded up to whole rounds of 8 patches
+        const long CT = ceil_div(w.NT, 8), RT = ceil_div(R, 256), patches = ceil_div(CT, 4) * ceil_div(RT, 8);
+        dim3 grid((unsigned)(round_up(patches, 8) * 32));
+        if (w.KT % 2 == 0) {      // asynchronous staging: four stages of two k-tiles
+            if (epi == BEPI_F32_BIAS) launch_shm(m, name, big_gemm3_f16_kernel<BEPI_F32_BIAS>, grid, dim3(256), shm, e);
+            else if (epi == BEPI_RESID) launch_shm(m, name, big_gemm3_f16_kernel<BEPI_RESID>, grid, dim3(256), shm, e);
+            else launch_shm(m, name, big_gemm3_f16_kernel<BEPI_ACT16>, grid, dim3(256), shm, e);
+            return;
+        }
+        if (epi == BEPI_F32_BIAS) launch_shm(m, name, big_gemm2_f16_kernel<BEPI_F32_BIAS, CK>, grid, dim3(256), shm, e);
+        else if (epi == BEPI_RESID) launch_shm(m, name, big_gemm2_f16_kernel<BEPI_RESID, CK>, grid, dim3(256), shm, e);
+        else launch_shm(m, name, big_gemm2_f16_kernel<BEPI_ACT16, CK>, grid, dim3(256), shm, e);
+        return;
+    }
+    dim3 grid((unsigned)ceil_div(w.NT, 4), (unsigned)(Rp / 128));
+    if (epi == BEPI_F32_BIAS) launch(m, name, big_gemm_f16_kernel<BEPI_F32_BIAS>, grid, dim3(256), e);
+    else if (epi == BEPI_RESID) launch(m, name, big_gemm_f16_kernel<BEPI_RESID>, grid, dim3(256), e);
+    else launch(m, name, big_gemm_f16_kernel<BEPI_ACT16>, grid, dim3(256), e);
+}
+
 typedef void (*AttnKernel)(AttnArgs);
 template <typename CT, typename AT, int D>
 static AttnKernel pick_attn_g(int G, bool prefill) {
@@ -485,6 +513,7 @@ static void launch_attn_decode(TSHipGpt* m, AttnArgs a, int B) {
 // MoE feed-forward at decode (MoEFeedForward.Process, Seq2SeqSharp/Layers/MoEFeedForward.cs:76-181)
 // ------------------------------------------------------------------------------------------------
 static void run_moe_ffn(TSHipGpt* m, LayerW& L, int rows, const ResidNormArgs& pre);
+static void run_moe_ffn_prefill(TSHipGpt* m, LayerW& L, int rows, const ResidNormArgs& pre, const int* last_rows, int n_last);
 static void moe_alloc(TSHipGpt* m);
 static void moe_get_routing(TSHipGpt* m, int layer, float* top_idx, float* top_val, float* probs);
 static void sample_tokens(TSHipGpt* m, int mode, float top_p, float temperature, const float* host_uniforms, const float* dev_uniforms, int B, int* gen_out, const int* d_step, bool record);
@@ -715,6 +744,11 @@ static void prefill(TSHipGpt* m, const int32_t* host_ids, int B, int Tp) {
     ids.reserve(R * sizeof(int));
     TSHIP_CHECK_HIP(hipMemcpyAsync(ids.p, host_ids, R * sizeof(int), hipMemcpyHostToDevice, stream()));
     record_history(m, ids.as<int>(), B, Tp, pos0);
+    std::vector<int> map(B);             // row of every sequence's last position
+    for (int b = 0; b < B; ++b) map[b] = Tp * (b + 1) - 1;
+    rowmap.reserve(B * sizeof(int));
+    TSHIP_CHECK_HIP(hipMemcpyAsync(rowmap.p, map.data(), B * sizeof(int), hipMemcpyHostToDevice, stream()));
+    TSHIP_CHECK_HIP(hipStreamSynchronize(stream()));       // (map is a local; the copy must not outlive it)
     px.reserve((size_t)Rp * h * sizeof(float));
     pxn.reserve((size_t)Rp * m->ldh * m->esz());
     pqkv.reserve((size_t)Rp * qp * sizeof(float));
@@ -756,30 +790,7 @@ static void prefill(TSHipGpt* m, const int32_t* host_ids, int B, int Tp) {
     auto producer = [&](BigArgs& e, const float* gamma) {        // residual GEMM that also emits the next GEMM's input
         e.xg16 = pxn.as<half_t>(); e.ld_xg = (int)m->ldh; e.gamma = gamma; e.ssq_out = pssq.as<float>(); e.ssq_ld = R;
     };
-    auto big = [&](const char* name, const GemmW& w, const void* X, long ldx, int epi, BigArgs e) {
-        e.W = w.buf.as<half_t>(); e.KT = w.KT; e.NT = w.NT; e.X = (const half_t*)X; e.ldx = (int)ldx; e.R = (int)R;
-        if (R >= 512) {       // LDS-tiled kernel, 256 x 256 block tile
-            constexpr int CK = 4;
-            const unsigned shm = 2u * 2u * 8u * CK * 1024u;
-            // one-dimensional grid of 8-row x 4-column tile patches, 32 blocks each, rounded up to whole rounds of 8 patches
-            const long CT = ceil_div(w.NT, 8), RT = ceil_div(R, 256), patches = ceil_div(CT, 4) * ceil_div(RT, 8);
-            dim3 grid((unsigned)(round_up(patches, 8) * 32));
-            if (w.KT % 2 == 0) {      // asynchronous staging: four stages of two k-tiles
-                if (epi == BEPI_F32_BIAS) launch_shm(m, name, big_gemm3_f16_kernel<BEPI_F32_BIAS>, grid, dim3(256), shm, e);
-                else if (epi == BEPI_RESID) launch_shm(m, name, big_gemm3_f16_kernel<BEPI_RESID>, grid, dim3(256), shm, e);
-                else launch_shm(m, name, big_gemm3_f16_kernel<BEPI_ACT16>, grid, dim3(256), shm, e);
-                return;
-            }
-            if (epi == BEPI_F32_BIAS) launch_shm(m, name, big_gemm2_f16_kernel<BEPI_F32_BIAS, CK>, grid, dim3(256), shm, e);
-            else if (epi == BEPI_RESID) launch_shm(m, name, big_gemm2_f16_kernel<BEPI_RESID, CK>, grid, dim3(256), shm, e);
-            else launch_shm(m, name, big_gemm2_f16_kernel<BEPI_ACT16, CK>, grid, dim3(256), shm, e);
-            return;
-        }
-        dim3 grid((unsigned)ceil_div(w.NT, 4), (unsigned)(Rp / 128));
-        if (epi == BEPI_F32_BIAS) launch(m, name, big_gemm_f16_kernel<BEPI_F32_BIAS>, grid, dim3(256), e);
-        else if (epi == BEPI_RESID) launch(m, name, big_gemm_f16_kernel<BEPI_RESID>, grid, dim3(256), e);
-        else launch(m, name, big_gemm_f16_kernel<BEPI_ACT16>, grid, dim3(256), e);
-    };
+    auto big = [&](const char* name, const GemmW& w, const void* X, long ldx, int epi, BigArgs e) { run_big_gemm(m, name, w, X, ldx, R, epi, e); };
     DevBuf& zero_bias = m->pw_zero_bias; zero_bias.reserve((size_t)std::max<long>(std::max<long>(qp, m->F13), round_up(h, 32)) * sizeof(float));
     for (int l = 0; l < c.n_layers; ++l) {
         LayerW& L = *m->L[l];
@@ -819,12 +830,18 @@ static void prefill(TSHipGpt* m, const int32_t* host_ids, int B, int Tp) {
             run_gemm_f32(m, "p_gemm_wo", L.wo, po.as<float>(), m->ldh, (int)R, pqkv.as<float>(), qp, 0, 1);
             a2.part = pqkv.as<float>(); a2.KS = 1; a2.ld_part = qp; a2.bias = L.bo.as<float>();
         }
-        if (L.moe) throw Error("TSHip_GptPrefill: MoE layers are prefilled token by token; use TSHip_GptDecode");
-        if (deferred) make_rinv("p_rinv_ffn"); else run_resid_norm(m, "p_norm_ffn", (int)R, a2);
         ResidNormArgs a3 = rn;
         if (l + 1 < c.n_layers) { a3.gamma = m->L[l + 1]->n1_g.as<float>(); a3.beta = m->L[l + 1]->n1_b.as<float>(); }
         else a3.xn = nullptr;
-        if (m->f16) {
+        if (L.moe) {
+            // the router kernel applies the pending attention output (fp32 models) and the layer's own LayerNorm; the
+            // combine kernel adds the experts' output to the residual stream
+            run_moe_ffn_prefill(m, L, (int)R, a2, rowmap.as<int>(), B);
+        } else if (deferred) make_rinv("p_rinv_ffn");
+        else run_resid_norm(m, "p_norm_ffn", (int)R, a2);
+        if (L.moe) {
+            // (nothing more: no dense feed-forward in this layer)
+        } else if (m->f16) {
             BigArgs e; std::memset(&e, 0, sizeof(e));
             e.bias = L.b1.as<float>(); e.bias2 = L.b3.as<float>(); e.out16 = pa.as<half_t>(); e.ld16 = (int)m->ldF;
             e.act = c.act; e.gated = m->gated; e.n_valid = F;
@@ -846,10 +863,6 @@ static void prefill(TSHipGpt* m, const int32_t* host_ids, int B, int Tp) {
         else if (l + 1 < c.n_layers || !m->f16) run_resid_norm(m, "p_norm_attn", (int)R, a3);
     }
     // last position of every sequence (Decoder.cs:705-716) -> final norm -> vocabulary projection
-    std::vector<int> map(B);
-    for (int b = 0; b < B; ++b) map[b] = Tp * (b + 1) - 1;
-    rowmap.reserve(B * sizeof(int));
-    TSHIP_CHECK_HIP(hipMemcpyAsync(rowmap.p, map.data(), B * sizeof(int), hipMemcpyHostToDevice, stream()));
     if (m->fused_norm) {
         FnPrepArgs a; std::memset(&a, 0, sizeof(a));
         a.x = m->x.as<float>(); a.ldx = h; a.h = h; a.src = px.as<float>(); a.ld_src = h; a.row_map = rowmap.as<int>();
@@ -1077,26 +1090,7 @@ TSHIP_API int TSHip_GptPrefill(TSHipGpt* m, const int32_t* host_ids, int batch, 
     TSHIP_REQUIRE(batch >= 1 && batch <= m->c.max_batch, "TSHip_GptPrefill: batch out of range");
     for (long i = 0; i < (long)batch * prompt_len; ++i)
         TSHIP_REQUIRE(host_ids[i] >= 0 && host_ids[i] < m->c.vocab, "TSHip_GptPrefill: token id out of range");
-    bool any_moe = false; for (auto& L : m->L) any_moe = any_moe || L->moe;
-    if (any_moe) {
-        // token-by-token: the MoE layer is built for decode-sized row counts
-        std::vector<int32_t> col(batch);
-        for (int t = 0; t < prompt_len; ++t) {
-            for (int b = 0; b < batch; ++b) col[b] = host_ids[(long)b * prompt_len + t];
-            TSHIP_CHECK_HIP(hipMemcpyAsync(m->ids.p, col.data(), batch * sizeof(int), hipMemcpyHostToDevice, stream()));
-            TSHIP_CHECK_HIP(hipStreamSynchronize(stream()));
-            if (t == 0) {
-                TSHIP_REQUIRE(m->pos == 0 || m->cur_batch == batch, "TSHip_GptPrefill: batch differs from the cached sequences; call TSHip_GptReset first");
-                TSHIP_REQUIRE(m->pos + prompt_len < m->c.max_seq_len, "TSHip_GptPrefill: prompt length exceeds max_seq_len");
-            }
-            record_history(m, m->ids.as<int>(), batch, 1, m->pos);
-            decode_step(m, m->ids.as<int>(), batch);
-        }
-        TSHIP_CHECK_HIP(hipStreamSynchronize(stream()));
-        m->cur_batch = batch;
-    } else {
-        prefill(m, host_ids, batch, prompt_len);
-    }
+    prefill(m, host_ids, batch, prompt_len);
     TSHIP_END
 }
 

@@ -9,11 +9,12 @@ struct MoeLayout {
     long ld4h, ldy;
 };
 
-static MoeLayout moe_layout(TSHipGpt* m) {
+// cap: rows the workspace is laid out for (the padded batch for decode steps, the padded row count of a prefill)
+static MoeLayout moe_layout(TSHipGpt* m, long cap) {
     auto& c = m->c;
     MoeLayout o; size_t at = 0;
     auto take = [&](size_t bytes) { size_t r = at; at += round_up((long)bytes, 256); return r; };
-    const long h = c.hidden, E = c.n_experts, k = c.experts_per_token, Bp = m->Bpad;
+    const long h = c.hidden, E = c.n_experts, k = c.experts_per_token, Bp = cap;
     o.ld4h = round_up(4 * h, 16); o.ldy = round_up(h, 32);
     o.xn32 = take(Bp * h * 4); o.probs = take(Bp * E * 4); o.top_val = take(Bp * k * 4); o.top_idx = take(Bp * k * 4);
     o.counts = take(E * 4); o.lists = take(E * Bp * 4); o.slot = take(Bp * k * 4);
@@ -28,12 +29,12 @@ static MoeLayout moe_layout(TSHipGpt* m) {
 
 static void moe_alloc(TSHipGpt* m) {
     TSHIP_REQUIRE(m->c.hidden <= 4096, "TSHip_GptCreate: MoE layers support hidden up to 4096");
-    m->moe_ws.alloc(moe_layout(m).total);
+    m->moe_ws.alloc(moe_layout(m, m->Bpad).total);
 }
 
 static void moe_get_routing(TSHipGpt* m, int layer, float* top_idx, float* top_val, float* probs) {
     (void)layer;   // the workspace holds the routing of the MoE layer that ran last; callers run one layer at a time
-    MoeLayout o = moe_layout(m);
+    MoeLayout o = moe_layout(m, m->Bpad);
     const int B = m->cur_batch, k = m->c.experts_per_token, E = m->c.n_experts;
     TSHIP_CHECK_HIP(hipStreamSynchronize(stream()));
     char* base = (char*)m->moe_ws.p;
@@ -43,11 +44,15 @@ static void moe_get_routing(TSHipGpt* m, int layer, float* top_idx, float* top_v
 }
 
 // `pre` carries the pending attention output (split-K partials + bias) and the LayerNorm parameters
-static void run_moe_ffn(TSHipGpt* m, LayerW& L, int rows, const ResidNormArgs& pre) {
+// batched (prefill, any number of rows): the workspace is m->pw_moe laid out for `cap` rows, the lists come from the
+// many-row kernel, the host reads the experts' row counts (the reference builds its lists on the host as well,
+// MoEFeedForward.cs:92-105) and every expert with rows runs the prefill GEMMs on its gathered rows
+static void run_moe_ffn_impl(TSHipGpt* m, LayerW& L, int rows, const ResidNormArgs& pre, bool batched, long cap, const int* last_rows, int n_last) {
     auto& c = m->c;
-    MoeLayout o = moe_layout(m);
-    char* base = (char*)m->moe_ws.p;
-    const int h = c.hidden, E = c.n_experts, k = c.experts_per_token, Bp = m->Bpad;
+    MoeLayout o = moe_layout(m, cap);
+    char* base = (char*)(batched ? m->pw_moe.p : m->moe_ws.p);
+    TSHIP_REQUIRE(rows <= cap && o.total <= (batched ? m->pw_moe.bytes : m->moe_ws.bytes), "internal: MoE workspace too small");
+    const int h = c.hidden, E = c.n_experts, k = c.experts_per_token; const long Bp = cap;
     float* xn32 = (float*)(base + o.xn32); float* probs = (float*)(base + o.probs);
     float* top_val = (float*)(base + o.top_val); float* top_idx = (float*)(base + o.top_idx);
     int* counts = (int*)(base + o.counts); int* lists = (int*)(base + o.lists); int* slot = (int*)(base + o.slot);
@@ -62,11 +67,31 @@ static void run_moe_ffn(TSHipGpt* m, LayerW& L, int rows, const ResidNormArgs& p
     r.router_lds = ((long)E * h <= 16384) ? 1 : 0;
     const unsigned router_shm = (unsigned)((2L * h + (r.router_lds ? (long)E * h : 0)) * sizeof(float));
     launch_shm(m, "moe_router", moe_router_kernel, dim3(rows), dim3(256), router_shm, r);
-    launch_shm(m, "moe_lists", moe_lists_kernel, dim3(1), dim3(64), (unsigned)(rows * k * sizeof(int)), (const float*)top_idx, rows, k, E, Bp, counts, lists, slot);
+    if (batched) launch(m, "moe_lists", moe_lists_big_kernel, dim3(E), dim3(1024), (const float*)top_idx, rows, k, (int)Bp, counts, lists, slot);
+    else launch_shm(m, "moe_lists", moe_lists_kernel, dim3(1), dim3(64), (unsigned)(rows * k * sizeof(int)), (const float*)top_idx, rows, k, E, (int)Bp, counts, lists, slot);
+    std::vector<int> n_e(E, rows);
+    if (batched) {
+        TSHIP_CHECK_HIP(hipMemcpyAsync(n_e.data(), counts, E * sizeof(int), hipMemcpyDeviceToHost, stream()));
+        TSHIP_CHECK_HIP(hipStreamSynchronize(stream()));
+        for (int e = 0; e < E; ++e) TSHIP_REQUIRE(n_e[e] >= 0 && n_e[e] <= rows, "internal: expert row count out of range");
+    }
     const long xg_stride = (long)Bp * m->ldh, mid_stride = (long)Bp * o.ld4h, y_stride = (long)Bp * o.ldy;
-    if (m->f16) {
+    if (m->f16 && batched) {
         half_t* xg = (half_t*)(base + o.xg); half_t* mid = (half_t*)(base + o.mid);
-        launch(m, "moe_gather", moe_gather_kernel<half_t>, dim3(rows, E), dim3(256), (const float*)xn32, h, (const int*)counts, (const int*)lists, Bp, xg,
+        launch(m, "moe_gather", moe_gather_kernel<half_t>, dim3(rows, E), dim3(256), (const float*)xn32, h, (const int*)counts, (const int*)lists, (int)Bp, xg,
+               m->ldh, xg_stride, 0);
+        for (int e = 0; e < E; ++e) {
+            if (n_e[e] == 0) continue;
+            BigArgs e1; std::memset(&e1, 0, sizeof(e1));
+            e1.bias = zero; e1.out16 = mid + e * mid_stride; e1.ld16 = (int)o.ld4h; e1.act = c.act; e1.gated = 0; e1.n_valid = 4 * h;
+            run_big_gemm(m, "moe_gemm1", *L.e1[e], xg + e * xg_stride, m->ldh, n_e[e], BEPI_ACT16, e1);
+            BigArgs e2; std::memset(&e2, 0, sizeof(e2));
+            e2.bias = zero; e2.out = y + e * y_stride; e2.ld_out = (int)o.ldy; e2.n_valid = h;
+            run_big_gemm(m, "moe_gemm2", *L.e2[e], mid + e * mid_stride, o.ld4h, n_e[e], BEPI_F32_BIAS, e2);
+        }
+    } else if (m->f16) {
+        half_t* xg = (half_t*)(base + o.xg); half_t* mid = (half_t*)(base + o.mid);
+        launch(m, "moe_gather", moe_gather_kernel<half_t>, dim3(rows, E), dim3(256), (const float*)xn32, h, (const int*)counts, (const int*)lists, (int)Bp, xg,
                m->ldh, xg_stride, (int)(m->ldh / 16));
         // pointer tables are written once per layer object (weights never move)
         std::vector<const half_t*> t1(E), t2(E);
@@ -95,21 +120,39 @@ static void run_moe_ffn(TSHipGpt* m, LayerW& L, int rows, const ResidNormArgs& p
         }
     } else {
         float* xg = (float*)(base + o.xg); float* mid = (float*)(base + o.mid);
-        launch(m, "moe_gather", moe_gather_kernel<float>, dim3(rows, E), dim3(256), (const float*)xn32, h, (const int*)counts, (const int*)lists, Bp, xg,
+        launch(m, "moe_gather", moe_gather_kernel<float>, dim3(rows, E), dim3(256), (const float*)xn32, h, (const int*)counts, (const int*)lists, (int)Bp, xg,
                m->ldh, xg_stride, 0);
         for (int e = 0; e < E; ++e) {
-            // fp32 models: every expert runs on `rows` rows; rows past the expert's count hold stale finite data
-            // and are never read back
+            // fp32 models, decode: every expert runs on `rows` rows (no host round trip for the counts); rows past the
+            // expert's count hold stale finite data and are never read back.  Batched: the expert's own rows.
+            const int er = n_e[e];
+            if (er == 0) continue;
             float* mid_e = mid + e * mid_stride;
-            run_gemm_f32(m, "moe_gemm1", *L.e1[e], xg + e * xg_stride, m->ldh, rows, mid_e, o.ld4h, 0, 1);
-            long tot = (long)rows * 4 * h;
+            run_gemm_f32(m, "moe_gemm1", *L.e1[e], xg + e * xg_stride, m->ldh, er, mid_e, o.ld4h, 0, 1);
+            long tot = (long)er * 4 * h;
             launch(m, "moe_act", ffn_act_kernel<float>, dim3((unsigned)ceil_div(tot, 256)), dim3(256), (const float*)mid_e, 1, 0L, o.ld4h,
-                   (const float*)zero, (const float*)zero, 4 * h, 0, (int)c.act, mid_e, o.ld4h, (long)rows);
-            run_gemm_f32(m, "moe_gemm2", *L.e2[e], mid_e, o.ld4h, rows, y + e * y_stride, o.ldy, 0, 1);
+                   (const float*)zero, (const float*)zero, 4 * h, 0, (int)c.act, mid_e, o.ld4h, (long)er);
+            run_gemm_f32(m, "moe_gemm2", *L.e2[e], mid_e, o.ld4h, er, y + e * y_stride, o.ldy, 0, 1);
         }
     }
     launch(m, "moe_combine", moe_combine_kernel, dim3(rows), dim3(256), pre.x, pre.ldx, h, (const float*)y, o.ldy, y_stride, (const float*)probs,
            (const float*)top_idx, (const int*)slot, k, E);
+    if (batched && last_rows) {
+        // what TSHip_GptGetMoeRouting reports after a prefill: the routing of every sequence's last position
+        MoeLayout d = moe_layout(m, m->Bpad);
+        char* db = (char*)m->moe_ws.p;
+        launch(m, "moe_last_rows", moe_rows_kernel, dim3(n_last), dim3(64), (const float*)probs, last_rows, (float*)(db + d.probs), E);
+        launch(m, "moe_last_rows", moe_rows_kernel, dim3(n_last), dim3(64), (const float*)top_val, last_rows, (float*)(db + d.top_val), k);
+        launch(m, "moe_last_rows", moe_rows_kernel, dim3(n_last), dim3(64), (const float*)top_idx, last_rows, (float*)(db + d.top_idx), k);
+    }
+}
+
+static void run_moe_ffn(TSHipGpt* m, LayerW& L, int rows, const ResidNormArgs& pre) { run_moe_ffn_impl(m, L, rows, pre, false, m->Bpad, nullptr, 0); }
+
+static void run_moe_ffn_prefill(TSHipGpt* m, LayerW& L, int rows, const ResidNormArgs& pre, const int* last_rows, int n_last) {
+    const long cap = round_up(rows, 128);
+    m->pw_moe.reserve(moe_layout(m, cap).total);
+    run_moe_ffn_impl(m, L, rows, pre, true, cap, last_rows, n_last);
 }
 
 // next tokens from the logits on the device -> m->ids (and gen_out); greedy or top-p.

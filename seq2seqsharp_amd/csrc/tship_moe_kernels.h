@@ -201,6 +201,41 @@ __global__ __launch_bounds__(64) void moe_lists_kernel(const float* __restrict__
     counts[e] = n;
 }
 
+// The same lists for many rows (prefill): one block of 1024 threads per expert walks the (token, choice) pairs in order,
+// 1024 at a time; a pair's place in the list is the number of the expert's pairs before it (ballots inside a wavefront,
+// wavefront totals through LDS), so the lists come out in ascending token order like the serial kernel's.
+__global__ __launch_bounds__(1024) void moe_lists_big_kernel(const float* __restrict__ top_idx, int rows, int k, int max_rows, int* __restrict__ counts,
+                                                              int* __restrict__ lists, int* __restrict__ slot) {
+    __shared__ int s_wave[16];
+    __shared__ int s_base;
+    const int e = blockIdx.x, t = threadIdx.x, lane = t & 63, w = t >> 6;
+    if (t == 0) s_base = 0;
+    __syncthreads();
+    const int n_pairs = rows * k;
+    for (int i0 = 0; i0 < n_pairs; i0 += 1024) {
+        const int i = i0 + t;
+        const bool hit = i < n_pairs && (int)top_idx[i] == e;
+        const unsigned long long bal = __ballot(hit);
+        const int before = __popcll(bal & ((1ull << lane) - 1ull));
+        if (lane == 0) s_wave[w] = __popcll(bal);
+        __syncthreads();
+        int off = s_base;
+        for (int j = 0; j < w; ++j) off += s_wave[j];
+        if (hit) { const int n = off + before; lists[(long)e * max_rows + n] = i / k; slot[i] = n; }
+        __syncthreads();
+        if (t == 0) { int tot = 0; for (int j = 0; j < 16; ++j) tot += s_wave[j]; s_base += tot; }
+        __syncthreads();
+    }
+    if (t == 0) counts[e] = s_base;
+}
+
+// rows row_map[b] of a [.., width] table -> rows b of another (the routing of each sequence's last prompt position, kept
+// where the decode step keeps its routing): grid (batch)
+__global__ void moe_rows_kernel(const float* __restrict__ src, const int* __restrict__ row_map, float* __restrict__ dst, int width) {
+    const int b = blockIdx.x;
+    for (int c = threadIdx.x; c < width; c += blockDim.x) dst[(long)b * width + c] = src[(long)row_map[b] * width + c];
+}
+
 // IndexSelect(inputNorm, tokenIdx_e) for every expert (MoEFeedForward.cs:155): grid (max_rows, E)
 template <typename AT>
 __global__ __launch_bounds__(256) void moe_gather_kernel(const float* __restrict__ xn32, int h, const int* __restrict__ counts,

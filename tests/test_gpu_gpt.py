@@ -356,6 +356,30 @@ def test_moe_model(G, oracle, dtype, act):
     gpu.close()
 
 
+@pytest.mark.parametrize("dtype,batch,prompt", [("f16", 4, 330), ("f16", 3, 70), ("f32", 2, 40)])
+def test_moe_prefill_runs_the_experts_on_gathered_rows(G, oracle, dtype, batch, prompt):
+    """Prefill of a model with MoE layers: all prompt rows are routed at once, every expert runs the prefill GEMMs on the
+    rows gathered for it (about 660 rows per expert in the first case: the LDS-tiled kernel; fewer than 512 in the
+    others), and the scaled outputs are added back in expert order.  Logits of the last position and the routing of the
+    last position against the oracle, then decode steps on top of the cache the prefill wrote."""
+    cfg = synth.tiny_config(n_layers=3, n_experts=4, experts_per_token=2, norm_type=synth.LAYERNORM, act=synth.RELU, dtype=dtype,
+                            batch=batch, prompt=prompt, vocab=300)
+    orc, gpu, out, cur = _teacher_forced(G, oracle, cfg, 61, 3)
+    for lg, gl in out:
+        if dtype == "f32":
+            assert _rel(gl, lg) <= FP32_REL
+        else:
+            assert np.abs(gl - lg).max() <= FP16_ABS
+    if dtype == "f32":
+        gpu.reset()
+        gpu.prefill(cur)
+        ti, tv, pr = gpu.moe_routing(2)                      # last MoE layer, last position of every sequence
+        oi, ov, op = orc.moe_trace(0, batch)
+        assert np.array_equal(ti, oi)
+        assert np.allclose(pr, op, rtol=1e-6)
+    gpu.close()
+
+
 def test_moe_tied_router_follows_topk_rule(G, oracle):
     cfg = synth.tiny_config(n_layers=3, n_experts=4, experts_per_token=2, norm_type=synth.LAYERNORM, act=synth.RELU, batch=5)
     w = synth.make_weights(cfg, 41, random_bias=True)
