@@ -512,7 +512,7 @@ static void launch_attn_decode(TSHipGpt* m, AttnArgs a, int B) {
 // ------------------------------------------------------------------------------------------------
 // MoE feed-forward at decode (MoEFeedForward.Process, Seq2SeqSharp/Layers/MoEFeedForward.cs:76-181)
 // ------------------------------------------------------------------------------------------------
-static void run_moe_ffn(TSHipGpt* m, LayerW& L, int rows, const ResidNormArgs& pre);
+static void run_moe_ffn(TSHipGpt* m, LayerW& L, int rows, const ResidNormArgs& pre, const ResidNormArgs* next);
 static void run_moe_ffn_prefill(TSHipGpt* m, LayerW& L, int rows, const ResidNormArgs& pre, const int* last_rows, int n_last);
 static void moe_alloc(TSHipGpt* m);
 static void moe_get_routing(TSHipGpt* m, int layer, float* top_idx, float* top_val, float* probs);
@@ -679,12 +679,11 @@ static void decode_step(TSHipGpt* m, const int* d_ids, int B) {
         const float* next_b = (l + 1 < c.n_layers) ? m->L[l + 1]->n1_b.as<float>() : m->fn_b.as<float>();
         if (L.moe) {
             a2.norm_type = 1;          // MoEFeedForward always uses LayerNormalization (MoEFeedForward.cs:49)
-            run_moe_ffn(m, L, B, a2);
-            // x already updated by the MoE combine; next norm
+            // the next norm's kernel adds the experts' outputs to x first
             ResidNormArgs a3 = rn;
             a3.gamma = next_g; a3.beta = next_b;
             if (l + 1 == c.n_layers) a3.advance_pos = m->d_pos.as<int>();
-            run_resid_norm(m, "norm_next", B, a3);
+            run_moe_ffn(m, L, B, a2, &a3);
             continue;
         }
         run_resid_norm(m, "resid_norm_ffn", B, a2);

@@ -47,7 +47,9 @@ static void moe_get_routing(TSHipGpt* m, int layer, float* top_idx, float* top_v
 // batched (prefill, any number of rows): the workspace is m->pw_moe laid out for `cap` rows, the lists come from the
 // many-row kernel, the host reads the experts' row counts (the reference builds its lists on the host as well,
 // MoEFeedForward.cs:92-105) and every expert with rows runs the prefill GEMMs on its gathered rows
-static void run_moe_ffn_impl(TSHipGpt* m, LayerW& L, int rows, const ResidNormArgs& pre, bool batched, long cap, const int* last_rows, int n_last) {
+// next: when given, the norm kernel that follows adds the experts' outputs itself (no separate combine launch)
+static void run_moe_ffn_impl(TSHipGpt* m, LayerW& L, int rows, const ResidNormArgs& pre, bool batched, long cap, const int* last_rows, int n_last,
+                             const ResidNormArgs* next = nullptr) {
     auto& c = m->c;
     MoeLayout o = moe_layout(m, cap);
     char* base = (char*)(batched ? m->pw_moe.p : m->moe_ws.p);
@@ -67,8 +69,10 @@ static void run_moe_ffn_impl(TSHipGpt* m, LayerW& L, int rows, const ResidNormAr
     r.router_lds = ((long)E * h <= 16384) ? 1 : 0;
     const unsigned router_shm = (unsigned)((2L * h + (r.router_lds ? (long)E * h : 0)) * sizeof(float));
     launch_shm(m, "moe_router", moe_router_kernel, dim3(rows), dim3(256), router_shm, r);
+    // decode-sized batches: the gather kernel builds the lists itself (one launch less)
+    const bool fused_lists = !batched && (long)rows * k <= 1024;
     if (batched) launch(m, "moe_lists", moe_lists_big_kernel, dim3(E), dim3(1024), (const float*)top_idx, rows, k, (int)Bp, counts, lists, slot);
-    else launch_shm(m, "moe_lists", moe_lists_kernel, dim3(1), dim3(64), (unsigned)(rows * k * sizeof(int)), (const float*)top_idx, rows, k, E, (int)Bp, counts, lists, slot);
+    else if (!fused_lists) launch_shm(m, "moe_lists", moe_lists_kernel, dim3(1), dim3(64), (unsigned)(rows * k * sizeof(int)), (const float*)top_idx, rows, k, E, (int)Bp, counts, lists, slot);
     std::vector<int> n_e(E, rows);
     if (batched) {
         TSHIP_CHECK_HIP(hipMemcpyAsync(n_e.data(), counts, E * sizeof(int), hipMemcpyDeviceToHost, stream()));
@@ -91,7 +95,9 @@ static void run_moe_ffn_impl(TSHipGpt* m, LayerW& L, int rows, const ResidNormAr
         }
     } else if (m->f16) {
         half_t* xg = (half_t*)(base + o.xg); half_t* mid = (half_t*)(base + o.mid);
-        launch(m, "moe_gather", moe_gather_kernel<half_t>, dim3(rows, E), dim3(256), (const float*)xn32, h, (const int*)counts, (const int*)lists, (int)Bp, xg,
+        if (fused_lists) launch(m, "moe_gather", moe_gather_lists_kernel<half_t>, dim3(rows, E), dim3(256), (const float*)top_idx, rows, k, (const float*)xn32, h,
+                                counts, lists, slot, (int)Bp, xg, m->ldh, xg_stride, (int)(m->ldh / 16));
+        else launch(m, "moe_gather", moe_gather_kernel<half_t>, dim3(rows, E), dim3(256), (const float*)xn32, h, (const int*)counts, (const int*)lists, (int)Bp, xg,
                m->ldh, xg_stride, (int)(m->ldh / 16));
         // pointer tables are written once per layer object (weights never move)
         std::vector<const half_t*> t1(E), t2(E);
@@ -120,7 +126,9 @@ static void run_moe_ffn_impl(TSHipGpt* m, LayerW& L, int rows, const ResidNormAr
         }
     } else {
         float* xg = (float*)(base + o.xg); float* mid = (float*)(base + o.mid);
-        launch(m, "moe_gather", moe_gather_kernel<float>, dim3(rows, E), dim3(256), (const float*)xn32, h, (const int*)counts, (const int*)lists, (int)Bp, xg,
+        if (fused_lists) launch(m, "moe_gather", moe_gather_lists_kernel<float>, dim3(rows, E), dim3(256), (const float*)top_idx, rows, k, (const float*)xn32, h,
+                                counts, lists, slot, (int)Bp, xg, m->ldh, xg_stride, 0);
+        else launch(m, "moe_gather", moe_gather_kernel<float>, dim3(rows, E), dim3(256), (const float*)xn32, h, (const int*)counts, (const int*)lists, (int)Bp, xg,
                m->ldh, xg_stride, 0);
         for (int e = 0; e < E; ++e) {
             // fp32 models, decode: every expert runs on `rows` rows (no host round trip for the counts); rows past the
@@ -135,8 +143,14 @@ static void run_moe_ffn_impl(TSHipGpt* m, LayerW& L, int rows, const ResidNormAr
             run_gemm_f32(m, "moe_gemm2", *L.e2[e], mid_e, o.ld4h, er, y + e * y_stride, o.ldy, 0, 1);
         }
     }
-    launch(m, "moe_combine", moe_combine_kernel, dim3(rows), dim3(256), pre.x, pre.ldx, h, (const float*)y, o.ldy, y_stride, (const float*)probs,
-           (const float*)top_idx, (const int*)slot, k, E);
+    if (next) {
+        ResidNormArgs a = *next;
+        a.moe_y = y; a.moe_ldy = o.ldy; a.moe_estride = y_stride; a.moe_probs = probs; a.moe_top = top_idx; a.moe_slot = slot; a.moe_k = k; a.moe_E = E;
+        run_resid_norm(m, "moe_combine_norm", rows, a);
+    } else {
+        launch(m, "moe_combine", moe_combine_kernel, dim3(rows), dim3(256), pre.x, pre.ldx, h, (const float*)y, o.ldy, y_stride, (const float*)probs,
+               (const float*)top_idx, (const int*)slot, k, E);
+    }
     if (batched && last_rows) {
         // what TSHip_GptGetMoeRouting reports after a prefill: the routing of every sequence's last position
         MoeLayout d = moe_layout(m, m->Bpad);
@@ -147,7 +161,7 @@ static void run_moe_ffn_impl(TSHipGpt* m, LayerW& L, int rows, const ResidNormAr
     }
 }
 
-static void run_moe_ffn(TSHipGpt* m, LayerW& L, int rows, const ResidNormArgs& pre) { run_moe_ffn_impl(m, L, rows, pre, false, m->Bpad, nullptr, 0); }
+static void run_moe_ffn(TSHipGpt* m, LayerW& L, int rows, const ResidNormArgs& pre, const ResidNormArgs* next) { run_moe_ffn_impl(m, L, rows, pre, false, m->Bpad, nullptr, 0, next); }
 
 static void run_moe_ffn_prefill(TSHipGpt* m, LayerW& L, int rows, const ResidNormArgs& pre, const int* last_rows, int n_last) {
     const long cap = round_up(rows, 128);

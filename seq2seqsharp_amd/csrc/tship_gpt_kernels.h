@@ -1018,6 +1018,10 @@ struct ResidNormArgs {
     int xn_kt;              // > 0 (fp16 only): xn is fragment packed with this many k-tiles; 0: row-major with ldxn
     const int* row_map;     // optional: block r works on row row_map[r] of x and writes row r of xn
     int* advance_pos;       // optional: block 0 increments this device counter (end of a decode step)
+    // optional source: x += the MoE experts' outputs, each scaled by its router probability and added in expert order
+    // (MoEFeedForward.cs:167-178; IndexSelectGrad, TensorApplyCPU.cs:1336-1356).  y[e][slot][col], slot[row * k + j] =
+    // place of the row in the list of its j-th expert
+    const float* moe_y; long moe_ldy; long moe_estride; const float* moe_probs; const float* moe_top; const int* moe_slot; int moe_k; int moe_E;
 };
 
 template <typename AT, int NPT>   // NPT * 256 >= hidden
@@ -1080,12 +1084,27 @@ __global__ __launch_bounds__(256) void resid_norm_kernel(ResidNormArgs a) {
             if (c < a.h) v[i] = (s[i] + a.bias[c]) + v[i];
         }
     }
+    if (a.moe_y) {
+#pragma clang fp contract(off)
+        for (int i = 0; i < NPT; ++i) {
+            const int c = t + i * 256;
+            if (c >= a.h) continue;
+            float out = 0.0f;
+            for (int e = 0; e < a.moe_E; ++e)
+                for (int j = 0; j < a.moe_k; ++j)
+                    if ((int)a.moe_top[xr * a.moe_k + j] == e) {
+                        float sc = a.moe_y[e * a.moe_estride + (long)a.moe_slot[xr * a.moe_k + j] * a.moe_ldy + c] * a.moe_probs[xr * a.moe_E + e];
+                        out += sc;
+                    }
+            v[i] = v[i] + out;
+        }
+    }
     float sum = 0.0f, sq = 0.0f;
 #pragma unroll
     for (int i = 0; i < NPT; ++i) {
         int c = t + i * 256;
         if (c < a.h) {
-            if (a.ids || part) a.x[xr * a.ldx + c] = v[i];
+            if (a.ids || part || a.moe_y) a.x[xr * a.ldx + c] = v[i];
             sum += v[i]; sq += v[i] * v[i];
         }
     }

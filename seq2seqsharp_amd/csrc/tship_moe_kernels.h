@@ -251,6 +251,46 @@ __global__ __launch_bounds__(256) void moe_gather_kernel(const float* __restrict
     }
 }
 
+// Lists and gather in one launch for decode-sized batches (at most 1024 (token, choice) pairs): block (j, e) finds the
+// j-th pair of expert e by itself (every block repeats the small ordered count: ballots inside a wavefront, wavefront
+// totals through LDS, pairs t, t + 256, ... in four rounds), records the pair's slot, and copies the token's row.
+// Block (0, e) stores the expert's count.  Same lists, same order as moe_lists_kernel.
+template <typename AT>
+__global__ __launch_bounds__(256) void moe_gather_lists_kernel(const float* __restrict__ top_idx, int rows, int k, const float* __restrict__ xn32, int h,
+                                                                int* __restrict__ counts, int* __restrict__ lists, int* __restrict__ slot, int max_rows,
+                                                                AT* __restrict__ xg, long ld, long estride, int packed_kt) {
+    __shared__ int s_wave[4];
+    __shared__ int s_pair;
+    const int j = blockIdx.x, e = blockIdx.y, t = threadIdx.x, lane = t & 63, w = t >> 6;
+    const int n_pairs = rows * k;
+    if (t == 0) s_pair = -1;
+    int base = 0;
+    for (int q = 0; q < 4; ++q) {
+        const int i = q * 256 + t;
+        const bool hit = i < n_pairs && (int)top_idx[i] == e;
+        const unsigned long long bal = __ballot(hit);
+        const int before = __popcll(bal & ((1ull << lane) - 1ull));
+        __syncthreads();                       // (s_wave of the round before has been read)
+        if (lane == 0) s_wave[w] = __popcll(bal);
+        __syncthreads();
+        int off = base;
+        for (int x = 0; x < w; ++x) off += s_wave[x];
+        if (hit && off + before == j) s_pair = i;
+        base += s_wave[0] + s_wave[1] + s_wave[2] + s_wave[3];
+    }
+    __syncthreads();
+    if (j == 0 && t == 0) counts[e] = base;
+    const int pair = s_pair;
+    if (pair < 0) return;                      // fewer than j + 1 tokens chose this expert
+    const int tok = pair / k;
+    if (t == 0) { slot[pair] = j; lists[e * max_rows + j] = tok; }
+    AT* dst = xg + e * estride;
+    for (int c = t; c < h; c += 256) {
+        if (packed_kt > 0) dst[xpack_index(j, c, packed_kt)] = (AT)xn32[(long)tok * h + c];
+        else dst[(long)j * ld + c] = (AT)xn32[(long)tok * h + c];
+    }
+}
+
 // EltMul by the expert's probability, scatter-add in expert-major order into zeros, then input + result
 // (MoEFeedForward.cs:167-178; IndexSelectGrad, TensorApplyCPU.cs:1336-1356): one block per token
 __global__ __launch_bounds__(256) void moe_combine_kernel(float* __restrict__ x, long ldx, int h, const float* __restrict__ y, long ldy, long estride,
