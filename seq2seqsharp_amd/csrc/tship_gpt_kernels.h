@@ -229,7 +229,17 @@ __global__ __launch_bounds__(NW * 64) void skinny_gemm_f16_kernel(SkinnyArgs a) 
         const int src = half_of[j] == 1 ? (lane & ~8) : half_of[j] == 2 ? (lane | 8) : lane;
         wp[j] = a.W + ((long)min(tile_of[j], a.NT - 1) * a.KT * 64 + src) * 8;
     }
-    const half_t* xp = a.X + lane * 8;
+    // Activation fragments: lane l holds row l % 32 of a 32-row tile.  Rows from rows_valid on need no bytes of their
+    // own: their lanes read the bytes of valid rows again (whole 8-lane, 128-byte runs; row tiles without a valid row
+    // read the last tile that has one), which costs no further request, and their sums are never stored.
+    const half_t* xp[BT];
+    {
+        const int rv = max(a.rows_valid, 1), last_bt = min((rv - 1) >> 5, BT - 1);
+        const int rv8 = min(32, (rv - last_bt * 32 + 7) & ~7);
+        const int dup = (lane & 32) | ((lane & 31) % rv8);
+#pragma unroll
+        for (int bt = 0; bt < BT; ++bt) xp[bt] = a.X + (long)min(bt, last_bt) * a.KT * 512 + (bt >= last_bt ? dup : lane) * 8;
+    }
     // Full batches of U k-tiles run without conditions: a request under a condition of its own would make every
     // later wait cover all requests, and the products could not start while the batch is still arriving.
     int kt = wk0;
@@ -241,7 +251,7 @@ __global__ __launch_bounds__(NW * 64) void skinny_gemm_f16_kernel(SkinnyArgs a) 
 #pragma unroll
             for (int j = 0; j < NJ; ++j) wf[u][j] = *(const half8*)(wp[j] + (long)(kt + u) * 512);
 #pragma unroll
-            for (int bt = 0; bt < BT; ++bt) xf[u][bt] = *(const half8*)(xp + ((long)bt * a.KT + kt + u) * 512);
+            for (int bt = 0; bt < BT; ++bt) xf[u][bt] = *(const half8*)(xp[bt] + (long)(kt + u) * 512);
         }
         __builtin_amdgcn_sched_barrier(0);       // all requests of the batch go out before its first product
 #pragma unroll
@@ -261,7 +271,7 @@ __global__ __launch_bounds__(NW * 64) void skinny_gemm_f16_kernel(SkinnyArgs a) 
 #pragma unroll
                 for (int j = 0; j < NJ; ++j) wf[u][j] = *(const half8*)(wp[j] + (long)(kt + u) * 512);
 #pragma unroll
-                for (int bt = 0; bt < BT; ++bt) xf[u][bt] = *(const half8*)(xp + ((long)bt * a.KT + kt + u) * 512);
+                for (int bt = 0; bt < BT; ++bt) xf[u][bt] = *(const half8*)(xp[bt] + (long)(kt + u) * 512);
             }
         }
 #pragma unroll
