@@ -138,6 +138,17 @@ def main():
     dom_bytes = float(cfg["hidden"]) * cfg["ffn_dim"] * nW13 * es      # the weights one launch streams, once
     dom_gbs = dom_bytes / (dom_ms / 1e3) / 1e9
     kernel_ms = {k: round(float(np.sum(v)) / n_prof, 4) for k, v in acc.items()}
+    # the attention kernel takes the largest share of the step at long contexts; its bytes grow with the context, so its
+    # figure is quoted at the context length of the profiled steps (keys and values of one layer, read once)
+    attn = None
+    if "attn_decode" in acc:
+        t_attn = T_end + 1 + (n_prof - 1) / 2.0
+        a_bytes = float(es) * B * cfg["n_kv_heads"] * d * 2 * t_attn
+        a_ms = float(np.mean(acc["attn_decode"]))
+        a_gbs = a_bytes / (a_ms / 1e3) / 1e9
+        attn = {"bound": "hbm", "achieved": round(a_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(a_gbs / HBM_PEAK_GBS, 4),
+                "traffic": None, "kernel": "attention (attn_decode)", "kv_len": t_attn, "bytes_per_launch": a_bytes, "avg_launch_ms": round(a_ms, 5),
+                "share_of_step": round(kernel_ms["attn_decode"] / sum(kernel_ms.values()), 3)}
 
     # a plain copy of known size: the reference point for scaling FETCH_SIZE / WRITE_SIZE in counter runs
     if not args.no_copy_calibration:
@@ -165,7 +176,9 @@ def main():
         "roofline": {"bound": "hbm", "achieved": round(dom_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(dom_gbs / HBM_PEAK_GBS, 4), "traffic": traffic,
                      "kernel": "skinny_gemm_f16_kernel<%d, EPI_ACT16> (%s)" % (1 if B <= 32 else 2 if B <= 64 else 4, dom),
-                     "bytes_per_launch": dom_bytes, "avg_launch_ms": round(dom_ms, 5)},
+                     "bytes_per_launch": dom_bytes, "avg_launch_ms": round(dom_ms, 5),
+                     "share_of_step": round(kernel_ms[dom] / sum(kernel_ms.values()), 3)},
+        "roofline_attention": attn,
         "whole_step": {"algorithmic_bytes": round(step_bytes), "achieved_GBps": round(step_gbs, 1),
                        "frac_of_hbm_peak": round(step_gbs / HBM_PEAK_GBS, 4), "host_wall_ms_per_step": round(wall / K * 1e3, 4)},
         "prefill": {"tokens_per_s": round(prefill_tok_s, 1), "seconds": round(t_prefill, 4),
