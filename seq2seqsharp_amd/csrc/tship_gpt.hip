@@ -414,10 +414,10 @@ static void run_big_gemm(TSHipGpt* m, const char* name, const GemmW& w, const vo
         // one-dimensional grid of 8-row x 4-column tile patches, 32 blocks each, rounded up to whole rounds of 8 patches
         const long CT = ceil_div(w.NT, 8), RT = ceil_div(R, 256), patches = ceil_div(CT, 4) * ceil_div(RT, 8);
         dim3 grid((unsigned)(round_up(patches, 8) * 32));
-        if (w.KT % 2 == 0) {      // asynchronous staging: four stages of two k-tiles
-            if (epi == BEPI_F32_BIAS) launch_shm(m, name, big_gemm3_f16_kernel<BEPI_F32_BIAS>, grid, dim3(256), shm, e);
-            else if (epi == BEPI_RESID) launch_shm(m, name, big_gemm3_f16_kernel<BEPI_RESID>, grid, dim3(256), shm, e);
-            else launch_shm(m, name, big_gemm3_f16_kernel<BEPI_ACT16>, grid, dim3(256), shm, e);
+        if (w.KT % 2 == 0) {      // asynchronous staging: four stages of two k-tiles, eight wavefronts
+            if (epi == BEPI_F32_BIAS) launch_shm(m, name, big_gemm3_f16_kernel<BEPI_F32_BIAS>, grid, dim3(512), shm, e);
+            else if (epi == BEPI_RESID) launch_shm(m, name, big_gemm3_f16_kernel<BEPI_RESID>, grid, dim3(512), shm, e);
+            else launch_shm(m, name, big_gemm3_f16_kernel<BEPI_ACT16>, grid, dim3(512), shm, e);
             return;
         }
         if (epi == BEPI_F32_BIAS) launch_shm(m, name, big_gemm2_f16_kernel<BEPI_F32_BIAS, CK>, grid, dim3(256), shm, e);
