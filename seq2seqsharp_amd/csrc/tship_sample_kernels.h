@@ -75,46 +75,70 @@ __device__ __forceinline__ float block_max_256(float v, float* s) {
     return fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3]));
 }
 
-__device__ __forceinline__ float block_max_1024(float v, float* s) {
+// Softmax statistics of a row, a row split over its nseg segments of 1024 elements so that the whole chip works on the
+// rows: per-segment maxima, then per-segment sums of exp(x / T - row maximum).  They live in the first floats of the
+// row's slice of `accp`, which the pick kernel only uses afterwards: maxima at [seg], sums at [nseg + seg].
+// grid (nseg, rows), 256 threads, four elements per thread.
+static __global__ __launch_bounds__(256) void topp_rowmax_kernel(TopPArgs a) {
+    __shared__ float sred[4];
+    const int seg = blockIdx.x, r = blockIdx.y, t = threadIdx.x;
+    const float* row = a.in + (long)r * a.ld;
+    float lm = -INFINITY;
 #pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
-    __syncthreads();
-    if ((threadIdx.x & 63) == 0) s[threadIdx.x >> 6] = v;
-    __syncthreads();
-    float m = s[0];
-#pragma unroll
-    for (int i = 1; i < 16; ++i) m = fmaxf(m, s[i]);
-    return m;
+    for (int it = 0; it < 4; ++it) {
+        const int i = seg * TOPP_SEG + it * 256 + t;
+        if (i < a.V) lm = fmaxf(lm, row[i] / a.temperature);
+    }
+    const float m = block_max_256(lm, sred);
+    if (t == 0) a.accp[(long)r * a.Vs + seg] = m;
 }
 
-// probabilities (TensorApplyCPU.Softmax, TensorApplyCPU.cs:1230-1268) written as sort keys: grid (rows), 1024 threads
-static __global__ __launch_bounds__(1024) void topp_keys_kernel(TopPArgs a) {
-    __shared__ float sred[16];
-    const int r = blockIdx.x, t = threadIdx.x, V = a.V;
+__device__ __forceinline__ float topp_row_max(const TopPArgs& a, int r) {
+    const float* sm = a.accp + (long)r * a.Vs;
+    float mx = sm[0];
+    for (int s2 = 1; s2 < a.nseg; ++s2) mx = fmaxf(mx, sm[s2]);
+    return mx;
+}
+
+static __global__ __launch_bounds__(256) void topp_rowsum_kernel(TopPArgs a) {
+    __shared__ float sred[4];
+    const int seg = blockIdx.x, r = blockIdx.y, t = threadIdx.x;
+    const float* row = a.in + (long)r * a.ld;
+    const float mx = topp_row_max(a, r);
+    float ls = 0.0f;
+#pragma unroll
+    for (int it = 0; it < 4; ++it) {
+        const int i = seg * TOPP_SEG + it * 256 + t;
+        if (i < a.V) ls += expf(row[i] / a.temperature - mx);
+    }
+    ls = wave_sum(ls);
+    if ((t & 63) == 0) sred[t >> 6] = ls;
+    __syncthreads();
+    if (t == 0) a.accp[(long)r * a.Vs + a.nseg + seg] = ((sred[0] + sred[1]) + sred[2]) + sred[3];
+}
+
+// probabilities (TensorApplyCPU.Softmax, TensorApplyCPU.cs:1230-1268) written as sort keys, and the digit counts of the
+// first sort pass: grid (nseg, rows), 256 threads.  The row's sum is the sum of the segment sums in segment order.
+static __global__ __launch_bounds__(256) void topp_keys_kernel(TopPArgs a) {
+    __shared__ unsigned s_key[TOPP_SEG];
+    __shared__ int s_hist[256];
+    const int seg = blockIdx.x, r = blockIdx.y, t = threadIdx.x, V = a.V;
+    const int i0 = seg * TOPP_SEG;
     const float* row = a.in + (long)r * a.ld;
     unsigned* kA = a.keysA + (long)r * a.Vs;
     int* iA = a.idxA + (long)r * a.Vs;
     float sum = 1.0f, mx = 0.0f;
     if (a.in_is_logits) {
-        float lm = -INFINITY;
-        for (int i = t; i < V; i += 1024) lm = fmaxf(lm, row[i] / a.temperature);
-        mx = block_max_1024(lm, sred);
-        float ls = 0.0f;
-        for (int i = t; i < V; i += 1024) ls += expf(row[i] / a.temperature - mx);
-        ls = wave_sum(ls);
-        __syncthreads();
-        if ((t & 63) == 0) sred[t >> 6] = ls;
-        __syncthreads();
-        sum = 0.0f;
-#pragma unroll
-        for (int i = 0; i < 16; ++i) sum += sred[i];
+        mx = topp_row_max(a, r);
+        const float* ss = a.accp + (long)r * a.Vs + a.nseg;
+        sum = ss[0];
+        for (int s2 = 1; s2 < a.nseg; ++s2) sum += ss[s2];
     }
     // Repeat penalty: few tokens of the vocabulary occur in the sequence, but almost every wavefront holds one of them, and
-    // the double-precision pow would be paid by all 64 lanes.  So the pass over the vocabulary only notes those tokens
+    // the double-precision pow would be paid by all 64 lanes.  So the pass over the segment only notes those tokens
     // (index and probability) in an LDS list, and the list is worked off densely afterwards.
-    constexpr int DECAY_CAP = 8192;          // 64 KiB of LDS; more distinct tokens than this in a sequence are decayed in place
-    __shared__ int s_didx[DECAY_CAP];
-    __shared__ float s_dp[DECAY_CAP];
+    __shared__ int s_didx[TOPP_SEG];
+    __shared__ float s_dp[TOPP_SEG];
     __shared__ int s_dn;
     const bool decay = a.last_pos && a.repeat_penalty != 0.0f;
     const int len = decay ? topp_seq_len(a, r) : 0;
@@ -129,28 +153,38 @@ static __global__ __launch_bounds__(1024) void topp_keys_kernel(TopPArgs a) {
     // p <= 0 is dropped by the reference: give it the largest key so that it sorts behind every candidate.
     auto key_of = [&](float p, int i) { return (p > 0.0f && !(a.blocked && a.blocked[i])) ? ~__float_as_uint(p) : 0xffffffffu; };
     if (t == 0) s_dn = 0;
+    s_hist[t] = 0;
     __syncthreads();
-    for (int i = t; i < V; i += 1024) {
-        float p = a.in_is_logits ? expf(row[i] / a.temperature - mx) / sum : row[i];
+#pragma unroll
+    for (int it = 0; it < 4; ++it) {
+        const int e = it * 256 + t, i = i0 + e;
+        if (i >= V) continue;
+        const float p = a.in_is_logits ? expf(row[i] / a.temperature - mx) / sum : row[i];
         if (decay && p > 0.0f) {
             const int lp = last[i];
-            if (lp >= 0) {
-                const int slot = atomicAdd(&s_dn, 1);
-                if (slot < DECAY_CAP) { s_didx[slot] = i; s_dp[slot] = p; }
-                else p = decayed(p, lp);                             // list full (sequences longer than the list): in place
-            }
+            if (lp >= 0) { const int slot = atomicAdd(&s_dn, 1); s_didx[slot] = e; s_dp[slot] = p; }      // (at most TOPP_SEG entries)
         }
-        kA[i] = key_of(p, i);
-        iA[i] = i;
+        s_key[e] = key_of(p, i);
     }
+    __syncthreads();
     if (decay) {
-        __syncthreads();
-        const int nd = min(s_dn, DECAY_CAP);
-        for (int e = t; e < nd; e += 1024) {
-            const int i = s_didx[e];
-            kA[i] = key_of(decayed(s_dp[e], last[i]), i);
+        const int nd = s_dn;
+        for (int k = t; k < nd; k += 256) {
+            const int e = s_didx[k], i = i0 + e;
+            s_key[e] = key_of(decayed(s_dp[k], last[i]), i);
         }
+        __syncthreads();
     }
+#pragma unroll
+    for (int it = 0; it < 4; ++it) {
+        const int e = it * 256 + t, i = i0 + e;
+        if (i >= V) continue;
+        const unsigned k = s_key[e];
+        kA[i] = k; iA[i] = i;
+        atomicAdd(&s_hist[k & 255u], 1);
+    }
+    __syncthreads();
+    a.hist[((long)r * a.nseg + seg) * 256 + t] = s_hist[t];
 }
 
 // digit counts of one segment: grid (nseg, rows), 256 threads
@@ -508,10 +542,15 @@ static __global__ __launch_bounds__(PICK_THREADS) void topp_pick_scan_kernel(Top
 // the whole pipeline; `launch_fn(name, kernel, grid, block, args)` puts one kernel on the library stream
 template <typename LaunchFn>
 inline void topp_run(TopPArgs a, int rows, LaunchFn&& launch_fn) {
-    launch_fn("topp_keys", topp_keys_kernel, dim3((unsigned)rows), dim3(1024), a);
+    const dim3 segs((unsigned)a.nseg, (unsigned)rows);
+    if (a.in_is_logits) {
+        launch_fn("topp_rowmax", topp_rowmax_kernel, segs, dim3(256), a);
+        launch_fn("topp_rowsum", topp_rowsum_kernel, segs, dim3(256), a);
+    }
+    launch_fn("topp_keys", topp_keys_kernel, segs, dim3(256), a);          // also the digit counts of pass 0
     for (int pass = 0; pass < 4; ++pass) {
         a.shift = pass * 8;
-        launch_fn("topp_hist", topp_hist_kernel, dim3((unsigned)a.nseg, (unsigned)rows), dim3(256), a);
+        if (pass > 0) launch_fn("topp_hist", topp_hist_kernel, dim3((unsigned)a.nseg, (unsigned)rows), dim3(256), a);
         launch_fn("topp_scan", topp_scan_kernel, dim3((unsigned)rows), dim3(256), a);
         launch_fn("topp_scatter", topp_scatter_kernel, dim3((unsigned)a.nseg, (unsigned)rows), dim3(256), a);
         unsigned* tk = a.keysA; a.keysA = a.keysB; a.keysB = tk;
