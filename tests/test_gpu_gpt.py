@@ -380,6 +380,18 @@ def test_moe_prefill_runs_the_experts_on_gathered_rows(G, oracle, dtype, batch, 
     gpu.close()
 
 
+@pytest.mark.parametrize("batch,experts", [(70, 4), (50, 2), (100, 2)])
+def test_moe_decode_batches_above_32_rows(G, oracle, batch, experts):
+    """Decode with MoE layers and more than 32 rows (two and four 32-row tiles per block in the expert GEMMs): 70 rows over
+    four experts; with two experts and two choices per token every expert gets all 50 or all 100 rows."""
+    cfg = synth.tiny_config(n_layers=3, n_experts=experts, experts_per_token=2, norm_type=synth.LAYERNORM, act=synth.RELU, dtype="f16",
+                            batch=batch, prompt=5, vocab=200)
+    orc, gpu, out, _ = _teacher_forced(G, oracle, cfg, 71, 3)
+    for lg, gl in out:
+        assert np.abs(gl - lg).max() <= FP16_ABS
+    gpu.close()
+
+
 def test_moe_tied_router_follows_topk_rule(G, oracle):
     cfg = synth.tiny_config(n_layers=3, n_experts=4, experts_per_token=2, norm_type=synth.LAYERNORM, act=synth.RELU, batch=5)
     w = synth.make_weights(cfg, 41, random_bias=True)
