@@ -2008,9 +2008,14 @@ __global__ __launch_bounds__(D == 128 ? 256 : 512) void attn_mfma_prefill_kernel
     const std::integral_constant<bool, false> plain; const std::integral_constant<bool, true> masked;
     const int n_own = active ? (T + 31) / 32 : 0;
     const int n_full = min(n_own, (pos_base + 1) / 32);
-    for (int c = 0; c < nchunks; ++c) {
+    // One loop per kind of chunk (unmasked, masked, not this wavefront's): with the kinds as branches of one loop the
+    // compiler copies the running outputs between registers around every branch, a third of the loop's instructions.
+    // Every wavefront passes the same nchunks barriers whatever its split.
+    auto step = [&](auto mode_c, int c) {
+        constexpr int MODE = decltype(mode_c)::value;         // 0: unmasked, 1: masked, 2: only the block's fetch and barrier
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");      // this wavefront's share of chunk c has landed
         __syncthreads();                                      // ... and everybody's; chunk c - 1 is consumed
+        if (MODE == 2) { if (c + 1 < nchunks) fetch(c + 1); return; }
         half8 kf[2][KD], vf[DT];
         const half_t* st = schunk[c & 1] + lane * 8;
 #pragma unroll
@@ -2024,8 +2029,13 @@ __global__ __launch_bounds__(D == 128 ? 256 : 512) void attn_mfma_prefill_kernel
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         __builtin_amdgcn_sched_barrier(0);
         if (c + 1 < nchunks) fetch(c + 1);
-        if (c < n_full) do_chunk(plain, c, kf, vf);
-        else if (c < n_own) do_chunk(masked, c, kf, vf);
+        if (MODE == 0) do_chunk(plain, c, kf, vf); else do_chunk(masked, c, kf, vf);
+    };
+    {
+        int c = 0;
+        for (; c < n_full; ++c) step(std::integral_constant<int, 0>{}, c);
+        for (; c < n_own; ++c) step(std::integral_constant<int, 1>{}, c);
+        for (; c < nchunks; ++c) step(std::integral_constant<int, 2>{}, c);
     }
     l_run += __shfl_xor(l_run, 16, 64);
     l_run += __shfl_xor(l_run, 32, 64);
