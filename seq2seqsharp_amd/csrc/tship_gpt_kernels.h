@@ -1710,7 +1710,8 @@ __global__ __launch_bounds__(D == 128 ? 256 : 512) void attn_mfma_kernel(AttnArg
                 const int vec = p / (D / 2), i = p % (D / 2);
                 float x0 = sIn[vec * D + 2 * i], x1 = sIn[vec * D + 2 * i + 1], y0 = x0, y1 = x1;
                 if (a.rope_cos) rope_pair(x0, x1, rc[pi], rs[pi], y0, y1);
-                if (vec < G) { sQ[vec][2 * i] = a.scale * y0; sQ[vec][2 * i + 1] = a.scale * y1; }
+                // (scores are kept in units of log 2, so that the exponentials below are bare v_exp_f32)
+                if (vec < G) { sQ[vec][2 * i] = (a.scale * 1.44269504f) * y0; sQ[vec][2 * i + 1] = (a.scale * 1.44269504f) * y1; }
                 else { Kb[kfrag_index(pos, 2 * i, D)] = (half_t)y0; Kb[kfrag_index(pos, 2 * i + 1, D)] = (half_t)y1; }
             }
         }
@@ -1724,10 +1725,9 @@ __global__ __launch_bounds__(D == 128 ? 256 : 512) void attn_mfma_kernel(AttnArg
 #pragma unroll
     for (int kd = 0; kd < KD; ++kd)
 #pragma unroll
-        for (int j = 0; j < 8; ++j) qf[kd][j] = (half_t)sQ[r16][kd * 32 + 8 * q + j];
-    // last position this lane's column may attend to
+        for (int j = 0; j < 8; ++j) qf[kd][j] = r16 < NCOL ? (half_t)sQ[r16][kd * 32 + 8 * q + j] : (half_t)0.0f;      // columns beyond the group: zero queries, scores 0
+    // last position the columns may attend to (the same for all: one query position per sequence)
     const int tmax = T - 1;
-    const bool col_ok = r16 < NCOL;
 
     float m_run = -INFINITY, l_run = 0.0f;
     floatx4 acc_o[DT];
@@ -1746,23 +1746,24 @@ __global__ __launch_bounds__(D == 128 ? 256 : 512) void attn_mfma_kernel(AttnArg
         float s[8];
 #pragma unroll
         for (int j = 0; j < 4; ++j) { s[j] = sA[j]; s[4 + j] = sB[j]; }
+        if (t0 + 31 > tmax) {          // only the chunk that holds the newest position has positions to hide
+#pragma unroll
+            for (int j = 0; j < 8; ++j) if (t0 + 8 * q + j > tmax) s[j] = -INFINITY;
+        }
         float cm = -INFINITY;
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            const int tj = t0 + 8 * q + j;
-            if (col_ok && tj > tmax) s[j] = -INFINITY;
-            if (!col_ok) s[j] = 0.0f;
-            cm = fmaxf(cm, s[j]);
-        }
+        for (int j = 0; j < 8; ++j) cm = fmaxf(cm, s[j]);
         cm = fmaxf(cm, __shfl_xor(cm, 16, 64));
         cm = fmaxf(cm, __shfl_xor(cm, 32, 64));
+        // (a chunk that is processed has a visible position, so m_new is finite; exp2(-inf) = 0 covers hidden positions
+        // and the first chunk's m_run)
         const float m_new = fmaxf(m_run, cm);
-        const float corr = (m_new == -INFINITY) ? 1.0f : __expf(m_run - m_new);     // m_run = -inf -> 0, and the sums are still 0
+        const float corr = __builtin_amdgcn_exp2f(m_run - m_new);
         half8 pf;
         float psum = 0.0f;
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
-            const float p = (s[j] == -INFINITY) ? 0.0f : __expf(s[j] - m_new);
+            const float p = __builtin_amdgcn_exp2f(s[j] - m_new);
             psum += p;
             pf[j] = (half_t)p;
         }
@@ -1838,7 +1839,7 @@ __global__ __launch_bounds__(D == 128 ? 256 : 512) void attn_mfma_kernel(AttnArg
             float L = 0.0f, O = 0.0f;
 #pragma unroll
             for (int i = 0; i < NW; ++i) {
-                const float wgt = (sM[i][col] == -INFINITY) ? 0.0f : __expf(sM[i][col] - M);
+                const float wgt = (sM[i][col] == -INFINITY) ? 0.0f : __builtin_amdgcn_exp2f(sM[i][col] - M);
                 L += sL[i][col] * wgt;
                 O += sO[i][d][col] * wgt;
             }
@@ -1862,7 +1863,7 @@ __global__ __launch_bounds__(D == 128 ? 256 : 512) void attn_mfma_kernel(AttnArg
             float L = 0.0f, O = 0.0f;
             for (int s = 0; s < a.S; ++s) {
                 const float ms = __hip_atomic_load(base + s * per + NCOL * D + col, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                const float wgt = (ms == -INFINITY) ? 0.0f : __expf(ms - M);
+                const float wgt = (ms == -INFINITY) ? 0.0f : __builtin_amdgcn_exp2f(ms - M);
                 L += __hip_atomic_load(base + s * per + NCOL * D + NCOL + col, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) * wgt;
                 O += __hip_atomic_load(base + s * per + idx, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) * wgt;
             }
@@ -1882,7 +1883,7 @@ __global__ __launch_bounds__(D == 128 ? 256 : 512) void attn_mfma_kernel(AttnArg
         float L = 0.0f, O = 0.0f;
 #pragma unroll
         for (int i = 0; i < NW; ++i) {
-            const float wgt = (sM[i][col] == -INFINITY) ? 0.0f : __expf(sM[i][col] - M);
+            const float wgt = (sM[i][col] == -INFINITY) ? 0.0f : __builtin_amdgcn_exp2f(sM[i][col] - M);
             L += sL[i][col] * wgt;
             O += sO[i][d][col] * wgt;
         }
