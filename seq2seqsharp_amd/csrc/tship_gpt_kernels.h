@@ -1628,12 +1628,11 @@ __global__ __launch_bounds__(D == 128 ? 256 : 512) void attn_mfma_kernel(AttnArg
     const int r16 = lane & 15, q = lane >> 4;
     const int HD = a.H * D, GD = a.Hkv * D;
     const int kvh = blockIdx.x, b = blockIdx.y;
-    const int pos_base = *a.d_pos, T = pos_base + 1;
+    // (the position is requested here and first used behind the prologue's other requests, which do not depend on it:
+    // one memory round trip for both instead of one after the other)
+    const int pos_base = *a.d_pos;
     half_t* Kb = (half_t*)a.kcache + ((long)b * a.Hkv + kvh) * a.max_len * D;
     half_t* Vt = (half_t*)a.vcache + ((long)b * a.Hkv + kvh) * (long)D * a.max_len;
-
-    // geometry needed by the early loads
-    const int nchunks = (T + 31) / 32;
     half8 kfA[2][KD], vfA[DT];
     auto load_chunk = [&](int c, half8 (&kf)[2][KD], half8 (&vf)[DT]) {
         const half_t* kc = Kb + (long)c * (32 * D) + lane * 8;
@@ -1651,17 +1650,19 @@ __global__ __launch_bounds__(D == 128 ? 256 : 512) void attn_mfma_kernel(AttnArg
     // behind them; every later chunk is requested right before the chunk ahead of it is processed.  The first request
     // is unconditional so that the waits below are counted exactly; a first chunk that holds the row being appended
     // is requested again after the prologue.
-    const int n_own = nchunks > gw ? (nchunks - gw + GS - 1) / GS : 0;
-    const bool validA = gw < nchunks - 1;
-
     for (int i = t; i < 16 * D; i += NTH) (&sQ[0][0])[i] = 0.0f;
+    int T, nchunks, n_own; bool validA;
     {
         constexpr int CPT = ((G + 2) * D + NTH - 1) / NTH;        // projection columns per thread
         constexpr int PPT = ((G + 1) * D / 2 + NTH - 1) / NTH;    // rotary pairs per thread
-        const int pos = pos_base;
         // every global load of the prologue is issued before the first use
-        float ssq_part = 0.0f;
-        if (a.ssq) for (int tt = lane; tt < a.ssq_nt; tt += 64) ssq_part += a.ssq[(long)tt * a.ssq_ld + b];
+        // (the first four tile sums of a lane are requested without a wait of their own: a load-and-add loop would cost a
+        // memory round trip ahead of every other request; they are added below in the same order)
+        float ssq_part = 0.0f, ssq_v[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+        if (a.ssq) {      // (unconditional requests at clamped indices; the values beyond the last tile are dropped below)
+#pragma unroll
+            for (int u = 0; u < 4; ++u) ssq_v[u] = a.ssq[(long)min(lane + 64 * u, a.ssq_nt - 1) * a.ssq_ld + b];
+        }
         float part[CPT][8], bias[CPT];
 #pragma unroll
         for (int ci = 0; ci < CPT; ++ci) {
@@ -1679,6 +1680,11 @@ __global__ __launch_bounds__(D == 128 ? 256 : 512) void attn_mfma_kernel(AttnArg
                 bias[ci] = a.bias[col];
             }
         }
+        __builtin_amdgcn_sched_barrier(0);
+        const int pos = pos_base;
+        T = pos_base + 1; nchunks = (T + 31) / 32;
+        n_own = nchunks > gw ? (nchunks - gw + GS - 1) / GS : 0;
+        validA = gw < nchunks - 1;
         float rc[PPT], rs[PPT];
 #pragma unroll
         for (int pi = 0; pi < PPT; ++pi) {
@@ -1691,7 +1697,13 @@ __global__ __launch_bounds__(D == 128 ? 256 : 512) void attn_mfma_kernel(AttnArg
         load_chunk(min(gw, (int)(a.max_len >> 5) - 1), kfA, vfA);
         __builtin_amdgcn_sched_barrier(0);
         float rinv = 1.0f;
-        if (a.ssq) rinv = 1.0f / sqrtf(wave_sum(ssq_part) * a.inv_h + a.eps);
+        if (a.ssq) {
+#pragma unroll
+            for (int u = 0; u < 4; ++u) if (lane + 64 * u >= a.ssq_nt) ssq_v[u] = 0.0f;
+            ssq_part = ((ssq_v[0] + ssq_v[1]) + ssq_v[2]) + ssq_v[3];
+            for (int tt = lane + 256; tt < a.ssq_nt; tt += 64) ssq_part += a.ssq[(long)tt * a.ssq_ld + b];
+            rinv = 1.0f / sqrtf(wave_sum(ssq_part) * a.inv_h + a.eps);
+        }
 #pragma unroll
         for (int ci = 0; ci < CPT; ++ci) {
             const int idx = t + ci * NTH;
