@@ -319,14 +319,20 @@ class OracleGpt:
     def set_cache(self, layer, which, data, BH, T, d):
         _chk(lib().orc_gpt_set_cache(self.h, layer, which, _f(data), BH, T, d))
 
-    def moe_trace(self, ordinal, R):
+    def moe_trace(self, ordinal, R=None):
+        """Routing of MoE layer number `ordinal` at the last step, for all rows that step fed (B at a cached step, B * len
+        at a full-sequence step).  R, when given, must be that row count."""
         k, E = self.cfg["experts_per_token"], self.cfg["n_experts"]
-        ti = np.empty((R, k), np.float32)
-        tv = np.empty((R, k), np.float32)
-        pr = np.empty((R, E), np.float32)
-        n = lib().orc_gpt_moe_trace(self.h, ordinal, _vp(ti), _vp(tv), _vp(pr), R * k)
+        n = lib().orc_gpt_moe_trace(self.h, ordinal, None, None, None, 0)
         if n < 0:
             raise IndexError("no such MoE layer trace")
+        rows = n // k
+        if R is not None and R != rows:
+            raise ValueError("the last step routed %d rows, not %d" % (rows, R))
+        ti = np.empty((rows, k), np.float32)
+        tv = np.empty((rows, k), np.float32)
+        pr = np.empty((rows, E), np.float32)
+        lib().orc_gpt_moe_trace(self.h, ordinal, _vp(ti), _vp(tv), _vp(pr), rows * k)
         return ti, tv, pr
 
     def moe_layer(self, layer, x):

@@ -1664,10 +1664,11 @@ __global__ __launch_bounds__(D == 128 ? 256 : 512) void attn_mfma_kernel(AttnArg
             for (int u = 0; u < 4; ++u) ssq_v[u] = a.ssq[(long)min(lane + 64 * u, a.ssq_nt - 1) * a.ssq_ld + b];
         }
         float part[CPT][8], bias[CPT];
+        int pcol[CPT];
 #pragma unroll
         for (int ci = 0; ci < CPT; ++ci) {
             const int idx = t + ci * NTH;
-            bias[ci] = 0.0f;
+            bias[ci] = 0.0f; pcol[ci] = 0;
 #pragma unroll
             for (int k = 0; k < 8; ++k) part[ci][k] = 0.0f;
             if (idx < (G + 2) * D) {
@@ -1675,6 +1676,7 @@ __global__ __launch_bounds__(D == 128 ? 256 : 512) void attn_mfma_kernel(AttnArg
                 if (idx < G * D) col = kvh * G * D + idx;
                 else if (idx < (G + 1) * D) col = HD + kvh * D + (idx - G * D);
                 else col = HD + GD + kvh * D + (idx - (G + 1) * D);
+                pcol[ci] = col;
 #pragma unroll
                 for (int k = 0; k < 8; ++k) if (k < a.KS) part[ci][k] = a.qkv[k * a.split_stride + (long)b * a.ldq + col];
                 bias[ci] = a.bias[col];
@@ -1711,6 +1713,7 @@ __global__ __launch_bounds__(D == 128 ? 256 : 512) void attn_mfma_kernel(AttnArg
                 float s = part[ci][0];
 #pragma unroll
                 for (int k = 1; k < 8; ++k) if (k < a.KS) s += part[ci][k];
+                for (int k = 8; k < a.KS; ++k) s += a.qkv[k * a.split_stride + (long)b * a.ldq + pcol[ci]];     // (more than eight splits: wide models at batches above 64)
                 sIn[idx] = s * rinv + bias[ci];
             }
         }

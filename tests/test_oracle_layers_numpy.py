@@ -1,0 +1,211 @@
+"""Arithmetic pins of the oracle's layer compositions: float64 NumPy restatements of one attention layer (grouped-query
+and classic multi-head), the dense feed-forward layer and the whole decoder step, written from the reference's layer
+code in a different form than the oracle (per-head loops on [B, T, ...] arrays instead of the reference's
+view / transpose / expand / batched-multiply sequence), so that a wrong score scale, a softmax over the wrong axis, a
+dropped bias, a wrong head-to-KV-head map or an activation on the wrong factor of the gate shows.
+
+Reference: Seq2SeqSharp/Layers/GroupQueryAttention.cs:114-233, Layers/MultiHeadAttention.cs:125-240,
+Layers/PositionwiseFeedForward.cs:72-116, Networks/GPTDecoder.cs:153-191, Applications/Decoder.cs:648-733,
+TensorSharp/TensorApplyCPU.cs:1148-1178 (RoPE), :1016-1036 (causal mask), :1360-1496 (norms)."""
+import numpy as np
+import pytest
+
+from seq2seqsharp_amd import synth
+
+F64 = np.float64
+
+
+def norm64(cfg, w, prefix, x):
+    g = w[prefix + ".m_alpha"].astype(F64).reshape(-1)
+    if cfg["norm_type"] == synth.LAYERNORM:
+        mu = x.mean(1, keepdims=True)
+        var = ((x - mu) ** 2).mean(1, keepdims=True)
+        return g * (x - mu) / np.sqrt(var + cfg["norm_eps"]) + w[prefix + ".m_beta"].astype(F64).reshape(-1)
+    return g * x / np.sqrt((x * x).mean(1, keepdims=True) + cfg["norm_eps"])
+
+
+def rope64(cfg, v, pos):
+    """v [..., d] at sequence position pos: pairs (2i, 2i+1) rotated by pos * base^(-2i/d); the angle is formed in
+    float32 as the reference does (theta and theta * m are floats), its cosine and sine in double."""
+    d = v.shape[-1]
+    i = np.arange(d // 2)
+    theta = np.power(F64(cfg["rope_base"]), -2.0 * i / d).astype(np.float32)
+    ang = (theta * np.float32(pos)).astype(np.float32).astype(F64)
+    c, s = np.cos(ang), np.sin(ang)
+    out = np.empty_like(v)
+    out[..., 0::2] = v[..., 0::2] * c - v[..., 1::2] * s
+    out[..., 1::2] = v[..., 1::2] * c + v[..., 0::2] * s
+    return out
+
+
+def attention64(cfg, w, layer, x, B, Tq, past=None, causal=True, mut=None):
+    """x [B*Tq, h] -> (x + attention output, (keys, values)) with keys/values [B, Hkv, T, d] after RoPE.
+    past: (keys, values) of earlier positions.  The new rows sit at positions len(past) .. len(past) + Tq - 1.
+    mut: a deliberate mistake (tests use it to show that the tolerance would catch that mistake)."""
+    name = f"GPTDecoder.SelfAttn_{layer}"
+    h, H, Hkv = cfg["hidden"], cfg["n_heads"], cfg["n_kv_heads"]
+    d = h // H
+    n = norm64(cfg, w, name + ".layerNormQ", x)
+    if cfg["attn_type"] == synth.GQA:
+        q = n @ w[name + ".Q"].astype(F64) + (0.0 if mut == "bias" else w[name + ".Qb"].astype(F64).reshape(-1))
+        k = n @ w[name + ".K"].astype(F64) + w[name + ".Kb"].astype(F64).reshape(-1)
+        v = n @ w[name + ".V"].astype(F64) + w[name + ".Vb"].astype(F64).reshape(-1)
+    else:                                                    # fused projection, columns ordered [3][H][d]
+        qkv = n @ w[name + ".QKV"].astype(F64) + (0.0 if mut == "bias" else w[name + ".QKVb"].astype(F64).reshape(-1))
+        q, k, v = qkv[:, :h], qkv[:, h:2 * h], qkv[:, 2 * h:]
+    q = q.reshape(B, Tq, H, d)
+    k = k.reshape(B, Tq, Hkv, d)
+    v = v.reshape(B, Tq, Hkv, d)
+    off = 0 if past is None else past[0].shape[2]
+    if cfg["use_rope"]:
+        for t in range(Tq):
+            q[:, t] = rope64(cfg, q[:, t], off + t)
+            k[:, t] = rope64(cfg, k[:, t], off + t)
+    keys = k.transpose(0, 2, 1, 3)
+    vals = v.transpose(0, 2, 1, 3)
+    if past is not None:
+        keys = np.concatenate([past[0], keys], 2)
+        vals = np.concatenate([past[1], vals], 2)
+    T = keys.shape[2]
+    out = np.zeros((B, Tq, H, d), F64)
+    for b in range(B):
+        for hh in range(H):
+            kv = hh % Hkv if mut == "headmap" else hh // (H // Hkv)
+            for t in range(Tq):
+                s = keys[b, kv] @ q[b, t, hh] / (F64(d) if mut == "scale" else np.sqrt(F64(d)))         # [T]
+                if causal and past is None:
+                    s = s + np.where(np.arange(T) <= t, 0.0, -30000.0)   # additive mask, only built without a cache
+                p = np.exp(s - s.max())
+                p = p / p.sum()
+                out[b, t, hh] = p @ vals[b, kv]
+    y = out.reshape(B * Tq, h) @ w[name + ".W0"].astype(F64) + w[name + ".b0"].astype(F64).reshape(-1)
+    return x + y, (keys, vals)
+
+
+def ffn64(cfg, w, layer, x):
+    name = f"GPTDecoder.PosFFN_{layer}"
+    n = norm64(cfg, w, name + ".layerNorm2", x)
+    a = n @ w[name + ".feedForwardLayer1.m_Whd"].astype(F64) + w[name + ".feedForwardLayer1.m_Bd"].astype(F64).reshape(-1)
+    act = cfg["act"]
+    if act == synth.RELU:
+        a = np.maximum(a, 0.0)
+    elif act in (synth.SILU, synth.SWIGLU_SILU):
+        a = a / (1.0 + np.exp(-a))
+    elif act == synth.LEAKYRELU:
+        a = np.where(a < 0, 0.01 * a, a)
+    # SWIGLU: the reference's RunActivateFunction has no branch for it, the first factor stays linear
+    if act in (synth.SWIGLU, synth.SWIGLU_SILU):
+        a = a * (n @ w[name + ".feedForwardLayer3.m_Whd"].astype(F64) + w[name + ".feedForwardLayer3.m_Bd"].astype(F64).reshape(-1))
+    y = a @ w[name + ".feedForwardLayer2.m_Whd"].astype(F64) + w[name + ".feedForwardLayer2.m_Bd"].astype(F64).reshape(-1)
+    return x + y
+
+
+def gpt64(cfg, w, seqs, past=None):
+    """Whole sequences (no cache) or the last token on top of `past` (one (keys, values) pair per layer).
+    Returns (logits [B, V], final-norm hidden [B, h], new past)."""
+    B, ln = seqs.shape
+    h = cfg["hidden"]
+    ids = seqs if past is None else seqs[:, -1:]
+    Tq = ids.shape[1]
+    x = w["TgtEmbeddings"].astype(F64)[ids.reshape(-1)] * F64(np.float32(np.sqrt(np.float32(h))))
+    new = []
+    for layer in range(cfg["n_layers"]):
+        x, kv = attention64(cfg, w, layer, x, B, Tq, None if past is None else past[layer])
+        new.append(kv)
+        x = ffn64(cfg, w, layer, x)
+    hid = norm64(cfg, w, "GPTDecoder.layerNorm", x).reshape(B, Tq, h)[:, -1]
+    logits = hid @ w["FeedForward_Decoder_0.m_Whd"].astype(F64) + w["FeedForward_Decoder_0.m_Bd"].astype(F64).reshape(-1)
+    return logits, hid, new
+
+
+def _sharpen(w):
+    """N(0, 0.02) projections give almost uniform attention, which hides mistakes in the scores: widen Q and K."""
+    out = dict(w)
+    for k, v in w.items():
+        if k.endswith((".Q", ".K", ".Qb", ".Kb", ".QKV", ".QKVb")):
+            out[k] = (v * np.float32(12.0)).astype(np.float32)
+    return out
+
+
+ATTN_CASES = {
+    "gqa_rms": dict(),
+    "gqa_ln_g4": dict(hidden=96, n_heads=12, n_kv_heads=3, norm_type=synth.LAYERNORM, act=synth.RELU),
+    "mha_rms": dict(attn_type=synth.MHA, n_kv_heads=4),
+    "mha_ln": dict(attn_type=synth.MHA, n_kv_heads=4, norm_type=synth.LAYERNORM, act=synth.RELU),
+    "gqa_no_rope": dict(use_rope=0),
+}
+
+
+@pytest.mark.parametrize("name", sorted(ATTN_CASES))
+def test_attention_layer_prefill_and_cached_step(oracle, name):
+    cfg = synth.tiny_config(n_layers=1, **ATTN_CASES[name])
+    w = _sharpen(synth.make_weights(cfg, 17, random_bias=True))
+    B, Tq, h = 3, 6, cfg["hidden"]
+    rng = np.random.default_rng(5)
+    x = rng.standard_normal((B * Tq, h)).astype(np.float32)
+    m = oracle.OracleGpt(cfg, w)
+    y = m.attn_layer(0, x, B, Tq, True, True)                      # causal prefill, fills the oracle's cache
+    y64, past = attention64(cfg, w, 0, x.astype(F64), B, Tq)
+    assert np.abs(y - y64).max() <= 1e-5
+    x1 = rng.standard_normal((B, h)).astype(np.float32)
+    y1 = m.attn_layer(0, x1, B, 1, False, True)                    # one cached step: no mask, RoPE offset Tq
+    y164, past2 = attention64(cfg, w, 0, x1.astype(F64), B, 1, past)
+    assert np.abs(y1 - y164).max() <= 1e-5
+    assert past2[0].shape[2] == Tq + 1 == m.cache_len()
+    # the comparison is sensitive to what it is meant to pin: each deliberate mistake moves the output far beyond 1e-5
+    for mut in ("scale", "bias") + (("headmap",) if cfg["n_kv_heads"] not in (1, cfg["n_heads"]) else ()):
+        bad, _ = attention64(cfg, w, 0, x.astype(F64), B, Tq, mut=mut)
+        assert np.abs(bad - y64).max() > 1e-3, mut
+
+
+@pytest.mark.parametrize("act", [synth.RELU, synth.SILU, synth.LEAKYRELU, synth.SWIGLU, synth.SWIGLU_SILU])
+@pytest.mark.parametrize("norm", [synth.RMSNORM, synth.LAYERNORM])
+def test_dense_ffn_layer(oracle, act, norm):
+    cfg = synth.tiny_config(n_layers=1, act=act, norm_type=norm)
+    w = synth.make_weights(cfg, 19, random_bias=True)
+    x = np.random.default_rng(7).standard_normal((7, cfg["hidden"])).astype(np.float32)
+    y = oracle.OracleGpt(cfg, w).ffn_layer(0, x)
+    y64 = ffn64(cfg, w, 0, x.astype(F64))
+    assert np.abs(y - y64).max() <= 1e-5
+    if act == synth.SWIGLU:
+        # the reference's "SwiGLU" differs from the textbook one (SiLU on the gate) by far more than the tolerance
+        assert np.abs(ffn64(dict(cfg, act=synth.SWIGLU_SILU), w, 0, x.astype(F64)) - y64).max() > 1e-3
+
+
+@pytest.mark.parametrize("name", ["gqa_rms", "mha_ln", "gqa_ln_g4"])
+def test_decoder_step_logits(oracle, name):
+    """Two layers, prompt through the mask path, then two steps on the cache: logits, final hidden state, greedy tokens."""
+    cfg = synth.tiny_config(n_layers=2, **ATTN_CASES[name])
+    w = _sharpen(synth.make_weights(cfg, 23, random_bias=True))
+    seqs = synth.make_prompts(cfg, 24)
+    m = oracle.OracleGpt(cfg, w)
+    p, lg, hid = m.step(seqs, use_cache=True, want_hidden=True)
+    lg64, hid64, past = gpt64(cfg, w, seqs)
+    assert np.abs(hid - hid64).max() <= 1e-5
+    assert np.abs(lg - lg64).max() <= 1e-5
+    sm = np.exp(lg64 - lg64.max(1, keepdims=True))
+    assert np.abs(p - sm / sm.sum(1, keepdims=True)).max() <= 1e-6
+    cur = seqs
+    for _ in range(2):
+        nxt = lg64.argmax(1).astype(np.int32)
+        assert np.array_equal(nxt, oracle.argmax(p).astype(np.int32))
+        cur = np.concatenate([cur, nxt[:, None]], 1)
+        p, lg = m.step(cur, use_cache=True)
+        lg64, _, past = gpt64(cfg, w, cur, past)
+        assert np.abs(lg - lg64).max() <= 1e-5
+    # without a cache the whole sequence is recomputed under the mask: same logits
+    lg_full, _, _ = gpt64(cfg, w, cur)
+    assert np.abs(lg_full - lg64).max() <= 1e-9
+
+
+def test_temperature_divides_logits_only_when_sampling(oracle):
+    """Decoder.cs:720-723: the division happens for DecodingStrategy == Sampling and temperature != 1 only."""
+    cfg = synth.tiny_config(n_layers=1)
+    w = synth.make_weights(cfg, 29, random_bias=True)
+    seqs = synth.make_prompts(cfg, 30)
+    lg64, _, _ = gpt64(cfg, w, seqs)
+    m = oracle.OracleGpt(cfg, w)
+    _, lg = m.step(seqs, use_cache=False, temperature=0.5, sampling=True)
+    assert np.abs(lg - lg64 / 0.5).max() <= 2e-5
+    _, lg = m.step(seqs, use_cache=False, temperature=0.5, sampling=False)
+    assert np.abs(lg - lg64).max() <= 1e-5
