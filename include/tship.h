@@ -116,6 +116,15 @@ TSHIP_API int TSHip_TopPSample(const TSHipTensor* result, const TSHipTensor* pro
 TSHIP_API int TSHip_TopPSampleEx(const TSHipTensor* result, const TSHipTensor* probs, const TSHipTensor* uniforms, float top_p, float repeat_penalty,
                                  const int32_t* host_seqs, const int32_t* host_seq_lens, int seq_ld);
 
+/* TSHip_TopPSample for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc): no counterpart in the reference.  Same arguments, same kernels and same result as
+ * TSHip_TopPSample, but the pipeline's scratch (sort keys, indices, running sums, digit counts) lives in a fixed 6 MiB
+ * device array inside the library instead of a per-call allocation, and nothing is allocated, freed or synchronised.
+ * Limit: rows * 20 * round_up(columns, 64) + rows * ceil(columns / 1024) * 1024 bytes must fit in 6 MiB (about 300000
+ * probabilities, e.g. 8 rows of 32000); larger inputs fail with an error.  TSHip_Init must have been called.  All calls
+ * on a GPU share that GPU's array: calls that overlap in time on one GPU race; calls on the library stream do not. */
+TSHIP_API int TSHip_TopPSampleNoAlloc(const TSHipTensor* result, const TSHipTensor* probs, const TSHipTensor* uniforms, float top_p);
+
 /* ---- fused GPTDecoder path: one object per model replica, preallocated compact KV cache, the whole
  *      token loop on the device (replaces GPT.RunForwardOnSingleDevice, Seq2SeqSharp/Applications/GPT.cs:212-335,
  *      Decoder.GPTDecode, Applications/Decoder.cs:648-794, and GPTDecoder.Decode, Networks/GPTDecoder.cs:153-191). ---- */

@@ -50,6 +50,8 @@ struct Error : std::runtime_error {
 // The library's ordered stream (created by TSHip_Init, default priority).
 hipStream_t stream();
 void ensure_init();
+int current_device();          // device the library was initialised on, -1 before TSHip_Init
+void noalloc_device_setup(int device);   // tship_ops.hip: address of the fixed scratch array, once per device
 int n_compute_units();
 
 typedef _Float16 half_t;

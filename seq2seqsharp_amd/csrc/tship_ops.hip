@@ -11,6 +11,25 @@
 
 namespace tship {
 
+// Scratch of TSHip_TopPSampleNoAlloc, the entry point that allocates nothing: sort keys, indices, running sums and digit
+// counts of the top-p pipeline.  Every GPU the library runs on holds its own copy of this array, at its own address, until
+// the process ends.  In host code the array's name is only a stand-in for that address: the address is asked for once per
+// device at initialisation (noalloc_device_setup) and only that pointer is ever handed to kernels.
+constexpr size_t NOALLOC_SCRATCH_BYTES = 6u << 20;
+static __device__ __align__(256) unsigned char scratch[NOALLOC_SCRATCH_BYTES];
+constexpr int NOALLOC_MAX_DEVICES = 64;
+static unsigned char* g_scratch_ptr[NOALLOC_MAX_DEVICES] = {};
+
+// called by TSHip_Init with `device` current
+void noalloc_device_setup(int device) {
+    TSHIP_REQUIRE(device >= 0 && device < NOALLOC_MAX_DEVICES, "TSHip_Init: device id beyond the per-device scratch table");
+    if (g_scratch_ptr[device]) return;
+    unsigned char* ptr = nullptr;
+    TSHIP_CHECK_HIP(hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(scratch)));
+    TSHIP_REQUIRE(ptr != nullptr, "TSHip_Init: the device scratch array has no address");
+    g_scratch_ptr[device] = ptr;
+}
+
 struct View {
     void* p; int dtype; int nd;
     long sz[TSHIP_MAX_DIMS]; long st[TSHIP_MAX_DIMS];
@@ -684,6 +703,34 @@ static int topp_sample_op(const char* who, const TSHipTensor* result, const TSHi
 
 TSHIP_API int TSHip_TopPSample(const TSHipTensor* result, const TSHipTensor* probs, const TSHipTensor* uniforms, float top_p) {
     return topp_sample_op("TSHip_TopPSample", result, probs, uniforms, top_p, 0.0f, nullptr, nullptr, 0);
+}
+
+TSHIP_API int TSHip_TopPSampleNoAlloc(const TSHipTensor* result, const TSHipTensor* probs, const TSHipTensor* uniforms, float top_p) {
+    TSHIP_BEGIN
+    const int dev = current_device();
+    TSHIP_REQUIRE(dev >= 0 && dev < NOALLOC_MAX_DEVICES && g_scratch_ptr[dev], "TSHip_TopPSampleNoAlloc: call TSHip_Init first (this entry point sets nothing up by itself)");
+    const char* who = "TSHip_TopPSampleNoAlloc";
+    View r = make_view(result, who), p = make_view(probs, who), u = make_view(uniforms, who);
+    TSHIP_REQUIRE(p.nd == 2 && p.dtype == TSHIP_F32 && p.st[1] == 1, "TSHip_TopPSampleNoAlloc: probs must be a Float32 matrix with contiguous rows");
+    const long rows = p.sz[0], K = p.sz[1];
+    TSHIP_REQUIRE(K >= 1 && K <= 65535, "TSHip_TopPSampleNoAlloc: between 1 and 65535 columns are supported");
+    TSHIP_REQUIRE(count(r) == rows && r.dtype == TSHIP_F32 && is_contiguous(r), "TSHip_TopPSampleNoAlloc: result must be a contiguous Float32 [rows,1] tensor");
+    TSHIP_REQUIRE(count(u) == rows && u.dtype == TSHIP_F32 && is_contiguous(u), "TSHip_TopPSampleNoAlloc: uniforms must be a contiguous Float32 [rows] tensor");
+    if (rows == 0) return 1;
+    const size_t need = topp_scratch_bytes(rows, K);
+    TSHIP_REQUIRE(need <= NOALLOC_SCRATCH_BYTES, "TSHip_TopPSampleNoAlloc: rows x columns needs " + std::to_string(need) + " bytes of scratch, the fixed scratch holds " +
+                                                     std::to_string(NOALLOC_SCRATCH_BYTES) + " (about 300000 probabilities); use TSHip_TopPSample");
+    TopPArgs a; std::memset(&a, 0, sizeof(a));
+    a.in = (const float*)p.p; a.ld = p.st[0]; a.V = (int)K; a.in_is_logits = 0; a.temperature = 1.0f;
+    a.uniforms = (const float*)u.p; a.top_p = top_p;
+    // (every kernel of the pipeline writes what it later reads, digit counts included: nothing has to start at zero)
+    topp_carve(a, g_scratch_ptr[dev], rows, K);
+    a.out_f32 = (float*)r.p;
+    topp_run(a, (int)rows, [&](const char*, void (*kernel)(TopPArgs), dim3 grid, dim3 block, const TopPArgs& args) {
+        hipLaunchKernelGGL(kernel, grid, block, 0, stream(), args);
+    });
+    TSHIP_CHECK_HIP(hipGetLastError());
+    TSHIP_END
 }
 
 TSHIP_API int TSHip_TopPSampleEx(const TSHipTensor* result, const TSHipTensor* probs, const TSHipTensor* uniforms, float top_p, float repeat_penalty,

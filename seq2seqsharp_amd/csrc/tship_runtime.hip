@@ -17,6 +17,7 @@ static hipStream_t g_stream = nullptr;
 static int g_cus = 0;
 
 hipStream_t stream() { return g_stream; }
+int current_device() { return g_initialised ? g_device : -1; }
 int n_compute_units() { return g_cus; }
 
 static void init_locked(int device_id) {
@@ -37,6 +38,7 @@ static void init_locked(int device_id) {
     if (arch.rfind("gfx950", 0) != 0)
         throw Error("TSHip_Init: this library is built for gfx950 (MI355X); device reports " + arch);
     g_cus = prop.multiProcessorCount;
+    noalloc_device_setup(device_id);
     TSHIP_CHECK_HIP(hipStreamCreateWithFlags(&g_stream, hipStreamNonBlocking));
     g_device = device_id;
     g_initialised = true;

@@ -44,6 +44,7 @@ def _p():
     L.TSHip_BuildSelfTriMask.argtypes = [T, T, C.c_int, C.c_float, C.c_float]
     L.TSHip_IsCorrupted.argtypes = [T, C.POINTER(C.c_int)]
     L.TSHip_TopPSample.argtypes = [T, T, T, C.c_float]
+    L.TSHip_TopPSampleNoAlloc.argtypes = [T, T, T, C.c_float]
     L.TSHip_TopPSampleEx.argtypes = [T, T, T, C.c_float, C.c_float, C.c_void_p, C.c_void_p, C.c_int]
     _ok = True
     return L
@@ -252,6 +253,13 @@ def toppsample(result, probs, uniforms, top_p, repeat_penalty=0.0, seqs=None, se
     check(_p().TSHip_TopPSampleEx(_d(r), _d(probs), _d(uniforms), float(top_p), float(repeat_penalty),
                                   seqs.ctypes.data_as(C.c_void_p), lens.ctypes.data_as(C.c_void_p), int(seqs.shape[1])))
     return r
+
+
+def toppsample_noalloc(result, probs, uniforms, top_p):
+    """TSHip_TopPSample on the library's fixed scratch array: nothing is allocated, so `result` must be supplied.  Not
+    synchronised: read the result after a synchronising call (HipTensor.numpy does)."""
+    check(_p().TSHip_TopPSampleNoAlloc(_d(result), _d(probs), _d(uniforms), float(top_p)))
+    return result
 
 
 def concat(dim, tensors):
