@@ -67,6 +67,8 @@ struct LayerW {
     // MoE (Seq2SeqSharp/Layers/MoEFeedForward.cs:49-55)
     DevBuf router, router_b;               // fp32 [h][E], [E]
     std::vector<std::unique_ptr<GemmW>> e1, e2;   // per expert [h][4h], [4h][h]
+    DevBuf wtab1, wtab2;                   // device tables of the experts' weight pointers (fp16 decode GEMMs batch over them); written once at Finalize
+    DevBuf route;                          // this layer's routing at the last step: probs [Bpad][E], top values [Bpad][k], top indices [Bpad][k]
 };
 
 struct Profiler {
@@ -1035,6 +1037,18 @@ TSHIP_API int TSHip_GptFinalize(TSHipGpt* m) {
             L->w2.KS = m->BT == 1 ? tail_ks(L->w2) : (L->w2.KS <= 2 ? 1 : L->w2.KS);
         }
     }
+    for (auto& L : m->L) {
+        if (!L->moe) continue;
+        const int E = m->c.n_experts, k = m->c.experts_per_token;
+        L->route.alloc((size_t)m->Bpad * (E + 2 * k) * sizeof(float));
+        if (!m->f16) continue;
+        std::vector<const void*> t1(E), t2(E);
+        for (int e = 0; e < E; ++e) { t1[e] = L->e1[e]->buf.p; t2[e] = L->e2[e]->buf.p; }
+        L->wtab1.alloc(E * sizeof(void*)); L->wtab2.alloc(E * sizeof(void*));
+        TSHIP_CHECK_HIP(hipMemcpyAsync(L->wtab1.p, t1.data(), E * sizeof(void*), hipMemcpyHostToDevice, stream()));
+        TSHIP_CHECK_HIP(hipMemcpyAsync(L->wtab2.p, t2.data(), E * sizeof(void*), hipMemcpyHostToDevice, stream()));
+        TSHIP_CHECK_HIP(hipStreamSynchronize(stream()));       // (the host tables are locals)
+    }
     m->finalized = true;
     TSHIP_END
 }
@@ -1144,8 +1158,7 @@ static int generate_impl(TSHipGpt* m, int n_steps, int mode, float top_p, float 
     TSHIP_CHECK_HIP(hipMemsetAsync(m->d_pos.as<int>() + 1, 0, sizeof(int), stream()));
     const int* d_step = m->d_pos.as<int>() + 1;
     const float* uni_base = mode == TSHIP_TOPP ? uni.as<float>() : nullptr;
-    bool any_moe = false; for (auto& L : m->L) any_moe = any_moe || L->moe;
-    const bool use_graph = !any_moe && std::getenv("TSHIP_NO_GRAPH") == nullptr;
+    const bool use_graph = std::getenv("TSHIP_NO_GRAPH") == nullptr;
     if (mode == TSHIP_TOPP) {      // scratch must exist before capture (no allocation inside a graph)
         const size_t need = topp_scratch_bytes(m->Bpad, m->c.vocab);
         if (m->topp_scratch.bytes < need) m->topp_scratch.alloc(need);

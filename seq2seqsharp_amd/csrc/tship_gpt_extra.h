@@ -5,7 +5,7 @@
 namespace tship {
 
 struct MoeLayout {
-    size_t xn32, probs, top_val, top_idx, counts, lists, slot, xg, mid, y, wtab1, wtab2, zero, total;
+    size_t xn32, probs, top_val, top_idx, counts, lists, slot, xg, mid, y, zero, total;
     long ld4h, ldy;
 };
 
@@ -21,7 +21,6 @@ static MoeLayout moe_layout(TSHipGpt* m, long cap) {
     o.xg = take(E * Bp * m->ldh * m->esz());
     o.mid = take(E * Bp * o.ld4h * m->esz());
     o.y = take(E * Bp * o.ldy * 4);
-    o.wtab1 = take(E * sizeof(void*)); o.wtab2 = take(E * sizeof(void*));
     o.zero = take(std::max<long>(4 * h, 64) * 4);
     o.total = at;
     return o;
@@ -33,14 +32,14 @@ static void moe_alloc(TSHipGpt* m) {
 }
 
 static void moe_get_routing(TSHipGpt* m, int layer, float* top_idx, float* top_val, float* probs) {
-    (void)layer;   // the workspace holds the routing of the MoE layer that ran last; callers run one layer at a time
-    MoeLayout o = moe_layout(m, m->Bpad);
+    LayerW& L = *m->L[layer];
     const int B = m->cur_batch, k = m->c.experts_per_token, E = m->c.n_experts;
+    TSHIP_REQUIRE(L.route.p, "TSHip_GptGetMoeRouting: call TSHip_GptFinalize first");
     TSHIP_CHECK_HIP(hipStreamSynchronize(stream()));
-    char* base = (char*)m->moe_ws.p;
-    if (top_idx) TSHIP_CHECK_HIP(hipMemcpy(top_idx, base + o.top_idx, (size_t)B * k * 4, hipMemcpyDeviceToHost));
-    if (top_val) TSHIP_CHECK_HIP(hipMemcpy(top_val, base + o.top_val, (size_t)B * k * 4, hipMemcpyDeviceToHost));
-    if (probs) TSHIP_CHECK_HIP(hipMemcpy(probs, base + o.probs, (size_t)B * E * 4, hipMemcpyDeviceToHost));
+    const float* base = L.route.as<float>();
+    if (probs) TSHIP_CHECK_HIP(hipMemcpy(probs, base, (size_t)B * E * 4, hipMemcpyDeviceToHost));
+    if (top_val) TSHIP_CHECK_HIP(hipMemcpy(top_val, base + (size_t)m->Bpad * E, (size_t)B * k * 4, hipMemcpyDeviceToHost));
+    if (top_idx) TSHIP_CHECK_HIP(hipMemcpy(top_idx, base + (size_t)m->Bpad * (E + k), (size_t)B * k * 4, hipMemcpyDeviceToHost));
 }
 
 // `pre` carries the pending attention output (split-K partials + bias) and the LayerNorm parameters
@@ -55,8 +54,13 @@ static void run_moe_ffn_impl(TSHipGpt* m, LayerW& L, int rows, const ResidNormAr
     char* base = (char*)(batched ? m->pw_moe.p : m->moe_ws.p);
     TSHIP_REQUIRE(rows <= cap && o.total <= (batched ? m->pw_moe.bytes : m->moe_ws.bytes), "internal: MoE workspace too small");
     const int h = c.hidden, E = c.n_experts, k = c.experts_per_token; const long Bp = cap;
-    float* xn32 = (float*)(base + o.xn32); float* probs = (float*)(base + o.probs);
-    float* top_val = (float*)(base + o.top_val); float* top_idx = (float*)(base + o.top_idx);
+    // decode steps write the routing straight into the layer's own buffers (TSHip_GptGetMoeRouting reads them); a prefill
+    // routes all rows in the workspace and copies every sequence's last position there afterwards
+    float* lroute = L.route.as<float>();
+    TSHIP_REQUIRE(lroute && (size_t)m->Bpad * (E + 2 * k) * sizeof(float) <= L.route.bytes, "internal: routing buffers missing (TSHip_GptFinalize allocates them)");
+    float* xn32 = (float*)(base + o.xn32); float* probs = batched ? (float*)(base + o.probs) : lroute;
+    float* top_val = batched ? (float*)(base + o.top_val) : lroute + (size_t)m->Bpad * E;
+    float* top_idx = batched ? (float*)(base + o.top_idx) : lroute + (size_t)m->Bpad * (E + k);
     int* counts = (int*)(base + o.counts); int* lists = (int*)(base + o.lists); int* slot = (int*)(base + o.slot);
     float* y = (float*)(base + o.y); float* zero = (float*)(base + o.zero);
 
@@ -68,7 +72,11 @@ static void run_moe_ffn_impl(TSHipGpt* m, LayerW& L, int rows, const ResidNormAr
     r.xn32 = xn32; r.probs = probs; r.top_val = top_val; r.top_idx = top_idx;
     r.router_lds = ((long)E * h <= 16384) ? 1 : 0;
     const unsigned router_shm = (unsigned)((2L * h + (r.router_lds ? (long)E * h : 0)) * sizeof(float));
-    launch_shm(m, "moe_router", moe_router_kernel, dim3(rows), dim3(256), router_shm, r);
+    if (m->f16) {      // tree-order sums: an fp16 model's routing input is not the reference's to the last bit anyway
+        if (h <= 1024) launch(m, "moe_router", moe_router_fast_kernel<4>, dim3(rows), dim3(256), r);
+        else if (h <= 2048) launch(m, "moe_router", moe_router_fast_kernel<8>, dim3(rows), dim3(256), r);
+        else launch(m, "moe_router", moe_router_fast_kernel<16>, dim3(rows), dim3(256), r);
+    } else launch_shm(m, "moe_router", moe_router_kernel, dim3(rows), dim3(256), router_shm, r);
     // decode-sized batches: the gather kernel builds the lists itself (one launch less)
     const bool fused_lists = !batched && (long)rows * k <= 1024;
     if (batched) launch(m, "moe_lists", moe_lists_big_kernel, dim3(E), dim3(1024), (const float*)top_idx, rows, k, (int)Bp, counts, lists, slot);
@@ -99,31 +107,27 @@ static void run_moe_ffn_impl(TSHipGpt* m, LayerW& L, int rows, const ResidNormAr
                                 counts, lists, slot, (int)Bp, xg, m->ldh, xg_stride, (int)(m->ldh / 16));
         else launch(m, "moe_gather", moe_gather_kernel<half_t>, dim3(rows, E), dim3(256), (const float*)xn32, h, (const int*)counts, (const int*)lists, (int)Bp, xg,
                m->ldh, xg_stride, (int)(m->ldh / 16));
-        // pointer tables are written once per layer object (weights never move)
-        std::vector<const half_t*> t1(E), t2(E);
-        for (int e = 0; e < E; ++e) { t1[e] = L.e1[e]->buf.as<half_t>(); t2[e] = L.e2[e]->buf.as<half_t>(); }
-        TSHIP_CHECK_HIP(hipMemcpyAsync(base + o.wtab1, t1.data(), E * sizeof(void*), hipMemcpyHostToDevice, stream()));
-        TSHIP_CHECK_HIP(hipMemcpyAsync(base + o.wtab2, t2.data(), E * sizeof(void*), hipMemcpyHostToDevice, stream()));
-        TSHIP_CHECK_HIP(hipStreamSynchronize(stream()));
+        // (the experts' weight pointer tables were written once, when the model was finalised: no host work in a step)
+        TSHIP_REQUIRE(L.wtab1.p && L.wtab2.p, "internal: expert pointer tables missing (TSHip_GptFinalize builds them)");
         SkinnyArgs e1; std::memset(&e1, 0, sizeof(e1));
-        e1.W = t1[0]; e1.KT = L.e1[0]->KT; e1.NT = L.e1[0]->NT; e1.X = xg; e1.ldx = (int)m->ldh; e1.KS = 1;
+        e1.W = L.e1[0]->buf.as<half_t>(); e1.KT = L.e1[0]->KT; e1.NT = L.e1[0]->NT; e1.X = xg; e1.ldx = (int)m->ldh; e1.KS = 1;
         e1.bias = zero; e1.out16 = mid; e1.ld16 = (int)o.ld4h; e1.out16_kt = L.e2[0]->KT; e1.act = c.act; e1.gated = 0; e1.n_valid = 4 * h;
-        e1.Wtab = (const half_t* const*)(base + o.wtab1); e1.x_estride = xg_stride; e1.out16_estride = mid_stride; e1.rows_tab = counts;
+        e1.Wtab = (const half_t* const*)L.wtab1.p; e1.x_estride = xg_stride; e1.out16_estride = mid_stride; e1.rows_tab = counts;
         SkinnyArgs e2; std::memset(&e2, 0, sizeof(e2));
-        e2.W = t2[0]; e2.KT = L.e2[0]->KT; e2.NT = L.e2[0]->NT; e2.X = mid; e2.ldx = (int)o.ld4h; e2.KS = 1;
+        e2.W = L.e2[0]->buf.as<half_t>(); e2.KT = L.e2[0]->KT; e2.NT = L.e2[0]->NT; e2.X = mid; e2.ldx = (int)o.ld4h; e2.KS = 1;
         e2.bias = zero; e2.out = y; e2.ld_out = (int)o.ldy; e2.n_valid = h;
-        e2.Wtab = (const half_t* const*)(base + o.wtab2); e2.x_estride = mid_stride; e2.out_estride = y_stride; e2.rows_tab = counts;
-        dim3 g1(e1.NT, E), g2(e2.NT, E);
-        if (m->BT == 1) {
-            launch(m, "moe_gemm1", skinny_gemm_f16_kernel<1, EPI_ACT16, 8>, g1, dim3(512), e1);
-            launch(m, "moe_gemm2", skinny_gemm_f16_kernel<1, EPI_F32_BIAS, 8>, g2, dim3(512), e2);
-        } else if (m->BT == 2) {
-            launch(m, "moe_gemm1", skinny_gemm_f16_kernel<2, EPI_ACT16, 8>, g1, dim3(512), e1);
-            launch(m, "moe_gemm2", skinny_gemm_f16_kernel<2, EPI_F32_BIAS, 8>, g2, dim3(512), e2);
-        } else {
-            launch(m, "moe_gemm1", skinny_gemm_f16_kernel<4, EPI_ACT16, 4>, g1, dim3(256), e1);
-            launch(m, "moe_gemm2", skinny_gemm_f16_kernel<4, EPI_F32_BIAS, 4>, g2, dim3(256), e2);
-        }
+        e2.Wtab = (const half_t* const*)L.wtab2.p; e2.x_estride = mid_stride; e2.out_estride = y_stride; e2.rows_tab = counts;
+        // Up projection: one 32-row tile per block with the tile number on blockIdx.z.  The experts of a decode step mostly
+        // hold fewer than 32 rows, so the kernel for one row tile does the work (single-barrier reduction) and the blocks of
+        // empty row tiles exit at once: 16.4 us against 24 us with two row tiles per block at 8 experts x 1024 x 4096.
+        // Measured and not used: 2 or 4 column tiles per block with one copy of the activations (20 and 23 us), and the same
+        // split for the down projection (19.1 against 17.9 us: its 256 blocks are one round either way).
+        e1.row_tiles_z = 1;
+        launch(m, "moe_gemm1", skinny_gemm_f16_kernel<1, EPI_ACT16, 8>, dim3(e1.NT, E, (unsigned)m->BT), dim3(512), e1);
+        dim3 g2(e2.NT, E);
+        if (m->BT == 1) launch(m, "moe_gemm2", skinny_gemm_f16_kernel<1, EPI_F32_BIAS, 8>, g2, dim3(512), e2);
+        else if (m->BT == 2) launch(m, "moe_gemm2", skinny_gemm_f16_kernel<2, EPI_F32_BIAS, 8>, g2, dim3(512), e2);
+        else launch(m, "moe_gemm2", skinny_gemm_f16_kernel<4, EPI_F32_BIAS, 4>, g2, dim3(256), e2);
     } else {
         float* xg = (float*)(base + o.xg); float* mid = (float*)(base + o.mid);
         if (fused_lists) launch(m, "moe_gather", moe_gather_lists_kernel<float>, dim3(rows, E), dim3(256), (const float*)top_idx, rows, k, (const float*)xn32, h,
@@ -153,11 +157,9 @@ static void run_moe_ffn_impl(TSHipGpt* m, LayerW& L, int rows, const ResidNormAr
     }
     if (batched && last_rows) {
         // what TSHip_GptGetMoeRouting reports after a prefill: the routing of every sequence's last position
-        MoeLayout d = moe_layout(m, m->Bpad);
-        char* db = (char*)m->moe_ws.p;
-        launch(m, "moe_last_rows", moe_rows_kernel, dim3(n_last), dim3(64), (const float*)probs, last_rows, (float*)(db + d.probs), E);
-        launch(m, "moe_last_rows", moe_rows_kernel, dim3(n_last), dim3(64), (const float*)top_val, last_rows, (float*)(db + d.top_val), k);
-        launch(m, "moe_last_rows", moe_rows_kernel, dim3(n_last), dim3(64), (const float*)top_idx, last_rows, (float*)(db + d.top_idx), k);
+        launch(m, "moe_last_rows", moe_rows_kernel, dim3(n_last), dim3(64), (const float*)probs, last_rows, lroute, E);
+        launch(m, "moe_last_rows", moe_rows_kernel, dim3(n_last), dim3(64), (const float*)top_val, last_rows, lroute + (size_t)m->Bpad * E, k);
+        launch(m, "moe_last_rows", moe_rows_kernel, dim3(n_last), dim3(64), (const float*)top_idx, last_rows, lroute + (size_t)m->Bpad * (E + k), k);
     }
 }
 

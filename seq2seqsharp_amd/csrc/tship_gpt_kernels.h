@@ -93,6 +93,7 @@ struct SkinnyArgs {
     // optional batch of independent problems (MoE experts) on blockIdx.y: weights from a pointer table,
     // activations / outputs at a fixed stride, row counts read on the device
     const half_t* const* Wtab; long x_estride; long out_estride; long out16_estride; const int* rows_tab;
+    int row_tiles_z;       // batched problems only: blockIdx.z selects a 32-row tile (kernels instantiated for one row tile)
     // deferred RMSNorm: the input rows were stored as half(gamma * x); the epilogue multiplies row b by
     // 1 / sqrt(sum_t ssq[t][b] / h + eps), the factor the norm would have applied (exact up to rounding)
     const float* ssq; int ssq_nt; int ssq_ld; float inv_h; float eps;
@@ -133,7 +134,17 @@ __global__ __launch_bounds__(NW * 64) void skinny_gemm_f16_kernel(SkinnyArgs a) 
     if (a.Wtab) {
         const int e = blockIdx.y;
         a.rows_valid = a.rows_tab[e];
-        if (a.rows_valid == 0) return;
+        if (a.row_tiles_z) {
+            // one 32-row tile per block, tile number on blockIdx.z: an expert with at most 32 rows (the usual case at decode)
+            // costs one block per column tile, the blocks of its empty row tiles leave at once; an expert with more rows
+            // has its weights streamed once per row tile
+            const int rt = blockIdx.z;
+            a.rows_valid -= 32 * rt;
+            a.X += (long)rt * a.KT * 512;
+            if (a.out) a.out += (long)rt * 32 * a.ld_out;
+            if (a.out16) a.out16 += a.out16_kt > 0 ? (long)rt * a.out16_kt * 512 : (long)rt * 32 * a.ld16;
+        }
+        if (a.rows_valid <= 0) return;
         a.W = a.Wtab[e]; a.X += e * a.x_estride;
         if (a.out) a.out += e * a.out_estride;
         if (a.out16) a.out16 += e * a.out16_estride;
@@ -1099,17 +1110,51 @@ __global__ __launch_bounds__(256) void resid_norm_kernel(ResidNormArgs a) {
     }
     if (a.moe_y) {
 #pragma clang fp contract(off)
-        for (int i = 0; i < NPT; ++i) {
-            const int c = t + i * 256;
-            if (c >= a.h) continue;
-            float out = 0.0f;
-            for (int e = 0; e < a.moe_E; ++e)
-                for (int j = 0; j < a.moe_k; ++j)
-                    if ((int)a.moe_top[xr * a.moe_k + j] == e) {
-                        float sc = a.moe_y[e * a.moe_estride + (long)a.moe_slot[xr * a.moe_k + j] * a.moe_ldy + c] * a.moe_probs[xr * a.moe_E + e];
-                        out += sc;
+        constexpr int MAXK = 4;
+        if (a.moe_k <= MAXK) {
+            // the row's choices, their slots and probabilities once; then every expert output at once; added in expert order
+            int te[MAXK], ts[MAXK]; float tp[MAXK], yv[MAXK][NPT];
+#pragma unroll
+            for (int j = 0; j < MAXK; ++j) {
+                te[j] = j < a.moe_k ? (int)a.moe_top[xr * a.moe_k + j] : -1;
+                ts[j] = j < a.moe_k ? a.moe_slot[xr * a.moe_k + j] : 0;
+            }
+#pragma unroll
+            for (int j = 0; j < MAXK; ++j) {
+                tp[j] = te[j] >= 0 ? a.moe_probs[xr * a.moe_E + te[j]] : 0.0f;
+#pragma unroll
+                for (int i = 0; i < NPT; ++i) {
+                    const int c = t + i * 256;
+                    yv[j][i] = (te[j] >= 0 && c < a.h) ? a.moe_y[te[j] * a.moe_estride + (long)ts[j] * a.moe_ldy + c] : 0.0f;
+                }
+            }
+            float out[NPT];
+#pragma unroll
+            for (int i = 0; i < NPT; ++i) out[i] = 0.0f;
+            for (int e = 0; e < a.moe_E; ++e) {
+#pragma unroll
+                for (int j = 0; j < MAXK; ++j) {
+                    if (te[j] == e) {
+#pragma unroll
+                        for (int i = 0; i < NPT; ++i) { const float sc = yv[j][i] * tp[j]; out[i] += sc; }
                     }
-            v[i] = v[i] + out;
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < NPT; ++i) v[i] = v[i] + out[i];
+        } else {
+            for (int i = 0; i < NPT; ++i) {
+                const int c = t + i * 256;
+                if (c >= a.h) continue;
+                float out = 0.0f;
+                for (int e = 0; e < a.moe_E; ++e)
+                    for (int j = 0; j < a.moe_k; ++j)
+                        if ((int)a.moe_top[xr * a.moe_k + j] == e) {
+                            float sc = a.moe_y[e * a.moe_estride + (long)a.moe_slot[xr * a.moe_k + j] * a.moe_ldy + c] * a.moe_probs[xr * a.moe_E + e];
+                            out += sc;
+                        }
+                v[i] = v[i] + out;
+            }
         }
     }
     float sum = 0.0f, sq = 0.0f;

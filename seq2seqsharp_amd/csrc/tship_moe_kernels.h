@@ -36,6 +36,7 @@ __global__ __launch_bounds__(256) void moe_router_kernel(MoeRouterArgs a) {
 #pragma clang fp contract(off)
     extern __shared__ __attribute__((aligned(16))) float moe_smem[];
     __shared__ float sr[64];
+    __shared__ float s_ov[64], s_oi[64];
     __shared__ float s_stat[2];
     const int r = blockIdx.x, t = threadIdx.x, h = a.h, E = a.E;
     float* sx = moe_smem;
@@ -163,15 +164,24 @@ __global__ __launch_bounds__(256) void moe_router_kernel(MoeRouterArgs a) {
         sr[t] = acc + (-65000.0f);
     }
     __syncthreads();
-    if (t == 0) {
-        const int k = a.k;
+    // the exponentials (evaluated in double, the expensive part) do not depend on each other: one lane per expert; only
+    // their sum has an order
+    if (t < 64) {
         float mx = sr[0];
         for (int e = 1; e < E; ++e) mx = fmaxf(mx, sr[e]);
+        const float ex = t < E ? (float)exp((double)(sr[t] - mx)) : 0.0f;
+        __builtin_amdgcn_wave_barrier();
+        if (t < E) sr[t] = ex;
+    }
+    __syncthreads();
+    if (t == 0) {
+        const int k = a.k;
         float sum = 0.0f;
-        for (int e = 0; e < E; ++e) { float ex = (float)exp((double)(sr[e] - mx)); sr[e] = ex; sum += ex; }
+        for (int e = 0; e < E; ++e) sum += sr[e];
         float* pr = a.probs + (long)r * E;
         for (int e = 0; e < E; ++e) { sr[e] = sr[e] / sum; pr[e] = sr[e]; }
-        float* ov = a.top_val + (long)r * k; float* oi = a.top_idx + (long)r * k;
+        // (the insertion works on LDS copies: on the global arrays every step would be a memory round trip)
+        float* ov = s_ov; float* oi = s_oi;
         for (int i = 0; i < k; ++i) { ov[i] = -1.70141e+38f; oi[i] = -1.70141e+38f; }
         for (int e = 0; e < E; ++e) {
             float data = sr[e];
@@ -183,6 +193,113 @@ __global__ __launch_bounds__(256) void moe_router_kernel(MoeRouterArgs a) {
             }
             if (j < 0) { ov[0] = data; oi[0] = (float)e; }
         }
+        for (int i = 0; i < k; ++i) { a.top_val[(long)r * k + i] = ov[i]; a.top_idx[(long)r * k + i] = oi[i]; }
+    }
+}
+
+// The same routing for fp16 models, one block of 256 threads per token row, everything requested in one memory round
+// trip and reduced as trees.  An fp16 model's activations differ from the fp32 reference's by the fp16 path's rounding
+// (about 1e-3), which already decides near-ties differently, so reproducing the reference's serial summation order (the
+// 1024-step chains of the kernel above) buys nothing there; that kernel remains the one fp32 models use, where routing
+// indices are bit-exact.  Same outputs: x updated with the pending attention output, LayerNorm in fp32, router logits
+// + (-65000), softmax with the exponentials evaluated in double, TopK by the reference's insertion rule.
+template <int NPT>      // NPT * 256 >= hidden
+__global__ __launch_bounds__(256) void moe_router_fast_kernel(MoeRouterArgs a) {
+    constexpr int MAXE = 64;
+    __shared__ float sred[4];
+    __shared__ float swe[4][MAXE];
+    __shared__ float sr[MAXE];
+    __shared__ float s_ov[MAXE], s_oi[MAXE];
+    const int r = blockIdx.x, t = threadIdx.x, h = a.h, E = a.E, lane = t & 63, w = t >> 6;
+    float v[NPT], g[NPT], bt[NPT];
+    {
+        float xv[NPT], bv[NPT], pv[NPT][4];
+#pragma unroll
+        for (int i = 0; i < NPT; ++i) {
+            const int c = t + i * 256; const bool ok = c < h;
+            xv[i] = ok ? a.x[(long)r * a.ldx + c] : 0.0f;
+            bv[i] = (ok && a.part) ? a.bias[c] : 0.0f;
+#pragma unroll
+            for (int k = 0; k < 4; ++k) pv[i][k] = (ok && a.part && k < a.KS) ? a.part[k * a.split_stride + (long)r * a.ld_part + c] : 0.0f;
+            g[i] = ok ? a.gamma[c] : 0.0f; bt[i] = ok ? a.beta[c] : 0.0f;
+        }
+#pragma unroll
+        for (int i = 0; i < NPT; ++i) {
+            const int c = t + i * 256;
+            v[i] = xv[i];
+            if (a.part && c < h) {
+                float s = pv[i][0];
+#pragma unroll
+                for (int k = 1; k < 4; ++k) if (k < a.KS) s += pv[i][k];
+                for (int k = 4; k < a.KS; ++k) s += a.part[k * a.split_stride + (long)r * a.ld_part + c];
+                v[i] = (s + bv[i]) + xv[i];
+                a.x[(long)r * a.ldx + c] = v[i];
+            }
+        }
+    }
+    float sum = 0.0f;
+#pragma unroll
+    for (int i = 0; i < NPT; ++i) sum += v[i];                 // (columns beyond h hold zeros)
+    const float mean = block_sum_256(sum, sred) / (float)h;
+    float d2 = 0.0f;
+#pragma unroll
+    for (int i = 0; i < NPT; ++i) { const int c = t + i * 256; if (c < h) { const float d = v[i] - mean; d2 += d * d; } }
+    const float sigma = sqrtf(a.eps + block_sum_256(d2, sred) / (float)h);
+    float y[NPT];
+#pragma unroll
+    for (int i = 0; i < NPT; ++i) {
+        const int c = t + i * 256;
+        y[i] = 0.0f;
+        if (c < h) { y[i] = g[i] * ((v[i] - mean) / sigma) + bt[i]; a.xn32[(long)r * h + c] = y[i]; }
+    }
+    // router logits: every thread's columns against all experts, then a tree over the block
+    for (int e0 = 0; e0 < E; e0 += 8) {
+        float acc[8], wv[NPT][8];
+#pragma unroll
+        for (int i = 0; i < NPT; ++i) {
+            const int c = t + i * 256;
+#pragma unroll
+            for (int u = 0; u < 8; ++u) wv[i][u] = (c < h && e0 + u < E) ? a.router[(long)c * E + e0 + u] : 0.0f;
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) acc[u] = 0.0f;
+#pragma unroll
+        for (int i = 0; i < NPT; ++i) {
+#pragma unroll
+            for (int u = 0; u < 8; ++u) acc[u] += y[i] * wv[i][u];
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) { acc[u] = wave_sum(acc[u]); if (lane == 0 && e0 + u < E) swe[w][e0 + u] = acc[u]; }
+    }
+    __syncthreads();
+    if (t < 64) {
+        float lg = -INFINITY;
+        if (t < E) lg = ((((swe[0][t] + swe[1][t]) + swe[2][t]) + swe[3][t]) + a.router_b[t]) + (-65000.0f);
+        const float mx = wave_max(lg);
+        const float ex = t < E ? (float)exp((double)(lg - mx)) : 0.0f;
+        if (t < E) sr[t] = ex;
+    }
+    __syncthreads();
+    if (t == 0) {
+        const int k = a.k;
+        float s = 0.0f;
+        for (int e = 0; e < E; ++e) s += sr[e];
+        float* pr = a.probs + (long)r * E;
+        for (int e = 0; e < E; ++e) { sr[e] = sr[e] / s; pr[e] = sr[e]; }
+        // (the insertion works on LDS copies: on the global arrays every step would be a memory round trip)
+        float* ov = s_ov; float* oi = s_oi;
+        for (int i = 0; i < k; ++i) { ov[i] = -1.70141e+38f; oi[i] = -1.70141e+38f; }
+        for (int e = 0; e < E; ++e) {
+            float data = sr[e];
+            if (data < ov[k - 1]) continue;
+            int j = k - 2;
+            for (; j >= 0; --j) {
+                if (data > ov[j]) { ov[j + 1] = ov[j]; oi[j + 1] = oi[j]; }
+                else { ov[j + 1] = data; oi[j + 1] = (float)e; break; }
+            }
+            if (j < 0) { ov[0] = data; oi[0] = (float)e; }
+        }
+        for (int i = 0; i < k; ++i) { a.top_val[(long)r * k + i] = ov[i]; a.top_idx[(long)r * k + i] = oi[i]; }
     }
 }
 
