@@ -160,6 +160,14 @@ TSHIP_API int TSHip_GptReset(TSHipGpt* m);
  * empty after Create / Reset; a later call continues the same sequences, e.g. the next turn of a dialogue whose cache
  * was kept, GPT.cs:236-247,312-328) and leaves the last-position logits on the device (Decoder.cs:679-716) */
 TSHIP_API int TSHip_GptPrefill(TSHipGpt* m, const int32_t* host_ids, int batch, int prompt_len);
+/* prefill of sequences of different lengths, as the reference runs them when padding is allowed (Decoder.cs:656, 687-690):
+ * ids [batch, padded_len] hold every sequence padded with the END tag to the longest (BuildInTokens.PadSentences,
+ * Corpus/BuildInTokens.cs:68-101), host_lens [batch] the original lengths.  Masking is BuildSelfTriMask's
+ * (TensorApplyCPU.cs:1040-1065): a row inside its sequence sees the columns up to itself, a padding row has every column
+ * masked (so it attends to the whole padded sequence).  As in the reference, all sequences continue from position
+ * padded_len: the logits are those of every row's LAST PADDED position and the padding stays in the cache.  The cache must
+ * be empty (Create / Reset). */
+TSHIP_API int TSHip_GptPrefillPadded(TSHipGpt* m, const int32_t* host_ids, const int32_t* host_lens, int batch, int padded_len);
 /* one decode step with the given tokens (Decoder.cs:661-678); leaves logits on the device */
 TSHIP_API int TSHip_GptDecode(TSHipGpt* m, const int32_t* host_ids, int batch);
 /* DecodingOptions.RepeatPenalty (Applications/DecodingOptions.cs:23, default 2.0 there; 0 here until set): top-p sampling

@@ -711,8 +711,10 @@ static Tensor decoder(const Model& m, Tensor x, const Tensor* mask, long B, Cach
 // seqs: B rows of `len` token ids (the whole sequence so far).  With a non-empty cache only the last token
 // of each row is fed (Decoder.cs:661-678); otherwise the whole sequence with a causal mask (:679-700).
 // Returns probs [B,V]; logits (before softmax, after the temperature division) are written to logitsOut if given.
+// lens (optional): the sequences' lengths before PadSentences made them `len` long (Decoder.cs:656); given, the mask of the
+// full-sequence branch is BuildSelfTriMask over them (Decoder.cs:687-690, PaddingType other than NoPadding, batch > 1).
 static Tensor gpt_step(const Model& m, const int* seqs, long B, long len, Cache* cache, float temperature, bool sampling,
-                       float* logitsOut, std::vector<MoETrace>* traces, float* hiddenOut) {
+                       float* logitsOut, std::vector<MoETrace>* traces, float* hiddenOut, const float* lens = nullptr) {
     long Tq; std::vector<float> ids;
     Tensor mask; bool haveMask = false;
     if (cache && !cache->empty()) {
@@ -721,9 +723,15 @@ static Tensor gpt_step(const Model& m, const int* seqs, long B, long len, Cache*
     } else {
         Tq = len; ids.resize(B * len);
         for (long i = 0; i < B * len; ++i) ids[i] = (float)seqs[i];
-        mask = Tensor(std::vector<long>{Tq, Tq});
-        buildtrimask(mask.p(), Tq, Tq, 0.0f, -30000.0f);                                // g.BuildTriMask, ComputeGraphTensor.cs:3932-3935
-        mask = mask.view({1, 1, Tq, Tq}); haveMask = true;
+        if (lens) {
+            mask = Tensor(std::vector<long>{B, Tq, Tq});
+            buildselftrimask(mask.p(), lens, B * Tq, Tq, (int)Tq, 0.0f, -30000.0f);     // g.BuildSelfTriMask, ComputeGraphTensor.cs:3903-3909
+            mask = mask.view({B, 1, Tq, Tq}); haveMask = true;
+        } else {
+            mask = Tensor(std::vector<long>{Tq, Tq});
+            buildtrimask(mask.p(), Tq, Tq, 0.0f, -30000.0f);                            // g.BuildTriMask, ComputeGraphTensor.cs:3932-3935
+            mask = mask.view({1, 1, Tq, Tq}); haveMask = true;
+        }
     }
     // TensorUtils.CreateTokensEmbeddings, Utils/TensorUtils.cs:44-162: IndexSelect then Mul(scalar) in place
     const Tensor& E = m.W("TgtEmbeddings");
@@ -878,6 +886,17 @@ ORC_API int orc_gpt_step(void* h, const int* seqs, long B, long len, int use_cac
     auto* g = (OrcGpt*)h;
     g->traces.clear();
     Tensor p = gpt_step(g->m, seqs, B, len, use_cache ? &g->cache : nullptr, temperature, sampling != 0, logits_out, &g->traces, hidden_out);
+    if (probs_out) std::memcpy(probs_out, p.p(), sizeof(float) * p.count());
+    ORC_CATCH
+}
+// The same call on sequences that PadSentences brought to one length: seqs [B, len] padded (with the END tag), lens [B]
+// their original lengths as floats (BuildInTokens.PadSentences returns them so).
+ORC_API int orc_gpt_step_padded(void* h, const int* seqs, long B, long len, const float* lens, int use_cache, float temperature, int sampling,
+                                float* probs_out, float* logits_out, float* hidden_out) {
+    ORC_TRY
+    auto* g = (OrcGpt*)h;
+    g->traces.clear();
+    Tensor p = gpt_step(g->m, seqs, B, len, use_cache ? &g->cache : nullptr, temperature, sampling != 0, logits_out, &g->traces, hidden_out, lens);
     if (probs_out) std::memcpy(probs_out, p.p(), sizeof(float) * p.count());
     ORC_CATCH
 }

@@ -75,6 +75,7 @@ def lib():
     L.orc_gpt_cache_len.argtypes = [C.c_void_p]
     L.orc_gpt_cache_len.restype = C.c_long
     L.orc_gpt_step.argtypes = [C.c_void_p, i32p, C.c_long, C.c_long, C.c_int, C.c_float, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]
+    L.orc_gpt_step_padded.argtypes = [C.c_void_p, i32p, C.c_long, C.c_long, f32p, C.c_int, C.c_float, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]
     L.orc_gpt_get_cache.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_long]
     L.orc_gpt_get_cache.restype = C.c_long
     L.orc_gpt_set_cache.argtypes = [C.c_void_p, C.c_int, C.c_int, f32p, C.c_long, C.c_long, C.c_long]
@@ -296,14 +297,20 @@ class OracleGpt:
     def cache_len(self):
         return lib().orc_gpt_cache_len(self.h)
 
-    def step(self, seqs, use_cache=True, temperature=1.0, sampling=False, want_hidden=False):
-        """seqs: int array [B, len] (whole sequences so far).  Returns (probs, logits[, hidden])."""
+    def step(self, seqs, use_cache=True, temperature=1.0, sampling=False, want_hidden=False, lens=None):
+        """seqs: int array [B, len] (whole sequences so far).  Returns (probs, logits[, hidden]).
+        lens: original lengths of sequences that were padded to `len` (the reference's PadSentences + BuildSelfTriMask
+        branch); only the first, full-sequence call looks at them."""
         seqs = np.ascontiguousarray(seqs, dtype=np.int32)
         B, ln = seqs.shape
         V = self.cfg["vocab"]
         probs = np.empty((B, V), np.float32)
         logits = np.empty((B, V), np.float32)
         hidden = np.empty((B, self.cfg["hidden"]), np.float32) if want_hidden else None
+        if lens is not None:
+            _chk(lib().orc_gpt_step_padded(self.h, seqs, B, ln, _f(lens), int(use_cache), temperature, int(sampling),
+                                           _vp(probs), _vp(logits), _vp(hidden)))
+            return (probs, logits, hidden) if want_hidden else (probs, logits)
         _chk(lib().orc_gpt_step(self.h, seqs, B, ln, int(use_cache), temperature, int(sampling),
                                 _vp(probs), _vp(logits), _vp(hidden)))
         return (probs, logits, hidden) if want_hidden else (probs, logits)

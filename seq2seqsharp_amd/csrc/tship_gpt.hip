@@ -99,7 +99,7 @@ struct TSHipGpt {
     // decode state
     DevBuf x, xn, o, a, part_qkv, part_h, part_f, logits, ids, d_pos, hidden;
     DevBuf moe_ws, topp_scratch, topp_uni, gen_buf, uni_buf, tile_count;
-    DevBuf pw_ids, pw_x, pw_xn, pw_qkv, pw_o, pw_a, pw_f, pw_rowmap, pw_ssq, pw_rinv, pw_zero_bias, pw_moe;     // prefill workspace
+    DevBuf pw_lens, pw_ids, pw_x, pw_xn, pw_qkv, pw_o, pw_a, pw_f, pw_rowmap, pw_ssq, pw_rinv, pw_zero_bias, pw_moe;     // prefill workspace
     DevBuf ssq;                    // deferred-norm path: per-column-tile sums of squares [h/32][Bpad]
     bool fused_norm = false;       // fp16 + RMSNorm + dense layers: residual/norm folded into the GEMM tails
     bool vt = false;               // fp16 cache with head_dim 64/128: keys and values stored fragment-major for the MFMA attention kernels
@@ -454,7 +454,15 @@ static AttnKernel pick_attn_d(int D, int G, bool prefill) {
     }
 }
 template <int D>
-static AttnKernel pick_attn_mfma(int G, bool prefill, bool split) {
+static AttnKernel pick_attn_mfma(int G, bool prefill, bool split, bool ragged) {
+    if (prefill && ragged) {
+        switch (G) {
+            case 1: return attn_mfma_prefill_kernel<D, 1, true>;
+            case 2: return attn_mfma_prefill_kernel<D, 2, true>;
+            case 4: return attn_mfma_prefill_kernel<D, 4, true>;
+            default: throw Error("query heads per KV head must be 1, 2 or 4");
+        }
+    }
     switch (G) {
         case 1: return prefill ? attn_mfma_prefill_kernel<D, 1> : split ? attn_mfma_kernel<D, 1, true> : attn_mfma_kernel<D, 1, false>;
         case 2: return prefill ? attn_mfma_prefill_kernel<D, 2> : split ? attn_mfma_kernel<D, 2, true> : attn_mfma_kernel<D, 2, false>;
@@ -462,8 +470,8 @@ static AttnKernel pick_attn_mfma(int G, bool prefill, bool split) {
         default: throw Error("query heads per KV head must be 1, 2 or 4");
     }
 }
-static AttnKernel pick_attn(TSHipGpt* m, bool prefill, bool split = false) {
-    if (m->vt) return m->D == 64 ? pick_attn_mfma<64>(m->G, prefill, split) : pick_attn_mfma<128>(m->G, prefill, split);
+static AttnKernel pick_attn(TSHipGpt* m, bool prefill, bool split = false, bool ragged = false) {
+    if (m->vt) return m->D == 64 ? pick_attn_mfma<64>(m->G, prefill, split, ragged) : pick_attn_mfma<128>(m->G, prefill, split, ragged);
     return m->f16 ? pick_attn_d<half_t, half_t>(m->D, m->G, prefill) : pick_attn_d<float, float>(m->D, m->G, prefill);
 }
 template <typename CT>
@@ -732,7 +740,8 @@ static void decode_step(TSHipGpt* m, const int* d_ids, int B) {
 // ------------------------------------------------------------------------------------------------
 // prefill: whole prompts, causal attention, cache filled for every position, logits of the last position
 // ------------------------------------------------------------------------------------------------
-static void prefill(TSHipGpt* m, const int32_t* host_ids, int B, int Tp) {
+// host_lens (optional): the sequences were padded to Tp tokens; their original lengths select BuildSelfTriMask's masking
+static void prefill(TSHipGpt* m, const int32_t* host_ids, int B, int Tp, const int32_t* host_lens = nullptr) {
     auto& c = m->c;
     const int h = c.hidden, F = c.ffn_dim;
     const long R = (long)B * Tp, Rp = round_up(R, 128);
@@ -749,7 +758,12 @@ static void prefill(TSHipGpt* m, const int32_t* host_ids, int B, int Tp) {
     for (int b = 0; b < B; ++b) map[b] = Tp * (b + 1) - 1;
     rowmap.reserve(B * sizeof(int));
     TSHIP_CHECK_HIP(hipMemcpyAsync(rowmap.p, map.data(), B * sizeof(int), hipMemcpyHostToDevice, stream()));
-    TSHIP_CHECK_HIP(hipStreamSynchronize(stream()));       // (map is a local; the copy must not outlive it)
+    if (host_lens) {
+        TSHIP_REQUIRE(pos0 == 0, "TSHip_GptPrefillPadded: padded prompts start a sequence; call TSHip_GptReset first");
+        m->pw_lens.reserve(B * sizeof(int));
+        TSHIP_CHECK_HIP(hipMemcpyAsync(m->pw_lens.p, host_lens, B * sizeof(int), hipMemcpyHostToDevice, stream()));
+    }
+    TSHIP_CHECK_HIP(hipStreamSynchronize(stream()));       // (map is a local; the copies must not outlive their sources)
     px.reserve((size_t)Rp * h * sizeof(float));
     pxn.reserve((size_t)Rp * m->ldh * m->esz());
     pqkv.reserve((size_t)Rp * qp * sizeof(float));
@@ -798,6 +812,7 @@ static void prefill(TSHipGpt* m, const int32_t* host_ids, int B, int Tp) {
         AttnArgs aa = attn_args(m, L);
         aa.qkv = pqkv.as<float>(); aa.KS = 1; aa.split_stride = 0; aa.ldq = qp; aa.pos0 = pos0; aa.Tq = Tp;
         aa.out = po.p; aa.ld_out = m->ldh;
+        aa.lens = host_lens ? m->pw_lens.as<int>() : nullptr;
         if (m->f16) {
             BigArgs e; std::memset(&e, 0, sizeof(e));
             e.out = pqkv.as<float>(); e.ld_out = (int)qp; e.bias = L.bqkv.as<float>(); e.n_valid = m->Nqkv;
@@ -817,7 +832,7 @@ static void prefill(TSHipGpt* m, const int32_t* host_ids, int B, int Tp) {
         }
         if (m->vt) {      // a wavefront per 16 / G query positions, 8 (head_dim 64) or 4 (head_dim 128) wavefronts per block
             const int per_block = (16 / m->G) * (m->D == 128 ? 4 : 8);
-            launch(m, "p_attn", pick_attn(m, true), dim3((unsigned)ceil_div(Tp, per_block), c.n_kv_heads, B), dim3(m->D == 128 ? 256 : 512), aa);
+            launch(m, "p_attn", pick_attn(m, true, false, host_lens != nullptr), dim3((unsigned)ceil_div(Tp, per_block), c.n_kv_heads, B), dim3(m->D == 128 ? 256 : 512), aa);
         }
         else launch(m, "p_attn", pick_attn(m, true), dim3(Tp, c.n_kv_heads, B), dim3(256), aa);
         ResidNormArgs a2 = rn;
@@ -1104,6 +1119,18 @@ TSHIP_API int TSHip_GptPrefill(TSHipGpt* m, const int32_t* host_ids, int batch, 
     for (long i = 0; i < (long)batch * prompt_len; ++i)
         TSHIP_REQUIRE(host_ids[i] >= 0 && host_ids[i] < m->c.vocab, "TSHip_GptPrefill: token id out of range");
     prefill(m, host_ids, batch, prompt_len);
+    TSHIP_END
+}
+
+TSHIP_API int TSHip_GptPrefillPadded(TSHipGpt* m, const int32_t* host_ids, const int32_t* host_lens, int batch, int padded_len) {
+    TSHIP_BEGIN
+    TSHIP_REQUIRE(m && host_ids && host_lens, "TSHip_GptPrefillPadded: null argument");
+    TSHIP_REQUIRE(m->finalized, "TSHip_GptPrefillPadded: call TSHip_GptFinalize first");
+    TSHIP_REQUIRE(batch >= 1 && batch <= m->c.max_batch, "TSHip_GptPrefillPadded: batch out of range");
+    for (int b = 0; b < batch; ++b) TSHIP_REQUIRE(host_lens[b] >= 0 && host_lens[b] <= padded_len, "TSHip_GptPrefillPadded: a sequence length lies outside 0..padded_len");
+    for (long i = 0; i < (long)batch * padded_len; ++i)
+        TSHIP_REQUIRE(host_ids[i] >= 0 && host_ids[i] < m->c.vocab, "TSHip_GptPrefillPadded: token id out of range");
+    prefill(m, host_ids, batch, padded_len, host_lens);
     TSHIP_END
 }
 

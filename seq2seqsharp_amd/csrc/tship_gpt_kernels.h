@@ -1315,6 +1315,11 @@ struct AttnArgs {
     int vt;      // 1: keys and values are stored fragment-major (kfrag_index / vfrag_index) for the MFMA attention kernels
     // decode with several blocks per (row, KV head): their number, the exchange area [pairs][S][G D + 2 G] floats and one counter per pair
     int S; float* xchg; int* xcount;
+    // prefill of sequences padded to one length (Decoder.cs:656, 687-690): original lengths [batch], null = none were padded.
+    // Query row r of sequence b sees columns c <= r while r < lens[b] (BuildSelfTriMask, TensorApplyCPU.cs:1040-1065); a row
+    // from lens[b] on has every column masked, which after the softmax means: it attends to ALL columns of the padded
+    // sequence, with scores rounded to multiples of 2^-9 by the float32 addition of -30000.
+    const int* lens;
 };
 
 // rotary embedding of one (even, odd) pair, two roundings per output like the reference's C# expression
@@ -1333,7 +1338,7 @@ __device__ __forceinline__ void rope_pair(float x0, float x1, float c, float s, 
 // sQ: LDS [G][D] queries, already rotated and scaled.  Result (fp32) is written to sOut [G][D] in LDS.
 template <typename CT, int D, int G, int NW>
 __device__ __forceinline__ void attn_core(const float* sQ, const CT* Kb, const CT* Vb, int T, float* sM, float* sL, float* sAcc,
-                                          float* sOut) {
+                                          float* sOut, bool quant = false) {
     constexpr int EPL = 16 / (int)sizeof(CT);
     constexpr int LPR = D / EPL;
     constexpr int RPW = 64 / LPR;
@@ -1409,7 +1414,7 @@ __device__ __forceinline__ void attn_core(const float* sQ, const CT* Kb, const C
                 }
 #pragma unroll
                 for (int o = LPR / 2; o > 0; o >>= 1) d += __shfl_xor(d, o, 64);
-                s[g] = d;
+                s[g] = quant ? d + (-30000.0f) : d;      // (a fully masked row: the float32 addition of the mask value rounds the score)
             }
             if (ok) {
 #pragma unroll
@@ -1638,7 +1643,8 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(AttnArgs a) {
     __syncthreads();
     const CT* Kb = (const CT*)a.kcache + ((long)b * a.Hkv + kvh) * a.max_len * D;
     const CT* Vb = (const CT*)a.vcache + ((long)b * a.Hkv + kvh) * a.max_len * D;
-    attn_core<CT, D, G, 4>(sm.q, Kb, Vb, pos + 1, sm.m, sm.l, sm.acc, sm.out);
+    const bool all_masked = a.lens && tq >= a.lens[b];          // (padded prompts start an empty cache: pos0 = 0)
+    attn_core<CT, D, G, 4>(sm.q, Kb, Vb, all_masked ? a.pos0 + a.Tq : pos + 1, sm.m, sm.l, sm.acc, sm.out, all_masked);
     AT* out = (AT*)a.out + row * a.ld_out + kvh * G * D;
     for (int idx = t; idx < G * D; idx += 256) out[idx] = (AT)sm.out[idx];
 }
@@ -1961,7 +1967,10 @@ __global__ __launch_bounds__(D == 128 ? 256 : 512) void attn_mfma_kernel(AttnArg
 // straight into LDS (two stages; wavefront w brings fragments w, w + NW, ...), and all wavefronts read their MFMA
 // operands from there.  (With every wavefront streaming its own prefix the kernel was bound by L2: the L1 holds two
 // chunks and the wavefronts drift apart.)  grid (ceil(Tq / (QB NW)), Hkv, batch).
-template <int D, int G>
+// RAGGED: sequences padded to one length (a.lens).  A query row at or beyond its sequence's length attends to every
+// column of the padded sequence with scores rounded as the float32 addition of -30000 rounds them; every chunk then
+// takes the masked path and a block that holds such a row walks all chunks.
+template <int D, int G, bool RAGGED = false>
 __global__ __launch_bounds__(D == 128 ? 256 : 512) void attn_mfma_prefill_kernel(AttnArgs a) {
     constexpr int NW = D == 128 ? 4 : 8;
     constexpr int QB = 16 / G, KD = D / 32, DT = D / 16;
@@ -1979,7 +1988,9 @@ __global__ __launch_bounds__(D == 128 ? 256 : 512) void attn_mfma_prefill_kernel
     const int pos_base = a.pos0 + tq0, T = min(pos_base + QB, a.pos0 + a.Tq);
     // chunks of the block: up to the last position of its last active wavefront
     const int tq_last = min(a.Tq, (int)(blockIdx.x + 1) * NW * QB);
-    const int nchunks = (a.pos0 + tq_last + 31) / 32;
+    const int len_b = RAGGED ? a.lens[b] : 0x7fffffff;
+    const int Ttot = a.pos0 + a.Tq;
+    const int nchunks = (RAGGED && tq_last > len_b) ? (Ttot + 31) / 32 : (a.pos0 + tq_last + 31) / 32;
     const half_t* Kb = (const half_t*)a.kcache + ((long)b * a.Hkv + kvh) * a.max_len * D;
     const half_t* Vt = (const half_t*)a.vcache + ((long)b * a.Hkv + kvh) * (long)D * a.max_len;
     typedef const void __attribute__((address_space(1)))* gptr_t;
@@ -2017,7 +2028,8 @@ __global__ __launch_bounds__(D == 128 ? 256 : 512) void attn_mfma_prefill_kernel
     for (int kd = 0; kd < KD; ++kd)
 #pragma unroll
         for (int j = 0; j < 8; ++j) qf[kd][j] = (half_t)sq[r16 * D + kd * 32 + 8 * q + j];
-    const int tmax = pos_base + r16 / G;      // last position this lane's column may attend to
+    const bool fully = RAGGED && tq0 + r16 / G >= len_b;                    // this lane's query row has every column masked
+    const int tmax = fully ? Ttot - 1 : pos_base + r16 / G;                 // last position this lane's column may attend to
 
     float m_run = -INFINITY, l_run = 0.0f;
     floatx4 acc_o[DT];
@@ -2039,6 +2051,10 @@ __global__ __launch_bounds__(D == 128 ? 256 : 512) void attn_mfma_prefill_kernel
         float cm = -INFINITY;
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
+            if (RAGGED && fully) {      // scores are in units of log 2 here: round in natural units as s + (-30000) does, and back
+                const float sn = s[j] * 0.69314718f + (-30000.0f);
+                s[j] = (sn - (-30000.0f)) * 1.44269504f;
+            }
             if (MASKED && t0 + 8 * q + j > tmax) s[j] = -INFINITY;       // causal mask (adding -30000 gives exactly 0 after exp in fp32 too)
             cm = fmaxf(cm, s[j]);
         }
@@ -2067,8 +2083,9 @@ __global__ __launch_bounds__(D == 128 ? 256 : 512) void attn_mfma_prefill_kernel
     // Chunks [0, n_full) lie entirely at or below this wavefront's first query position; chunks from n_own on lie
     // entirely behind its last one (the block's later wavefronts still need them).
     const std::integral_constant<bool, false> plain; const std::integral_constant<bool, true> masked;
-    const int n_own = active ? (T + 31) / 32 : 0;
-    const int n_full = min(n_own, (pos_base + 1) / 32);
+    const bool wave_fully = RAGGED && active && min(tq0 + QB, a.Tq) > len_b;      // its last query row lies beyond the sequence's length
+    const int n_own = active ? (wave_fully ? (Ttot + 31) / 32 : (T + 31) / 32) : 0;
+    const int n_full = RAGGED ? 0 : min(n_own, (pos_base + 1) / 32);
     // One loop per kind of chunk (unmasked, masked, not this wavefront's): with the kinds as branches of one loop the
     // compiler copies the running outputs between registers around every branch, a third of the loop's instructions.
     // Every wavefront passes the same nchunks barriers whatever its split.

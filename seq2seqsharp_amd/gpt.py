@@ -29,6 +29,7 @@ def _protos():
     L.TSHip_GptFinalize.argtypes = [vp]
     L.TSHip_GptReset.argtypes = [vp]
     L.TSHip_GptPrefill.argtypes = [vp, vp, C.c_int, C.c_int]
+    L.TSHip_GptPrefillPadded.argtypes = [vp, vp, vp, C.c_int, C.c_int]
     L.TSHip_GptDecode.argtypes = [vp, vp, C.c_int]
     L.TSHip_GptSample.argtypes = [vp, C.c_int, C.c_float, C.c_float, vp, vp]
     L.TSHip_GptSetRepeatPenalty.argtypes = [vp, C.c_float]
@@ -95,11 +96,28 @@ class HipGpt:
         check(lib().TSHip_GptReset(self.h))
         self.batch = 0
 
-    def prefill(self, ids):
+    def prefill(self, ids, lens=None):
+        """ids [batch, len]; lens: original lengths of sequences that were padded to `len` with the END tag
+        (BuildInTokens.PadSentences): the reference's masking for padded batches then applies."""
         ids = np.ascontiguousarray(ids, dtype=np.int32)
         B, T = ids.shape
-        check(lib().TSHip_GptPrefill(self.h, _ptr(ids), B, T))
+        if lens is None:
+            check(lib().TSHip_GptPrefill(self.h, _ptr(ids), B, T))
+        else:
+            lens = np.ascontiguousarray(lens, dtype=np.int32).reshape(-1)
+            assert lens.size == B
+            check(lib().TSHip_GptPrefillPadded(self.h, _ptr(ids), _ptr(lens), B, T))
         self.batch = B
+
+    @staticmethod
+    def pad_sentences(seqs, pad_id=0):
+        """BuildInTokens.PadSentences (Corpus/BuildInTokens.cs:68-101): lists of token ids -> (ids [batch, longest] padded
+        with `pad_id`, the END tag in the reference; original lengths)."""
+        lens = np.array([len(s) for s in seqs], np.int32)
+        out = np.full((len(seqs), int(lens.max())), pad_id, np.int32)
+        for i, s in enumerate(seqs):
+            out[i, :len(s)] = s
+        return out, lens
 
     def decode(self, ids):
         ids = np.ascontiguousarray(ids, dtype=np.int32).reshape(-1)

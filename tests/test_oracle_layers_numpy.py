@@ -38,7 +38,7 @@ def rope64(cfg, v, pos):
     return out
 
 
-def attention64(cfg, w, layer, x, B, Tq, past=None, causal=True, mut=None):
+def attention64(cfg, w, layer, x, B, Tq, past=None, causal=True, mut=None, lens=None):
     """x [B*Tq, h] -> (x + attention output, (keys, values)) with keys/values [B, Hkv, T, d] after RoPE.
     past: (keys, values) of earlier positions.  The new rows sit at positions len(past) .. len(past) + Tq - 1.
     mut: a deliberate mistake (tests use it to show that the tolerance would catch that mistake)."""
@@ -73,7 +73,18 @@ def attention64(cfg, w, layer, x, B, Tq, past=None, causal=True, mut=None):
             kv = hh % Hkv if mut == "headmap" else hh // (H // Hkv)
             for t in range(Tq):
                 s = keys[b, kv] @ q[b, t, hh] / (F64(d) if mut == "scale" else np.sqrt(F64(d)))         # [T]
-                if causal and past is None:
+                if causal and past is None and lens is not None:
+                    # BuildSelfTriMask (TensorApplyCPU.cs:1040-1065): visible iff column and row lie inside the sequence's
+                    # original length and column <= row.  The addition happens in float32, where -30000 swallows the low
+                    # bits of the score: a row beyond the length (everything masked) attends to ALL columns with scores
+                    # rounded to multiples of 2^-9.
+                    c = np.arange(T)
+                    vis = (c < lens[b]) & (t < lens[b]) & (c <= t)
+                    if mut == "pad_causal":
+                        vis = c <= t
+                    m32 = np.where(vis, np.float32(0.0), np.float32(-30000.0)).astype(np.float32)
+                    s = (s.astype(np.float32) + m32).astype(np.float32).astype(F64)
+                elif causal and past is None:
                     s = s + np.where(np.arange(T) <= t, 0.0, -30000.0)   # additive mask, only built without a cache
                 p = np.exp(s - s.max())
                 p = p / p.sum()
@@ -100,7 +111,7 @@ def ffn64(cfg, w, layer, x):
     return x + y
 
 
-def gpt64(cfg, w, seqs, past=None):
+def gpt64(cfg, w, seqs, past=None, lens=None, mut=None):
     """Whole sequences (no cache) or the last token on top of `past` (one (keys, values) pair per layer).
     Returns (logits [B, V], final-norm hidden [B, h], new past)."""
     B, ln = seqs.shape
@@ -110,7 +121,7 @@ def gpt64(cfg, w, seqs, past=None):
     x = w["TgtEmbeddings"].astype(F64)[ids.reshape(-1)] * F64(np.float32(np.sqrt(np.float32(h))))
     new = []
     for layer in range(cfg["n_layers"]):
-        x, kv = attention64(cfg, w, layer, x, B, Tq, None if past is None else past[layer])
+        x, kv = attention64(cfg, w, layer, x, B, Tq, None if past is None else past[layer], lens=lens, mut=mut)
         new.append(kv)
         x = ffn64(cfg, w, layer, x)
     hid = norm64(cfg, w, "GPTDecoder.layerNorm", x).reshape(B, Tq, h)[:, -1]
@@ -209,3 +220,35 @@ def test_temperature_divides_logits_only_when_sampling(oracle):
     assert np.abs(lg - lg64 / 0.5).max() <= 2e-5
     _, lg = m.step(seqs, use_cache=False, temperature=0.5, sampling=False)
     assert np.abs(lg - lg64).max() <= 1e-5
+
+
+@pytest.mark.parametrize("name", ["gqa_rms", "mha_ln"])
+def test_padded_batch_takes_the_self_tri_mask(oracle, name):
+    """Sequences of different lengths (Decoder.cs:656, 687-690): padded with the END tag to the longest, masked per row by
+    BuildSelfTriMask, logits read at the last padded position of every row, then decoding goes on from the padded
+    sequences without a mask.  The restatement forms the mask from its definition and adds it in float32."""
+    cfg = synth.tiny_config(n_layers=2, batch=4, **ATTN_CASES[name])
+    w = _sharpen(synth.make_weights(cfg, 31, random_bias=True))
+    lens = np.array([5, 8, 1, 8], np.float32)
+    T = 8
+    seqs = synth.make_prompts(cfg, 32, batch=4, length=T)
+    for b in range(4):
+        seqs[b, int(lens[b]):] = 0                          # the END tag's id (Utils/Vocab.cs:23-30)
+    m = oracle.OracleGpt(cfg, w)
+    p, lg, hid = m.step(seqs, use_cache=True, want_hidden=True, lens=lens)
+    lg64, hid64, past = gpt64(cfg, w, seqs, lens=lens)
+    assert np.abs(hid - hid64).max() <= 5e-5 and np.abs(lg - lg64).max() <= 5e-5
+    # rows as long as the batch's longest see the plain causal mask; shorter rows do not
+    lg_plain, _, _ = gpt64(cfg, w, seqs)
+    assert np.abs(lg_plain[[1, 3]] - lg64[[1, 3]]).max() <= 1e-6       # (the float32 addition rounds the visible scores too)
+    assert np.abs(lg_plain[[0, 2]] - lg64[[0, 2]]).max() > 1e-3
+    bad, _, _ = gpt64(cfg, w, seqs, lens=lens, mut="pad_causal")
+    assert np.abs(bad - lg64).max() > 1e-3
+    # the loop continues on the padded sequences (no mask with a cache: the padding stays visible)
+    cur = seqs
+    for _ in range(2):
+        nxt = oracle.argmax(p).astype(np.int32)
+        cur = np.concatenate([cur, nxt[:, None]], 1)
+        p, lg = m.step(cur, use_cache=True)
+        lg64, _, past = gpt64(cfg, w, cur, past)
+        assert np.abs(lg - lg64).max() <= 5e-5
