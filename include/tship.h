@@ -194,6 +194,22 @@ TSHIP_API int TSHip_GptGenerate(TSHipGpt* m, int n_steps, int mode, float top_p,
  * tokens, which costs one small copy and one synchronisation per step. */
 TSHIP_API int TSHip_GptGenerateUntil(TSHipGpt* m, int max_steps, int eos_id, int mode, float top_p, float temperature,
                                      const float* host_uniforms, int32_t* host_ids_out, int* steps_done, float* elapsed_ms);
+/* ---- beam search (Decoder.cs:756-792, GPT.cs:264-297, Utils/BeamSearch.cs:36-46).  Hypotheses are rows of the cached batch. ----
+ * TSHip_GptBeamPick: from the logits on the device, n_picks picks per row as the reference makes them: probabilities =
+ * softmax (after the division by the temperature when sampling), pick = Argmax (greedy) or TopPSample (with the repeat
+ * penalty and the blocked tokens set on the model; host_uniforms [n_picks, batch]), ScatterFill(probs, 0) at the picked
+ * index before the next pick.  host_ids_out [n_picks, batch]; host_logp_out [n_picks, batch] = log of the picked
+ * probability (the reference adds its negative to the hypothesis' score).  Nothing is appended to the sequences. */
+TSHIP_API int TSHip_GptBeamPick(TSHipGpt* m, int n_picks, int mode, float top_p, float temperature, const float* host_uniforms,
+                                int32_t* host_ids_out, float* host_logp_out);
+/* Gather the cached sequences: row i of the new batch continues old row host_src_rows[i] (rows may repeat: a hypothesis
+ * with several surviving children; new_batch may differ from the old batch, at most max_batch).  KV cache and token
+ * history move; the logits on the device are stale until the next TSHip_GptDecode. */
+TSHIP_API int TSHip_GptReorderRows(TSHipGpt* m, const int32_t* host_src_rows, int new_batch);
+/* BeamSearch.GetTopNBSS: indices of the top_n lowest scores among scores[0..n), in the order the reference's
+ * FixedSizePriorityQueue enumerates them (AdvUtils/FixedSizePriorityQueue.cs; not sorted).  kept: top_n entries. */
+TSHIP_API int TSHip_BeamTopN(const float* scores, int n, int top_n, int32_t* kept, int* n_kept);
+
 /* inspection for parity tests */
 TSHIP_API int TSHip_GptGetLogits(TSHipGpt* m, float* host_out /* [batch, vocab] */);
 TSHIP_API int TSHip_GptGetHidden(TSHipGpt* m, float* host_out /* [batch, hidden], after the final norm */);

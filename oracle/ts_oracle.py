@@ -364,3 +364,175 @@ class OracleGpt:
         y = np.empty_like(x)
         _chk(lib().orc_ffn_layer(self.h, layer, x, x.shape[0], y))
         return y
+
+
+# ---- beam search (pure Python: small cases only) ------------------------------------------------
+class FixedSizePriorityQueue:
+    """AdvUtils/FixedSizePriorityQueue.cs:10-341 with ComparableItemComparer(false) (Seq2SeqSharp/Tools/ComparableItem.cs:31-50),
+    as BeamSearch.GetTopNBSS uses it (Utils/BeamSearch.cs:36-46).  Items are (score, payload); lower scores are better.
+    Two array heaps: `top` (better half, best at the root) and `bottom` (worst at the root); enumeration = top in array
+    order, then bottom in reverse array order."""
+
+    def __init__(self, capacity):
+        assert capacity >= 1
+        self.cap, self.count, self.nb, self.nt = capacity, 0, 0, 0
+        bcap = max(capacity // 2, 1)
+        self.top = [None] * max(capacity - bcap, 1)
+        self.bottom = [None] * bcap
+
+    @staticmethod
+    def _better(a, b, f_top):
+        d = np.float32(a[0]) - np.float32(b[0])
+        c = -(1 if d > 0 else (-1 if d < 0 else 0))         # Compare(x, y) = -Math.Sign(x.Score - y.Score)
+        return c > 0 if f_top else c < 0
+
+    def _up(self, arr, i, f_top):                           # UpHeapify :198-208
+        while i > 0:
+            p = (i - 1) // 2
+            if not self._better(arr[i], arr[p], f_top):
+                return i
+            arr[i], arr[p] = arr[p], arr[i]
+            i = p
+        return i
+
+    def _down(self, arr, i, size, f_top):                   # DownHeapify :210-224
+        while True:
+            l, r, best = 2 * i + 1, 2 * i + 2, i
+            if l < size and self._better(arr[l], arr[best], f_top):
+                best = l
+            if r < size and self._better(arr[r], arr[best], f_top):
+                best = r
+            if best == i:
+                return i
+            arr[i], arr[best] = arr[best], arr[i]
+            i = best
+
+    def _top1(self, i):                                     # TopNode1 :176-182
+        return 2 * i + 1 if self.nb <= 2 * i + 1 < self.nt else i
+
+    def _top2(self, i):                                     # TopNode2 :184-195
+        if i == self.nb - 1 and i % 2 == 1 and self.nt > self.nb:
+            return i + 1
+        return 2 * i + 1 if self.nb <= 2 * i + 1 < self.nt else i
+
+    def _boundary_up(self, bpos):                           # CheckBoundaryUpwards :226-249
+        t1, t2, b = self._top1(bpos), self._top2(bpos), -1
+        if self._better(self.bottom[bpos], self.top[t1], True):
+            b = t1
+        if self._better(self.bottom[bpos], self.top[t2], True) and (b == -1 or self._better(self.top[t1], self.top[t2], True)):
+            b = t2
+        if b == -1:
+            return -1
+        self.top[b], self.bottom[bpos] = self.bottom[bpos], self.top[b]
+        return b
+
+    def _boundary_down(self, tpos):                         # CheckBoundaryDownwards :251-268, BottomNode :163-174
+        if tpos < self.nb:
+            bpos = tpos
+        else:
+            bpos = (tpos - 1) // 2 if tpos % 2 == 1 else tpos - 1
+        if bpos == -1:
+            return -1
+        if bpos >= self.nb or not self._better(self.bottom[bpos], self.top[tpos], True):
+            return -1
+        self.top[tpos], self.bottom[bpos] = self.bottom[bpos], self.top[tpos]
+        return bpos
+
+    def enqueue(self, item):                                # Enqueue :56-149
+        if self.cap == self.count:
+            if self.cap == 1:
+                if not self._better(item, self.top[0], True):
+                    return False
+                self.top[0] = item
+                return True
+            if not self._better(item, self.bottom[0], True):
+                return False
+            self.bottom[0] = item
+            upd = self._down(self.bottom, 0, self.nb, False)
+            if not (2 * upd + 2 >= self.nb):                # SemiLeaf
+                return True
+            it = self._boundary_up(upd)
+            if it == -1:
+                return True
+            self._up(self.top, it, True)
+            return True
+        self.count += 1
+        if self.nb < self.nt:
+            pos = self.nb
+            self.nb += 1
+            self.bottom[pos] = item
+            up = self._boundary_up(pos)
+            if up == -1:
+                self._up(self.bottom, pos, False)
+            else:
+                self._up(self.top, up, True)
+            return True
+        pos = self.nt
+        self.nt += 1
+        self.top[pos] = item
+        bt = self._boundary_down(pos)
+        if bt == -1:
+            self._up(self.top, pos, True)
+        else:
+            self._up(self.bottom, bt, False)
+        return True
+
+    def items(self):                                        # GetEnumerator :306-312
+        return [self.top[i] for i in range(self.nt)] + [self.bottom[i] for i in range(self.nb - 1, -1, -1)]
+
+
+def get_top_n(scores, top_n):
+    """BeamSearch.GetTopNBSS on a list of scores: indices of the survivors in the queue's enumeration order."""
+    q = FixedSizePriorityQueue(top_n)
+    for i, s in enumerate(scores):
+        q.enqueue((np.float32(s), i))
+    return [it[1] for it in q.items()]
+
+
+def beam_picks(probs, n_picks, top_p=None, repeat_penalty=0.0, seqs=None, uniforms=None):
+    """The pick loop of Decoder.GPTDecode (Applications/Decoder.cs:756-792): Argmax (top_p None) or TopPSample, Gather + Log of
+    the picked probability, ScatterFill(probs, 0) at the pick before the next one.  probs [B, V] (blocked tokens already
+    lowered by 1).  Returns (ids [n_picks, B], log p [n_picks, B])."""
+    p = _f(probs).copy()
+    B = p.shape[0]
+    ids = np.zeros((n_picks, B), np.int32)
+    logp = np.zeros((n_picks, B), np.float32)
+    for i in range(n_picks):
+        if top_p is None:
+            pick = argmax(p).astype(np.int32)
+        else:
+            pick = toppsample(p, top_p, repeat_penalty, seqs, uniforms[i]).astype(np.int32)
+        ids[i] = pick
+        with np.errstate(divide="ignore"):
+            logp[i] = np.log(p[np.arange(B), pick].astype(np.float64)).astype(np.float32)      # (float)Math.Log
+        p[np.arange(B), pick] = 0.0
+    return ids, logp
+
+
+def gpt_beam_search(orc, prompts, beam_size, max_len, eos_id=0, top_p=None, repeat_penalty=0.0, uniforms=None, temperature=1.0):
+    """GPT.RunForwardOnSingleDevice for BeamSearchSize > 1 (Applications/GPT.cs:264-302) on an OracleGpt: no KV cache (the
+    dictionary only exists for beam size 1, :238-241), every beam's batch recomputed from its first token each step.
+    uniforms [steps, beam_size picks, beams * batch] (beam-major rows).  Returns (hypotheses [batch][beam], scores)."""
+    prompts = np.ascontiguousarray(prompts, dtype=np.int32)
+    B, T0 = prompts.shape
+    beams = [[(list(map(int, prompts[b])), np.float32(1.0)) for b in range(B)]]       # beam2batchStatus; Score starts at 1.0f
+    step = 0
+    for _ in range(T0, max_len):
+        per_batch = [[] for _ in range(B)]
+        for j, batch_status in enumerate(beams):
+            seqs = np.array([h[0] for h in batch_status], np.int32)
+            p, _ = orc.step(seqs, use_cache=False, temperature=temperature, sampling=top_p is not None)
+            u = None if uniforms is None else [uniforms[step][i][j * B:(j + 1) * B] for i in range(beam_size)]
+            ids, logp = beam_picks(p, beam_size, top_p, repeat_penalty, seqs if top_p is not None else None, u)
+            for b in range(B):
+                for i in range(beam_size):
+                    per_batch[b].append((batch_status[b][0] + [int(ids[i, b])], np.float32(batch_status[b][1] + np.float32(-1.0) * logp[i, b])))
+        if beam_size > 1:
+            per_batch = [[c[k] for k in get_top_n([h[1] for h in c], beam_size)] for c in per_batch]
+        beams = [[per_batch[b][j] for b in range(B)] for j in range(len(per_batch[0]))]
+        step += 1
+        if all(h[0][-1] == eos_id for bs in beams for h in bs):
+            break
+    hyp = [[beams[j][b][0] for j in range(len(beams))] for b in range(B)]
+    sc = [[float(beams[j][b][1]) for j in range(len(beams))] for b in range(B)]
+    return hyp, sc

@@ -116,6 +116,7 @@ struct TSHipGpt {
     bool any_blocked = false;
     DevBuf blocked;                // one byte per token, non-zero = DecodingOptions.BlockedTokens (allocated with the model: graphs keep its address)
     int cur_batch = 0;
+    DevBuf beam_probs, beam_ids, beam_out, beam_uni, reorder_tmp, reorder_src;      // beam search: probabilities the picks consume, picks, gather temporaries
     Profiler* prof = nullptr;
 
     size_t esz() const { return f16 ? 2 : 4; }
@@ -910,6 +911,7 @@ static void prefill(TSHipGpt* m, const int32_t* host_ids, int B, int Tp, const i
 }  // namespace tship
 
 #include "tship_gpt_extra.h"
+#include "tship_beam.h"
 
 // =================================================================================================
 // exported functions
@@ -1258,6 +1260,100 @@ TSHIP_API int TSHip_GptGenerateUntil(TSHipGpt* m, int max_steps, int eos_id, int
     if (m && (eos_id < 0 || eos_id >= m->c.vocab)) { set_last_error("TSHip_GptGenerateUntil: eos_id out of range"); return 0; }
     if (!steps_done) { set_last_error("TSHip_GptGenerateUntil: null argument"); return 0; }
     return generate_impl(m, max_steps, mode, top_p, temperature, host_uniforms, host_ids_out, elapsed_ms, eos_id, steps_done);
+}
+
+TSHIP_API int TSHip_GptBeamPick(TSHipGpt* m, int n_picks, int mode, float top_p, float temperature, const float* host_uniforms,
+                                int32_t* host_ids_out, float* host_logp_out) {
+    TSHIP_BEGIN
+    TSHIP_REQUIRE(m && host_ids_out && host_logp_out, "TSHip_GptBeamPick: null argument");
+    TSHIP_REQUIRE(m->cur_batch > 0, "TSHip_GptBeamPick: no logits yet; prefill or decode first");
+    TSHIP_REQUIRE(n_picks >= 1 && n_picks <= m->c.vocab, "TSHip_GptBeamPick: n_picks must lie in 1..vocab");
+    TSHIP_REQUIRE(mode == TSHIP_GREEDY || (mode == TSHIP_TOPP && host_uniforms), "TSHip_GptBeamPick: top-p needs one uniform draw per row and pick");
+    TSHIP_REQUIRE(mode == TSHIP_GREEDY || m->c.vocab <= 65535, "top-p sampling supports vocabularies up to 65535");
+    TSHIP_REQUIRE(temperature > 0.0f, "temperature must be positive");
+    const int B = m->cur_batch, V = m->c.vocab;
+    const long Vp = round_up(V, 32);
+    m->beam_probs.reserve((size_t)m->Bpad * Vp * sizeof(float));
+    m->beam_ids.reserve((size_t)m->Bpad * sizeof(int));
+    m->beam_out.reserve((size_t)n_picks * B * (sizeof(int) + sizeof(float)));
+    int* d_ids_out = m->beam_out.as<int>(); float* d_logp = (float*)(d_ids_out + (size_t)n_picks * B);
+    float* probs = m->beam_probs.as<float>();
+    // Decoder.cs:720-723: the logits are divided by the temperature only when sampling
+    launch(m, "beam_probs", beam_probs_kernel, dim3(B), dim3(1024), (const float*)m->logits.as<float>(), Vp, V, temperature,
+           (int)(mode == TSHIP_TOPP && temperature != 1.0f), probs, Vp);
+    const unsigned char* blocked = m->any_blocked ? (const unsigned char*)m->blocked.p : nullptr;
+    if (mode == TSHIP_TOPP) {
+        m->beam_uni.reserve((size_t)n_picks * B * sizeof(float));
+        TSHIP_CHECK_HIP(hipMemcpyAsync(m->beam_uni.p, host_uniforms, (size_t)n_picks * B * sizeof(float), hipMemcpyHostToDevice, stream()));
+        const size_t need = topp_scratch_bytes(m->Bpad, V);
+        if (m->topp_scratch.bytes < need) m->topp_scratch.alloc(need);
+    }
+    for (int i = 0; i < n_picks; ++i) {
+        if (mode == TSHIP_GREEDY) {
+            // Argmax over the probabilities, first maximum (TensorApplyCPU.cs:339-360); nothing is recorded: the caller decides
+            // which picks survive
+            launch(m, "beam_argmax", greedy_kernel, dim3(B), dim3(1024), (const float*)probs, Vp, V, m->beam_ids.as<int>(), (int*)nullptr, (const int*)nullptr,
+                   (int*)nullptr, 0L, (const int*)nullptr, blocked);
+        } else {
+            TopPArgs a; std::memset(&a, 0, sizeof(a));
+            a.in = probs; a.ld = Vp; a.V = V; a.in_is_logits = 0; a.temperature = 1.0f;
+            a.uniforms = m->beam_uni.as<float>() + (size_t)i * B; a.top_p = top_p;
+            topp_carve(a, m->topp_scratch.p, m->Bpad, V);
+            a.next_ids = m->beam_ids.as<int>();
+            a.blocked = blocked;
+            a.repeat_penalty = m->repeat_penalty; a.last_pos = m->last_pos.as<int>(); a.last_ld = m->last_ld; a.d_len = m->d_pos.as<int>(); a.record = 0;
+            topp_run(a, B, [&](const char* name, void (*kernel)(TopPArgs), dim3 grid, dim3 block, const TopPArgs& args) { launch(m, name, kernel, grid, block, args); });
+        }
+        launch(m, "beam_take", beam_take_kernel, dim3((unsigned)ceil_div(B, 64)), dim3(64), probs, Vp, (const int*)m->beam_ids.as<int>(), B,
+               d_ids_out + (size_t)i * B, d_logp + (size_t)i * B);
+    }
+    TSHIP_CHECK_HIP(hipMemcpyAsync(host_ids_out, d_ids_out, (size_t)n_picks * B * sizeof(int), hipMemcpyDeviceToHost, stream()));
+    TSHIP_CHECK_HIP(hipMemcpyAsync(host_logp_out, d_logp, (size_t)n_picks * B * sizeof(float), hipMemcpyDeviceToHost, stream()));
+    TSHIP_CHECK_HIP(hipStreamSynchronize(stream()));
+    TSHIP_END
+}
+
+TSHIP_API int TSHip_GptReorderRows(TSHipGpt* m, const int32_t* host_src_rows, int new_batch) {
+    TSHIP_BEGIN
+    TSHIP_REQUIRE(m && host_src_rows, "TSHip_GptReorderRows: null argument");
+    TSHIP_REQUIRE(m->cur_batch > 0, "TSHip_GptReorderRows: no cached sequences");
+    TSHIP_REQUIRE(new_batch >= 1 && new_batch <= m->c.max_batch, "TSHip_GptReorderRows: new batch out of range (max_batch)");
+    bool identity = new_batch == m->cur_batch;
+    for (int i = 0; i < new_batch; ++i) {
+        TSHIP_REQUIRE(host_src_rows[i] >= 0 && host_src_rows[i] < m->cur_batch, "TSHip_GptReorderRows: source row out of range");
+        identity = identity && host_src_rows[i] == i;
+    }
+    if (!identity) {
+        m->reorder_src.reserve((size_t)m->c.max_batch * sizeof(int));
+        TSHIP_CHECK_HIP(hipMemcpyAsync(m->reorder_src.p, host_src_rows, (size_t)new_batch * sizeof(int), hipMemcpyHostToDevice, stream()));
+        TSHIP_CHECK_HIP(hipStreamSynchronize(stream()));       // (the caller's array may go away)
+        // cache rows: [batch][kv head][ML * D] elements; the first round_up(pos, 32) positions of every head are live
+        // (fragment-major caches keep positions in chunks of 32)
+        const long head_bytes = (long)m->ML * m->D * (long)m->esz(), row_bytes = head_bytes * m->c.n_kv_heads;
+        const long used = std::min<long>(head_bytes, round_up(std::max(m->pos, 1), 32) * (long)m->D * (long)m->esz());
+        m->reorder_tmp.reserve((size_t)std::max<long>(row_bytes, m->last_pos.p ? m->last_ld * (long)sizeof(int) : 0) * m->c.max_batch);
+        const int* src = m->reorder_src.as<int>();
+        auto gather = [&](void* table, long stride, long chunk, long live, long pieces) {
+            launch(m, "rows_gather", rows_gather_kernel, dim3((unsigned)pieces, (unsigned)new_batch), dim3(256), (const char*)table, stride, chunk, live, src, m->reorder_tmp.as<char>(), 1);
+            launch(m, "rows_gather", rows_gather_kernel, dim3((unsigned)pieces, (unsigned)new_batch), dim3(256), (const char*)table, stride, chunk, live, src, m->reorder_tmp.as<char>(), 0);
+        };
+        for (auto& L : m->L) { gather(L->kc.p, row_bytes, head_bytes, used, m->c.n_kv_heads); gather(L->vc.p, row_bytes, head_bytes, used, m->c.n_kv_heads); }
+        if (m->last_pos.p) gather(m->last_pos.p, m->last_ld * (long)sizeof(int), m->last_ld * (long)sizeof(int), m->last_ld * (long)sizeof(int), 1);
+        TSHIP_CHECK_HIP(hipStreamSynchronize(stream()));
+    }
+    m->cur_batch = new_batch;
+    TSHIP_END
+}
+
+TSHIP_API int TSHip_BeamTopN(const float* scores, int n, int top_n, int32_t* kept, int* n_kept) {
+    TSHIP_BEGIN
+    TSHIP_REQUIRE(scores && kept && n_kept && n >= 0 && top_n >= 1, "TSHip_BeamTopN: bad argument");
+    TopNQueue q(top_n);
+    for (int i = 0; i < n; ++i) q.enqueue(TopNQueue::Item{scores[i], i});
+    const auto items = q.enumerate();
+    for (size_t i = 0; i < items.size(); ++i) kept[i] = items[i].index;
+    *n_kept = (int)items.size();
+    TSHIP_END
 }
 
 TSHIP_API int TSHip_GptGetLogits(TSHipGpt* m, float* host_out) {

@@ -36,6 +36,9 @@ def _protos():
     L.TSHip_GptSetBlockedTokens.argtypes = [vp, vp, C.c_int]
     L.TSHip_GptGenerateUntil.argtypes = [vp, C.c_int, C.c_int, C.c_int, C.c_float, C.c_float, vp, vp, C.POINTER(C.c_int), C.POINTER(C.c_float)]
     L.TSHip_GptGenerate.argtypes = [vp, C.c_int, C.c_int, C.c_float, C.c_float, vp, vp, C.POINTER(C.c_float)]
+    L.TSHip_GptBeamPick.argtypes = [vp, C.c_int, C.c_int, C.c_float, C.c_float, vp, vp, vp]
+    L.TSHip_GptReorderRows.argtypes = [vp, vp, C.c_int]
+    L.TSHip_BeamTopN.argtypes = [vp, C.c_int, C.c_int, vp, C.POINTER(C.c_int)]
     L.TSHip_GptGetLogits.argtypes = [vp, vp]
     L.TSHip_GptGetHidden.argtypes = [vp, vp]
     L.TSHip_GptGetSeqLen.argtypes = [vp, C.POINTER(C.c_int)]
@@ -156,6 +159,76 @@ class HipGpt:
         done = C.c_int(0)
         check(lib().TSHip_GptGenerateUntil(self.h, max_steps, eos_id, mode, top_p, temperature, _ptr(u), _ptr(out), C.byref(done), C.byref(ms)))
         return out[:done.value], ms.value
+
+    def beam_pick(self, n_picks, mode=GREEDY, top_p=0.0, temperature=1.0, uniforms=None):
+        """n_picks picks per cached row from the current logits, the reference's way (pick, zero the picked probability,
+        pick again: Decoder.cs:756-792).  Returns (ids [n_picks, batch], log of the picked probabilities [n_picks, batch])."""
+        ids = np.empty((n_picks, self.batch), np.int32)
+        logp = np.empty((n_picks, self.batch), np.float32)
+        u = None if uniforms is None else np.ascontiguousarray(uniforms, dtype=np.float32)
+        check(lib().TSHip_GptBeamPick(self.h, n_picks, mode, top_p, temperature, _ptr(u), _ptr(ids), _ptr(logp)))
+        return ids, logp
+
+    def reorder_rows(self, src_rows):
+        """Row i of the new batch continues old row src_rows[i] (KV cache and token history are gathered)."""
+        src = np.ascontiguousarray(src_rows, dtype=np.int32).reshape(-1)
+        check(lib().TSHip_GptReorderRows(self.h, _ptr(src), int(src.size)))
+        self.batch = int(src.size)
+
+    def beam_search(self, prompts, beam_size, max_len, eos_id=0, mode=GREEDY, top_p=0.0, temperature=1.0, uniforms=None, lens=None):
+        """The loop of GPT.RunForwardOnSingleDevice for BeamSearchSize > 1 (Applications/GPT.cs:264-302): every step makes
+        beam_size picks from every hypothesis, scores them (previous score - log p; a hypothesis starts at 1.0,
+        Utils/BeamSearch.cs:29), keeps the beam_size best per sequence (BeamSearch.GetTopNBSS) and stops when every
+        hypothesis ends in the END tag or at max_len tokens.  prompts [batch, len].  uniforms [steps, beam_size picks,
+        beam_size * batch rows] for top-p.  Returns (hypotheses [batch][beam] as token lists, scores [batch][beam]),
+        beams in the reference's order."""
+        prompts = np.ascontiguousarray(prompts, dtype=np.int32)
+        B, T0 = prompts.shape
+        assert beam_size >= 1 and B * beam_size <= self.max_batch, "max_batch must hold batch x beam_size rows"
+        self.reset()
+        self.prefill(prompts, lens=lens)
+        # rows are hypotheses in beam-major order: row j * B + b = hypothesis j of sequence b
+        hyp = [[list(map(int, prompts[b])) for b in range(B)]]
+        score = [[np.float32(1.0) for _ in range(B)]]
+        step = 0
+        for _ in range(T0, max_len):
+            nb = len(hyp)
+            u = None if uniforms is None else np.ascontiguousarray(uniforms[step][:, :nb * B])
+            ids, logp = self.beam_pick(beam_size, mode, top_p, temperature, u)
+            new_hyp = [[None] * B for _ in range(beam_size)]
+            new_score = [[None] * B for _ in range(beam_size)]
+            src = np.zeros((beam_size, B), np.int32)
+            tok = np.zeros((beam_size, B), np.int32)
+            for b in range(B):
+                cand = []                                   # (score, parent beam, token) in the reference's order: beams outer, picks inner
+                for j in range(nb):
+                    for i in range(beam_size):
+                        r = j * B + b
+                        cand.append((np.float32(score[j][b] + np.float32(-1.0) * logp[i, r]), j, int(ids[i, r])))
+                if beam_size > 1:
+                    sc = np.array([c[0] for c in cand], np.float32)
+                    kept = np.empty((beam_size,), np.int32)
+                    nk = C.c_int(0)
+                    check(lib().TSHip_BeamTopN(_ptr(sc), len(cand), beam_size, _ptr(kept), C.byref(nk)))
+                    order = [int(k) for k in kept[:nk.value]]
+                else:
+                    order = [0]
+                for jn, k in enumerate(order):
+                    s_, j, t = cand[k]
+                    new_hyp[jn][b] = hyp[j][b] + [t]
+                    new_score[jn][b] = s_
+                    src[jn, b] = j * B + b
+                    tok[jn, b] = t
+            hyp, score = new_hyp, new_score
+            step += 1
+            done = all(h[-1] == eos_id for beam in hyp for h in beam)
+            if done or len(hyp[0][0]) >= max_len:
+                break
+            self.reorder_rows(src.reshape(-1))
+            self.decode(tok.reshape(-1))
+        out_h = [[hyp[j][b] for j in range(len(hyp))] for b in range(B)]
+        out_s = [[float(score[j][b]) for j in range(len(hyp))] for b in range(B)]
+        return out_h, out_s
 
     def logits(self):
         out = np.empty((self.batch, self.cfg["vocab"]), np.float32)
