@@ -10,6 +10,9 @@
  *   - no C++ exception crosses the boundary                              (ggml_ops.cpp:4707-4722)
  *   - the caller owns every tensor buffer; the library keeps no tensor pointer after a call returns
  *   - calls are ordered on one library stream; functions that hand data to the host synchronise
+ *   - any thread may call: a call holds the library's lock from entry to return, so calls from several threads
+ *     (the reference issues ops from Parallel.For workers, BaseSeq2SeqFramework.cs:912-941) are serialised, each
+ *     seeing its own last-error string; one TSHipGpt object is meant for one thread at a time, like a ggml context
  *
  * Tensor arguments are strided views (sizes and strides in ELEMENTS, outermost dimension first, exactly
  * TensorSharp.Tensor's Sizes/Strides, TensorSharp/Tensor.cs:12-125).  `data` is a DEVICE pointer already
@@ -45,8 +48,14 @@ typedef struct TSHipTensor {
 TSHIP_API const char* TSHip_GetLastError(void);                               /* cf. TSGgml_GetLastError */
 TSHIP_API int TSHip_GetDeviceCount(int* count);
 TSHIP_API int TSHip_Init(int device_id);                                      /* once per process; cf. ggml_ops.cpp:256-280 */
+/* Device memory comes from a pool (cf. TensorSharp.CUDA/ContextState/PoolingDeviceAllocator.cs): freed blocks are cached
+ * by size class and handed out again without a driver call or a device synchronisation (every use of a block is ordered
+ * on the library stream).  TSHip_Free rejects pointers that TSHip_Malloc did not hand out. */
 TSHIP_API int TSHip_Malloc(void** ptr, size_t bytes);                         /* IAllocator.Allocate */
 TSHIP_API int TSHip_Free(void* ptr);                                          /* Storage.Destroy */
+TSHIP_API int TSHip_PoolTrim(void);                                           /* give every cached block back to the driver */
+/* number of hipMalloc calls the pool has made, bytes handed out, bytes cached for reuse (any pointer may be NULL) */
+TSHIP_API int TSHip_GetPoolStats(size_t* device_allocations, size_t* bytes_in_use, size_t* bytes_cached);
 TSHIP_API int TSHip_MemcpyH2D(void* dst, const void* src, size_t bytes);      /* Storage.CopyToStorage / SetElementsAsFloat */
 TSHIP_API int TSHip_MemcpyD2H(void* dst, const void* src, size_t bytes);      /* Storage.CopyFromStorage / GetElementsAsFloat */
 TSHIP_API int TSHip_MemcpyD2D(void* dst, const void* src, size_t bytes);

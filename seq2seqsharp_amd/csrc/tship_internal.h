@@ -8,6 +8,7 @@
 
 #include <cstdint>
 #include <cstdio>
+#include <mutex>
 #include <stdexcept>
 #include <string>
 
@@ -33,8 +34,15 @@ struct Error : std::runtime_error {
         if (!(cond)) throw ::tship::Error(std::string(msg));                                          \
     } while (0)
 
+// One lock for every exported call that touches the device: the library drives one ordered stream, and a call may span
+// many launches that must not interleave with another thread's (a HIP graph capture records whatever lands on the stream
+// meanwhile; a model's buffers are written by consecutive kernels).  Callers on several threads, as the reference's
+// Parallel.For over devices (BaseSeq2SeqFramework.cs:912-941), are serialised here; the lock is recursive because
+// exported calls nest.
+std::recursive_mutex& api_mutex();
+
 // Every exported function is wrapped: 1 on success, 0 on failure with the message stored per thread.
-#define TSHIP_BEGIN try {
+#define TSHIP_BEGIN try { std::lock_guard<std::recursive_mutex> tship_api_lock(::tship::api_mutex());
 #define TSHIP_END                                                                                     \
     return 1;                                                                                         \
     }                                                                                                 \

@@ -3,12 +3,18 @@
 // TensorSharp/Storage.cs:32-47); the error convention follows TensorSharp.GGML.Native/ggml_ops.cpp:211-224.
 #include "tship_internal.h"
 
+#include <map>
 #include <mutex>
+#include <unordered_map>
+#include <vector>
 
 namespace tship {
 
 static thread_local std::string t_last_error;
 void set_last_error(const std::string& msg) { t_last_error = msg; }
+
+static std::recursive_mutex g_api_mutex;
+std::recursive_mutex& api_mutex() { return g_api_mutex; }
 
 static std::mutex g_init_mutex;
 static bool g_initialised = false;
@@ -49,6 +55,74 @@ void ensure_init() {
     if (!g_initialised) init_locked(0);
 }
 
+// ------------------------------------------------------------------------------------------------
+// Device memory pool behind TSHip_Malloc / TSHip_Free (the role of TensorSharp.CUDA/ContextState/PoolingDeviceAllocator.cs:
+// tensors come and go about 45 times per layer and step on the per-op surface, and hipMalloc / hipFree cost tens of
+// microseconds each and synchronise the device).
+// Blocks are cached by size class and never returned to the driver while the process runs (TSHip_PoolTrim and an
+// allocation failure release them).  A freed block may be handed out again at once without waiting for the GPU: every
+// kernel and copy of this library runs on the one library stream, so whatever still reads the block was enqueued before
+// whatever the next owner enqueues.
+// Size classes: multiples of 256 bytes up to 4 KiB, then four classes per power of two (at most 19 % slack).
+// ------------------------------------------------------------------------------------------------
+static std::mutex g_pool_mutex;
+static std::unordered_map<void*, size_t> g_pool_live;                 // block -> class size
+static std::map<size_t, std::vector<void*>> g_pool_free;              // class size -> cached blocks
+static size_t g_pool_device_allocs = 0, g_pool_bytes_cached = 0, g_pool_bytes_live = 0;
+
+static size_t pool_class(size_t bytes) {
+    if (bytes <= 4096) return (bytes + 255) / 256 * 256;
+    size_t p = 4096;
+    while (p * 2 < bytes) p *= 2;                                        // p < bytes <= 2p
+    const size_t step = p / 4;
+    return p + (bytes - p + step - 1) / step * step;
+}
+
+static void pool_release_cached_locked() {
+    for (auto& kv : g_pool_free) for (void* p : kv.second) (void)hipFree(p);
+    g_pool_free.clear();
+    g_pool_bytes_cached = 0;
+}
+
+static void* pool_malloc(size_t bytes) {
+    const size_t cls = pool_class(bytes == 0 ? 4 : bytes);
+    std::lock_guard<std::mutex> lk(g_pool_mutex);
+    auto it = g_pool_free.find(cls);
+    if (it != g_pool_free.end() && !it->second.empty()) {
+        void* p = it->second.back(); it->second.pop_back();
+        g_pool_bytes_cached -= cls; g_pool_bytes_live += cls;
+        g_pool_live[p] = cls;
+        return p;
+    }
+    void* p = nullptr;
+    hipError_t e = hipMalloc(&p, cls);
+    if (e != hipSuccess) {
+        // give the cached blocks back and try once more (the GPU may still be using them: wait for it first)
+        (void)hipGetLastError();
+        (void)hipStreamSynchronize(stream());
+        pool_release_cached_locked();
+        e = hipMalloc(&p, cls);
+    }
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        throw Error("out of device memory: hipMalloc(" + std::to_string(cls) + " bytes) failed: " + hipGetErrorString(e));
+    }
+    ++g_pool_device_allocs;
+    g_pool_bytes_live += cls;
+    g_pool_live[p] = cls;
+    return p;
+}
+
+static void pool_free(void* p) {
+    std::lock_guard<std::mutex> lk(g_pool_mutex);
+    auto it = g_pool_live.find(p);
+    if (it == g_pool_live.end()) throw Error("TSHip_Free: pointer was not allocated by TSHip_Malloc (or was freed before)");
+    const size_t cls = it->second;
+    g_pool_live.erase(it);
+    g_pool_free[cls].push_back(p);
+    g_pool_bytes_live -= cls; g_pool_bytes_cached += cls;
+}
+
 }  // namespace tship
 
 using namespace tship;
@@ -79,12 +153,7 @@ TSHIP_API int TSHip_Malloc(void** ptr, size_t bytes) {
     TSHIP_REQUIRE(ptr != nullptr, "TSHip_Malloc: ptr is null");
     ensure_init();
     *ptr = nullptr;
-    if (bytes == 0) bytes = 4;
-    hipError_t e = hipMalloc(ptr, bytes);
-    if (e != hipSuccess) {
-        (void)hipGetLastError();
-        throw Error("out of device memory: hipMalloc(" + std::to_string(bytes) + " bytes) failed: " + hipGetErrorString(e));
-    }
+    *ptr = pool_malloc(bytes);
     TSHIP_END
 }
 
@@ -92,9 +161,26 @@ TSHIP_API int TSHip_Free(void* ptr) {
     TSHIP_BEGIN
     if (ptr) {
         ensure_init();
-        TSHIP_CHECK_HIP(hipStreamSynchronize(stream()));
-        TSHIP_CHECK_HIP(hipFree(ptr));
+        pool_free(ptr);
     }
+    TSHIP_END
+}
+
+TSHIP_API int TSHip_PoolTrim(void) {
+    TSHIP_BEGIN
+    ensure_init();
+    TSHIP_CHECK_HIP(hipStreamSynchronize(stream()));
+    std::lock_guard<std::mutex> lk(g_pool_mutex);
+    pool_release_cached_locked();
+    TSHIP_END
+}
+
+TSHIP_API int TSHip_GetPoolStats(size_t* device_allocations, size_t* bytes_in_use, size_t* bytes_cached) {
+    TSHIP_BEGIN
+    std::lock_guard<std::mutex> lk(g_pool_mutex);
+    if (device_allocations) *device_allocations = g_pool_device_allocs;
+    if (bytes_in_use) *bytes_in_use = g_pool_bytes_live;
+    if (bytes_cached) *bytes_cached = g_pool_bytes_cached;
     TSHIP_END
 }
 
