@@ -192,6 +192,68 @@ __global__ __launch_bounds__(256) void gemm_strided_kernel(MatView C, MatView S,
     }
 }
 
+// ---- GEMM on the matrix cores for fp16 operands with contiguous rows (what Affine and Mul issue on fp16 models) -------
+// C[M,N] = beta * S + alpha * A[M,K] B[K,N], fp32 accumulation.  Block tile 128 x 64, four wavefronts, each a 32-row
+// strip of the tile and both of its 32-column halves; k advances 16 per step with v_mfma_f32_32x32x16_f16:
+//   A operand (32 rows x 16 k): lane l holds row l % 32, k = 8 (l / 32) .. + 7: 16 contiguous bytes of a row of A, read
+//     straight from global memory;
+//   B operand (16 k x 32 columns): lane l holds column l % 32, k = 8 (l / 32) .. + 7, a column walk in row-major B: the
+//     block stages the 16 x 64 tile of B in LDS transposed ([column][k], two stages), so that a lane reads its 8 values
+//     as one 16-byte LDS load;
+//   D: lane l, register v holds row 8 (v / 4) + 4 (l / 32) + v % 4, column l % 32: a register is a run of 32 columns.
+// The host takes this path when K % 8 == 0, N % 4 == 0, the leading dimensions keep 16-byte (A) and 8-byte (B) alignment
+// and inner strides are 1; everything else goes to the generic kernel above.
+__global__ __launch_bounds__(256) void gemm_f16_mfma_kernel(MatView C, MatView S, MatView A, MatView B, int M, int N, int K, float alpha, float beta) {
+    __shared__ __attribute__((aligned(16))) half_t Bs[2][64][24];        // [stage][column][k (16, padded to 24: conflict-free 16-byte reads)]
+    const int t = threadIdx.x, lane = t & 63, w = t >> 6;
+    const int col0 = blockIdx.x * 64, row0 = blockIdx.y * 128 + w * 32; const long bz = blockIdx.z;
+    const half_t* Ab = (const half_t*)A.p + bz * A.sb;
+    const half_t* Bb = (const half_t*)B.p + bz * B.sb;
+    floatx16 acc[2];
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[j][v] = 0.0f;
+    const int am = row0 + (lane & 31), ak = 8 * (lane >> 5);
+    const bool a_ok = am < M;
+    // staging of B: thread t brings 4 columns of one k row
+    const int bk = t >> 4, bn = (t & 15) * 4;
+    const bool b_ok = col0 + bn < N;            // (N is a multiple of 4: a group of 4 columns is inside or outside)
+    const int nk = (K + 15) / 16;
+    auto stage_b = [&](int kt, int st) {
+        half4 v = half4{0, 0, 0, 0};
+        const int k = kt * 16 + bk;
+        if (b_ok && k < K) v = *(const half4*)(Bb + (long)k * B.s0 + col0 + bn);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) Bs[st][bn + i][bk] = v[i];
+    };
+    stage_b(0, 0);
+    for (int kt = 0; kt < nk; ++kt) {
+        half8 af = half8{0, 0, 0, 0, 0, 0, 0, 0};
+        if (a_ok && kt * 16 + ak < K) af = *(const half8*)(Ab + (long)am * A.s0 + kt * 16 + ak);      // (K is a multiple of 8)
+        __syncthreads();                        // stage kt & 1 is complete; the other one has been consumed
+        if (kt + 1 < nk) stage_b(kt + 1, (kt + 1) & 1);
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const half8 bf = *(const half8*)(&Bs[kt & 1][j * 32 + (lane & 31)][ak]);
+            acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af, bf, acc[j], 0, 0, 0);
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        const int c = col0 + j * 32 + (lane & 31);
+        if (c >= N) continue;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            const int r = row0 + 8 * (v / 4) + 4 * (lane >> 5) + (v % 4);
+            if (r >= M) continue;
+            float o = alpha * acc[j][v];
+            if (beta != 0.0f) o += beta * ld(S.p, S.dtype, bz * S.sb + (long)r * S.s0 + (long)c * S.s1);
+            ((half_t*)C.p)[bz * C.sb + (long)r * C.s0 + c] = (half_t)o;
+        }
+    }
+}
+
 // ---- row kernels: one 256-thread block per row ----------------------------------------------------
 __global__ __launch_bounds__(256) void softmax_rows_kernel(RowView r, RowView s) {
     __shared__ float sred[4];
@@ -406,8 +468,17 @@ static void addmm_common(const char* what, const TSHipTensor* result, float beta
     const int M = (int)s.sz[o], N = (int)s.sz[o + 1], K = (int)a.sz[o + 1];
     if (M == 0 || N == 0 || nb == 0) return;
     auto mv = [&](const View& v) { MatView m; m.p = v.p; m.dtype = v.dtype; m.s0 = v.st[o]; m.s1 = v.st[o + 1]; m.sb = nd == 3 ? v.st[0] : 0; return m; };
-    dim3 grid((unsigned)ceil_div(N, 64), (unsigned)ceil_div(M, 64), (unsigned)nb);
-    hipLaunchKernelGGL(gemm_strided_kernel, grid, dim3(256), 0, stream(), mv(r), mv(s), mv(a), mv(b), M, N, K, alpha, beta);
+    // fp16 operands with contiguous rows (Affine, Mul and AddmmBatch with an untransposed right operand): matrix cores
+    const bool mfma = s.dtype == TSHIP_F16 && a.st[o + 1] == 1 && b.st[o + 1] == 1 && r.st[o + 1] == 1 && K % 8 == 0 && N % 4 == 0 && K >= 16 &&
+                      a.st[o] % 8 == 0 && b.st[o] % 4 == 0 && ((uintptr_t)a.p % 16) == 0 && ((uintptr_t)b.p % 8) == 0 &&
+                      (nd == 2 || (a.st[0] % 8 == 0 && b.st[0] % 4 == 0));
+    if (mfma) {
+        dim3 grid((unsigned)ceil_div(N, 64), (unsigned)ceil_div(M, 128), (unsigned)nb);
+        hipLaunchKernelGGL(gemm_f16_mfma_kernel, grid, dim3(256), 0, stream(), mv(r), mv(s), mv(a), mv(b), M, N, K, alpha, beta);
+    } else {
+        dim3 grid((unsigned)ceil_div(N, 64), (unsigned)ceil_div(M, 64), (unsigned)nb);
+        hipLaunchKernelGGL(gemm_strided_kernel, grid, dim3(256), 0, stream(), mv(r), mv(s), mv(a), mv(b), M, N, K, alpha, beta);
+    }
     check_launch();
 }
 

@@ -13,7 +13,7 @@ import math
 import numpy as np
 
 from . import ops
-from .tensor import F32, HipTensor
+from .tensor import F16, F32, HipTensor
 
 
 class ComputeGraph:
@@ -86,8 +86,10 @@ class ComputeGraph:
 class DeviceWeights:
     """The model's parameters as device tensors under the reference's names."""
 
-    def __init__(self, weights):
-        self.t = {k: HipTensor.from_numpy(np.asarray(v, np.float32)) for k, v in weights.items()}
+    def __init__(self, weights, dtype=F32):
+        """dtype F16: the model as the reference holds it with AMP (every parameter Float16, Applications/GPT.cs:122-130)."""
+        self.dtype = dtype
+        self.t = {k: HipTensor.from_numpy(np.asarray(v, np.float32), dtype) for k, v in weights.items()}
 
     def __getitem__(self, k):
         return self.t[k]
@@ -110,11 +112,18 @@ def _attn_tail(g, cfg, W, name, Qs, Ks, Vs, mask, B, Tq, H, d, inputQ, cache):
         cache[vn] = Vs
     Tkv = Ks.sizes[2]
     scale = np.float32(1.0) / np.float32(math.sqrt(d))
+    use_f16 = Qs.dtype == F16                     # GroupQueryAttention.cs:196-201: scores, mask and softmax run in Float32
+    if use_f16:
+        Qs, Ks = ops.half2float(None, Qs), ops.half2float(None, Ks)
     attn = g.MulBatch(Qs, Ks, float(scale))
     attn = g.View(attn, [B, H, Tq, Tkv])
     if mask is not None:
+        if use_f16:
+            mask = ops.half2float(None, mask)     # :209-212 (the expanded view is materialised by the conversion)
         attn = g.Add(attn, mask, in_place=True)
     attn = g.Softmax(attn, in_place=True)
+    if use_f16:
+        attn = ops.float2half(None, attn)         # :216-219
     attn = g.View(attn, [B * H, Tq, Tkv])
     o = g.View(g.MulBatch(attn, Vs), [B, H, Tq, d])
     Wt = g.View(g.AsContiguous(g.Transpose(o, 1, 2)), [B * Tq, H * d])
@@ -180,7 +189,9 @@ def positionwise_feed_forward(g, cfg, W, layer, x):
 
 def gpt_decode_step(g, cfg, W, seqs, cache):
     """Decoder.GPTDecode up to the probabilities (Seq2SeqSharp/Applications/Decoder.cs:648-732), dense layers only.
-    seqs: int array [B, len].  Returns (probs, logits) as device tensors."""
+    seqs: int array [B, len].  Returns (probs, logits) as device tensors.  With Float16 weights (DeviceWeights(..., F16))
+    this is the AMP run: every tensor Float16 except the attention scores and the logits handed to the softmax."""
+    amp = getattr(W, "dtype", F32) == F16
     seqs = np.asarray(seqs)
     B, ln = seqs.shape
     H = cfg["n_heads"]
@@ -189,7 +200,7 @@ def gpt_decode_step(g, cfg, W, seqs, cache):
         Tq, ids = 1, seqs[:, -1].astype(np.float32)
     else:
         Tq, ids = ln, seqs.reshape(-1).astype(np.float32)
-        m = ops.buildtrimask(HipTensor([Tq, Tq]), 0.0, -30000.0)
+        m = ops.buildtrimask(HipTensor([Tq, Tq], F16 if amp else F32), 0.0, -30000.0)      # Decoder.cs:685: the mask has the model's type
         mask = m.view(1, 1, Tq, Tq).expand(B, H, Tq, Tq)
     idx = HipTensor.from_numpy(ids.reshape(-1, 1))
     x = g.IndexSelect(W["TgtEmbeddings"], idx)
@@ -202,5 +213,7 @@ def gpt_decode_step(g, cfg, W, seqs, cache):
     last = HipTensor.from_numpy(np.array([Tq * (i + 1) - 1 for i in range(B)], np.float32).reshape(-1, 1))
     x = g.IndexSelect(x, last)
     logits = g.Affine(x, W["FeedForward_Decoder_0.m_Whd"], W["FeedForward_Decoder_0.m_Bd"])
+    if amp:
+        logits = ops.half2float(None, logits)     # Decoder.cs:725-730
     probs = ops.softmax(None, logits)
     return probs, logits

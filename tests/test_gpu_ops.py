@@ -107,6 +107,39 @@ def test_addmm(T, oracle):
         ops.addmm(None, 0.0, HT([2, 3]), 1.0, HT([2, 4]), HT([5, 3]))
 
 
+@pytest.mark.parametrize("M,K,N", [(1, 16, 4), (33, 24, 68), (130, 512, 256), (64, 2048, 96), (200, 40, 8)])
+def test_addmm_fp16_on_the_matrix_cores(T, M, K, N):
+    """Float16 operands with contiguous rows take the MFMA kernel (K a multiple of 8, N of 4): partial row, column and k
+    tiles, alpha / beta, an expanded bias, result aliasing src, and the batched form.  Against float64 products of the same
+    Float16 values; the result is rounded to Float16 once."""
+    HT, ops = T
+    from seq2seqsharp_amd.tensor import F16
+    rng = np.random.default_rng(M + K + N)
+    a = rng.standard_normal((M, K)).astype(np.float16)
+    b = rng.standard_normal((K, N)).astype(np.float16)
+    bias = rng.standard_normal((1, N)).astype(np.float16)
+    want = a.astype(np.float64) @ b.astype(np.float64)
+    tol = 2e-3 * np.sqrt(K) + 1e-2
+    ta, tb = HT.from_numpy(a.astype(np.float32), F16), HT.from_numpy(b.astype(np.float32), F16)
+    got = ops.addmm(None, 1.0, HT.from_numpy(bias.astype(np.float32), F16).expand(M, N), 1.0, ta, tb)
+    assert got.dtype == F16
+    assert np.abs(got.numpy() - (want + bias.astype(np.float64))).max() <= tol
+    r = HT.from_numpy(np.ones((M, N), np.float32), F16)
+    got = ops.addmm(r, 0.5, r, -2.0, ta, tb).numpy()                      # result aliases src
+    assert np.abs(got - (0.5 - 2.0 * want)).max() <= 2 * tol
+    # same product through the generic kernel (a transposed view of a transposed copy is not row-contiguous)
+    tbt = HT.from_numpy(np.ascontiguousarray(b.T).astype(np.float32), F16).transpose(0, 1)
+    gen = ops.addmm(None, 0.0, HT([M, N], F16), 1.0, ta, tbt).numpy()
+    mf = ops.addmm(None, 0.0, HT([M, N], F16), 1.0, ta, tb).numpy()
+    assert np.abs(gen - mf).max() <= tol
+    # batched: attention weights x values (MulBatch(attn, Vs))
+    q = rng.standard_normal((5, M, K)).astype(np.float16)
+    v = rng.standard_normal((5, K, N)).astype(np.float16)
+    z = HT([5, M, N], F16)
+    got = ops.addmmbatch(z, 0.0, z, 1.0, HT.from_numpy(q.astype(np.float32), F16), HT.from_numpy(v.astype(np.float32), F16)).numpy()
+    assert np.abs(got - np.einsum("bik,bkj->bij", q.astype(np.float64), v.astype(np.float64))).max() <= tol
+
+
 def test_addmmbatch(T, oracle):
     HT, ops = T
     m1 = np.arange(1, 13, dtype=np.float32).reshape(2, 3, 2)
