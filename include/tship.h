@@ -112,6 +112,11 @@ TSHIP_API int TSHip_Unary(int op, const TSHipTensor* result, const TSHipTensor* 
 TSHIP_API int TSHip_BuildTriMask(const TSHipTensor* result, float value, float masked_value);
 TSHIP_API int TSHip_BuildSelfTriMask(const TSHipTensor* result, const TSHipTensor* original_lengths,
                                      int padded_seq_len, float value, float masked_value);
+/* "gather": result[.., j, ..] = src[.., (long)indices[.., j, ..], ..] along `dim`; "scatter_fill": result[.., (long)indices[..], ..] =
+ * value (CpuIndexingOps.cs:23-56, :141-167; TensorApplyCPU.cs:200-257).  The beam search loop issues them on the probabilities
+ * (Decoder.cs:766, :788).  An index outside the dimension fails the call. */
+TSHIP_API int TSHip_Gather(const TSHipTensor* result, const TSHipTensor* src, int dim, const TSHipTensor* indices);
+TSHIP_API int TSHip_ScatterFill(const TSHipTensor* result, float value, int dim, const TSHipTensor* indices);
 /* "iscorrupted": *corrupted = 1 if any element is not finite (TensorApplyCPU.cs:1212-1228) */
 TSHIP_API int TSHip_IsCorrupted(const TSHipTensor* src, int* corrupted);
 

@@ -7,6 +7,7 @@
 #include "tship_sample_kernels.h"
 
 #include <cstring>
+#include <functional>
 #include <vector>
 
 namespace tship {
@@ -141,6 +142,35 @@ __global__ void ew_scalar_kernel(View r, View a, float s, int op, long n) {
     long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= n) return;
     st(r.p, r.dtype, view_offset(r, i), binary_apply(op, ld(a.p, a.dtype, view_offset(a, i)), s));
+}
+
+// ---- gather / scatter_fill along one dimension (TensorApplyCPU.cs:200-257 through ApplyDim2 / ApplyDim3) -------------
+// One thread per element of `indices`.  gather: result[.., j, ..] = src[.., (long)indices[.., j, ..], ..];
+// scatter_fill: result[.., (long)indices[.., j, ..], ..] = value.  An index outside the dimension (the reference throws
+// IndexOutOfRangeException) sets *bad and is skipped.
+__global__ void gather_kernel(View r, View s, View ix, int dim, long n, int* bad) {
+    long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const long idx = (long)ld(ix.p, ix.dtype, view_offset(ix, i));
+    if (idx < 0 || idx >= s.sz[dim]) { *bad = 1; return; }
+    long lin = i, so = 0;
+#pragma unroll
+    for (int d = TSHIP_MAX_DIMS - 1; d >= 0; --d) {
+        if (d < ix.nd) { const long q = lin / ix.sz[d]; const long c = lin - q * ix.sz[d]; so += (d == dim ? idx : c) * s.st[d]; lin = q; }
+    }
+    st(r.p, r.dtype, view_offset(r, i), ld(s.p, s.dtype, so));
+}
+__global__ void scatter_fill_kernel(View r, View ix, int dim, float value, long n, int* bad) {
+    long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const long idx = (long)ld(ix.p, ix.dtype, view_offset(ix, i));
+    if (idx < 0 || idx >= r.sz[dim]) { *bad = 1; return; }
+    long lin = i, ro = 0;
+#pragma unroll
+    for (int d = TSHIP_MAX_DIMS - 1; d >= 0; --d) {
+        if (d < ix.nd) { const long q = lin / ix.sz[d]; const long c = lin - q * ix.sz[d]; ro += (d == dim ? idx : c) * r.st[d]; lin = q; }
+    }
+    st(r.p, r.dtype, ro, value);
 }
 
 // ---- GEMM over strided 2-D views, optional batch (blockIdx.z) ---------------------------------------
@@ -694,6 +724,50 @@ TSHIP_API int TSHip_BuildSelfTriMask(const TSHipTensor* result, const TSHipTenso
     if (n == 0) return 1;
     hipLaunchKernelGGL(trimask_kernel, grid1(n), dim3(256), 0, stream(), r, r.sz[0], r.sz[1], value, masked_value, (const void*)l.p, l.dtype, padded_seq_len);
     check_launch();
+    TSHIP_END
+}
+
+// shared by gather and scatter_fill: a device flag for indices outside the dimension, read back after the kernel
+static void run_indexed(const char* what, const std::function<void(int*)>& launch_fn) {
+    int* flag = nullptr;
+    TSHIP_CHECK_HIP(hipMalloc(&flag, sizeof(int)));
+    int host = 0;
+    hipError_t e = hipMemsetAsync(flag, 0, sizeof(int), stream());
+    if (e == hipSuccess) { launch_fn(flag); e = hipGetLastError(); }
+    if (e == hipSuccess) e = hipMemcpyAsync(&host, flag, sizeof(int), hipMemcpyDeviceToHost, stream());
+    if (e == hipSuccess) e = hipStreamSynchronize(stream());
+    (void)hipFree(flag);
+    TSHIP_CHECK_HIP(e);
+    if (host) throw Error(std::string(what) + ": an index lies outside the dimension");
+}
+
+TSHIP_API int TSHip_Gather(const TSHipTensor* result, const TSHipTensor* src, int dim, const TSHipTensor* indices) {
+    TSHIP_BEGIN
+    ensure_init();
+    View r = make_view(result, "TSHip_Gather"), s = make_view(src, "TSHip_Gather"), ix = make_view(indices, "TSHip_Gather");
+    // CpuIndexingOps.Gather, TensorSharp/Cpu/CpuIndexingOps.cs:23-56
+    TSHIP_REQUIRE(r.nd == s.nd, "result and src must have same number of dimensions");
+    TSHIP_REQUIRE(dim >= 0 && dim < r.nd, "TSHip_Gather: dim out of range");
+    TSHIP_REQUIRE(ix.nd == s.nd, "src and indices must have same number of dimensions");
+    TSHIP_REQUIRE(same_shape(r, ix), "result and indices must be the same size");
+    for (int d = 0; d < r.nd; ++d) TSHIP_REQUIRE(d == dim || s.sz[d] == r.sz[d], "result and src must be the same size except in dimension dim");
+    const long n = count(ix);
+    if (n == 0) return 1;
+    run_indexed("TSHip_Gather", [&](int* flag) { hipLaunchKernelGGL(gather_kernel, grid1(n), dim3(256), 0, stream(), r, s, ix, dim, n, flag); });
+    TSHIP_END
+}
+
+TSHIP_API int TSHip_ScatterFill(const TSHipTensor* result, float value, int dim, const TSHipTensor* indices) {
+    TSHIP_BEGIN
+    ensure_init();
+    View r = make_view(result, "TSHip_ScatterFill"), ix = make_view(indices, "TSHip_ScatterFill");
+    // CpuIndexingOps.ScatterFill, TensorSharp/Cpu/CpuIndexingOps.cs:141-167
+    TSHIP_REQUIRE(dim >= 0 && dim < r.nd, "TSHip_ScatterFill: dim out of range");
+    TSHIP_REQUIRE(ix.nd == r.nd, "result and indices must have same number of dimensions");
+    for (int d = 0; d < r.nd; ++d) TSHIP_REQUIRE(d == dim || ix.sz[d] == r.sz[d], "result and indices must be the same size except in dimension dim");
+    const long n = count(ix);
+    if (n == 0) return 1;
+    run_indexed("TSHip_ScatterFill", [&](int* flag) { hipLaunchKernelGGL(scatter_fill_kernel, grid1(n), dim3(256), 0, stream(), r, ix, dim, value, n, flag); });
     TSHIP_END
 }
 

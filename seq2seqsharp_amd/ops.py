@@ -44,6 +44,8 @@ def _p():
     L.TSHip_BuildSelfTriMask.argtypes = [T, T, C.c_int, C.c_float, C.c_float]
     L.TSHip_IsCorrupted.argtypes = [T, C.POINTER(C.c_int)]
     L.TSHip_TopPSample.argtypes = [T, T, T, C.c_float]
+    L.TSHip_Gather.argtypes = [T, T, C.c_int, T]
+    L.TSHip_ScatterFill.argtypes = [T, C.c_float, C.c_int, T]
     L.TSHip_TopPSampleNoAlloc.argtypes = [T, T, T, C.c_float]
     L.TSHip_TopPSampleEx.argtypes = [T, T, T, C.c_float, C.c_float, C.c_void_p, C.c_void_p, C.c_int]
     _ok = True
@@ -239,6 +241,17 @@ def iscorrupted(src):                                    # "iscorrupted"
     flag = C.c_int(0)
     check(_p().TSHip_IsCorrupted(_d(src), C.byref(flag)))
     return bool(flag.value)
+
+
+def gather(result, src, dim, indices):                   # "gather", CpuIndexingOps.cs:23-56
+    r = _target(result, indices.sizes, src.dtype)
+    check(_p().TSHip_Gather(_d(r), _d(src), int(dim), _d(indices)))
+    return r
+
+
+def scatter_fill(result, value, dim, indices):           # "scatter_fill", CpuIndexingOps.cs:141-167
+    check(_p().TSHip_ScatterFill(_d(result), float(value), int(dim), _d(indices)))
+    return result
 
 
 def toppsample(result, probs, uniforms, top_p, repeat_penalty=0.0, seqs=None, seq_lens=None):

@@ -323,3 +323,28 @@ def test_error_paths(T):
         ops.add(None, HT([2, 3]), HT([3, 2]))
     with pytest.raises(TSHipError):
         ops.topk(None, None, HT([2, 3]), 4)
+
+
+def test_gather_and_scatter_fill(T):
+    """The two indexing ops of the beam search loop (Decoder.cs:766 Gather(probs, idx, 1), :788 ScatterFill(probs, 0, idx, 1)),
+    on contiguous and strided tensors, against NumPy's take_along_axis / put_along_axis; an index outside the dimension fails."""
+    HT, ops = T
+    rng = np.random.default_rng(30)
+    p = rng.random((5, 97)).astype(np.float32)
+    idx = rng.integers(0, 97, size=(5, 1)).astype(np.float32)
+    got = ops.gather(None, HT.from_numpy(p), 1, HT.from_numpy(idx)).numpy()
+    assert np.array_equal(got, np.take_along_axis(p, idx.astype(np.int64), 1))
+    t = HT.from_numpy(p)
+    ops.scatter_fill(t, 0.0, 1, HT.from_numpy(idx))
+    want = p.copy()
+    np.put_along_axis(want, idx.astype(np.int64), 0.0, 1)
+    assert np.array_equal(t.numpy(), want)
+    a = rng.random((4, 6, 7)).astype(np.float32)
+    for dim in range(3):
+        shape = list(a.shape)
+        shape[dim] = 3
+        ix = rng.integers(0, a.shape[dim], size=shape).astype(np.float32)
+        for src in (HT.from_numpy(a), HT.from_numpy(np.ascontiguousarray(a.transpose(0, 2, 1))).transpose(1, 2)):
+            assert np.array_equal(ops.gather(None, src, dim, HT.from_numpy(ix)).numpy(), np.take_along_axis(a, ix.astype(np.int64), dim))
+    with pytest.raises(Exception, match="outside"):
+        ops.gather(None, HT.from_numpy(p), 1, HT.from_numpy(np.full((5, 1), 97, np.float32)))
