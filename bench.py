@@ -6,8 +6,8 @@
 A "step" is one decode step of the whole batch (one new token per sequence) on synthetic data:
 seeded N(0, 0.02) weights of the named architecture and uniform-random prompts, KV cache filled by a real
 prefill of the prompts.  Prints ONE JSON line: decode tokens/s (whole batch), the roofline of the
-dominant kernel (the weight-streaming decode GEMM of the FFN up/gate projection) measured live with device
-events, and the CPU baseline (the oracle's restatement of the reference's CPU backend, single thread,
+dominant kernel (the one with the largest share of the step; every streaming kernel is listed in roofline_all)
+measured live with device events, and the CPU baseline (the oracle's restatement of the reference's CPU backend, single thread,
 timed on a bounded sample on this host).
 """
 import argparse
@@ -73,6 +73,7 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-topp", action="store_true")
     ap.add_argument("--prompt", type=int, default=0, help="override the prompt length")
+    ap.add_argument("--structure-probe", action="store_true", help="also time the step's launch structure with pure streaming reads of the same bytes")
     ap.add_argument("--no-copy-calibration", action="store_true",
                     help="skip the 256 MiB plain copy that gives rocprofv3 counter runs a kernel of known traffic")
     args = ap.parse_args()
@@ -125,30 +126,46 @@ def main():
     step_bytes = wbytes + kv_per_pos * (T_start + T_end + 1) / 2.0
     step_gbs = step_bytes / (ms_per_step / 1e3) / 1e9
 
-    # per-kernel device times of single decode steps -> roofline of the dominant kernel
+    # per-kernel device times of single decode steps (device events attached to every dispatch on the library stream) ->
+    # roofline of every streaming kernel; the dominant kernel is the one with the largest share of the step
     nxt = gpu.sample()
     acc = {}
     n_prof = 5
+    symbols = {}
     for _ in range(n_prof):
-        for name, t in gpu.profile_decode(nxt):
+        prof = gpu.profile_decode(nxt)
+        syms = gpu.profile_symbols()
+        for (name, t), sym in zip(prof, syms):
             acc.setdefault(name, []).append(t)
-    dom = "gemm_ffn13" if "gemm_ffn13" in acc else max(acc, key=lambda k: sum(acc[k]))
-    dom_ms = float(np.mean(acc[dom]))
-    nW13 = 2 if cfg["act"] in (3, 4) else 1
-    dom_bytes = float(cfg["hidden"]) * cfg["ffn_dim"] * nW13 * es      # the weights one launch streams, once
-    dom_gbs = dom_bytes / (dom_ms / 1e3) / 1e9
+            symbols[name] = sym
     kernel_ms = {k: round(float(np.sum(v)) / n_prof, 4) for k, v in acc.items()}
-    # the attention kernel takes the largest share of the step at long contexts; its bytes grow with the context, so its
-    # figure is quoted at the context length of the profiled steps (keys and values of one layer, read once)
-    attn = None
-    if "attn_decode" in acc:
-        t_attn = T_end + 1 + (n_prof - 1) / 2.0
-        a_bytes = float(es) * B * cfg["n_kv_heads"] * d * 2 * t_attn
-        a_ms = float(np.mean(acc["attn_decode"]))
-        a_gbs = a_bytes / (a_ms / 1e3) / 1e9
-        attn = {"bound": "hbm", "achieved": round(a_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(a_gbs / HBM_PEAK_GBS, 4),
-                "traffic": None, "kernel": "attention (attn_decode)", "kv_len": t_attn, "bytes_per_launch": a_bytes, "avg_launch_ms": round(a_ms, 5),
-                "share_of_step": round(kernel_ms["attn_decode"] / sum(kernel_ms.values()), 3)}
+    step_sum = sum(kernel_ms.values())
+    t_attn = T_end + 1 + (n_prof - 1) / 2.0                  # mean KV length of the profiled steps
+    h, F, V, Hq, Hkv = cfg["hidden"], cfg["ffn_dim"], cfg["vocab"], cfg["n_heads"], cfg["n_kv_heads"]
+    nW13 = 2 if cfg["act"] in (3, 4) else 1
+    E = cfg.get("n_experts", 1)
+    # algorithmic bytes of one launch: the weights (or the cache) it must read once
+    launch_bytes = {
+        "gemm_qkv": float(h) * (Hq + 2 * Hkv) * d * es,
+        "attn_decode": float(es) * B * Hkv * d * 2 * t_attn,
+        "gemm_wo": float(h) * h * es,
+        "gemm_ffn13": float(h) * F * nW13 * es,
+        "gemm_ffn2": float(F) * h * es,
+        "gemm_head": float(h) * V * es,
+        "moe_gemm1": float(min(E, B * cfg.get("experts_per_token", 1))) * h * 4 * h * es,
+        "moe_gemm2": float(min(E, B * cfg.get("experts_per_token", 1))) * 4 * h * h * es,
+    }
+    roofline_all = {}
+    for name, ts in acc.items():
+        if name not in launch_bytes:
+            continue
+        ms_avg = float(np.mean(ts))
+        gbs = launch_bytes[name] / (ms_avg / 1e3) / 1e9
+        roofline_all[name] = {"kernel": symbols.get(name, ""), "bytes_per_launch": launch_bytes[name], "avg_launch_us": round(ms_avg * 1e3, 2),
+                              "launches_per_step": len(ts) // n_prof, "achieved_GBps": round(gbs, 1), "frac": round(gbs / HBM_PEAK_GBS, 4),
+                              "share_of_step": round(kernel_ms[name] / step_sum, 3)}
+    dom = max(roofline_all, key=lambda k: roofline_all[k]["share_of_step"])
+    dom_r = roofline_all[dom]
 
     # a plain copy of known size: the reference point for scaling FETCH_SIZE / WRITE_SIZE in counter runs
     if not args.no_copy_calibration:
@@ -161,10 +178,35 @@ def main():
         src.dispose()
         dst.dispose()
 
-    traffic = None
-    tpath = os.path.join(ROOT, "profiles", "decode_%s_ffn13_traffic.json" % args.config)
+    # HBM traffic per launch of the dominant kernel comes from hardware counters, which a separate rocprofv3 --pmc run of this
+    # script collects; the figure printed here is the one from the committed summary of that run (named beside it), never
+    # a value measured in this process
+    traffic, traffic_source = None, None
+    tpath = os.path.join(ROOT, "profiles", "decode_%s_%s_traffic.json" % (args.config, dom))
     if os.path.exists(tpath):
         traffic = json.load(open(tpath)).get("traffic_bytes_per_launch")
+        traffic_source = "profiles/" + os.path.basename(tpath)
+
+    structure = None
+    if args.structure_probe:
+        # the step's launch structure with pure streaming reads of the same bytes (see TSHip_StreamStructureProbe)
+        from seq2seqsharp_amd.gpt import stream_structure_probe
+        per_layer = [("gemm_qkv", 64), ("attn_decode", 4), ("gemm_wo", 32), ("gemm_ffn13", 128), ("gemm_ffn2", 90)]
+        pb, ak = [], []
+        for _ in range(cfg["n_layers"]):
+            for name, kib in per_layer:
+                pb.append(launch_bytes[name])
+                ak.append(kib)
+        pb.append(launch_bytes["gemm_head"])
+        ak.append(128)
+        ms3 = stream_structure_probe(pb, ak, repeats=6)
+        ms3_noact = stream_structure_probe(pb, [0] * len(ak), repeats=6)
+        structure = {"phases": len(pb), "bytes": float(sum(pb)),
+                     "one_launch_per_phase_ms": round(ms3[0], 4), "persistent_grid_barrier_ms": round(ms3[1], 4), "persistent_prefetch_before_barrier_ms": round(ms3[2], 4),
+                     "one_launch_per_phase_cache_resident_ms": round(ms3[3], 4),
+                     "without_shared_activation_reads": {"one_launch_per_phase_ms": round(ms3_noact[0], 4), "persistent_grid_barrier_ms": round(ms3_noact[1], 4),
+                                                         "persistent_prefetch_before_barrier_ms": round(ms3_noact[2], 4),
+                                                         "one_launch_per_phase_cache_resident_ms": round(ms3_noact[3], 4)}}
 
     out = {
         "metric": "decode tokens/s on 1 GPU (1B GQA fp16, batch 32)" if args.config == "cfg2_1b_gqa_f16" else "decode tokens/s on 1 GPU",
@@ -173,18 +215,19 @@ def main():
         "dtype": cfg["dtype"], "data": "synthetic",
         "config": {"workload": args.config, "batch": B, "prompt_len": Tp, "kv_len_start": T_start, "kv_len_end": T_end,
                    "sampling": "greedy", "rope_base": cfg["rope_base"]},
-        "roofline": {"bound": "hbm", "achieved": round(dom_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(dom_gbs / HBM_PEAK_GBS, 4), "traffic": traffic,
-                     "kernel": "skinny_gemm_f16_kernel<%d, EPI_ACT16> (%s)" % (1 if B <= 32 else 2 if B <= 64 else 4, dom),
-                     "bytes_per_launch": dom_bytes, "avg_launch_ms": round(dom_ms, 5),
-                     "share_of_step": round(kernel_ms[dom] / sum(kernel_ms.values()), 3)},
-        "roofline_attention": attn,
+        "roofline": {"bound": "hbm", "achieved": dom_r["achieved_GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": dom_r["frac"],
+                     "traffic": traffic, "traffic_source": traffic_source, "kernel": dom_r["kernel"], "launch": dom,
+                     "bytes_per_launch": dom_r["bytes_per_launch"], "avg_launch_ms": round(dom_r["avg_launch_us"] / 1e3, 5),
+                     "timing": "device events attached to each dispatch of 5 profiled steps (a rocprofv3 kernel trace of the graph replays reads about 5 % longer)",
+                     "kv_len": t_attn if dom == "attn_decode" else None, "share_of_step": dom_r["share_of_step"]},
+        "roofline_all": roofline_all,
         "whole_step": {"algorithmic_bytes": round(step_bytes), "achieved_GBps": round(step_gbs, 1),
                        "frac_of_hbm_peak": round(step_gbs / HBM_PEAK_GBS, 4), "host_wall_ms_per_step": round(wall / K * 1e3, 4)},
         "prefill": {"tokens_per_s": round(prefill_tok_s, 1), "seconds": round(t_prefill, 4),
                     "algorithmic_TFLOPs": round(prefill_tflops, 2),
                     "frac_of_fp16_mfma_peak": round(prefill_tflops / MFMA_FP16_PEAK_TFLOPS, 4) if cfg["dtype"] == "f16" else None},
         "kernel_ms_per_step": kernel_ms,
+        "launch_structure_probe": structure,
         "load_seconds": round(t_load, 1),
     }
     if not args.no_topp:

@@ -129,7 +129,11 @@ namespace TensorSharp.HIP
         [DllImport(Dll, CallingConvention = CC)] internal static extern int TSHip_GptSetSeqLen(IntPtr model, int batch, int len);
         [DllImport(Dll, CallingConvention = CC)] internal static extern int TSHip_GptGetMoeRouting(IntPtr model, int layer, float[] topIdx, float[] topVal, float[] probs);
         [DllImport(Dll, CallingConvention = CC)] internal static extern int TSHip_GptProfileDecode(IntPtr model, int[] hostIds, int batch, byte[] names, float[] ms, int nMax, out int n);
+        [DllImport(Dll, CallingConvention = CC)] internal static extern int TSHip_GptProfileSymbols(IntPtr model, byte[] symbols, int stride, int nMax, out int n);
         [DllImport(Dll, CallingConvention = CC)] internal static extern int TSHip_GptStepBytes(IntPtr model, int batch, out double weightBytes, out double kvBytes);
+
+        // ---- measurement aid ----
+        [DllImport(Dll, CallingConvention = CC)] internal static extern int TSHip_StreamStructureProbe(int nPhases, double[] phaseBytes, int[] actKib, int repeats, float[] msOut);
 
         internal static string LastError() => Marshal.PtrToStringAnsi(TSHip_GetLastError()) ?? string.Empty;
 

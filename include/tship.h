@@ -238,8 +238,19 @@ TSHIP_API int TSHip_GptGetMoeRouting(TSHipGpt* m, int layer, float* top_idx, flo
 /* per-kernel device times of one decode step (events around every launch on the library stream).
  * names: buffer of n_max entries of 48 chars; ms: n_max floats; *n receives the number of launches. */
 TSHIP_API int TSHip_GptProfileDecode(TSHipGpt* m, const int32_t* host_ids, int batch, char* names, float* ms, int n_max, int* n);
+/* the launched kernel symbols (demangled, as a profiler's kernel trace names them) of the step TSHip_GptProfileDecode timed
+ * last, in launch order: n_max entries of `stride` chars */
+TSHIP_API int TSHip_GptProfileSymbols(TSHipGpt* m, char* symbols, int stride, int n_max, int* n);
 /* algorithmic bytes one decode step moves at the current sequence length (weights once, compact KV once) */
 TSHIP_API int TSHip_GptStepBytes(TSHipGpt* m, int batch, double* weight_bytes, double* kv_bytes);
+
+/* Measurement aid (no counterpart in the reference): the cost of a decode step's launch structure on this machine with
+ * every kernel replaced by a pure streaming read.  phase_bytes[i] bytes are read once in phase i, every block also reads
+ * act_kib[i] KiB shared by all blocks, and every phase depends on the one before.  ms_out[0]: one launch per phase;
+ * ms_out[1]: one persistent kernel with a grid-wide barrier between phases (bounded polling); ms_out[2]: the same with
+ * the next phase's first loads requested before the barrier; ms_out[3]: one launch per phase with every phase reading
+ * the same region (cache resident where it fits).  Best of `repeats` runs each; ms_out holds four floats. */
+TSHIP_API int TSHip_StreamStructureProbe(int n_phases, const double* phase_bytes, const int* act_kib, int repeats, float* ms_out);
 
 #ifdef __cplusplus
 }

@@ -12,7 +12,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(HERE, "build")
 LIB = os.path.join(HERE, "libtship.so")
-SOURCES = ["tship_runtime.hip", "tship_gpt.hip", "tship_ops.hip"]
+SOURCES = ["tship_runtime.hip", "tship_gpt.hip", "tship_ops.hip", "tship_probe.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 # -packed-fp32-ops off: keep the compiler from forming packed fp32 instructions out of scalar float code
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden",

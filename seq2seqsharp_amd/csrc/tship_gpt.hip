@@ -15,6 +15,7 @@
 
 #include <cmath>
 #include <cstdlib>
+#include <cxxabi.h>
 #include <cstring>
 #include <map>
 #include <memory>
@@ -71,8 +72,19 @@ struct LayerW {
     DevBuf route;                          // this layer's routing at the last step: probs [Bpad][E], top values [Bpad][k], top indices [Bpad][k]
 };
 
+// demangled name of the device function behind a __global__ host stub (what a profiler's kernel trace shows)
+static std::string kernel_symbol(const void* host_fn) {
+    const char* raw = hipKernelNameRefByPtr(host_fn, stream());
+    if (!raw) { (void)hipGetLastError(); return std::string(); }
+    int status = 0;
+    char* dem = abi::__cxa_demangle(raw, nullptr, nullptr, &status);
+    std::string out = (status == 0 && dem) ? dem : raw;
+    std::free(dem);
+    return out;
+}
+
 struct Profiler {
-    std::vector<std::string> names;
+    std::vector<std::string> names, symbols;
     std::vector<hipEvent_t> ev0, ev1;
     ~Profiler() { for (auto e : ev0) (void)hipEventDestroy(e); for (auto e : ev1) (void)hipEventDestroy(e); }
 };
@@ -116,6 +128,7 @@ struct TSHipGpt {
     bool any_blocked = false;
     DevBuf blocked;                // one byte per token, non-zero = DecodingOptions.BlockedTokens (allocated with the model: graphs keep its address)
     int cur_batch = 0;
+    std::vector<std::string> last_symbols;      // launched symbols of the last profiled step, in launch order
     DevBuf beam_probs, beam_ids, beam_out, beam_uni, reorder_tmp, reorder_src;      // beam search: probabilities the picks consume, picks, gather temporaries
     Profiler* prof = nullptr;
 
@@ -131,6 +144,7 @@ static void launch(TSHipGpt* m, const char* name, void (*kernel)(KArgs...), dim3
         TSHIP_CHECK_HIP(hipEventCreate(&e0));
         TSHIP_CHECK_HIP(hipEventCreate(&e1));
         m->prof->names.push_back(name);
+        m->prof->symbols.push_back(kernel_symbol((const void*)kernel));
         m->prof->ev0.push_back(e0);
         m->prof->ev1.push_back(e1);
     }
@@ -154,6 +168,7 @@ static void launch_shm(TSHipGpt* m, const char* name, void (*kernel)(KArgs...), 
         TSHIP_CHECK_HIP(hipEventCreate(&e0));
         TSHIP_CHECK_HIP(hipEventCreate(&e1));
         m->prof->names.push_back(name);
+        m->prof->symbols.push_back(kernel_symbol((const void*)kernel));
         m->prof->ev0.push_back(e0);
         m->prof->ev1.push_back(e1);
     }
@@ -1482,6 +1497,7 @@ TSHIP_API int TSHip_GptProfileDecode(TSHipGpt* m, const int32_t* host_ids, int b
     TSHIP_CHECK_HIP(hipStreamSynchronize(stream()));
     m->cur_batch = batch;
     int cnt = (int)prof.names.size();
+    m->last_symbols = prof.symbols;
     *n = cnt;
     for (int i = 0; i < cnt && i < n_max; ++i) {
         float t = 0.0f;
@@ -1489,6 +1505,17 @@ TSHIP_API int TSHip_GptProfileDecode(TSHipGpt* m, const int32_t* host_ids, int b
         ms[i] = t;
         std::strncpy(names + (size_t)i * 48, prof.names[i].c_str(), 47);
         names[(size_t)i * 48 + 47] = 0;
+    }
+    TSHIP_END
+}
+
+TSHIP_API int TSHip_GptProfileSymbols(TSHipGpt* m, char* symbols, int stride, int n_max, int* n) {
+    TSHIP_BEGIN
+    TSHIP_REQUIRE(m && symbols && n && stride >= 2, "TSHip_GptProfileSymbols: bad argument");
+    *n = (int)m->last_symbols.size();
+    for (int i = 0; i < *n && i < n_max; ++i) {
+        std::strncpy(symbols + (size_t)i * stride, m->last_symbols[i].c_str(), stride - 1);
+        symbols[(size_t)i * stride + stride - 1] = 0;
     }
     TSHIP_END
 }

@@ -47,6 +47,8 @@ def _protos():
     L.TSHip_GptSetSeqLen.argtypes = [vp, C.c_int, C.c_int]
     L.TSHip_GptGetMoeRouting.argtypes = [vp, C.c_int, vp, vp, vp]
     L.TSHip_GptProfileDecode.argtypes = [vp, vp, C.c_int, vp, vp, C.c_int, C.POINTER(C.c_int)]
+    L.TSHip_GptProfileSymbols.argtypes = [vp, vp, C.c_int, C.c_int, C.POINTER(C.c_int)]
+    L.TSHip_StreamStructureProbe.argtypes = [C.c_int, vp, vp, C.c_int, vp]
     L.TSHip_GptStepBytes.argtypes = [vp, C.c_int, C.POINTER(C.c_double), C.POINTER(C.c_double)]
     L.TSHip_Synchronize.argtypes = []
     _proto_done = True
@@ -83,6 +85,15 @@ class HipGpt:
             check(L.TSHip_GptSetWeight(self.h, name.encode(), _ptr(w), w.ndim, sizes))
         check(L.TSHip_GptFinalize(self.h))
         self.batch = 0
+
+    @classmethod
+    def from_model_file(cls, path, max_batch, max_seq_len, dtype=None, device=0):
+        """A replica from a model file the reference saved (see seq2seqsharp_amd.model_file); returns (model, target vocabulary).
+        dtype None keeps the file's storage type: Float16 files run in fp16, as the reference demands AMP for them
+        (Models/Model.cs:267-270)."""
+        from . import model_file
+        cfg, weights, vocab = model_file.load_gpt(path, dtype)
+        return cls(cfg, weights, max_batch=max_batch, max_seq_len=max_seq_len, device=device), vocab
 
     def close(self):
         if getattr(self, "h", None):
@@ -283,8 +294,29 @@ class HipGpt:
             out.append((names.raw[i * 48:(i + 1) * 48].split(b"\0", 1)[0].decode(), float(ms[i])))
         return out
 
+    def profile_symbols(self, n_max=4096, stride=256):
+        """Launched kernel symbols of the step profile_decode timed last, in launch order."""
+        buf = C.create_string_buffer(stride * n_max)
+        n = C.c_int(0)
+        check(lib().TSHip_GptProfileSymbols(self.h, C.cast(buf, C.c_void_p), stride, n_max, C.byref(n)))
+        return [buf.raw[i * stride:(i + 1) * stride].split(b"\0", 1)[0].decode() for i in range(min(n.value, n_max))]
+
     def step_bytes(self, batch=None):
         """Algorithmic bytes of one decode step at the current length: (weight bytes, KV bytes)."""
         w, k = C.c_double(0), C.c_double(0)
         check(lib().TSHip_GptStepBytes(self.h, batch or self.batch, C.byref(w), C.byref(k)))
         return w.value, k.value
+
+
+def stream_structure_probe(phase_bytes, act_kib, repeats=5):
+    """TSHip_StreamStructureProbe: milliseconds of (one launch per phase, persistent kernel with grid barriers, the same with
+    the next phase's first loads requested before the barrier, one launch per phase with every phase reading the same
+    cache-resident region) for a chain of pure streaming phases."""
+    _protos()
+    pb = np.ascontiguousarray(phase_bytes, dtype=np.float64)
+    ak = np.ascontiguousarray(act_kib, dtype=np.int32)
+    assert pb.size == ak.size
+    out = np.zeros((4,), np.float32)
+    check(lib().TSHip_Init(0))
+    check(lib().TSHip_StreamStructureProbe(int(pb.size), _ptr(pb), _ptr(ak), int(repeats), _ptr(out)))
+    return [float(x) for x in out]
