@@ -180,9 +180,12 @@ static void launch_shm(TSHipGpt* m, const char* name, void (*kernel)(KArgs...), 
 // decode GEMM split-K: a block has NW wavefronts of 8 k-tiles each in flight; split K across blocks until one
 // pass covers the block's range (keeps partial-sum traffic small: K = 2048 needs no split at batch <= 32)
 static int pick_ks_f16(int NT, int KT, int BT) {
-    (void)NT;
     const int NW = BT <= 2 ? 8 : 4;
     int ks = (int)ceil_div(KT, NW * 8);
+    // few column tiles (small models): split further, up to one block per compute unit, while every wavefront keeps two
+    // k-tiles (32 blocks that each walk the whole K are bound by one block's latency, not by bandwidth)
+    const int fill = std::min(n_compute_units() / std::max(1, NT), KT / (NW * 2));
+    ks = std::max(ks, fill);
     return std::max(1, std::min(ks, 16));
 }
 static int pick_ks_f32(int N, int K) {
@@ -1093,6 +1096,7 @@ TSHIP_API int TSHip_GptReset(TSHipGpt* m) {
     if (m->tile_count.p) TSHIP_CHECK_HIP(hipMemsetAsync(m->tile_count.p, 0, m->tile_count.bytes, stream()));
     if (m->last_pos.p) TSHIP_CHECK_HIP(hipMemsetAsync(m->last_pos.p, 0xff, m->last_pos.bytes, stream()));      // -1: no token seen
     if (m->attn_count.p) TSHIP_CHECK_HIP(hipMemsetAsync(m->attn_count.p, 0, m->attn_count.bytes, stream()));
+    if (m->moe_ws.p) TSHIP_CHECK_HIP(hipMemsetAsync((char*)m->moe_ws.p + moe_layout(m, m->Bpad).counts, 0, (size_t)m->c.n_experts * sizeof(int), stream()));
     TSHIP_CHECK_HIP(hipStreamSynchronize(stream()));
     TSHIP_END
 }
@@ -1216,6 +1220,10 @@ static int generate_impl(TSHipGpt* m, int n_steps, int mode, float top_p, float 
         }
         if (!m->step_graph) {
             hipGraph_t graph = nullptr;
+            // the arrival counters of the one-launch reductions are zero between launches; a step that ended in an error
+            // may have left them otherwise, and every replay of the graph starts from what is there
+            if (m->tile_count.p) TSHIP_CHECK_HIP(hipMemsetAsync(m->tile_count.p, 0, m->tile_count.bytes, stream()));
+            if (m->attn_count.p) TSHIP_CHECK_HIP(hipMemsetAsync(m->attn_count.p, 0, m->attn_count.bytes, stream()));
             TSHIP_CHECK_HIP(hipStreamSynchronize(stream()));
             TSHIP_CHECK_HIP(hipStreamBeginCapture(stream(), hipStreamCaptureModeThreadLocal));
             const int saved_pos = m->pos;

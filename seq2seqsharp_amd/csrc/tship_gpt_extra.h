@@ -29,6 +29,8 @@ static MoeLayout moe_layout(TSHipGpt* m, long cap) {
 static void moe_alloc(TSHipGpt* m) {
     TSHIP_REQUIRE(m->c.hidden <= 4096, "TSHip_GptCreate: MoE layers support hidden up to 4096");
     m->moe_ws.alloc(moe_layout(m, m->Bpad).total);
+    // the experts' row counters start at zero and every layer's combine kernel leaves them so (the fp16 router adds to them)
+    TSHIP_CHECK_HIP(hipMemsetAsync(m->moe_ws.p, 0, m->moe_ws.bytes, stream()));
 }
 
 static void moe_get_routing(TSHipGpt* m, int layer, float* top_idx, float* top_val, float* probs) {
@@ -71,23 +73,26 @@ static void run_moe_ffn_impl(TSHipGpt* m, LayerW& L, int rows, const ResidNormAr
     r.router = L.router.as<float>(); r.router_b = L.router_b.as<float>(); r.E = E; r.k = k;
     r.xn32 = xn32; r.probs = probs; r.top_val = top_val; r.top_idx = top_idx;
     r.router_lds = ((long)E * h <= 16384) ? 1 : 0;
+    const long xg_stride = (long)Bp * m->ldh, mid_stride = (long)Bp * o.ld4h, y_stride = (long)Bp * o.ldy;
+    // fp16 decode steps: the router kernel also takes the row's place in its experts' batches and writes the row there
+    const bool fused_route = m->f16 && h % 4 == 0 && !batched && k <= 64;
+    if (fused_route) { r.xg16 = (half_t*)(base + o.xg); r.xg_estride = xg_stride; r.packed_kt = (int)(m->ldh / 16); r.counts = counts; r.slot = slot; r.max_rows = (int)Bp; }
     const unsigned router_shm = (unsigned)((2L * h + (r.router_lds ? (long)E * h : 0)) * sizeof(float));
-    if (m->f16) {      // tree-order sums: an fp16 model's routing input is not the reference's to the last bit anyway
-        if (h <= 1024) launch(m, "moe_router", moe_router_fast_kernel<4>, dim3(rows), dim3(256), r);
-        else if (h <= 2048) launch(m, "moe_router", moe_router_fast_kernel<8>, dim3(rows), dim3(256), r);
-        else launch(m, "moe_router", moe_router_fast_kernel<16>, dim3(rows), dim3(256), r);
+    if (m->f16 && h % 4 == 0) {      // tree-order sums: an fp16 model's routing input is not the reference's to the last bit anyway
+        if (h <= 1024) launch(m, "moe_router", moe_router_fast_kernel<1>, dim3(rows), dim3(256), r);
+        else if (h <= 2048) launch(m, "moe_router", moe_router_fast_kernel<2>, dim3(rows), dim3(256), r);
+        else launch(m, "moe_router", moe_router_fast_kernel<4>, dim3(rows), dim3(256), r);
     } else launch_shm(m, "moe_router", moe_router_kernel, dim3(rows), dim3(256), router_shm, r);
     // decode-sized batches: the gather kernel builds the lists itself (one launch less)
-    const bool fused_lists = !batched && (long)rows * k <= 1024;
+    const bool fused_lists = !batched && !fused_route && (long)rows * k <= 1024;
     if (batched) launch(m, "moe_lists", moe_lists_big_kernel, dim3(E), dim3(1024), (const float*)top_idx, rows, k, (int)Bp, counts, lists, slot);
-    else if (!fused_lists) launch_shm(m, "moe_lists", moe_lists_kernel, dim3(1), dim3(64), (unsigned)(rows * k * sizeof(int)), (const float*)top_idx, rows, k, E, (int)Bp, counts, lists, slot);
+    else if (!fused_lists && !fused_route) launch_shm(m, "moe_lists", moe_lists_kernel, dim3(1), dim3(64), (unsigned)(rows * k * sizeof(int)), (const float*)top_idx, rows, k, E, (int)Bp, counts, lists, slot);
     std::vector<int> n_e(E, rows);
     if (batched) {
         TSHIP_CHECK_HIP(hipMemcpyAsync(n_e.data(), counts, E * sizeof(int), hipMemcpyDeviceToHost, stream()));
         TSHIP_CHECK_HIP(hipStreamSynchronize(stream()));
         for (int e = 0; e < E; ++e) TSHIP_REQUIRE(n_e[e] >= 0 && n_e[e] <= rows, "internal: expert row count out of range");
     }
-    const long xg_stride = (long)Bp * m->ldh, mid_stride = (long)Bp * o.ld4h, y_stride = (long)Bp * o.ldy;
     if (m->f16 && batched) {
         half_t* xg = (half_t*)(base + o.xg); half_t* mid = (half_t*)(base + o.mid);
         launch(m, "moe_gather", moe_gather_kernel<half_t>, dim3(rows, E), dim3(256), (const float*)xn32, h, (const int*)counts, (const int*)lists, (int)Bp, xg,
@@ -103,7 +108,8 @@ static void run_moe_ffn_impl(TSHipGpt* m, LayerW& L, int rows, const ResidNormAr
         }
     } else if (m->f16) {
         half_t* xg = (half_t*)(base + o.xg); half_t* mid = (half_t*)(base + o.mid);
-        if (fused_lists) launch(m, "moe_gather", moe_gather_lists_kernel<half_t>, dim3(rows, E), dim3(256), (const float*)top_idx, rows, k, (const float*)xn32, h,
+        if (fused_route) {}
+        else if (fused_lists) launch(m, "moe_gather", moe_gather_lists_kernel<half_t>, dim3(rows, E), dim3(256), (const float*)top_idx, rows, k, (const float*)xn32, h,
                                 counts, lists, slot, (int)Bp, xg, m->ldh, xg_stride, (int)(m->ldh / 16));
         else launch(m, "moe_gather", moe_gather_kernel<half_t>, dim3(rows, E), dim3(256), (const float*)xn32, h, (const int*)counts, (const int*)lists, (int)Bp, xg,
                m->ldh, xg_stride, (int)(m->ldh / 16));
@@ -150,10 +156,11 @@ static void run_moe_ffn_impl(TSHipGpt* m, LayerW& L, int rows, const ResidNormAr
     if (next) {
         ResidNormArgs a = *next;
         a.moe_y = y; a.moe_ldy = o.ldy; a.moe_estride = y_stride; a.moe_probs = probs; a.moe_top = top_idx; a.moe_slot = slot; a.moe_k = k; a.moe_E = E;
+        a.moe_clear_counts = fused_route ? counts : nullptr;
         run_resid_norm(m, "moe_combine_norm", rows, a);
     } else {
         launch(m, "moe_combine", moe_combine_kernel, dim3(rows), dim3(256), pre.x, pre.ldx, h, (const float*)y, o.ldy, y_stride, (const float*)probs,
-               (const float*)top_idx, (const int*)slot, k, E);
+               (const float*)top_idx, (const int*)slot, k, E, fused_route ? counts : (int*)nullptr);
     }
     if (batched && last_rows) {
         // what TSHip_GptGetMoeRouting reports after a prefill: the routing of every sequence's last position

@@ -1046,6 +1046,7 @@ struct ResidNormArgs {
     // (MoEFeedForward.cs:167-178; IndexSelectGrad, TensorApplyCPU.cs:1336-1356).  y[e][slot][col], slot[row * k + j] =
     // place of the row in the list of its j-th expert
     const float* moe_y; long moe_ldy; long moe_estride; const float* moe_probs; const float* moe_top; const int* moe_slot; int moe_k; int moe_E;
+    int* moe_clear_counts;  // optional: block 0 clears the experts' row counters for the next router launch
 };
 
 template <typename AT, int NPT>   // NPT * 256 >= hidden
@@ -1057,7 +1058,22 @@ __global__ __launch_bounds__(256) void resid_norm_kernel(ResidNormArgs a) {
     const float* __restrict__ xin = a.x + xr * a.ldx;
     float v[NPT];
     long erow = a.ids ? (long)a.ids[r] : 0;
-    // all loads first (independent), then the arithmetic, then the stores
+    // all loads first (independent), then the arithmetic, then the stores; the MoE choices head the longest chain of
+    // dependent loads (choice -> slot -> expert output), so they are requested before anything else
+    constexpr int MAXK = 4;
+    int te[MAXK], ts[MAXK];
+#pragma unroll
+    for (int j = 0; j < MAXK; ++j) {
+        te[j] = (a.moe_y && j < a.moe_k && a.moe_k <= MAXK) ? (int)a.moe_top[xr * a.moe_k + j] : -1;
+        ts[j] = (a.moe_y && j < a.moe_k && a.moe_k <= MAXK) ? a.moe_slot[xr * a.moe_k + j] : 0;
+    }
+    float gm[NPT], bt[NPT];
+#pragma unroll
+    for (int i = 0; i < NPT; ++i) {
+        const int c = t + i * 256;
+        gm[i] = (a.xn && c < a.h) ? a.gamma[c] : 0.0f;
+        bt[i] = (a.xn && a.beta && c < a.h) ? a.beta[c] : 0.0f;
+    }
 #pragma unroll
     for (int i = 0; i < NPT; ++i) {
         int c = t + i * 256;
@@ -1110,15 +1126,10 @@ __global__ __launch_bounds__(256) void resid_norm_kernel(ResidNormArgs a) {
     }
     if (a.moe_y) {
 #pragma clang fp contract(off)
-        constexpr int MAXK = 4;
+        if (a.moe_clear_counts && blockIdx.x == 0 && t < a.moe_E) a.moe_clear_counts[t] = 0;
         if (a.moe_k <= MAXK) {
             // the row's choices, their slots and probabilities once; then every expert output at once; added in expert order
-            int te[MAXK], ts[MAXK]; float tp[MAXK], yv[MAXK][NPT];
-#pragma unroll
-            for (int j = 0; j < MAXK; ++j) {
-                te[j] = j < a.moe_k ? (int)a.moe_top[xr * a.moe_k + j] : -1;
-                ts[j] = j < a.moe_k ? a.moe_slot[xr * a.moe_k + j] : 0;
-            }
+            float tp[MAXK], yv[MAXK][NPT];
 #pragma unroll
             for (int j = 0; j < MAXK; ++j) {
                 tp[j] = te[j] >= 0 ? a.moe_probs[xr * a.moe_E + te[j]] : 0.0f;
@@ -1176,8 +1187,8 @@ __global__ __launch_bounds__(256) void resid_norm_kernel(ResidNormArgs a) {
         for (int i = 0; i < NPT; ++i) {
             int c = t + i * 256;
             if (c < a.h) {
-                float y = a.gamma[c] * (v[i] / rms);
-                if (a.beta) y += a.beta[c];
+                float y = gm[i] * (v[i] / rms);
+                if (a.beta) y += bt[i];
                 if (a.xn_kt > 0) ((AT*)a.xn)[xpack_index(r, c, a.xn_kt)] = (AT)y; else out[c] = (AT)y;
             }
         }
@@ -1194,8 +1205,8 @@ __global__ __launch_bounds__(256) void resid_norm_kernel(ResidNormArgs a) {
         for (int i = 0; i < NPT; ++i) {
             int c = t + i * 256;
             if (c < a.h) {
-                float y = a.gamma[c] * ((v[i] - mean) / sigma);
-                if (a.beta) y += a.beta[c];
+                float y = gm[i] * ((v[i] - mean) / sigma);
+                if (a.beta) y += bt[i];
                 if (a.xn_kt > 0) ((AT*)a.xn)[xpack_index(r, c, a.xn_kt)] = (AT)y; else out[c] = (AT)y;
             }
         }

@@ -20,6 +20,9 @@ struct MoeRouterArgs {
     const float* router; const float* router_b; int E; int k;
     float* xn32; float* probs; float* top_val; float* top_idx;
     int router_lds;      // 1: the launch reserved LDS for the router matrix
+    // fast kernel only, when xg16 is set: the row's place in each chosen expert's batch is taken from the expert's counter
+    // and the normalised row is written there in fp16 (fragment packed), so that no list or gather launch follows
+    half_t* xg16; long xg_estride; int packed_kt; int* counts; int* slot; int max_rows;
 };
 
 __device__ __forceinline__ float tree8(float v) {
@@ -203,103 +206,234 @@ __global__ __launch_bounds__(256) void moe_router_kernel(MoeRouterArgs a) {
 // 1024-step chains of the kernel above) buys nothing there; that kernel remains the one fp32 models use, where routing
 // indices are bit-exact.  Same outputs: x updated with the pending attention output, LayerNorm in fp32, router logits
 // + (-65000), softmax with the exponentials evaluated in double, TopK by the reference's insertion rule.
-template <int NPT>      // NPT * 256 >= hidden
+// v of lane `l`, the same l in every lane (a register read, no trip through the cross-lane network)
+__device__ __forceinline__ float lane_value(float v, int l) { return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), l)); }
+
+// The reference's TopK (TensorApplyCPU.cs TopK: keep the K largest by insertion, walking the row once) with the row spread
+// over the lanes of a wavefront (lane e holds element e) and the K kept values in registers of every lane.  An element
+// equal to the smallest kept value still enters (and takes the last place); an element equal to a larger kept value goes
+// behind it.  pos = the number of kept values, among the first K - 1, that the element does not exceed.
+template <int K>
+__device__ __forceinline__ void topk_by_insertion(float p, int E, float (&ov)[4], float (&oi)[4]) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) { ov[i] = -1.70141e+38f; oi[i] = -1.70141e+38f; }
+    for (int e = 0; e < E; ++e) {
+        const float data = lane_value(p, e);
+        if (data < ov[K - 1]) continue;
+        int pos = 0;
+#pragma unroll
+        for (int j = 0; j < K - 1; ++j) pos += (data > ov[j]) ? 0 : 1;
+#pragma unroll
+        for (int i = K - 1; i >= 0; --i) {
+            if (i > pos) { if (i >= 1) { ov[i] = ov[i > 0 ? i - 1 : 0]; oi[i] = oi[i > 0 ? i - 1 : 0]; } }
+            else if (i == pos) { ov[i] = data; oi[i] = (float)e; }
+        }
+    }
+}
+
+// Sums of eight values per lane over the wavefront with ten cross-lane moves instead of forty-eight: every step halves the
+// number of values a lane carries (the upper half of the lanes keeps the upper half of the values), and once one value is
+// left three more steps finish it.  Afterwards lane L holds the total of value ((L >> 5) & 1) * 4 + ((L >> 4) & 1) * 2 +
+// ((L >> 3) & 1).
+__device__ __forceinline__ float wave_sum8(const float (&acc)[8], int lane) {
+    float r4[4], r2[2];
+    const bool h5 = lane & 32, h4 = lane & 16, h3 = lane & 8;
+#pragma unroll
+    for (int u = 0; u < 4; ++u) { const float mine = h5 ? acc[u + 4] : acc[u], other = h5 ? acc[u] : acc[u + 4]; r4[u] = mine + __shfl_xor(other, 32, 64); }
+#pragma unroll
+    for (int u = 0; u < 2; ++u) { const float mine = h4 ? r4[u + 2] : r4[u], other = h4 ? r4[u] : r4[u + 2]; r2[u] = mine + __shfl_xor(other, 16, 64); }
+    float r1 = (h3 ? r2[1] : r2[0]) + __shfl_xor(h3 ? r2[0] : r2[1], 8, 64);
+    r1 += __shfl_xor(r1, 4, 64);
+    r1 += __shfl_xor(r1, 2, 64);
+    r1 += __shfl_xor(r1, 1, 64);
+    return r1;
+}
+
+// Thread t works on the column groups g = t, t + 256, ... of four neighbouring columns (16-byte requests; a row of 1024
+// columns is one request per tensor and thread), so hidden must be a multiple of four.
+template <int NG>      // NG * 1024 >= hidden
 __global__ __launch_bounds__(256) void moe_router_fast_kernel(MoeRouterArgs a) {
     constexpr int MAXE = 64;
     __shared__ float sred[4];
     __shared__ float swe[4][MAXE];
     __shared__ float sr[MAXE];
     __shared__ float s_ov[MAXE], s_oi[MAXE];
+    __shared__ int s_slot[MAXE];
     const int r = blockIdx.x, t = threadIdx.x, h = a.h, E = a.E, lane = t & 63, w = t >> 6;
-    float v[NPT], g[NPT], bt[NPT];
+    floatx4 v[NG], g[NG], bt[NG];
+    floatx4 wv0[NG][4][2];       // router weights of experts 0-7 for the thread's columns (E == 8: 32 bytes per column)
+    const bool e8 = E == 8;
+#pragma unroll
+    for (int i = 0; i < NG; ++i) {
+        const int c = 4 * (t + i * 256);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            if (e8 && c < h) {
+                const floatx4* src = (const floatx4*)(a.router + (long)(c + q) * 8);
+                wv0[i][q][0] = src[0]; wv0[i][q][1] = src[1];
+            } else {
+#pragma unroll
+                for (int u = 0; u < 8; ++u) wv0[i][q][u >> 2][u & 3] = (c < h && u < E) ? a.router[(long)(c + q) * E + u] : 0.0f;
+            }
+        }
+    }
     {
-        float xv[NPT], bv[NPT], pv[NPT][4];
+        floatx4 xv[NG], bv[NG], pv[NG][8];       // up to eight split-K partials requested at once
+        const floatx4 zero4 = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-        for (int i = 0; i < NPT; ++i) {
-            const int c = t + i * 256; const bool ok = c < h;
-            xv[i] = ok ? a.x[(long)r * a.ldx + c] : 0.0f;
-            bv[i] = (ok && a.part) ? a.bias[c] : 0.0f;
+        for (int i = 0; i < NG; ++i) {
+            const int c = 4 * (t + i * 256); const bool ok = c < h;
+            xv[i] = ok ? *(const floatx4*)(a.x + (long)r * a.ldx + c) : zero4;
+            bv[i] = (ok && a.part) ? *(const floatx4*)(a.bias + c) : zero4;
 #pragma unroll
-            for (int k = 0; k < 4; ++k) pv[i][k] = (ok && a.part && k < a.KS) ? a.part[k * a.split_stride + (long)r * a.ld_part + c] : 0.0f;
-            g[i] = ok ? a.gamma[c] : 0.0f; bt[i] = ok ? a.beta[c] : 0.0f;
+            for (int k = 0; k < 8; ++k) pv[i][k] = (ok && a.part && k < a.KS) ? *(const floatx4*)(a.part + k * a.split_stride + (long)r * a.ld_part + c) : zero4;
+            g[i] = ok ? *(const floatx4*)(a.gamma + c) : zero4; bt[i] = ok ? *(const floatx4*)(a.beta + c) : zero4;
         }
 #pragma unroll
-        for (int i = 0; i < NPT; ++i) {
-            const int c = t + i * 256;
+        for (int i = 0; i < NG; ++i) {
+            const int c = 4 * (t + i * 256);
             v[i] = xv[i];
             if (a.part && c < h) {
-                float s = pv[i][0];
+                floatx4 s = pv[i][0];
 #pragma unroll
-                for (int k = 1; k < 4; ++k) if (k < a.KS) s += pv[i][k];
-                for (int k = 4; k < a.KS; ++k) s += a.part[k * a.split_stride + (long)r * a.ld_part + c];
+                for (int k = 1; k < 8; ++k) if (k < a.KS) s += pv[i][k];
+                for (int k = 8; k < a.KS; ++k) s += *(const floatx4*)(a.part + k * a.split_stride + (long)r * a.ld_part + c);
                 v[i] = (s + bv[i]) + xv[i];
-                a.x[(long)r * a.ldx + c] = v[i];
+                *(floatx4*)(a.x + (long)r * a.ldx + c) = v[i];
             }
         }
     }
     float sum = 0.0f;
 #pragma unroll
-    for (int i = 0; i < NPT; ++i) sum += v[i];                 // (columns beyond h hold zeros)
+    for (int i = 0; i < NG; ++i) sum += (v[i][0] + v[i][1]) + (v[i][2] + v[i][3]);          // (columns beyond h hold zeros)
     const float mean = block_sum_256(sum, sred) / (float)h;
     float d2 = 0.0f;
 #pragma unroll
-    for (int i = 0; i < NPT; ++i) { const int c = t + i * 256; if (c < h) { const float d = v[i] - mean; d2 += d * d; } }
-    const float sigma = sqrtf(a.eps + block_sum_256(d2, sred) / (float)h);
-    float y[NPT];
+    for (int i = 0; i < NG; ++i) {
+        if (4 * (t + i * 256) < h) {
 #pragma unroll
-    for (int i = 0; i < NPT; ++i) {
-        const int c = t + i * 256;
-        y[i] = 0.0f;
-        if (c < h) { y[i] = g[i] * ((v[i] - mean) / sigma) + bt[i]; a.xn32[(long)r * h + c] = y[i]; }
+            for (int q = 0; q < 4; ++q) { const float d = v[i][q] - mean; d2 += d * d; }
+        }
+    }
+    const float sigma = sqrtf(a.eps + block_sum_256(d2, sred) / (float)h);
+    floatx4 y[NG];
+#pragma unroll
+    for (int i = 0; i < NG; ++i) {
+        const int c = 4 * (t + i * 256);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) y[i][q] = c < h ? g[i][q] * ((v[i][q] - mean) / sigma) + bt[i][q] : 0.0f;
+        if (c < h && !a.xg16) *(floatx4*)(a.xn32 + (long)r * h + c) = y[i];
     }
     // router logits: every thread's columns against all experts, then a tree over the block
     for (int e0 = 0; e0 < E; e0 += 8) {
-        float acc[8], wv[NPT][8];
-#pragma unroll
-        for (int i = 0; i < NPT; ++i) {
-            const int c = t + i * 256;
-#pragma unroll
-            for (int u = 0; u < 8; ++u) wv[i][u] = (c < h && e0 + u < E) ? a.router[(long)c * E + e0 + u] : 0.0f;
-        }
+        float acc[8];
 #pragma unroll
         for (int u = 0; u < 8; ++u) acc[u] = 0.0f;
 #pragma unroll
-        for (int i = 0; i < NPT; ++i) {
+        for (int i = 0; i < NG; ++i) {
+            const int c = 4 * (t + i * 256);
 #pragma unroll
-            for (int u = 0; u < 8; ++u) acc[u] += y[i] * wv[i][u];
-        }
+            for (int q = 0; q < 4; ++q) {
 #pragma unroll
-        for (int u = 0; u < 8; ++u) { acc[u] = wave_sum(acc[u]); if (lane == 0 && e0 + u < E) swe[w][e0 + u] = acc[u]; }
-    }
-    __syncthreads();
-    if (t < 64) {
-        float lg = -INFINITY;
-        if (t < E) lg = ((((swe[0][t] + swe[1][t]) + swe[2][t]) + swe[3][t]) + a.router_b[t]) + (-65000.0f);
-        const float mx = wave_max(lg);
-        const float ex = t < E ? (float)exp((double)(lg - mx)) : 0.0f;
-        if (t < E) sr[t] = ex;
-    }
-    __syncthreads();
-    if (t == 0) {
-        const int k = a.k;
-        float s = 0.0f;
-        for (int e = 0; e < E; ++e) s += sr[e];
-        float* pr = a.probs + (long)r * E;
-        for (int e = 0; e < E; ++e) { sr[e] = sr[e] / s; pr[e] = sr[e]; }
-        // (the insertion works on LDS copies: on the global arrays every step would be a memory round trip)
-        float* ov = s_ov; float* oi = s_oi;
-        for (int i = 0; i < k; ++i) { ov[i] = -1.70141e+38f; oi[i] = -1.70141e+38f; }
-        for (int e = 0; e < E; ++e) {
-            float data = sr[e];
-            if (data < ov[k - 1]) continue;
-            int j = k - 2;
-            for (; j >= 0; --j) {
-                if (data > ov[j]) { ov[j + 1] = ov[j]; oi[j + 1] = oi[j]; }
-                else { ov[j + 1] = data; oi[j + 1] = (float)e; break; }
+                for (int u = 0; u < 8; ++u) {
+                    const float wgt = e0 == 0 ? wv0[i][q][u >> 2][u & 3] : ((c < h && e0 + u < E) ? a.router[(long)(c + q) * E + e0 + u] : 0.0f);
+                    acc[u] += y[i][q] * wgt;
+                }
             }
-            if (j < 0) { ov[0] = data; oi[0] = (float)e; }
         }
-        for (int i = 0; i < k; ++i) { a.top_val[(long)r * k + i] = ov[i]; a.top_idx[(long)r * k + i] = oi[i]; }
+        const float tot = wave_sum8(acc, lane);
+        const int eu = ((lane >> 5) & 1) * 4 + ((lane >> 4) & 1) * 2 + ((lane >> 3) & 1);
+        if ((lane & 7) == 0 && e0 + eu < E) swe[w][e0 + eu] = tot;
+    }
+    __syncthreads();
+    if (a.k <= 4) {
+        // softmax and TopK inside the first wavefront, in registers: lane e holds expert e, the serial steps of the reference
+        // (the sum in expert order, the insertion rule) run on all lanes alike with the values read across lanes
+        if (t < 64) {
+            float lg = -INFINITY;
+            if (t < E) lg = ((((swe[0][t] + swe[1][t]) + swe[2][t]) + swe[3][t]) + a.router_b[t]) + (-65000.0f);
+            const float mx = wave_max(lg);
+            const float ex = t < E ? (float)exp((double)(lg - mx)) : 0.0f;
+            float ssum = 0.0f;
+            for (int e = 0; e < E; ++e) ssum += lane_value(ex, e);
+            const float p = ex / ssum;
+            if (t < E) a.probs[(long)r * E + t] = p;
+            float ov[4], oi[4];
+            switch (a.k) {
+                case 1: topk_by_insertion<1>(p, E, ov, oi); break;
+                case 2: topk_by_insertion<2>(p, E, ov, oi); break;
+                case 3: topk_by_insertion<3>(p, E, ov, oi); break;
+                default: topk_by_insertion<4>(p, E, ov, oi); break;
+            }
+            if (t == 0) {
+                const int k = a.k;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) if (i < k) { a.top_val[(long)r * k + i] = ov[i]; a.top_idx[(long)r * k + i] = oi[i]; s_oi[i] = oi[i]; }
+                if (a.xg16) {
+                    // The row's place in each chosen expert's batch: the order in which rows arrive differs from run to run,
+                    // the results do not (a row's product does not depend on its place, and the combine step adds a token's
+                    // experts in expert order whatever their places).  The counters are zero on entry: the combine kernel
+                    // clears them.  All requests go out before the first answer is needed.
+                    int sl[4];
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) sl[i] = i < k ? (int)__hip_atomic_fetch_add(a.counts + (int)oi[i], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0;
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) if (i < k) { s_slot[i] = sl[i]; a.slot[(long)r * k + i] = sl[i]; }
+                }
+            }
+        }
+    } else {
+        if (t < 64) {
+            float lg = -INFINITY;
+            if (t < E) lg = ((((swe[0][t] + swe[1][t]) + swe[2][t]) + swe[3][t]) + a.router_b[t]) + (-65000.0f);
+            const float mx = wave_max(lg);
+            const float ex = t < E ? (float)exp((double)(lg - mx)) : 0.0f;
+            if (t < E) sr[t] = ex;
+        }
+        __syncthreads();
+        if (t == 0) {
+            const int k = a.k;
+            float s = 0.0f;
+            for (int e = 0; e < E; ++e) s += sr[e];
+            float* pr = a.probs + (long)r * E;
+            for (int e = 0; e < E; ++e) { sr[e] = sr[e] / s; pr[e] = sr[e]; }
+            // (the insertion works on LDS copies: on the global arrays every step would be a memory round trip)
+            float* ov = s_ov; float* oi = s_oi;
+            for (int i = 0; i < k; ++i) { ov[i] = -1.70141e+38f; oi[i] = -1.70141e+38f; }
+            for (int e = 0; e < E; ++e) {
+                float data = sr[e];
+                if (data < ov[k - 1]) continue;
+                int j = k - 2;
+                for (; j >= 0; --j) {
+                    if (data > ov[j]) { ov[j + 1] = ov[j]; oi[j + 1] = oi[j]; }
+                    else { ov[j + 1] = data; oi[j + 1] = (float)e; break; }
+                }
+                if (j < 0) { ov[0] = data; oi[0] = (float)e; }
+            }
+            for (int i = 0; i < k; ++i) { a.top_val[(long)r * k + i] = ov[i]; a.top_idx[(long)r * k + i] = oi[i]; }
+            if (a.xg16) {
+                for (int i = 0; i < k; ++i) {
+                    const int sl = (int)__hip_atomic_fetch_add(a.counts + (int)oi[i], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    s_slot[i] = sl; a.slot[(long)r * k + i] = sl;
+                }
+            }
+        }
+    }
+    if (a.xg16) {
+        __syncthreads();
+        for (int i = 0; i < a.k; ++i) {
+            half_t* dst = a.xg16 + (long)(int)s_oi[i] * a.xg_estride;
+            const int sl = s_slot[i];
+            if (sl >= a.max_rows) continue;
+#pragma unroll
+            for (int q = 0; q < NG; ++q) {
+                const int c = 4 * (t + q * 256);
+                if (c < h) {
+                    half4 hv = {(half_t)y[q][0], (half_t)y[q][1], (half_t)y[q][2], (half_t)y[q][3]};
+                    *(half4*)(dst + xpack_index(sl, c, a.packed_kt)) = hv;       // (four neighbouring columns are neighbours in a fragment)
+                }
+            }
+        }
     }
 }
 
@@ -412,9 +546,10 @@ __global__ __launch_bounds__(256) void moe_gather_lists_kernel(const float* __re
 // (MoEFeedForward.cs:167-178; IndexSelectGrad, TensorApplyCPU.cs:1336-1356): one block per token
 __global__ __launch_bounds__(256) void moe_combine_kernel(float* __restrict__ x, long ldx, int h, const float* __restrict__ y, long ldy, long estride,
                                                            const float* __restrict__ probs, const float* __restrict__ top_idx, const int* __restrict__ slot,
-                                                           int k, int E) {
+                                                           int k, int E, int* __restrict__ clear_counts) {
 #pragma clang fp contract(off)
     const int i = blockIdx.x;
+    if (clear_counts && i == 0 && (int)threadIdx.x < E) clear_counts[threadIdx.x] = 0;       // for the next router launch
     for (int c = threadIdx.x; c < h; c += 256) {
         float out = 0.0f;
         for (int e = 0; e < E; ++e)
