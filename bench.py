@@ -181,10 +181,12 @@ def main():
     # HBM traffic per launch of the dominant kernel comes from hardware counters, which a separate rocprofv3 --pmc run of this
     # script collects; the figure printed here is the one from the committed summary of that run (named beside it), never
     # a value measured in this process
-    traffic, traffic_source = None, None
+    traffic, traffic_source, traffic_kv_len = None, None, None
     tpath = os.path.join(ROOT, "profiles", "decode_%s_%s_traffic.json" % (args.config, dom))
     if os.path.exists(tpath):
-        traffic = json.load(open(tpath)).get("traffic_bytes_per_launch")
+        tj = json.load(open(tpath))
+        traffic = tj.get("traffic_bytes_per_launch")
+        traffic_kv_len = tj.get("kv_len")                    # attention: the KV length of the counter run (its bytes grow with it)
         traffic_source = "profiles/" + os.path.basename(tpath)
 
     structure = None
@@ -216,7 +218,7 @@ def main():
         "config": {"workload": args.config, "batch": B, "prompt_len": Tp, "kv_len_start": T_start, "kv_len_end": T_end,
                    "sampling": "greedy", "rope_base": cfg["rope_base"]},
         "roofline": {"bound": "hbm", "achieved": dom_r["achieved_GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": dom_r["frac"],
-                     "traffic": traffic, "traffic_source": traffic_source, "kernel": dom_r["kernel"], "launch": dom,
+                     "traffic": traffic, "traffic_source": traffic_source, "traffic_kv_len": traffic_kv_len, "kernel": dom_r["kernel"], "launch": dom,
                      "bytes_per_launch": dom_r["bytes_per_launch"], "avg_launch_ms": round(dom_r["avg_launch_us"] / 1e3, 5),
                      "timing": "device events attached to each dispatch of 5 profiled steps (a rocprofv3 kernel trace of the graph replays reads about 5 % longer)",
                      "kv_len": t_attn if dom == "attn_decode" else None, "share_of_step": dom_r["share_of_step"]},
