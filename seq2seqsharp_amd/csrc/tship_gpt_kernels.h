@@ -360,6 +360,21 @@ __global__ __launch_bounds__(NW * 64) void skinny_gemm_f16_kernel(SkinnyArgs a) 
         const float rinv = a.ssq ? srinv[b] : 1.0f;
         if (EPI == EPI_SPLIT_TAIL) {
             // publish this block's partial sums, then find out whether it is the last of its column tile
+            //
+            // Memory model: the C++ model would want a release on the counter add and an acquire in the last block; that
+            // fence costs a write-back of the whole L2 here (measured > 10 us).  What this code relies on instead is the
+            // instruction sequence itself, on gfx950 (the build refuses other targets, tship_internal.h):
+            //   1. the data stores are agent-scope atomic stores: global_store_dword ... sc1, written through to the point of
+            //      coherence shared by the XCDs' L2s;
+            //   2. s_waitcnt vmcnt(0) (the asm below; "memory" keeps the compiler from moving accesses across it): vmcnt
+            //      counts stores on this target, so every store of this wavefront has been acknowledged there;
+            //   3. the block barrier: all wavefronts of the block are past (2);
+            //   4. one thread's agent-scope atomic add on the tile's counter: performed at that same point of coherence,
+            //      after this block's data;
+            //   5. the last arriver (control dependent on the counter's value, which no wavefront has before its
+            //      s_waitcnt for the returned data) reads all partials with agent-scope atomic loads (... sc1: they do
+            //      not hit stale lines of its own L2).
+            // The counter is back at zero when the launch ends, and is cleared by TSHip_GptReset and before graph capture.
             __shared__ int s_last;
             // (exchange layout [split][tile][2][512 threads]: a wavefront's store is 256 contiguous bytes)
             float* o = a.out + ((long)ks * a.NT + nt) * 1024 + threadIdx.x;
@@ -1926,6 +1941,8 @@ __global__ __launch_bounds__(D == 128 ? 256 : 512) void attn_mfma_kernel(AttnArg
                 __hip_atomic_store(mine + NCOL * D + NCOL + col, L, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             }
         }
+        // (same publication protocol as the split-K projections' exchange, whose comment lists the instruction sequence it
+        // rests on: write-through atomic stores, vmcnt(0), block barrier, atomic add, atomic loads in the last arriver)
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");            // the stores have reached the point of coherence
         __syncthreads();
         if (t == 0) s_last = __hip_atomic_fetch_add(a.xcount + pair, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == a.S - 1;

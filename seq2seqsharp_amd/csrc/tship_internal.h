@@ -63,6 +63,9 @@ void noalloc_device_setup(int device);   // tship_ops.hip: address of the fixed 
 int n_compute_units();
 
 typedef _Float16 half_t;
+#if defined(__HIP_DEVICE_COMPILE__) && !defined(__gfx950__)
+#error "libtship's device code is written for gfx950 only: MFMA shapes, direct-to-LDS loads, and cross-block exchanges whose ordering rests on this target's instruction behaviour"
+#endif
 typedef half_t half8 __attribute__((ext_vector_type(8)));
 typedef half_t half4 __attribute__((ext_vector_type(4)));
 typedef half_t half2v __attribute__((ext_vector_type(2)));
