@@ -227,6 +227,22 @@ def sigmoid(result, src):
     return _unary(SIGMOID, result, src)
 
 
+def neg(result, src):
+    return _unary(NEG, result, src)
+
+
+def tanh(result, src):
+    return _unary(TANH, result, src)
+
+
+def sqrt(result, src):
+    return _unary(SQRT, result, src)
+
+
+def abs(result, src):                                    # "abs" (the op registry's name)
+    return _unary(ABS, result, src)
+
+
 def buildtrimask(result, value, masked_value):           # "buildtrimask"
     check(_p().TSHip_BuildTriMask(_d(result), float(value), float(masked_value)))
     return result

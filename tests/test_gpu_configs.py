@@ -255,3 +255,32 @@ def test_wide_model_more_than_eight_qkv_splits(G, oracle):
     _, gpu, out, _ = teacher_forced(G, oracle, cfg, 13, 2)
     check_fp16(out)
     gpu.close()
+
+
+def test_cfg3_full_depth_graph_replay_equals_stepwise(G):
+    """Configuration 3 at its full depth (12 layers, 10 of them MoE) and batch: the captured step graph (router with the
+    counter-based places, expert GEMMs over the pointer tables, combine) gives the tokens and the logits of explicit
+    decode calls, and a second model object repeats them bit for bit -- the places rows take in their experts' batches
+    differ from run to run, the results must not."""
+    cfg = dict(synth.CONFIGS["cfg3_moe_f16"], vocab=4096, prompt=24)
+    B = cfg["batch"]
+    w = synth.make_weights(cfg, 21, random_bias=True)
+    ids = synth.make_prompts(cfg, 4)
+    runs = []
+    for rep in range(2):
+        gpu = G.HipGpt(cfg, w, max_batch=B, max_seq_len=cfg["prompt"] + 12)
+        gpu.prefill(ids)
+        toks, _ = gpu.generate(6)
+        runs.append((toks, gpu.logits()))
+        gpu.close()
+    assert np.array_equal(runs[0][0], runs[1][0]) and np.array_equal(runs[0][1], runs[1][1])
+    step = G.HipGpt(cfg, w, max_batch=B, max_seq_len=cfg["prompt"] + 12)
+    step.prefill(ids)
+    for s in range(6):
+        nxt = step.sample()
+        assert np.array_equal(nxt, runs[0][0][s])
+        step.decode(nxt)
+    assert np.array_equal(step.logits(), runs[0][1])
+    ti, tv, pr = step.moe_routing(5)
+    assert ti.shape == (B, cfg["experts_per_token"]) and np.allclose(pr.sum(1), 1.0, atol=1e-5)
+    step.close()

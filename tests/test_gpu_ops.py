@@ -64,13 +64,14 @@ def test_binary_ops(T, op):
     assert np.array_equal(ops.add(None, HT.from_numpy(a), row).numpy(), a + b[:1])
 
 
-@pytest.mark.parametrize("name", ["relu", "silu", "leakyrelu", "exp", "log", "sigmoid"])
+@pytest.mark.parametrize("name", ["relu", "silu", "leakyrelu", "exp", "log", "sigmoid", "neg", "tanh", "sqrt", "abs"])
 def test_unary_ops(T, oracle, name):
     HT, ops = T
     x = np.random.default_rng(2).standard_normal((5, 7)).astype(np.float32)
-    if name == "log":
+    if name in ("log", "sqrt"):
         x = np.abs(x) + 0.1
-    ref = {"exp": np.exp, "log": np.log, "sigmoid": lambda v: 1 / (1 + np.exp(-v))}.get(name)
+    ref = {"exp": np.exp, "log": np.log, "sigmoid": lambda v: 1 / (1 + np.exp(-v)), "neg": np.negative, "tanh": np.tanh, "sqrt": np.sqrt,
+           "abs": np.abs}.get(name)
     want = oracle.unary(name, x) if ref is None else ref(x.astype(np.float64))
     for t in _both_layouts(HT, x):
         assert np.allclose(getattr(ops, name)(None, t).numpy(), want, rtol=2e-6, atol=1e-7)

@@ -136,3 +136,30 @@ def test_two_models_on_two_threads():
     assert not fails, fails
     for m in models:
         m.close()
+
+
+def test_profile_reports_the_launched_symbols():
+    """TSHip_GptProfileDecode / TSHip_GptProfileSymbols: one entry per launch of a decode step, the symbol being the kernel
+    the runtime resolved for the launched function (what a profiler's kernel trace prints)."""
+    from seq2seqsharp_amd import synth
+    from seq2seqsharp_amd.gpt import HipGpt
+    cfg = synth.tiny_config(dtype="f16")
+    gpu = HipGpt(cfg, synth.make_weights(cfg, 1), max_batch=cfg["batch"], max_seq_len=32)
+    gpu.prefill(synth.make_prompts(cfg, 2))
+    prof = gpu.profile_decode(gpu.sample())
+    syms = gpu.profile_symbols()
+    assert len(prof) == len(syms) > 0
+    names = [n for n, _ in prof]
+    assert "attn_decode" in names and all(t >= 0 for _, t in prof)
+    assert "attn" in syms[names.index("attn_decode")] and all("tship::" in s or "kernel" in s for s in syms)
+    gpu.close()
+
+
+def test_stream_structure_probe_runs_and_orders_sensibly():
+    """The measurement aid: four timings for a small chain; every block of the persistent variants leaves its bounded
+    barrier (the call fails otherwise)."""
+    from seq2seqsharp_amd.gpt import stream_structure_probe
+    ms = stream_structure_probe([4e6, 1e6, 8e6, 2e6] * 3, [16, 4, 32, 8] * 3, repeats=2)
+    assert len(ms) == 4 and all(0 < m < 50 for m in ms)
+    with pytest.raises(Exception):
+        stream_structure_probe([1e6] * 200, [0] * 200)          # more phases than the probe's plan holds
