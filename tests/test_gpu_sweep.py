@@ -1,0 +1,69 @@
+"""Seeded sweep over model shapes the fused path accepts: head sizes 16-128, 1/2/4 query heads per KV head, both
+attention layers, both norms, all activations, MoE layers, odd vocabulary sizes and feed-forward widths, batches on both
+sides of the 32- and 64-row tiles, prompts on both sides of the 32-position cache chunks.  Prefill and three decode steps
+against the CPU oracle, fp32 and fp16 bars as everywhere else."""
+import numpy as np
+import pytest
+
+from parity_util import top1_agreement
+from seq2seqsharp_amd import synth
+
+pytestmark = pytest.mark.gpu
+
+
+def _random_cfg(seed):
+    rng = np.random.default_rng(1000 + seed)
+    d = int(rng.choice([16, 32, 64, 128]))
+    g = int(rng.choice([1, 2, 4]))
+    hkv = int(rng.choice([1, 2, 3, 4, 8]))
+    mha = bool(rng.integers(0, 3) == 0)
+    heads = hkv if mha else hkv * g
+    moe = bool(rng.integers(0, 4) == 0)
+    norm = int(rng.choice([synth.RMSNORM, synth.LAYERNORM]))
+    act = int(rng.choice([synth.RELU, synth.SILU, synth.LEAKYRELU] if moe else [synth.RELU, synth.SILU, synth.LEAKYRELU, synth.SWIGLU, synth.SWIGLU_SILU]))
+    cfg = synth._cfg(n_layers=int(rng.integers(1, 4)) if not moe else 3, hidden=heads * d, n_heads=heads, n_kv_heads=heads if mha else hkv,
+                     ffn_dim=int(rng.choice([48, 96, 176, 200, 264])), vocab=int(rng.choice([61, 97, 130, 257, 1000])),
+                     attn_type=synth.MHA if mha else synth.GQA, norm_type=norm, act=act,
+                     n_experts=int(rng.choice([2, 4, 8])) if moe else 1, experts_per_token=int(rng.choice([1, 2])) if moe else 1,
+                     batch=int(rng.choice([1, 2, 7, 31, 32, 33, 40, 64, 65, 100, 128])), prompt=int(rng.choice([1, 3, 31, 32, 33, 47])), steps=3,
+                     use_rope=int(rng.integers(0, 5) != 0), dtype="f16" if seed % 3 else "f32")
+    return cfg
+
+
+@pytest.mark.parametrize("seed", range(72))
+def test_random_shape_against_oracle(oracle, seed):
+    from seq2seqsharp_amd import gpt as G
+    cfg = _random_cfg(seed)
+    w = synth.make_weights(cfg, seed, random_bias=True)
+    orc = oracle.OracleGpt(cfg, w)
+    gpu = G.HipGpt(cfg, w, max_batch=cfg["batch"], max_seq_len=cfg["prompt"] + 6)
+    cur = synth.make_prompts(cfg, 200 + seed)
+    lens = None
+    if seed % 5 == 4 and cfg["prompt"] > 1:      # the reference's padded batches: BuildSelfTriMask per row
+        lens = np.random.default_rng(seed).integers(1, cfg["prompt"] + 1, cfg["batch"]).astype(np.int32)
+        lens[0] = cfg["prompt"]
+        for b in range(cfg["batch"]):
+            cur[b, lens[b]:] = 0                  # the END tag pads (BuildInTokens.PadSentences)
+    p, lg = orc.step(cur, use_cache=True, lens=lens)
+    gpu.prefill(cur, lens)
+    moe16 = cfg["dtype"] == "f16" and cfg["n_experts"] > 1
+    for step in range(4):
+        gl = gpu.logits()
+        if cfg["dtype"] == "f32":
+            assert float(np.abs(gl - lg).max() / max(np.abs(lg).max(), 1e-6)) <= 1e-4, (cfg, step)
+            a, b = gl.argmax(1), lg.argmax(1)
+            rows = np.arange(len(a))
+            assert ((a == b) | (lg[rows, b] - lg[rows, a] <= 1e-5 * np.abs(lg).max())).all(), (cfg, step)
+        elif not moe16:
+            assert np.abs(gl - lg).max() <= 3e-2, (cfg, step)
+            assert top1_agreement(gl, lg)[0] >= 0.99 or cfg["batch"] < 8, (cfg, step)
+        else:
+            # fp16 routing may flip near-ties (judged at cfg3's shape with the oracle's margins); here: most rows agree
+            assert np.median(np.abs(gl - lg).max(1)) <= 3e-2, (cfg, step)
+        if step == 3:
+            break
+        nxt = oracle.argmax(p).astype(np.int32)
+        cur = np.concatenate([cur, nxt[:, None]], 1)
+        p, lg = orc.step(cur, use_cache=True)
+        gpu.decode(nxt)
+    gpu.close()
