@@ -604,8 +604,97 @@ __global__ __launch_bounds__(256) void big_gemm_f16_kernel(BigArgs a) {
 }
 
 // Epilogue shared by the LDS-tiled prefill GEMMs.
+// Gated activation output of one wavefront (64 rows x 4 column tiles = 64 consecutive fp16 outputs per row) through LDS, so
+// that rows leave as whole 128-byte lines (eight lanes x 16 bytes per row, eight rows per store instruction) instead of
+// 32 pieces of 16 bytes per instruction: the fragmented form takes four times the store requests.  `stage`: 64 rows x 72
+// halfs of LDS owned by this wavefront (row stride 144 bytes: 16-byte aligned pieces, rows spread over the banks).  Whole tiles only.
+__device__ __forceinline__ void gated_store_lines(const BigArgs& a, floatx16 (&acc)[4][2], int nt_first, long row_first, int lane, half_t* stage,
+                                                  const float (&rinv2)[2]) {
+    constexpr int LDSROW = 72;
+    const int lh = lane >> 5, r = lane & 31;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        float b1[8], b2[8];
+#pragma unroll
+        for (int v = 0; v < 8; ++v) {
+            const int f = (nt_first + j) * 16 + 8 * (v / 4) + 4 * lh + (v % 4);
+            b1[v] = a.bias[f]; b2[v] = a.bias2[f];
+        }
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+#pragma unroll
+            for (int g = 0; g < 2; ++g) {
+                half4v o;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) o[e] = (half_t)(act_apply(a.act, acc[j][i][4 * g + e] * rinv2[i] + b1[4 * g + e]) * (acc[j][i][4 * g + e + 8] * rinv2[i] + b2[4 * g + e]));
+                *(half4v*)(stage + (32 * i + r) * LDSROW + 16 * j + 8 * g + 4 * lh) = o;
+            }
+        }
+    }
+    __builtin_amdgcn_wave_barrier();
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    const int piece = lane & 7, rr = lane >> 3;
+    half8 line[8];
+#pragma unroll
+    for (int ps = 0; ps < 8; ++ps) line[ps] = *(const half8*)(stage + (8 * ps + rr) * LDSROW + 8 * piece);
+#pragma unroll
+    for (int ps = 0; ps < 8; ++ps) *(half8*)(a.out16 + (row_first + 8 * ps + rr) * a.ld16 + (long)nt_first * 16 + 8 * piece) = line[ps];
+}
+
+// The same for one 32-column tile of a residual projection (64 rows x 32 fp32 columns = one 128-byte line per row): the
+// old residual values are requested in line layout first, the accumulators cross through LDS (64 rows x 36 floats), and
+// x, half(gamma x) and the tile's sums of squares leave from the line layout (a row's 32 columns sit in eight lanes).
+// Same arithmetic per element as the direct form (acc * rinv + bias, then + old); the sums of squares add in another order.
+template <bool RESID>     // false: plain fp32 output with bias (no old values, no fp16 copy)
+__device__ __forceinline__ void resid_store_lines(const BigArgs& a, const floatx16 (&acc2)[2], int nt, long row_first, int lane, float* stage,
+                                                  const float (&rinv2)[2]) {
+    constexpr int LDSROW = 36;
+    const int lh = lane >> 5, r = lane & 31, piece = lane & 7, rr = lane >> 3;
+    floatx4 old[8];
+#pragma unroll
+    for (int ps = 0; ps < 8; ++ps) old[ps] = RESID ? *(const floatx4*)(a.out + (row_first + 8 * ps + rr) * a.ld_out + (long)nt * 32 + 4 * piece) : floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+    float bb[16];
+#pragma unroll
+    for (int v = 0; v < 16; ++v) bb[v] = a.bias[nt * 32 + 8 * (v / 4) + 4 * lh + (v % 4)];
+    const floatx4 gm = (RESID && a.xg16) ? *(const floatx4*)(a.gamma + nt * 32 + 4 * piece) : floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            floatx4 sv;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) sv[e] = acc2[i][4 * g + e] * rinv2[i] + bb[4 * g + e];
+            *(floatx4*)(stage + (32 * i + r) * LDSROW + 8 * g + 4 * lh) = sv;
+        }
+    __builtin_amdgcn_wave_barrier();
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    floatx4 v[8];
+#pragma unroll
+    for (int ps = 0; ps < 8; ++ps) v[ps] = *(const floatx4*)(stage + (8 * ps + rr) * LDSROW + 4 * piece);
+#pragma unroll
+    for (int ps = 0; ps < 8; ++ps) {
+        const long row = row_first + 8 * ps + rr;
+        floatx4 sv;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) sv[e] = RESID ? v[ps][e] + old[ps][e] : v[ps][e];
+        *(floatx4*)(a.out + row * a.ld_out + (long)nt * 32 + 4 * piece) = sv;
+        if (RESID && a.xg16) {
+            half4v xg;
+            float q = 0.0f;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) { xg[e] = (half_t)(gm[e] * sv[e]); q += sv[e] * sv[e]; }
+            *(half4v*)(a.xg16 + row * a.ld_xg + (long)nt * 32 + 4 * piece) = xg;
+            q += __shfl_xor(q, 1, 64);
+            q += __shfl_xor(q, 2, 64);
+            q += __shfl_xor(q, 4, 64);
+            if (piece == 0) a.ssq_out[(long)nt * a.ssq_ld + row] = q;
+        }
+    }
+    __builtin_amdgcn_wave_barrier();          // the next tile's accumulators overwrite the stage
+}
+
 template <int EPI, int NI = 4>      // NI: 32-row tiles per wavefront (the wavefront's rows start at 32 NI wr)
-__device__ __forceinline__ void big_gemm_store(const BigArgs& a, floatx16 (&acc)[4][NI], int nt0, long row0, int wr, int wn, int lane) {
+__device__ __forceinline__ void big_gemm_store(const BigArgs& a, floatx16 (&acc)[4][NI], int nt0, long row0, int wr, int wn, int lane, half_t* stage = nullptr) {
     // accumulator (j, i), lane l, register v = 4 g + e: column (nt0 + 4 wn + j) * 32 + 8 g + 4 (l / 32) + e,
     // row row0 + 128 wr + 32 i + l % 32.  Biases (and the residual) are fetched in batches before the first store
     // of a column tile, and the four consecutive columns of a group go out as one 16-byte (fp32) or 8-byte (fp16) store.
@@ -616,6 +705,29 @@ __device__ __forceinline__ void big_gemm_store(const BigArgs& a, floatx16 (&acc)
     for (int i = 0; i < NI; ++i) {
         const long row = row0 + 32 * NI * wr + 32 * i + (lane & 31);
         rinv4[i] = (a.rinv && row < a.R) ? a.rinv[row] : 1.0f;
+    }
+    if constexpr (EPI == BEPI_ACT16 && NI == 2) {
+        // whole 64 x 64 output block of a gated projection with 16-byte aligned rows: line stores through LDS
+        const long rf = row0 + 64 * wr;
+        const int ntf = nt0 + 4 * wn;
+        if (stage && a.gated && rf + 64 <= a.R && ntf + 4 <= a.NT && (ntf + 4) * 16 <= a.n_valid && (a.ld16 & 7) == 0) {
+            const float r2[2] = {rinv4[0], rinv4[1]};
+            gated_store_lines(a, acc, ntf, rf, lane, stage, r2);
+            return;
+        }
+    }
+    if constexpr ((EPI == BEPI_RESID || EPI == BEPI_F32_BIAS) && NI == 2) {
+        const long rf = row0 + 64 * wr;
+        const int ntf = nt0 + 4 * wn;
+        constexpr bool RS = EPI == BEPI_RESID;
+        if (stage && rf + 64 <= a.R && ntf + 4 <= a.NT && (ntf + 4) * 32 <= a.n_valid && (a.ld_out & 3) == 0 && (!RS || !a.xg16 || (a.ld_xg & 3) == 0)) {
+            const float r2[2] = {rinv4[0], rinv4[1]};
+            resid_store_lines<RS>(a, acc[0], ntf + 0, rf, lane, (float*)stage, r2);
+            resid_store_lines<RS>(a, acc[1], ntf + 1, rf, lane, (float*)stage, r2);
+            resid_store_lines<RS>(a, acc[2], ntf + 2, rf, lane, (float*)stage, r2);
+            resid_store_lines<RS>(a, acc[3], ntf + 3, rf, lane, (float*)stage, r2);
+            return;
+        }
     }
     // one column tile per call with a compile-time tile number: the accumulators must only ever be indexed statically
     auto tile_out = [&](auto J) {
@@ -961,7 +1073,9 @@ __global__ __launch_bounds__(512) void big_gemm3_f16_kernel(BigArgs a) {
 #pragma unroll
             for (int i = 0; i < 2; ++i) acc[j][i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wfB[j], xfB[i], acc[j][i], 0, 0, 0);
     }
-    big_gemm_store<EPI, 2>(a, acc, nt0, row0, wr, wn, lane);
+    // (the stages are dead once every wavefront has left the loop: each wavefront then owns 64 x 72 halfs of them)
+    __builtin_amdgcn_s_barrier();
+    big_gemm_store<EPI, 2>(a, acc, nt0, row0, wr, wn, lane, big_smem + w * (64 * 72));
 }
 
 // ------------------------------------------------------------------------------------------------
