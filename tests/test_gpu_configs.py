@@ -284,3 +284,20 @@ def test_cfg3_full_depth_graph_replay_equals_stepwise(G):
     ti, tv, pr = step.moe_routing(5)
     assert ti.shape == (B, cfg["experts_per_token"]) and np.allclose(pr.sum(1), 1.0, atol=1e-5)
     step.close()
+
+
+@pytest.mark.parametrize("batch,prompt,hidden,heads,kv,ffn,act", [
+    (3, 200, 192, 3, 3, 256, synth.SWIGLU),        # 600 rows: partial 256-row tiles; 6 and 8 column tiles (partial groups of four)
+    (2, 300, 256, 4, 2, 264, synth.SWIGLU_SILU),   # odd number of k-tiles in the down projection (the register-staged kernel)
+    (5, 128, 512, 8, 2, 1024, synth.SWIGLU),       # 640 rows, whole 64-row blocks, whole groups of four column tiles (line stores)
+    (9, 64, 128, 2, 1, 512, synth.RELU),           # 576 rows, ungated activation
+])
+def test_prefill_tile_edges_against_oracle(G, oracle, batch, prompt, hidden, heads, kv, ffn, act):
+    """Prompts of 512 rows and more take the LDS-tiled prefill GEMMs, whose epilogues write whole 64 x 128-byte blocks
+    through LDS where a wavefront's block is complete and element-wise elsewhere: row counts that are no multiple of
+    the tile sizes and widths that leave partial column groups, against the oracle."""
+    cfg = synth._cfg(n_layers=2, hidden=hidden, n_heads=heads, n_kv_heads=kv, ffn_dim=ffn, vocab=211, attn_type=synth.GQA,
+                     norm_type=synth.RMSNORM, act=act, batch=batch, prompt=prompt, steps=2, dtype="f16")
+    _, gpu, out, _ = teacher_forced(G, oracle, cfg, 31, 2)
+    check_fp16(out)
+    gpu.close()
