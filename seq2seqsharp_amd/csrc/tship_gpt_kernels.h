@@ -693,6 +693,41 @@ __device__ __forceinline__ void resid_store_lines(const BigArgs& a, const floatx
     __builtin_amdgcn_wave_barrier();          // the next tile's accumulators overwrite the stage
 }
 
+// Ungated activation output (ReLU / SiLU / LeakyReLU feed-forward, MoE experts): a wavefront's 64 rows x 128 columns go
+// out in two halves of 64 columns (one 128-byte line per row each) through the same 64 x 72 halfs of LDS.
+__device__ __forceinline__ void act_store_lines(const BigArgs& a, floatx16 (&acc)[4][2], int nt_first, long row_first, int lane, half_t* stage,
+                                                const float (&rinv2)[2]) {
+    constexpr int LDSROW = 72;
+    const int lh = lane >> 5, r = lane & 31, piece = lane & 7, rr = lane >> 3;
+#pragma unroll
+    for (int hj = 0; hj < 2; ++hj) {
+#pragma unroll
+        for (int jj = 0; jj < 2; ++jj) {
+            const int j = 2 * hj + jj;
+            float bb[16];
+#pragma unroll
+            for (int v = 0; v < 16; ++v) bb[v] = a.bias[(nt_first + j) * 32 + 8 * (v / 4) + 4 * lh + (v % 4)];
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    half4v o;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) o[e] = (half_t)act_apply(a.act, acc[j][i][4 * g + e] * rinv2[i] + bb[4 * g + e]);
+                    *(half4v*)(stage + (32 * i + r) * LDSROW + 32 * jj + 8 * g + 4 * lh) = o;
+                }
+        }
+        __builtin_amdgcn_wave_barrier();
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        half8 line[8];
+#pragma unroll
+        for (int ps = 0; ps < 8; ++ps) line[ps] = *(const half8*)(stage + (8 * ps + rr) * LDSROW + 8 * piece);
+#pragma unroll
+        for (int ps = 0; ps < 8; ++ps) *(half8*)(a.out16 + (row_first + 8 * ps + rr) * a.ld16 + (long)(nt_first + 2 * hj) * 32 + 8 * piece) = line[ps];
+        __builtin_amdgcn_wave_barrier();          // the second half overwrites the stage
+    }
+}
+
 template <int EPI, int NI = 4>      // NI: 32-row tiles per wavefront (the wavefront's rows start at 32 NI wr)
 __device__ __forceinline__ void big_gemm_store(const BigArgs& a, floatx16 (&acc)[4][NI], int nt0, long row0, int wr, int wn, int lane, half_t* stage = nullptr) {
     // accumulator (j, i), lane l, register v = 4 g + e: column (nt0 + 4 wn + j) * 32 + 8 g + 4 (l / 32) + e,
@@ -713,6 +748,11 @@ __device__ __forceinline__ void big_gemm_store(const BigArgs& a, floatx16 (&acc)
         if (stage && a.gated && rf + 64 <= a.R && ntf + 4 <= a.NT && (ntf + 4) * 16 <= a.n_valid && (a.ld16 & 7) == 0) {
             const float r2[2] = {rinv4[0], rinv4[1]};
             gated_store_lines(a, acc, ntf, rf, lane, stage, r2);
+            return;
+        }
+        if (stage && !a.gated && rf + 64 <= a.R && ntf + 4 <= a.NT && (ntf + 4) * 32 <= a.n_valid && (a.ld16 & 7) == 0) {
+            const float r2[2] = {rinv4[0], rinv4[1]};
+            act_store_lines(a, acc, ntf, rf, lane, stage, r2);
             return;
         }
     }
