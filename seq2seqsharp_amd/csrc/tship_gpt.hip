@@ -420,6 +420,13 @@ static void run_gemm_f32(TSHipGpt* m, const char* name, const GemmW& w, const fl
     g.bias = KS == 1 ? bias : nullptr;
     g.A = X; g.lda = ldx; g.B = w.buf.as<float>(); g.ldb = w.ld; g.C = out; g.ldc = ld_out; g.split_stride = split_stride;
     g.M = rows; g.N = w.N; g.K = w.K; g.KS = KS;
+    if (rows <= 32) {      // decode steps: every weight element once, up to 32 rows in registers
+        dim3 sgrid((unsigned)ceil_div(w.N, 64), 1, KS);
+        if (rows <= 8) launch(m, name, skinny_gemm_f32_kernel<8>, sgrid, dim3(256), g);
+        else if (rows <= 16) launch(m, name, skinny_gemm_f32_kernel<16>, sgrid, dim3(256), g);
+        else launch(m, name, skinny_gemm_f32_kernel<32>, sgrid, dim3(256), g);
+        return;
+    }
     dim3 grid((unsigned)ceil_div(w.N, 64), (unsigned)ceil_div(rows, 64), KS);
     launch(m, name, gemm_f32_kernel, grid, dim3(256), g);
 }

@@ -1128,6 +1128,87 @@ struct F32GemmArgs {
     const float* bias;     // optional, added when the result is final (KS == 1)
 };
 
+// The same product for up to 32 rows (decode steps of fp32 models): the weights are what costs, every element is read
+// once, 16 bytes per thread.  Block = 64 columns x one K range (blockIdx.z of KS): thread (tx, ty) owns columns
+// 4 tx .. 4 tx + 3 and the k = ty, ty + 16, ... of the range, with the rows' activations broadcast from LDS; the sixteen
+// k-lanes are added in a fixed order (lanes 16 and 32 apart inside a wavefront, then the four wavefronts), so the result
+// does not depend on scheduling.  Same split-K output convention as the kernel below.
+template <int MR>      // rows held in registers: 8, 16 or 32
+__global__ __launch_bounds__(256) void skinny_gemm_f32_kernel(F32GemmArgs a) {
+    constexpr int KC = 8192 / MR;                       // k per staging pass: MR x KC floats = 32 KiB
+    __shared__ float sX[MR * KC];
+    __shared__ float red[4][MR][64];
+    const int t = threadIdx.x, tx = t & 15, ty = t >> 4, lane = t & 63, w = t >> 6;
+    const int col0 = blockIdx.x * 64 + tx * 4, ks = blockIdx.z;
+    const int kper = (int)round_up(ceil_div(a.K, a.KS), 16);
+    const int kb = ks * kper, ke = min(a.K, kb + kper);
+    const bool vec = (a.ldb & 3) == 0 && col0 + 3 < a.N;
+    float acc[MR][4];
+#pragma unroll
+    for (int m = 0; m < MR; ++m)
+#pragma unroll
+        for (int c = 0; c < 4; ++c) acc[m][c] = 0.0f;
+    for (int k0 = kb; k0 < ke; k0 += KC) {
+        const int kn = min(KC, ke - k0);
+        __syncthreads();                                // the pass before is consumed
+        for (int idx = t; idx < MR * kn; idx += 256) {
+            const int m = idx / kn, k = idx - m * kn;
+            sX[m * KC + k] = m < a.M ? a.A[(long)m * a.lda + k0 + k] : 0.0f;
+        }
+        __syncthreads();
+        for (int k = ty; k < kn; k += 64) {
+            // four weight rows in flight per thread
+            floatx4 wv[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int kk = k + 16 * u;
+                const float* src = a.B + (long)(k0 + kk) * a.ldb + col0;
+                if (kk < kn && vec) wv[u] = *(const floatx4*)src;
+                else {
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) wv[u][c] = (kk < kn && col0 + c < a.N) ? src[c] : 0.0f;
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int kk = k + 16 * u;
+                if (kk >= kn) break;
+#pragma unroll
+                for (int m = 0; m < MR; ++m) {
+                    const float xv = sX[m * KC + kk];
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) acc[m][c] = fmaf(xv, wv[u][c], acc[m][c]);
+                }
+            }
+        }
+    }
+    // k-lanes: ty = 4 w + (lane / 16): add the lanes 16 and 32 apart, then the wavefronts through LDS
+#pragma unroll
+    for (int m = 0; m < MR; ++m)
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            float v = acc[m][c];
+            v += __shfl_xor(v, 16, 64);
+            v += __shfl_xor(v, 32, 64);
+            acc[m][c] = v;
+        }
+    if (lane < 16) {
+#pragma unroll
+        for (int m = 0; m < MR; ++m)
+#pragma unroll
+            for (int c = 0; c < 4; ++c) red[w][m][tx * 4 + c] = acc[m][c];
+    }
+    __syncthreads();
+    for (int idx = t; idx < MR * 64; idx += 256) {
+        const int m = idx >> 6, c = idx & 63, col = blockIdx.x * 64 + c;
+        if (m < a.M && col < a.N) {
+            float v = ((red[0][m][c] + red[1][m][c]) + red[2][m][c]) + red[3][m][c];
+            if (a.bias) v += a.bias[col];
+            a.C[ks * a.split_stride + (long)m * a.ldc + col] = v;
+        }
+    }
+}
+
 __global__ __launch_bounds__(256) void gemm_f32_kernel(F32GemmArgs a) {
     __shared__ float As[16][64 + 4];
     __shared__ float Bs[16][64 + 4];
