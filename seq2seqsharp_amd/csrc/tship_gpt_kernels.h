@@ -1156,11 +1156,11 @@ __global__ __launch_bounds__(256) void skinny_gemm_f32_kernel(F32GemmArgs a) {
             sX[m * KC + k] = m < a.M ? a.A[(long)m * a.lda + k0 + k] : 0.0f;
         }
         __syncthreads();
-        for (int k = ty; k < kn; k += 64) {
-            // four weight rows in flight per thread
-            floatx4 wv[4];
+        constexpr int U = MR <= 16 ? 8 : 4;             // weight rows in flight per thread
+        for (int k = ty; k < kn; k += 16 * U) {
+            floatx4 wv[U];
 #pragma unroll
-            for (int u = 0; u < 4; ++u) {
+            for (int u = 0; u < U; ++u) {
                 const int kk = k + 16 * u;
                 const float* src = a.B + (long)(k0 + kk) * a.ldb + col0;
                 if (kk < kn && vec) wv[u] = *(const floatx4*)src;
@@ -1170,7 +1170,7 @@ __global__ __launch_bounds__(256) void skinny_gemm_f32_kernel(F32GemmArgs a) {
                 }
             }
 #pragma unroll
-            for (int u = 0; u < 4; ++u) {
+            for (int u = 0; u < U; ++u) {
                 const int kk = k + 16 * u;
                 if (kk >= kn) break;
 #pragma unroll
