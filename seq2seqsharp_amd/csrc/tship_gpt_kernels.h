@@ -1344,28 +1344,26 @@ __global__ __launch_bounds__(256) void resid_norm_kernel(ResidNormArgs a) {
             int c = t + i * 256;
             s[i] = (c < a.h) ? part[(long)r * a.ld_part + c] : 0.0f;
         }
-        // splits are added in index order; four at a time so that their loads are in flight together
-        int k = 1;
-        for (; k + 3 < a.KS; k += 4) {
-            float p0[NPT], p1[NPT], p2[NPT], p3[NPT];
+        // splits are added in index order; a batch of them is requested together (unconditionally, the index clamped to the
+        // last split, so that the batch's loads are all in flight before the first is waited for)
+        constexpr int GROUP = NPT <= 4 ? 8 : 4;
+        for (int k = 1; k < a.KS; k += GROUP) {
+            float p[GROUP][NPT];
 #pragma unroll
-            for (int i = 0; i < NPT; ++i) {
-                int c = t + i * 256;
-                const float* q = part + (long)r * a.ld_part + c;
-                bool ok = c < a.h;
-                p0[i] = ok ? q[k * a.split_stride] : 0.0f;
-                p1[i] = ok ? q[(k + 1) * a.split_stride] : 0.0f;
-                p2[i] = ok ? q[(k + 2) * a.split_stride] : 0.0f;
-                p3[i] = ok ? q[(k + 3) * a.split_stride] : 0.0f;
+            for (int j = 0; j < GROUP; ++j) {
+                const int kk = min(k + j, a.KS - 1);
+#pragma unroll
+                for (int i = 0; i < NPT; ++i) {
+                    const int c = min(t + i * 256, a.h - 1);
+                    p[j][i] = part[kk * a.split_stride + (long)r * a.ld_part + c];
+                }
             }
 #pragma unroll
-            for (int i = 0; i < NPT; ++i) s[i] = (((s[i] + p0[i]) + p1[i]) + p2[i]) + p3[i];
-        }
-        for (; k < a.KS; ++k) {
+            for (int j = 0; j < GROUP; ++j) {
+                if (k + j < a.KS) {
 #pragma unroll
-            for (int i = 0; i < NPT; ++i) {
-                int c = t + i * 256;
-                if (c < a.h) s[i] += part[k * a.split_stride + (long)r * a.ld_part + c];
+                    for (int i = 0; i < NPT; ++i) s[i] += p[j][i];
+                }
             }
         }
 #pragma unroll
