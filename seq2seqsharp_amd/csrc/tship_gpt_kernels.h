@@ -1265,14 +1265,20 @@ __global__ void ffn_act_kernel(const float* __restrict__ part, int KS, long spli
     long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;
     if (idx >= R * F) return;
     long r = idx / F; int f = (int)(idx % F);
-    float s = 0.0f;
-    for (int k = 0; k < KS; ++k) s += part[k * split_stride + r * ldp + f];
-    s = act_apply(act, s + b1[f]);
-    if (gated) {
-        float c = 0.0f;
-        for (int k = 0; k < KS; ++k) c += part[k * split_stride + r * ldp + F + f];
-        s *= (c + b3[f]);
-    }
+    // split-K partials in index order, eight requested at a time (unconditionally, the index clamped to the last split)
+    auto sum_splits = [&](long off) {
+        float acc = 0.0f;
+        for (int k = 0; k < KS; k += 8) {
+            float pk[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) pk[j] = part[min(k + j, KS - 1) * split_stride + off];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) if (k + j < KS) acc += pk[j];
+        }
+        return acc;
+    };
+    float s = act_apply(act, sum_splits(r * ldp + f) + b1[f]);
+    if (gated) s *= (sum_splits(r * ldp + F + f) + b3[f]);
     out[r * ld_out + f] = (AT)s;
 }
 
@@ -1761,8 +1767,15 @@ __global__ __launch_bounds__(1024) void attn_decode_kernel(AttnArgs a) {
         if (idx < G * D) col = kvh * G * D + idx;
         else if (idx < (G + 1) * D) col = HD + kvh * D + (idx - G * D);
         else col = HD + GD + kvh * D + (idx - (G + 1) * D);
+        // split-K partials in index order, eight requested at a time (unconditionally, the index clamped to the last split)
         float s = a.qkv[(long)b * a.ldq + col];
-        for (int k = 1; k < a.KS; ++k) s += a.qkv[k * a.split_stride + (long)b * a.ldq + col];
+        for (int k = 1; k < a.KS; k += 8) {
+            float pk[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) pk[j] = a.qkv[min(k + j, a.KS - 1) * a.split_stride + (long)b * a.ldq + col];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) if (k + j < a.KS) s += pk[j];
+        }
         sm.in[idx] = s * rinv + a.bias[col];
     }
     __syncthreads();
