@@ -1541,18 +1541,24 @@ __global__ __launch_bounds__(256) void fn_prepare_kernel(FnPrepArgs a) {
     const int r = blockIdx.x, t = threadIdx.x;
     const long erow = a.ids ? (long)a.ids[r] : 0;
     const long srow = a.row_map ? a.row_map[r] : r;
+    // all requests first (unconditional, the column clamped), then the arithmetic and the stores
+    float vin[NPT], gmv[NPT];
+#pragma unroll
+    for (int i = 0; i < NPT; ++i) {
+        const int c = min(t + i * 256, a.h - 1);
+        if (a.ids) vin[i] = a.emb_f16 ? (float)((const half_t*)a.emb)[erow * a.h + c] : ((const float*)a.emb)[erow * a.h + c];
+        else vin[i] = a.src[srow * a.ld_src + c];
+        gmv[i] = a.gamma[c];
+    }
 #pragma unroll
     for (int i = 0; i < NPT; ++i) {
         const int c = t + i * 256;
         float v = 0.0f;
         if (c < a.h) {
-            if (a.ids) {
-                float e = a.emb_f16 ? (float)((const half_t*)a.emb)[erow * a.h + c] : ((const float*)a.emb)[erow * a.h + c];
-                v = e * a.emb_scale;
-            } else v = a.src[srow * a.ld_src + c];
+            v = a.ids ? vin[i] * a.emb_scale : vin[i];
             a.x[(long)r * a.ldx + c] = v;
-            if (a.xg_kt > 0) a.xg16[xpack_index(r, c, a.xg_kt)] = (half_t)(a.gamma[c] * v);
-            else a.xg16[(long)r * a.xg_ld + c] = (half_t)(a.gamma[c] * v);
+            if (a.xg_kt > 0) a.xg16[xpack_index(r, c, a.xg_kt)] = (half_t)(gmv[i] * v);
+            else a.xg16[(long)r * a.xg_ld + c] = (half_t)(gmv[i] * v);
         }
         float q = v * v;
 #pragma unroll
@@ -2430,8 +2436,18 @@ __global__ __launch_bounds__(1024) void greedy_kernel(const float* __restrict__ 
     float best = -INFINITY; int bi = 0x7fffffff;
     for (int i0 = t; i0 < V; i0 += 1024 * 8) {
         float v[8];
+        // (unconditional requests with clamped indices: all eight are in flight before the first comparison)
 #pragma unroll
-        for (int u = 0; u < 8; ++u) { int i = i0 + u * 1024; v[u] = (i < V && !(blocked && blocked[i])) ? row[i] : -INFINITY; }
+        for (int u = 0; u < 8; ++u) v[u] = row[min(i0 + u * 1024, V - 1)];
+        if (blocked) {
+            unsigned char bl[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) bl[u] = blocked[min(i0 + u * 1024, V - 1)];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) if (bl[u]) v[u] = -INFINITY;
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) if (i0 + u * 1024 >= V) v[u] = -INFINITY;
 #pragma unroll
         for (int u = 0; u < 8; ++u) { int i = i0 + u * 1024; if (i < V && (v[u] > best || (v[u] == best && i < bi))) { best = v[u]; bi = i; } }
     }
