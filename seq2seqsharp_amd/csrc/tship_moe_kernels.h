@@ -200,12 +200,6 @@ __global__ __launch_bounds__(256) void moe_router_kernel(MoeRouterArgs a) {
     }
 }
 
-// The same routing for fp16 models, one block of 256 threads per token row, everything requested in one memory round
-// trip and reduced as trees.  An fp16 model's activations differ from the fp32 reference's by the fp16 path's rounding
-// (about 1e-3), which already decides near-ties differently, so reproducing the reference's serial summation order (the
-// 1024-step chains of the kernel above) buys nothing there; that kernel remains the one fp32 models use, where routing
-// indices are bit-exact.  Same outputs: x updated with the pending attention output, LayerNorm in fp32, router logits
-// + (-65000), softmax with the exponentials evaluated in double, TopK by the reference's insertion rule.
 // v of lane `l`, the same l in every lane (a register read, no trip through the cross-lane network)
 __device__ __forceinline__ float lane_value(float v, int l) { return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), l)); }
 
@@ -249,8 +243,16 @@ __device__ __forceinline__ float wave_sum8(const float (&acc)[8], int lane) {
     return r1;
 }
 
+// The same routing for fp16 models, one block of 256 threads per token row, everything requested in one memory round
+// trip and reduced as trees.  An fp16 model's activations differ from the fp32 reference's by the fp16 path's rounding
+// (about 1e-3), which already decides near-ties differently, so reproducing the reference's serial summation order (the
+// 1024-step chains of the kernel above) buys nothing there; that kernel remains the one fp32 models use, where routing
+// indices are bit-exact.  Same outputs: x updated with the pending attention output, LayerNorm in fp32, router logits
+// + (-65000), softmax with the exponentials evaluated in double, TopK by the reference's insertion rule.
 // Thread t works on the column groups g = t, t + 256, ... of four neighbouring columns (16-byte requests; a row of 1024
-// columns is one request per tensor and thread), so hidden must be a multiple of four.
+// columns is one request per tensor and thread: as 4-byte requests strided by the expert count the router matrix alone
+// took 3.5 us), so hidden must be a multiple of four.  With xg16 set (decode steps) the kernel also gives the row its
+// place in each chosen expert's batch and writes it there (see MoeRouterArgs).
 template <int NG>      // NG * 1024 >= hidden
 __global__ __launch_bounds__(256) void moe_router_fast_kernel(MoeRouterArgs a) {
     constexpr int MAXE = 64;
