@@ -1299,7 +1299,7 @@ TSHIP_API int TSHip_GptBeamPick(TSHipGpt* m, int n_picks, int mode, float top_p,
     TSHIP_REQUIRE(m->cur_batch > 0, "TSHip_GptBeamPick: no logits yet; prefill or decode first");
     TSHIP_REQUIRE(n_picks >= 1 && n_picks <= m->c.vocab, "TSHip_GptBeamPick: n_picks must lie in 1..vocab");
     TSHIP_REQUIRE(mode == TSHIP_GREEDY || (mode == TSHIP_TOPP && host_uniforms), "TSHip_GptBeamPick: top-p needs one uniform draw per row and pick");
-    TSHIP_REQUIRE(mode == TSHIP_GREEDY || m->c.vocab <= 65535, "top-p sampling supports vocabularies up to 65535");
+    TSHIP_REQUIRE(mode == TSHIP_GREEDY || m->c.vocab <= 262144, "top-p sampling supports vocabularies up to 262144");
     TSHIP_REQUIRE(temperature > 0.0f, "temperature must be positive");
     const int B = m->cur_batch, V = m->c.vocab;
     const long Vp = round_up(V, 32);

@@ -192,7 +192,7 @@ static void sample_tokens(TSHipGpt* m, int mode, float top_p, float temperature,
         return;
     }
     TSHIP_REQUIRE(mode == TSHIP_TOPP, "unknown sampling mode");
-    TSHIP_REQUIRE(m->c.vocab <= 65535, "top-p sampling supports vocabularies up to 65535");
+    TSHIP_REQUIRE(m->c.vocab <= 262144, "top-p sampling supports vocabularies up to 262144");
     TSHIP_REQUIRE(temperature > 0.0f, "temperature must be positive");
     const size_t need = topp_scratch_bytes(m->Bpad, m->c.vocab);
     if (m->topp_scratch.bytes < need) m->topp_scratch.alloc(need);

@@ -797,7 +797,7 @@ static int topp_sample_op(const char* who, const TSHipTensor* result, const TSHi
     View r = make_view(result, who), p = make_view(probs, who), u = make_view(uniforms, who);
     TSHIP_REQUIRE(p.nd == 2 && p.dtype == TSHIP_F32 && p.st[1] == 1, "TSHip_TopPSample: probs must be a Float32 matrix with contiguous rows");
     const long rows = p.sz[0], K = p.sz[1];
-    TSHIP_REQUIRE(K >= 1 && K <= 65535, "TSHip_TopPSample: between 1 and 65535 columns are supported");
+    TSHIP_REQUIRE(K >= 1 && K <= 262144, "TSHip_TopPSample: between 1 and 262144 columns are supported");
     TSHIP_REQUIRE(count(r) == rows && r.dtype == TSHIP_F32 && is_contiguous(r), "TSHip_TopPSample: result must be a contiguous Float32 [rows,1] tensor");
     TSHIP_REQUIRE(count(u) == rows && u.dtype == TSHIP_F32 && is_contiguous(u), "TSHip_TopPSample: uniforms must be a contiguous Float32 [rows] tensor");
     TSHIP_REQUIRE(std::isfinite(repeat_penalty), "TSHip_TopPSampleEx: the penalty must be finite");
@@ -858,7 +858,7 @@ TSHIP_API int TSHip_TopPSampleNoAlloc(const TSHipTensor* result, const TSHipTens
     View r = make_view(result, who), p = make_view(probs, who), u = make_view(uniforms, who);
     TSHIP_REQUIRE(p.nd == 2 && p.dtype == TSHIP_F32 && p.st[1] == 1, "TSHip_TopPSampleNoAlloc: probs must be a Float32 matrix with contiguous rows");
     const long rows = p.sz[0], K = p.sz[1];
-    TSHIP_REQUIRE(K >= 1 && K <= 65535, "TSHip_TopPSampleNoAlloc: between 1 and 65535 columns are supported");
+    TSHIP_REQUIRE(K >= 1 && K <= 262144, "TSHip_TopPSampleNoAlloc: between 1 and 262144 columns are supported");
     TSHIP_REQUIRE(count(r) == rows && r.dtype == TSHIP_F32 && is_contiguous(r), "TSHip_TopPSampleNoAlloc: result must be a contiguous Float32 [rows,1] tensor");
     TSHIP_REQUIRE(count(u) == rows && u.dtype == TSHIP_F32 && is_contiguous(u), "TSHip_TopPSampleNoAlloc: uniforms must be a contiguous Float32 [rows] tensor");
     if (rows == 0) return 1;

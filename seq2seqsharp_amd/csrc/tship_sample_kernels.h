@@ -508,7 +508,7 @@ static __global__ __launch_bounds__(PICK_THREADS) void topp_pick_scan_kernel(Top
     const long slot = (a.d_step ? (long)*a.d_step * gridDim.x : 0) + r;
     const float u = a.uniforms[slot];
     // first k < n with accp[k] / acc >= u.  The running sum never decreases, so the test is monotone in k: the last
-    // elements of 512 equal segments locate the segment, its (at most 128) elements the index: two loads per thread.
+    // elements of 512 equal segments locate the segment, its (at most 512) elements the index: two loads per thread.
     auto block_min = [&](int v) {
 #pragma unroll
         for (int o = 32; o > 0; o >>= 1) { const int other = __shfl_xor(v, o, 64); if (other < v) v = other; }
@@ -522,7 +522,7 @@ static __global__ __launch_bounds__(PICK_THREADS) void topp_pick_scan_kernel(Top
     };
     int pick = 0x7fffffff;
     if (n > 0) {
-        const int seg = (n + PICK_THREADS - 1) / PICK_THREADS;           // <= 128: vocabularies have at most 65535 entries
+        const int seg = (n + PICK_THREADS - 1) / PICK_THREADS;           // <= 512 = PICK_THREADS: at most 262144 entries (checked by the callers)
         const int last = min(n, (t + 1) * seg) - 1;                      // last element of segment t (empty segments repeat n - 1)
         const int hit_seg = block_min((t * seg < n && accp[last] / acc >= u) ? t : 0x7fffffff);
         if (hit_seg != 0x7fffffff) {

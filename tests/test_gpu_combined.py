@@ -81,3 +81,24 @@ def test_reordered_rows_continue_like_their_sources():
     assert np.abs(got - np.stack(want)).max() <= 2e-3       # (batch 1 and batch 6 take different GEMM tilings: fp16 rounding apart)
     assert np.array_equal(got[0], got[4])                    # same source, same token: identical rows
     ref.close()
+
+
+def test_vocabulary_beyond_sixteen_bits(oracle):
+    """A vocabulary of 70 000 entries: greedy and top-p picks index past 65 535 (every probability gets a 32-bit index in the
+    sort keys), against the oracle with the shared uniform stream."""
+    from seq2seqsharp_amd.gpt import HipGpt, TOPP
+    cfg = synth.tiny_config(dtype="f32", n_layers=1, hidden=32, n_heads=2, n_kv_heads=1, ffn_dim=48, vocab=70000, batch=3, prompt=5)
+    w = synth.make_weights(cfg, 8)
+    w["FeedForward_Decoder_0.m_Bd"] = np.linspace(-2.0, 6.0, 70000, dtype=np.float32).reshape(1, -1)      # favour the high indices
+    ids = synth.make_prompts(cfg, 3)
+    orc = oracle.OracleGpt(cfg, w)
+    gpu = HipGpt(cfg, w, max_batch=3, max_seq_len=16)
+    p, lg = orc.step(ids, use_cache=True)
+    gpu.prefill(ids)
+    assert np.abs(gpu.logits() - lg).max() <= 1e-4 * np.abs(lg).max()
+    assert np.array_equal(gpu.sample(), oracle.argmax(p).astype(np.int32)) and gpu.sample().min() > 65535
+    u = synth.make_uniforms(4, 3, 1)[0]
+    want = oracle.toppsample(p, 0.9, 0.0, None, u)
+    got = gpu.sample(mode=TOPP, top_p=0.9, temperature=1.0, uniforms=u)
+    assert np.array_equal(got, want.astype(np.int32))
+    gpu.close()

@@ -349,3 +349,20 @@ def test_gather_and_scatter_fill(T):
             assert np.array_equal(ops.gather(None, src, dim, HT.from_numpy(ix)).numpy(), np.take_along_axis(a, ix.astype(np.int64), dim))
     with pytest.raises(Exception, match="outside"):
         ops.gather(None, HT.from_numpy(p), 1, HT.from_numpy(np.full((5, 1), 97, np.float32)))
+
+
+def test_toppsample_wide_rows(T, oracle):
+    """Rows of 200 000 and 262 144 probabilities (vocabularies beyond 16 bits): nearly flat, so that the running sum walks
+    most of the row and the pick lands far beyond index 65 535 of the sorted order; bit-exact against the oracle."""
+    HT, ops = T
+    rng = np.random.default_rng(11)
+    for K in (200000, 262144):
+        p = rng.random((3, K)).astype(np.float32) + 0.5
+        p[1, :1000] = 0.0                                        # some non-candidates
+        p /= p.sum(1, keepdims=True)
+        u = np.array([0.999, 0.5, 0.93], np.float32)
+        want = oracle.toppsample(p, 0.97, 0.0, None, u)
+        got = ops.toppsample(None, HT.from_numpy(p), HT.from_numpy(u.reshape(-1, 1)), 0.97).numpy().reshape(-1)
+        assert np.array_equal(got, want), K
+    with pytest.raises(Exception):
+        ops.toppsample(None, HT.from_numpy(np.ones((1, 262145), np.float32)), HT.from_numpy(np.array([[0.5]], np.float32)), 0.9)
