@@ -466,7 +466,8 @@ static AttnKernel pick_attn_g(int G, bool prefill) {
         case 1: return prefill ? attn_prefill_kernel<CT, AT, D, 1> : attn_decode_kernel<CT, AT, D, 1>;
         case 2: return prefill ? attn_prefill_kernel<CT, AT, D, 2> : attn_decode_kernel<CT, AT, D, 2>;
         case 4: return prefill ? attn_prefill_kernel<CT, AT, D, 4> : attn_decode_kernel<CT, AT, D, 4>;
-        default: throw Error("query heads per KV head must be 1, 2 or 4");
+        case 8: return prefill ? attn_prefill_kernel<CT, AT, D, 8> : attn_decode_kernel<CT, AT, D, 8>;
+        default: throw Error("query heads per KV head must be 1, 2, 4 or 8");
     }
 }
 template <typename CT, typename AT>
@@ -486,14 +487,16 @@ static AttnKernel pick_attn_mfma(int G, bool prefill, bool split, bool ragged) {
             case 1: return attn_mfma_prefill_kernel<D, 1, true>;
             case 2: return attn_mfma_prefill_kernel<D, 2, true>;
             case 4: return attn_mfma_prefill_kernel<D, 4, true>;
-            default: throw Error("query heads per KV head must be 1, 2 or 4");
+            case 8: return attn_mfma_prefill_kernel<D, 8, true>;
+            default: throw Error("query heads per KV head must be 1, 2, 4 or 8");
         }
     }
     switch (G) {
         case 1: return prefill ? attn_mfma_prefill_kernel<D, 1> : split ? attn_mfma_kernel<D, 1, true> : attn_mfma_kernel<D, 1, false>;
         case 2: return prefill ? attn_mfma_prefill_kernel<D, 2> : split ? attn_mfma_kernel<D, 2, true> : attn_mfma_kernel<D, 2, false>;
         case 4: return prefill ? attn_mfma_prefill_kernel<D, 4> : split ? attn_mfma_kernel<D, 4, true> : attn_mfma_kernel<D, 4, false>;
-        default: throw Error("query heads per KV head must be 1, 2 or 4");
+        case 8: return prefill ? attn_mfma_prefill_kernel<D, 8> : split ? attn_mfma_kernel<D, 8, true> : attn_mfma_kernel<D, 8, false>;
+        default: throw Error("query heads per KV head must be 1, 2, 4 or 8");
     }
 }
 static AttnKernel pick_attn(TSHipGpt* m, bool prefill, bool split = false, bool ragged = false) {
@@ -964,7 +967,7 @@ TSHIP_API int TSHip_GptCreate(const TSHipGptConfig* cfg, TSHipGpt** out) {
     m->D = c.hidden / c.n_heads;
     m->G = c.n_heads / c.n_kv_heads;
     TSHIP_REQUIRE(m->D == 16 || m->D == 32 || m->D == 64 || m->D == 128, "TSHip_GptCreate: head_dim must be 16, 32, 64 or 128");
-    TSHIP_REQUIRE(m->G == 1 || m->G == 2 || m->G == 4, "TSHip_GptCreate: query heads per KV head must be 1, 2 or 4");
+    TSHIP_REQUIRE(m->G == 1 || m->G == 2 || m->G == 4 || m->G == 8, "TSHip_GptCreate: query heads per KV head must be 1, 2, 4 or 8");
     m->Nqkv = (c.n_heads + 2 * c.n_kv_heads) * m->D;
     m->BT = c.max_batch <= 32 ? 1 : (c.max_batch <= 64 ? 2 : 4);
     m->Bpad = m->BT * 32;

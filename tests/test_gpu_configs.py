@@ -301,3 +301,23 @@ def test_prefill_tile_edges_against_oracle(G, oracle, batch, prompt, hidden, hea
     _, gpu, out, _ = teacher_forced(G, oracle, cfg, 31, 2)
     check_fp16(out)
     gpu.close()
+
+
+@pytest.mark.parametrize("dtype,hidden,heads,kv,batch,prompt", [
+    ("f16", 512, 8, 1, 5, 70),        # head size 64, eight query heads on one KV head: the MFMA attention kernels
+    ("f16", 1024, 8, 1, 33, 40),      # head size 128
+    ("f16", 1024, 16, 2, 3, 530),     # two KV heads; 530 rows of prompt take the LDS-tiled prefill GEMMs
+    ("f32", 256, 8, 1, 4, 37),        # the fp32 (VALU) attention kernels
+    ("f16", 256, 8, 1, 2, 33),        # head size 32: VALU kernels on an fp16 cache
+])
+def test_eight_query_heads_per_kv_head(G, oracle, dtype, hidden, heads, kv, batch, prompt):
+    """Group size 8 (Llama-3-70B-like head layouts), prefill and decode, both cache layouts."""
+    cfg = synth._cfg(n_layers=2, hidden=hidden, n_heads=heads, n_kv_heads=kv, ffn_dim=2 * hidden, vocab=173, attn_type=synth.GQA,
+                     norm_type=synth.RMSNORM, act=synth.SWIGLU, batch=batch, prompt=prompt, steps=3, dtype=dtype)
+    _, gpu, out, _ = teacher_forced(G, oracle, cfg, 41, 3)
+    if dtype == "f16":
+        check_fp16(out)
+    else:
+        for lg, gl in out:
+            assert float(np.abs(gl - lg).max() / np.abs(lg).max()) <= FP32_REL
+    gpu.close()
