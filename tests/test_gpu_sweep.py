@@ -25,7 +25,7 @@ def _random_cfg(seed):
     cfg = synth._cfg(n_layers=int(rng.integers(1, 4)) if not moe else 3, hidden=heads * d, n_heads=heads, n_kv_heads=heads if mha else hkv,
                      ffn_dim=int(rng.choice([48, 96, 176, 200, 264])), vocab=int(rng.choice([61, 97, 130, 257, 1000])),
                      attn_type=synth.MHA if mha else synth.GQA, norm_type=norm, act=act,
-                     n_experts=int(rng.choice([2, 4, 8])) if moe else 1, experts_per_token=int(rng.choice([1, 2])) if moe else 1,
+                     n_experts=int(rng.choice([2, 4, 8, 12, 16])) if moe else 1, experts_per_token=int(rng.choice([1, 2])) if moe else 1,
                      batch=int(rng.choice([1, 2, 7, 31, 32, 33, 40, 64, 65, 100, 128])), prompt=int(rng.choice([1, 3, 31, 32, 33, 47])), steps=3,
                      use_rope=int(rng.integers(0, 5) != 0), dtype="f16" if seed % 3 else "f32")
     return cfg
@@ -67,4 +67,41 @@ def test_random_shape_against_oracle(oracle, seed):
         cur = np.concatenate([cur, nxt[:, None]], 1)
         p, lg = orc.step(cur, use_cache=True)
         gpu.decode(nxt)
+    gpu.close()
+
+
+@pytest.mark.parametrize("experts,k,batch,dtype", [(16, 4, 9, "f16"), (12, 3, 40, "f16"), (16, 4, 33, "f32"), (3, 3, 5, "f16"), (64, 2, 7, "f16")])
+def test_moe_expert_counts_beyond_eight(oracle, experts, k, batch, dtype):
+    """More than eight experts (the fp16 router walks them in groups of eight), counts that are no multiple of eight, as many
+    picks as experts, and the maximum of 64.  fp32: routing bit-exact; fp16: probabilities within 2e-3 and every differing
+    choice a near-tie of the oracle's own probabilities."""
+    from seq2seqsharp_amd import gpt as G
+    cfg = synth._cfg(n_layers=3, hidden=128, n_heads=4, n_kv_heads=2, ffn_dim=256, vocab=151, attn_type=synth.GQA, norm_type=synth.LAYERNORM,
+                     act=synth.RELU, n_experts=experts, experts_per_token=k, batch=batch, prompt=6, steps=2, dtype=dtype)
+    w = synth.make_weights(cfg, 77, random_bias=True)
+    orc = oracle.OracleGpt(cfg, w)
+    gpu = G.HipGpt(cfg, w, max_batch=batch, max_seq_len=16)
+    cur = synth.make_prompts(cfg, 78)
+    p, lg = orc.step(cur, use_cache=True)
+    gpu.prefill(cur)
+    for step in range(3):
+        nxt = oracle.argmax(p).astype(np.int32)
+        cur = np.concatenate([cur, nxt[:, None]], 1)
+        p, lg = orc.step(cur, use_cache=True)
+        gpu.decode(nxt)
+        ti, tv, pr = gpu.moe_routing(2)
+        oi, ov, op = orc.moe_trace(0)
+        gl = gpu.logits()
+        if dtype == "f32":
+            assert np.array_equal(ti, oi) and np.allclose(pr, op, rtol=1e-6)
+            assert float(np.abs(gl - lg).max() / np.abs(lg).max()) <= 1e-4
+        else:
+            assert np.abs(pr - op).max() <= 2e-3
+            same = np.array([set(ti[r]) == set(oi[r]) for r in range(batch)])
+            if k < experts:
+                srt = -np.sort(-op, axis=1)
+                assert ((srt[:, k - 1] - srt[:, k])[~same] < 2e-3).all()
+            else:
+                assert same.all()
+            assert np.abs(gl[same] - lg[same]).max() <= 3e-2
     gpu.close()
