@@ -201,14 +201,18 @@ def main():
                 ak.append(kib)
         pb.append(launch_bytes["gemm_head"])
         ak.append(128)
-        ms3 = stream_structure_probe(pb, ak, repeats=6)
-        ms3_noact = stream_structure_probe(pb, [0] * len(ak), repeats=6)
+        # half-layer fusion: the output projection with the FFN up projection, the FFN down projection with what follows
+        fuse = [1 if name in ("gemm_wo", "gemm_ffn2") else 0 for _ in range(cfg["n_layers"]) for name, _k in per_layer] + [0]
+        ms3 = stream_structure_probe(pb, ak, repeats=6, fuse_with_next=fuse)
+        ms3_noact = stream_structure_probe(pb, [0] * len(ak), repeats=6, fuse_with_next=fuse)
         structure = {"phases": len(pb), "bytes": float(sum(pb)),
                      "one_launch_per_phase_ms": round(ms3[0], 4), "persistent_grid_barrier_ms": round(ms3[1], 4), "persistent_prefetch_before_barrier_ms": round(ms3[2], 4),
                      "one_launch_per_phase_cache_resident_ms": round(ms3[3], 4),
+                     "half_layer_fusion_ms": round(ms3[4], 4),
                      "without_shared_activation_reads": {"one_launch_per_phase_ms": round(ms3_noact[0], 4), "persistent_grid_barrier_ms": round(ms3_noact[1], 4),
                                                          "persistent_prefetch_before_barrier_ms": round(ms3_noact[2], 4),
-                                                         "one_launch_per_phase_cache_resident_ms": round(ms3_noact[3], 4)}}
+                                                         "one_launch_per_phase_cache_resident_ms": round(ms3_noact[3], 4),
+                                                         "half_layer_fusion_ms": round(ms3_noact[4], 4)}}
 
     out = {
         "metric": "decode tokens/s on 1 GPU (1B GQA fp16, batch 32)" if args.config == "cfg2_1b_gqa_f16" else "decode tokens/s on 1 GPU",

@@ -6,6 +6,10 @@
 //   1: one persistent kernel, one block per compute unit, phases separated by a grid-wide barrier (an agent-scope counter,
 //      bounded polling);
 //   2: the same with every wavefront requesting its first batch of the next phase before it arrives at the barrier;
+//   4: one launch per phase, except that the phases marked in `fuse_with_next` share a launch with their successor: a
+//      resident kernel (one block per compute unit) runs both with one grid-wide barrier in between, every wavefront
+//      requesting its first batch of the second phase before it arrives at the barrier (half-layer fusion: the output
+//      projection with the FFN up projection, the FFN down projection with the next QKV projection);
 //   3: one launch per phase again, but every phase reads the same region from offset 0, so that after the first phases the
 //      bytes come from the memory-side cache where they fit: what is left is the cost of the launch edges themselves, and
 //      the distance to (0) is what prefetching the next phase's weights into that cache could gain at most.
@@ -103,11 +107,47 @@ __global__ __launch_bounds__(PROBE_NT) void probe_persistent_kernel(const floatx
     if (total[0] + total[1] + total[2] + total[3] + carry == 1234.5f) sink[0] = total[0];
 }
 
+// two phases in one launch, one grid barrier between them (bounded polling); grid = one block per compute unit
+__global__ __launch_bounds__(PROBE_NT) void probe_pair_kernel(const floatx4* __restrict__ src, ProbePhase pa, ProbePhase pb, int p, const floatx4* __restrict__ act,
+                                                               float* xa, const float* xr, float* xb, unsigned* counter, int* err, float* sink, int spin_limit) {
+    const int t = threadIdx.x, lane = t & 63, w = t >> 6, blk = blockIdx.x, nb = gridDim.x;
+    float carry = xr ? xr[(long)((blk + 37) % nb) * PROBE_NT + t] : 0.0f;
+    floatx4 v[PROBE_U];
+    floatx4 a0 = {0, 0, 0, 0};
+    if (xr) for (int i = t; i < pa.act_kib * 64; i += PROBE_NT) a0 += act[(long)(p & 3) * 16384 + i];
+    floatx4 acc = probe_stream(src, pa, nb, blk, lane, w, v, false) + a0;
+    // first batch of the second phase, requested before the barrier
+    bool have = false;
+    {
+        const long pern = (pb.chunks + nb - 1) / nb;
+        const long n0 = blk * pern, n1 = min(n0 + pern, pb.chunks);
+        if (n0 + (long)w * PROBE_U < n1) { probe_load(src, pb.off16, n0 + (long)w * PROBE_U, n1, lane, v); have = true; }
+    }
+    __hip_atomic_store(xa + (long)blk * PROBE_NT + t, acc[0] + carry, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (t == 0) {
+        __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        int spins = 0;
+        while (__hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < (unsigned)nb) {
+            __builtin_amdgcn_s_sleep(1);
+            if (++spins > spin_limit) { *err = 1; break; }          // bounded: every block leaves the loop and the kernel ends
+        }
+    }
+    __syncthreads();
+    carry = __hip_atomic_load(xa + (long)((blk + 37) % nb) * PROBE_NT + t, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    floatx4 b0 = {0, 0, 0, 0};
+    for (int i = t; i < pb.act_kib * 64; i += PROBE_NT) b0 += act[(long)((p + 1) & 3) * 16384 + i];
+    floatx4 acc2 = probe_stream(src, pb, nb, blk, lane, w, v, have) + b0;
+    xb[(long)blk * PROBE_NT + t] = acc2[0] + carry;
+    if (acc[0] + acc2[0] + acc2[1] + acc2[2] + acc2[3] == 1234.5f) sink[0] = acc[0];
+}
+
 }  // namespace tship
 
 using namespace tship;
 
-extern "C" TSHIP_API int TSHip_StreamStructureProbe(int n_phases, const double* phase_bytes, const int* act_kib, int repeats, float* ms_out /* [4] */) {
+extern "C" TSHIP_API int TSHip_StreamStructureProbe(int n_phases, const double* phase_bytes, const int* act_kib, const int* fuse_with_next, int repeats, float* ms_out /* [5] */) {
     TSHIP_BEGIN
     TSHIP_REQUIRE(phase_bytes && act_kib && ms_out, "TSHip_StreamStructureProbe: null argument");
     TSHIP_REQUIRE(n_phases >= 1 && n_phases <= PROBE_MAXP && repeats >= 1, "TSHip_StreamStructureProbe: between 1 and 128 phases");
@@ -136,7 +176,8 @@ extern "C" TSHIP_API int TSHip_StreamStructureProbe(int n_phases, const double* 
         float* xb = (float*)xbuf;
         hipEvent_t e0, e1;
         TSHIP_CHECK_HIP(hipEventCreate(&e0)); TSHIP_CHECK_HIP(hipEventCreate(&e1));
-        for (int variant = 0; variant < 4; ++variant) {
+        for (int variant = 0; variant < 5; ++variant) {
+            if (variant == 4 && !fuse_with_next) { ms_out[4] = 0.0f; continue; }
             float best = 1e30f;
             for (int it = 0; it < repeats; ++it) {
                 TSHIP_CHECK_HIP(hipMemsetAsync(misc, 0, 4096, stream()));
@@ -147,6 +188,20 @@ extern "C" TSHIP_API int TSHip_StreamStructureProbe(int n_phases, const double* 
                         if (variant == 3) ph.off16 = 0;
                         hipLaunchKernelGGL(probe_phase_kernel, dim3(nb), dim3(PROBE_NT), 0, stream(), (const floatx4*)buf, ph, p, (const floatx4*)act,
                                            xb + (long)(p & 1) * nb * PROBE_NT, p ? xb + (long)((p - 1) & 1) * nb * PROBE_NT : (const float*)nullptr, sink);
+                    }
+                } else if (variant == 4) {
+                    unsigned* counters = (unsigned*)((char*)misc + 1024);          // one counter per fused launch
+                    int slot = 0;
+                    for (int p = 0; p < plan.n; ++p) {
+                        float* xw = xb + (long)(p & 1) * nb * PROBE_NT;
+                        const float* xr = p ? xb + (long)((p - 1) & 1) * nb * PROBE_NT : (const float*)nullptr;
+                        if (fuse_with_next[p] && p + 1 < plan.n) {
+                            hipLaunchKernelGGL(probe_pair_kernel, dim3(nb), dim3(PROBE_NT), 0, stream(), (const floatx4*)buf, plan.p[p], plan.p[p + 1], p, (const floatx4*)act,
+                                               xw, xr, xb + (long)((p + 1) & 1) * nb * PROBE_NT, counters + slot, err, sink, 2000000);
+                            ++slot; ++p;
+                        } else {
+                            hipLaunchKernelGGL(probe_phase_kernel, dim3(nb), dim3(PROBE_NT), 0, stream(), (const floatx4*)buf, plan.p[p], p, (const floatx4*)act, xw, xr, sink);
+                        }
                     }
                 } else if (variant == 1) {
                     hipLaunchKernelGGL(probe_persistent_kernel<false>, dim3(nb), dim3(PROBE_NT), 0, stream(), (const floatx4*)buf, plan, (const floatx4*)act, xb, counter, err, sink, 2000000);
