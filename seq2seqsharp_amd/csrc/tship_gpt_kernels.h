@@ -1008,10 +1008,12 @@ __global__ __launch_bounds__(256) void big_gemm2_f16_kernel(BigArgs a) {
 // fragment reads and their waits are written out by hand.  Needs an even number of k-tiles; rows and column tiles
 // beyond the matrix are clamped to the last valid one on load and dropped on store.
 // Eight wavefronts, two per SIMD: wavefront (wr, wn) owns 64 rows x 128 columns (4 x 2 MFMA tiles of 32 x 32, 128
-// accumulator registers), so that one wavefront's fragment reads, waits and barrier overlap the other's MFMAs on the
-// same SIMD.  Per k-tile a wavefront reads 4 weight and 2 activation fragments for 8 MFMAs.  (Four wavefronts of
-// 128 x 128 each, 16 fragment reads per 32 MFMAs and two thirds of the LDS traffic, measured 4 % slower: the loop is
-// bound by exposed waits, not by LDS bandwidth.)
+// accumulator registers).  Per k-tile a wavefront reads 4 weight and 2 activation fragments for 8 MFMAs.  The two
+// wavefronts of a SIMD work half a period apart (see the loop): one reads fragments while the other multiplies.  With
+// both in step (barrier, reads, products) all eight wavefronts read LDS at once while the matrix pipes idle, and then
+// queue for the pipes: the gated up projection of 32 768 x 2048 x 11 264 took 1.21 ms that way against 1.07 ms.
+// (Four wavefronts of 128 x 128 each, 16 fragment reads per 32 MFMAs and two thirds of the LDS traffic, measured
+// slower still: the loop is bound by exposed waits, not by LDS bandwidth.)
 __device__ __forceinline__ void lds_read_frags(unsigned wa, unsigned xa, half8 (&wf)[4], half8 (&xf)[2]) {
     asm volatile(
         "ds_read_b128 %0, %6\n\t"
@@ -1089,31 +1091,65 @@ __global__ __launch_bounds__(512) void big_gemm3_f16_kernel(BigArgs a) {
     issue(0);
     if (NC > 1) issue(1);
     if (NC > 2) issue(2);
-    for (int c = 0; c < NC; ++c) {
-        // chunk c has landed once at most the loads of the chunks issued after it (4 per chunk) are outstanding
-        const int later = min(2, NC - 1 - c);
+    // Two groups of four wavefronts (one per SIMD each; wavefronts w and w + 4 share a SIMD: grouping by w % 2 instead
+    // measured 30 % slower) run the same chunks half a period apart with one block barrier per chunk: behind barrier c
+    // the first group reads its fragments of chunk c from LDS while the second multiplies chunk c - 1 out of its
+    // registers, then the first multiplies chunk c while the second reads it.  Before barrier c every wavefront has
+    // waited for its own part of chunk c and has read chunk c - 1, so the loads of chunk c + 3 may overwrite that stage.
+    // Both groups pass the same number of barriers.
+    const int g = w >> 2;
+    half8 wfA[4], xfA[2], wfB[4], xfB[2];
+    auto R = [&](int c) {
+        const unsigned sb = lds0 + (unsigned)((c & (NST - 1)) * STAGE * 2);
+        lds_read_frags(sb + woff, sb + xoff0, wfA, xfA);                   // k-tile 0
+        lds_read_frags(sb + woff + 1024, sb + xoff1, wfB, xfB);            // k-tile 1
+        if (c + 3 < NC) issue(c + 3);
+        const int later = max(0, min(2, NC - 2 - c));
         if (later == 2) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
         else if (later == 1) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
         else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        __builtin_amdgcn_s_barrier();          // every wavefront's part of chunk c is in LDS, and chunk c - 1 is consumed
-        if (c + 3 < NC) issue(c + 3);           // into the stage chunk c - 1 used
-        const unsigned sb = lds0 + (unsigned)((c & (NST - 1)) * STAGE * 2);
-        half8 wfA[4], xfA[2], wfB[4], xfB[2];
-        lds_read_frags(sb + woff, sb + xoff0, wfA, xfA);                   // k-tile 0
-        lds_read_frags(sb + woff + 1024, sb + xoff1, wfB, xfB);            // k-tile 1
-        lds_wait_frags<6>(wfA, xfA);
+        lds_wait_frags<0>(wfA, xfA);
+        lds_wait_frags<0>(wfB, xfB);
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    auto M = [&]() {
+        __builtin_amdgcn_sched_barrier(0);
+        __builtin_amdgcn_s_setprio(1);
 #pragma unroll
         for (int j = 0; j < 4; ++j)
 #pragma unroll
             for (int i = 0; i < 2; ++i) acc[j][i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wfA[j], xfA[i], acc[j][i], 0, 0, 0);
-        __builtin_amdgcn_sched_barrier(0);
-        lds_wait_frags<0>(wfB, xfB);
 #pragma unroll
         for (int j = 0; j < 4; ++j)
 #pragma unroll
             for (int i = 0; i < 2; ++i) acc[j][i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wfB[j], xfB[i], acc[j][i], 0, 0, 0);
+        __builtin_amdgcn_s_setprio(0);
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    {
+        const int later = min(2, NC - 1);
+        if (later == 2) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+        else if (later == 1) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+        else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     }
-    // (the stages are dead once every wavefront has left the loop: each wavefront then owns 64 x 72 halfs of them)
+    __builtin_amdgcn_s_barrier();                       // chunk 0 is in LDS
+    if (g == 0) {
+        for (int c = 0; c < NC; ++c) {
+            if (c) { __builtin_amdgcn_s_barrier(); __builtin_amdgcn_sched_barrier(0); }
+            R(c);
+            M();
+        }
+    } else {
+        R(0);
+        for (int c = 1; c < NC; ++c) {
+            __builtin_amdgcn_s_barrier();
+            M();
+            R(c);
+        }
+        M();
+    }
+    // (the first group is here while the second may still be reading the last chunk: the stages are dead, and each
+    // wavefront owns 64 x 72 halfs of them for its epilogue, once every wavefront has passed this barrier)
     __builtin_amdgcn_s_barrier();
     big_gemm_store<EPI, 2>(a, acc, nt0, row0, wr, wn, lane, big_smem + w * (64 * 72));
 }
