@@ -1037,7 +1037,7 @@ __device__ __forceinline__ void lds_wait_frags(half8 (&wf)[4], half8 (&xf)[2]) {
 template <int EPI>
 __global__ __launch_bounds__(512) void big_gemm3_f16_kernel(BigArgs a) {
     extern __shared__ __attribute__((aligned(16))) half_t big_smem[];
-    constexpr int CK = 2, NST = 4, FR = 8 * CK;          // k-tiles per stage, stages, fragments per operand and stage
+    constexpr int CK = 2, NST = 4, FR = 8 * CK, PF = NST - 1;          // k-tiles per stage, stages, fragments per operand and stage, chunks requested ahead
     constexpr int STAGE = 2 * FR * 512;                  // halfs per stage: weight fragments, then activation fragments
     const int t = threadIdx.x, lane = t & 63, w = __builtin_amdgcn_readfirstlane(t >> 6);
     const int wr = w >> 1, wn = w & 1;                   // 4 x 2 wavefronts
@@ -1073,7 +1073,7 @@ __global__ __launch_bounds__(512) void big_gemm3_f16_kernel(BigArgs a) {
     typedef const void __attribute__((address_space(1)))* gptr_t;
     typedef void __attribute__((address_space(3)))* lptr_t;
     auto issue = [&](int c) {
-        half_t* st = big_smem + (c & (NST - 1)) * STAGE;
+        half_t* st = big_smem + (c % NST) * STAGE;
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
             const int f = i * 8 + w;
@@ -1099,15 +1099,18 @@ __global__ __launch_bounds__(512) void big_gemm3_f16_kernel(BigArgs a) {
     // Both groups pass the same number of barriers.
     const int g = w >> 2;
     half8 wfA[4], xfA[2], wfB[4], xfB[2];
-    auto R = [&](int c) {
-        const unsigned sb = lds0 + (unsigned)((c & (NST - 1)) * STAGE * 2);
-        lds_read_frags(sb + woff, sb + xoff0, wfA, xfA);                   // k-tile 0
-        lds_read_frags(sb + woff + 1024, sb + xoff1, wfB, xfB);            // k-tile 1
-        if (c + 3 < NC) issue(c + 3);
-        const int later = max(0, min(2, NC - 2 - c));
+    auto wait_loads = [&](int c) {          // this wavefront's part of chunk c + 1 has landed
+        const int later = max(0, min(PF - 1, NC - 2 - c));
         if (later == 2) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
         else if (later == 1) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
         else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    };
+    auto R = [&](int c, bool wait_now) {
+        const unsigned sb = lds0 + (unsigned)((c % NST) * STAGE * 2);
+        lds_read_frags(sb + woff, sb + xoff0, wfA, xfA);                   // k-tile 0
+        lds_read_frags(sb + woff + 1024, sb + xoff1, wfB, xfB);            // k-tile 1
+        if (c + PF < NC) issue(c + PF);
+        if (wait_now) wait_loads(c);
         lds_wait_frags<0>(wfA, xfA);
         lds_wait_frags<0>(wfB, xfB);
         __builtin_amdgcn_sched_barrier(0);
@@ -1126,25 +1129,21 @@ __global__ __launch_bounds__(512) void big_gemm3_f16_kernel(BigArgs a) {
         __builtin_amdgcn_s_setprio(0);
         __builtin_amdgcn_sched_barrier(0);
     };
-    {
-        const int later = min(2, NC - 1);
-        if (later == 2) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
-        else if (later == 1) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
-        else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    }
+    wait_loads(-1);
     __builtin_amdgcn_s_barrier();                       // chunk 0 is in LDS
     if (g == 0) {
         for (int c = 0; c < NC; ++c) {
             if (c) { __builtin_amdgcn_s_barrier(); __builtin_amdgcn_sched_barrier(0); }
-            R(c);
+            R(c, false);
             M();
+            wait_loads(c);          // (behind the products: half a period more for the loads than in front of them)
         }
     } else {
-        R(0);
+        R(0, true);
         for (int c = 1; c < NC; ++c) {
             __builtin_amdgcn_s_barrier();
             M();
-            R(c);
+            R(c, true);
         }
         M();
     }
@@ -2321,21 +2320,47 @@ __global__ __launch_bounds__(D == 128 ? 256 : 512) void attn_mfma_prefill_kernel
     };
     fetch(0);
 
-    // queries: projection + bias, rotary embedding, 1 / sqrt(d); columns beyond the prompt stay zero
+    // queries: projection + bias, rotary embedding, 1 / sqrt(d); columns beyond the prompt stay zero.  A lane takes
+    // four consecutive elements (two rotary pairs) of a column at a time; the requests of four such pieces go out
+    // together (one memory round trip per batch: piece by piece the block spent longer here than in its chunks)
     float* sq = sbuf[w];
-    for (int i = lane; i < 16 * D; i += 64) sq[i] = 0.0f;
-    if (active) {
-        for (int p = lane; p < 16 * D / 2; p += 64) {
-            const int col = p / (D / 2), i = p % (D / 2);
-            const int qi = col / G, g = col % G;
-            if (tq0 + qi >= a.Tq) continue;
-            const long row = (long)b * a.Tq + tq0 + qi;
-            const int pos = pos_base + qi;
-            const int c0 = (kvh * G + g) * D + 2 * i;
-            float x0 = a.qkv[row * a.ldq + c0] + a.bias[c0], x1 = a.qkv[row * a.ldq + c0 + 1] + a.bias[c0 + 1], y0 = x0, y1 = x1;
-            if (a.rope_cos) rope_pair(x0, x1, a.rope_cos[(long)pos * (D / 2) + i], a.rope_sin[(long)pos * (D / 2) + i], y0, y1);
-            // (scores are kept in units of log 2, so that the exponentials below are bare v_exp_f32)
-            sq[col * D + 2 * i] = (a.scale * 1.44269504f) * y0; sq[col * D + 2 * i + 1] = (a.scale * 1.44269504f) * y1;
+    {
+        constexpr int PIECES = 16 * D / 4 / 64, BATCH = 4;       // pieces per lane, pieces requested together
+        static_assert(PIECES % BATCH == 0, "whole batches");
+        const float qs = a.scale * 1.44269504f;                  // (scores are kept in units of log 2, so that the exponentials below are bare v_exp_f32)
+#pragma unroll
+        for (int b0 = 0; b0 < PIECES; b0 += BATCH) {
+            floatx4 xv[BATCH], bv[BATCH]; floatx2 cv[BATCH], sv[BATCH]; bool ok[BATCH];
+#pragma unroll
+            for (int u = 0; u < BATCH; ++u) {
+                const int p = lane + 64 * (b0 + u);
+                const int col = p / (D / 4), i4 = p % (D / 4);
+                const int qi = col / G, g = col % G;
+                ok[u] = active && tq0 + qi < a.Tq;
+                const int qic = ok[u] ? qi : 0;                  // (a valid address either way; the value is dropped)
+                const long row = (long)b * a.Tq + min(tq0, a.Tq - 1) + (ok[u] ? qic : 0);
+                const int c0 = (kvh * G + g) * D + 4 * i4;
+                xv[u] = *(const floatx4*)(a.qkv + row * a.ldq + c0);
+                bv[u] = *(const floatx4*)(a.bias + c0);
+                if (a.rope_cos) {
+                    const long ro = (long)(min(pos_base, a.pos0 + a.Tq - 1) + qic) * (D / 2) + 2 * i4;
+                    cv[u] = *(const floatx2*)(a.rope_cos + ro); sv[u] = *(const floatx2*)(a.rope_sin + ro);
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < BATCH; ++u) {
+                const int p = lane + 64 * (b0 + u);
+                const int col = p / (D / 4), i4 = p % (D / 4);
+                floatx4 y;
+#pragma unroll
+                for (int pr = 0; pr < 2; ++pr) {
+                    const float x0 = xv[u][2 * pr] + bv[u][2 * pr], x1 = xv[u][2 * pr + 1] + bv[u][2 * pr + 1];
+                    float y0 = x0, y1 = x1;
+                    if (a.rope_cos) rope_pair(x0, x1, cv[u][pr], sv[u][pr], y0, y1);
+                    y[2 * pr] = ok[u] ? qs * y0 : 0.0f; y[2 * pr + 1] = ok[u] ? qs * y1 : 0.0f;
+                }
+                *(floatx4*)(sq + col * D + 4 * i4) = y;
+            }
         }
     }
     __builtin_amdgcn_wave_barrier();
