@@ -102,10 +102,13 @@ def main():
     if not args.no_topp:
         gpu.set_repeat_penalty(2.0)        # DecodingOptions.RepeatPenalty's default; only the top-p leg below applies it
     gpu.prefill(prompts)                   # untimed: loads every kernel and sizes the prefill workspace
-    gpu.reset()
-    t0 = time.perf_counter()
-    gpu.prefill(prompts)
-    t_prefill = time.perf_counter() - t0
+    prefill_runs = []
+    for _ in range(3):                     # host wall clock of the whole call (token upload and final sync included)
+        gpu.reset()
+        t0 = time.perf_counter()
+        gpu.prefill(prompts)
+        prefill_runs.append(time.perf_counter() - t0)
+    t_prefill = min(prefill_runs)
     prefill_tok_s = B * Tp / t_prefill
     prefill_tflops = algorithmic_prefill_flops(cfg, B, Tp) / t_prefill / 1e12
 
@@ -229,7 +232,7 @@ def main():
         "roofline_all": roofline_all,
         "whole_step": {"algorithmic_bytes": round(step_bytes), "achieved_GBps": round(step_gbs, 1),
                        "frac_of_hbm_peak": round(step_gbs / HBM_PEAK_GBS, 4), "host_wall_ms_per_step": round(wall / K * 1e3, 4)},
-        "prefill": {"tokens_per_s": round(prefill_tok_s, 1), "seconds": round(t_prefill, 4),
+        "prefill": {"tokens_per_s": round(prefill_tok_s, 1), "seconds": round(t_prefill, 4), "runs": [round(t, 4) for t in prefill_runs],
                     "algorithmic_TFLOPs": round(prefill_tflops, 2),
                     "frac_of_fp16_mfma_peak": round(prefill_tflops / MFMA_FP16_PEAK_TFLOPS, 4) if cfg["dtype"] == "f16" else None},
         "kernel_ms_per_step": kernel_ms,

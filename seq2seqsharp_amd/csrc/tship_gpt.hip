@@ -842,16 +842,28 @@ static void prefill(TSHipGpt* m, const int32_t* host_ids, int B, int Tp, const i
         aa.qkv = pqkv.as<float>(); aa.KS = 1; aa.split_stride = 0; aa.ldq = qp; aa.pos0 = pos0; aa.Tq = Tp;
         aa.out = po.p; aa.ld_out = m->ldh;
         aa.lens = host_lens ? m->pw_lens.as<int>() : nullptr;
+        // The LDS-tiled QKV projection writes keys and values into the fragment-major cache itself (rotation included)
+        // when its wavefronts' 64 x 128 tiles are whole chunks of whole heads; otherwise a kernel of its own does.
+        const int HD = c.n_heads * m->D, GD = c.n_kv_heads * m->D;
+        const bool fuse_kv = m->f16 && m->vt && pos0 % 32 == 0 && Tp % 32 == 0 && HD % 128 == 0 && GD % 128 == 0 && R >= 512 && L.qkv.KT % 2 == 0 &&
+                             (m->D == 64 || m->D == 128) && !std::getenv("TSHIP_NO_KV_FUSE");
         if (m->f16) {
             BigArgs e; std::memset(&e, 0, sizeof(e));
             e.out = pqkv.as<float>(); e.ld_out = (int)qp; e.bias = L.bqkv.as<float>(); e.n_valid = m->Nqkv;
             if (deferred) e.rinv = prinv.as<float>();
+            if (fuse_kv) {
+                TSHIP_REQUIRE((long)round_up(pos0 + Tp, 32) <= m->ML, "internal: cache chunk beyond the allocation");
+                e.kcache = (half_t*)L.kc.p; e.vcache = (half_t*)L.vc.p; e.kv_max_len = m->ML; e.kv_col0 = HD; e.kv_gd = GD; e.kv_D = m->D;
+                e.kv_hkv = c.n_kv_heads; e.kv_Tq = Tp; e.kv_pos0 = pos0; e.rope_cos = aa.rope_cos; e.rope_sin = aa.rope_sin;
+            }
             big("p_gemm_qkv", L.qkv, pxn.p, m->ldh, BEPI_F32_BIAS, e);
             aa.bias = zero_bias.as<float>();      // bias already added by the GEMM epilogue
         } else {
             run_gemm_f32(m, "p_gemm_qkv", L.qkv, pxn.as<float>(), m->ldh, (int)R, pqkv.as<float>(), qp, 0, 1);
         }
-        if (m->vt && aa.pos0 % 32 == 0) {      // whole fragments, one block per 32-position chunk
+        if (fuse_kv) {
+            // (cache written by the projection)
+        } else if (m->vt && aa.pos0 % 32 == 0) {      // whole fragments, one block per 32-position chunk
             TSHIP_REQUIRE(qp % 4 == 0 && (long)round_up(aa.pos0 + Tp, 32) <= m->ML, "internal: cache chunk beyond the allocation");
             dim3 grid((unsigned)ceil_div(Tp, 32), c.n_kv_heads, B);
             if (m->D == 64) launch(m, "p_kv_write", kv_write_frag_kernel<64>, grid, dim3(256), aa);

@@ -27,6 +27,14 @@ __device__ __forceinline__ float act_apply(int act, float w) {
     return w;
 }
 
+// rotary embedding of one (even, odd) pair, two roundings per output like the reference's C# expression
+// (TensorSharp/TensorApplyCPU.cs:1166-1173)
+__device__ __forceinline__ void rope_pair(float x0, float x1, float c, float s, float& y0, float& y1) {
+#pragma clang fp contract(off)
+    y0 = x0 * c - x1 * s;
+    y1 = x1 * c + x0 * s;
+}
+
 // GEMM inputs of the fp16 decode path are stored "fragment packed": for every k-tile of 16 the 32 rows form the
 // 1 KiB B-operand fragment of v_mfma_f32_32x32x16_f16 (lane l holds row l%32, k = kt*16 + 8*(l/32) .. +7), so a
 // wavefront fetches it with one coalesced 16-byte load per lane.  Index of element (row b, column k):
@@ -553,6 +561,13 @@ struct BigArgs {
     // into xg16 and the sum of squares of every (32-column tile, row) into ssq_out[tile * ssq_ld + row].
     const float* rinv;
     half_t* xg16; int ld_xg; const float* gamma; float* ssq_out; long ssq_ld;
+    // QKV projection of a prefill (BEPI_F32_BIAS, LDS-tiled kernel) writing the cache itself: columns from kv_col0 on are
+    // kv_gd key columns, then kv_gd value columns (head size kv_D, both counts multiples of 128); row r is position
+    // kv_pos0 + r % kv_Tq of sequence r / kv_Tq (kv_pos0 and kv_Tq multiples of 32).  Keys are rotated (rope_cos /
+    // rope_sin [position][kv_D / 2], null: not) and both leave as whole fragments of the fragment-major fp16 cache
+    // [sequence][kv_hkv heads][kv_max_len x kv_D]; only the query columns are stored to `out`.  kcache null: off.
+    half_t* kcache; half_t* vcache; long kv_max_len; int kv_col0, kv_gd, kv_D, kv_hkv, kv_Tq, kv_pos0;
+    const float* rope_cos; const float* rope_sin;
 };
 
 template <int EPI>
@@ -728,6 +743,109 @@ __device__ __forceinline__ void act_store_lines(const BigArgs& a, floatx16 (&acc
     }
 }
 
+// Keys or values of one wavefront of a QKV projection (64 rows = two 32-position chunks, 128 columns) into the
+// fragment-major fp16 cache, in two passes of 64 columns through the wavefront's 64 x 72 halfs of LDS: the accumulators
+// go in row-major (keys rotated first: a lane holds both elements of a pair), whole fragments come out, 16 bytes per lane
+// and 1 KiB per store instruction.  Key fragment (tile, kd) of a chunk: lane (r, qq) holds position 8 (r / 4) + 4 tile +
+// r % 4, elements 32 kd + 8 qq .. + 7; value fragment dt: lane (r, qq) holds element 16 dt + r at positions 8 qq .. + 7
+// (the layouts kv_write_frag_kernel writes).  Same arithmetic per element as the unfused path: acc * rinv + bias, rotation
+// with two roundings per output, one rounding to fp16.
+template <int D, bool IS_K>
+__device__ __forceinline__ void kv_store_frags(const BigArgs& a, floatx16 (&acc)[4][2], int nt_first, long row_first, int lane, half_t* stage,
+                                               const float (&rinv2)[2]) {
+    constexpr int LDSROW = 72, KD = D / 32;
+    const int lh = lane >> 5, r = lane & 31, r16 = lane & 15, qq = lane >> 4;
+    const int rel0 = nt_first * 32 - a.kv_col0 - (IS_K ? 0 : a.kv_gd);        // first column within the key (value) block
+    long cbase[2]; int pos[2]; bool rows_ok[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const long row = row_first + 32 * i;
+        rows_ok[i] = row < a.R;
+        const long rc = rows_ok[i] ? row : 0;
+        const int bq = (int)(rc / a.kv_Tq), tq = (int)(rc % a.kv_Tq);
+        pos[i] = a.kv_pos0 + tq + r;
+        cbase[i] = (long)bq * a.kv_hkv * a.kv_max_len * D + (long)((a.kv_pos0 + tq) >> 5) * (32 * D);
+    }
+#pragma unroll
+    for (int cg = 0; cg < 2; ++cg) {
+        const int relc = rel0 + 64 * cg, kvh = relc / D, dofs = relc % D;
+        floatx4 bb[2][4]; floatx2 cs[2][2][4], sn[2][2][4];
+#pragma unroll
+        for (int jj = 0; jj < 2; ++jj)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                bb[jj][g] = *(const floatx4*)(a.bias + (nt_first + 2 * cg + jj) * 32 + 8 * g + 4 * lh);
+                if (IS_K && a.rope_cos) {
+#pragma unroll
+                    for (int i = 0; i < 2; ++i) {
+                        const long ro = (long)pos[i] * (D / 2) + (dofs + 32 * jj + 8 * g + 4 * lh) / 2;
+                        cs[i][jj][g] = *(const floatx2*)(a.rope_cos + ro); sn[i][jj][g] = *(const floatx2*)(a.rope_sin + ro);
+                    }
+                }
+            }
+#pragma unroll
+        for (int jj = 0; jj < 2; ++jj)
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    float x[4];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) x[e] = acc[2 * cg + jj][i][4 * g + e] * rinv2[i] + bb[jj][g][e];
+                    half4v o;
+                    if (IS_K && a.rope_cos) {
+#pragma unroll
+                        for (int pr = 0; pr < 2; ++pr) {
+                            float y0, y1;
+                            rope_pair(x[2 * pr], x[2 * pr + 1], cs[i][jj][g][pr], sn[i][jj][g][pr], y0, y1);
+                            o[2 * pr] = (half_t)y0; o[2 * pr + 1] = (half_t)y1;
+                        }
+                    } else {
+                        // (the fp32 value is rounded before the conversion, as it is when the projection's output passes
+                        // through memory: a multiply-add fused with the conversion rounds once and differs in one of 2^13 cases)
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) { float xe = x[e]; asm volatile("" : "+v"(xe)); o[e] = (half_t)xe; }
+                    }
+                    *(half4v*)(stage + (32 * i + r) * LDSROW + 32 * jj + 8 * g + 4 * lh) = o;
+                }
+        __builtin_amdgcn_wave_barrier();
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        if (IS_K) {
+            half8 fr[2][2][2];
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int tile = 0; tile < 2; ++tile)
+#pragma unroll
+                    for (int kdl = 0; kdl < 2; ++kdl)
+                        fr[i][tile][kdl] = *(const half8*)(stage + (32 * i + 8 * (r16 >> 2) + 4 * tile + (r16 & 3)) * LDSROW + 32 * kdl + 8 * qq);
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                if (!rows_ok[i]) continue;
+                half_t* dst = a.kcache + cbase[i] + (long)kvh * a.kv_max_len * D + lane * 8;
+#pragma unroll
+                for (int tile = 0; tile < 2; ++tile)
+#pragma unroll
+                    for (int kdl = 0; kdl < 2; ++kdl) *(half8*)(dst + (tile * KD + dofs / 32 + kdl) * 512) = fr[i][tile][kdl];
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                half8 fr[4];
+#pragma unroll
+                for (int dtl = 0; dtl < 4; ++dtl)
+#pragma unroll
+                    for (int jx = 0; jx < 8; ++jx) fr[dtl][jx] = stage[(32 * i + 8 * qq + jx) * LDSROW + 16 * dtl + r16];
+                if (!rows_ok[i]) continue;
+                half_t* dst = a.vcache + cbase[i] + (long)kvh * a.kv_max_len * D + lane * 8;
+#pragma unroll
+                for (int dtl = 0; dtl < 4; ++dtl) *(half8*)(dst + (dofs / 16 + dtl) * 512) = fr[dtl];
+            }
+        }
+        __builtin_amdgcn_wave_barrier();          // the second pass overwrites the stage
+    }
+}
+
 template <int EPI, int NI = 4>      // NI: 32-row tiles per wavefront (the wavefront's rows start at 32 NI wr)
 __device__ __forceinline__ void big_gemm_store(const BigArgs& a, floatx16 (&acc)[4][NI], int nt0, long row0, int wr, int wn, int lane, half_t* stage = nullptr) {
     // accumulator (j, i), lane l, register v = 4 g + e: column (nt0 + 4 wn + j) * 32 + 8 g + 4 (l / 32) + e,
@@ -760,6 +878,18 @@ __device__ __forceinline__ void big_gemm_store(const BigArgs& a, floatx16 (&acc)
         const long rf = row0 + 64 * wr;
         const int ntf = nt0 + 4 * wn;
         constexpr bool RS = EPI == BEPI_RESID;
+        if constexpr (!RS) {
+            // key and value columns of a QKV projection that writes the cache itself (whole wavefronts: the column counts
+            // are multiples of 128, the launch code checks the rest)
+            if (stage && a.kcache && ntf * 32 >= a.kv_col0) {
+                if (ntf >= a.NT) return;
+                const float r2[2] = {rinv4[0], rinv4[1]};
+                const bool is_k = ntf * 32 < a.kv_col0 + a.kv_gd;
+                if (a.kv_D == 64) { if (is_k) kv_store_frags<64, true>(a, acc, ntf, rf, lane, stage, r2); else kv_store_frags<64, false>(a, acc, ntf, rf, lane, stage, r2); }
+                else { if (is_k) kv_store_frags<128, true>(a, acc, ntf, rf, lane, stage, r2); else kv_store_frags<128, false>(a, acc, ntf, rf, lane, stage, r2); }
+                return;
+            }
+        }
         if (stage && rf + 64 <= a.R && ntf + 4 <= a.NT && (ntf + 4) * 32 <= a.n_valid && (a.ld_out & 3) == 0 && (!RS || !a.xg16 || (a.ld_xg & 3) == 0)) {
             const float r2[2] = {rinv4[0], rinv4[1]};
             resid_store_lines<RS>(a, acc[0], ntf + 0, rf, lane, (float*)stage, r2);
@@ -1628,14 +1758,6 @@ struct AttnArgs {
     const int* lens;
 };
 
-// rotary embedding of one (even, odd) pair, two roundings per output like the reference's C# expression
-// (TensorSharp/TensorApplyCPU.cs:1166-1173)
-__device__ __forceinline__ void rope_pair(float x0, float x1, float c, float s, float& y0, float& y1) {
-#pragma clang fp contract(off)
-    y0 = x0 * c - x1 * s;
-    y1 = x1 * c + x0 * s;
-}
-
 // Single-query attention of G query heads that share one KV head over T cached positions.
 // Lanes are grouped LPR to a cache row (16-byte loads, head_dim contiguous); a wavefront covers RPW rows per
 // load and keeps UR loads of keys and of values in flight, refilling each register as soon as it is consumed.
@@ -2467,12 +2589,21 @@ __global__ __launch_bounds__(D == 128 ? 256 : 512) void attn_mfma_prefill_kernel
         for (int i = 0; i < 4; ++i) sq[(dt * 16 + 4 * q + i) * 16 + r16] = acc_o[dt][i];
     __builtin_amdgcn_wave_barrier();
     if (!active) return;
-    for (int col = 0; col < 16; ++col) {
+    // four lanes per column: lane (col, part) divides once and writes D / 4 consecutive outputs of its column as 16-byte pieces
+    {
+        const int col = lane >> 2, part = lane & 3;
         const int qi = col / G, g = col % G;
-        if (tq0 + qi >= a.Tq) break;
-        half_t* out = (half_t*)a.out + ((long)b * a.Tq + tq0 + qi) * a.ld_out + (kvh * G + g) * D;
-        const float inv = 1.0f / sl[w][col];
-        for (int d = lane; d < D; d += 64) out[d] = (half_t)(sq[d * 16 + col] * inv);
+        if (tq0 + qi < a.Tq) {
+            half_t* out = (half_t*)a.out + ((long)b * a.Tq + tq0 + qi) * a.ld_out + (kvh * G + g) * D + part * (D / 4);
+            const float inv = 1.0f / sl[w][col];
+#pragma unroll
+            for (int d8 = 0; d8 < D / 4; d8 += 8) {
+                half8 o;
+#pragma unroll
+                for (int j = 0; j < 8; ++j) o[j] = (half_t)(sq[(part * (D / 4) + d8 + j) * 16 + col] * inv);
+                *(half8*)(out + d8) = o;
+            }
+        }
     }
 }
 

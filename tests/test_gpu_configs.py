@@ -321,3 +321,40 @@ def test_eight_query_heads_per_kv_head(G, oracle, dtype, hidden, heads, kv, batc
         for lg, gl in out:
             assert float(np.abs(gl - lg).max() / np.abs(lg).max()) <= FP32_REL
     gpu.close()
+
+
+@pytest.mark.parametrize("hidden,heads,kv,batch,prompt", [
+    (512, 8, 2, 5, 128),       # head size 64, 640 rows: the last 256-row tile holds one 64-row block and a half
+    (1024, 8, 2, 3, 192),      # head size 128: a wavefront's 128 columns are one head, written in two passes
+    (512, 8, 4, 1, 544),       # one sequence of 17 chunks: the last wavefront's second chunk lies beyond the rows
+])
+def test_projection_writes_the_cache_like_the_separate_kernel(G, oracle, monkeypatch, hidden, heads, kv, batch, prompt):
+    """From 512 rows on, with whole 32-position chunks, the QKV projection's epilogue rotates the keys and writes keys and
+    values into the fragment-major cache itself.  Same cache contents and logits as with the separate cache-write kernel
+    (TSHIP_NO_KV_FUSE=1), and the cache against the oracle's keys and values."""
+    cfg = synth._cfg(n_layers=2, hidden=hidden, n_heads=heads, n_kv_heads=kv, ffn_dim=2 * hidden, vocab=157, attn_type=synth.GQA,
+                     norm_type=synth.RMSNORM, act=synth.SWIGLU, batch=batch, prompt=prompt, steps=2, dtype="f16")
+    w = synth.make_weights(cfg, 77, random_bias=True)
+    seqs = synth.make_prompts(cfg, 78)
+    gpu = G.HipGpt(cfg, w, max_batch=batch, max_seq_len=prompt + 40)
+    gpu.prefill(seqs)
+    fused = [(gpu.get_kv(l, 0), gpu.get_kv(l, 1)) for l in range(2)]
+    lg_fused = gpu.logits()
+    monkeypatch.setenv("TSHIP_NO_KV_FUSE", "1")
+    gpu.reset()
+    gpu.prefill(seqs)
+    monkeypatch.delenv("TSHIP_NO_KV_FUSE")
+    for l in range(2):
+        k, v = gpu.get_kv(l, 0), gpu.get_kv(l, 1)
+        assert np.array_equal(fused[l][0], k), "keys of layer %d" % l
+        assert np.array_equal(fused[l][1], v), "values of layer %d" % l
+    assert np.array_equal(lg_fused, gpu.logits())
+    # appended tokens behind the fused prefill (fewer than 512 rows: the separate kernel) continue the same cache
+    more = synth.make_prompts(dict(cfg, prompt=32), 79)
+    gpu.reset()
+    gpu.prefill(seqs)
+    gpu.prefill(more)
+    orc = oracle.OracleGpt(cfg, w)
+    _, lg = orc.step(np.concatenate([seqs, more], 1), use_cache=True)
+    assert np.abs(gpu.logits() - lg).max() <= FP16_ABS
+    gpu.close()
