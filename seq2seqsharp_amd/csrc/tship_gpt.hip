@@ -13,6 +13,7 @@
 #include "tship_moe_kernels.h"
 #include "tship_sample_kernels.h"
 
+#include <algorithm>
 #include <cmath>
 #include <cstdlib>
 #include <cxxabi.h>
@@ -433,15 +434,20 @@ static void run_gemm_f32(TSHipGpt* m, const char* name, const GemmW& w, const fl
 
 // Y = X * W for many rows (prefill), fp16: LDS-tiled MFMA kernels from 512 rows on, 128 x 128 tiles below.  X row-major
 // with at least round_up(R, 128) rows allocated (the small-tile kernel reads whole row tiles; rows from R on are never stored).
-static void run_big_gemm(TSHipGpt* m, const char* name, const GemmW& w, const void* X, long ldx, long R, int epi, BigArgs e) {
+// n_problems > 1 (LDS-tiled asynchronous kernel only, see big_gemm_batched_ok): e.Wtab / rows_tab / strides describe that many
+// problems of the same shape and at most R rows each, run by one launch.
+static bool big_gemm_batched_ok(const GemmW& w, long R) { return R >= 512 && w.KT % 2 == 0; }
+static void run_big_gemm(TSHipGpt* m, const char* name, const GemmW& w, const void* X, long ldx, long R, int epi, BigArgs e, int n_problems = 1) {
     const long Rp = round_up(R, 128);
     e.W = w.buf.as<half_t>(); e.KT = w.KT; e.NT = w.NT; e.X = (const half_t*)X; e.ldx = (int)ldx; e.R = (int)R;
+    TSHIP_REQUIRE(n_problems == 1 || big_gemm_batched_ok(w, R), "internal: batched launch of a GEMM shape the LDS-tiled kernel does not take");
     if (R >= 512) {       // LDS-tiled kernel, 256 x 256 block tile
         constexpr int CK = 4;
         const unsigned shm = 2u * 2u * 8u * CK * 1024u;
         // one-dimensional grid of 8-row x 4-column tile patches, 32 blocks each, rounded up to whole rounds of 8 patches
         const long CT = ceil_div(w.NT, 8), RT = ceil_div(R, 256), patches = ceil_div(CT, 4) * ceil_div(RT, 8);
         dim3 grid((unsigned)(round_up(patches, 8) * 32));
+        if (n_problems > 1) { e.blocks_per_problem = (int)grid.x; grid.x *= (unsigned)n_problems; }
         if (w.KT % 2 == 0) {      // asynchronous staging: four stages of two k-tiles, eight wavefronts
             if (epi == BEPI_F32_BIAS) launch_shm(m, name, big_gemm3_f16_kernel<BEPI_F32_BIAS>, grid, dim3(512), shm, e);
             else if (epi == BEPI_RESID) launch_shm(m, name, big_gemm3_f16_kernel<BEPI_RESID>, grid, dim3(512), shm, e);

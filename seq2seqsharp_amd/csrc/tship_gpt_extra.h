@@ -97,14 +97,28 @@ static void run_moe_ffn_impl(TSHipGpt* m, LayerW& L, int rows, const ResidNormAr
         half_t* xg = (half_t*)(base + o.xg); half_t* mid = (half_t*)(base + o.mid);
         launch(m, "moe_gather", moe_gather_kernel<half_t>, dim3(rows, E), dim3(256), (const float*)xn32, h, (const int*)counts, (const int*)lists, (int)Bp, xg,
                m->ldh, xg_stride, 0);
-        for (int e = 0; e < E; ++e) {
-            if (n_e[e] == 0) continue;
+        const int n_max = *std::max_element(n_e.begin(), n_e.end());
+        if (big_gemm_batched_ok(*L.e1[0], n_max) && big_gemm_batched_ok(*L.e2[0], n_max) && L.wtab1.p && L.wtab2.p && !std::getenv("TSHIP_NO_MOE_BATCH")) {
+            // all experts in one launch per projection (row counts read on the device): the down projection of one expert
+            // is 64 tiles at 8 x 4096 rows, a quarter of the compute units
             BigArgs e1; std::memset(&e1, 0, sizeof(e1));
-            e1.bias = zero; e1.out16 = mid + e * mid_stride; e1.ld16 = (int)o.ld4h; e1.act = c.act; e1.gated = 0; e1.n_valid = 4 * h;
-            run_big_gemm(m, "moe_gemm1", *L.e1[e], xg + e * xg_stride, m->ldh, n_e[e], BEPI_ACT16, e1);
+            e1.bias = zero; e1.out16 = mid; e1.ld16 = (int)o.ld4h; e1.act = c.act; e1.gated = 0; e1.n_valid = 4 * h;
+            e1.Wtab = (const half_t* const*)L.wtab1.p; e1.rows_tab = counts; e1.x_estride = xg_stride; e1.out16_estride = mid_stride;
+            run_big_gemm(m, "moe_gemm1", *L.e1[0], xg, m->ldh, n_max, BEPI_ACT16, e1, E);
             BigArgs e2; std::memset(&e2, 0, sizeof(e2));
-            e2.bias = zero; e2.out = y + e * y_stride; e2.ld_out = (int)o.ldy; e2.n_valid = h;
-            run_big_gemm(m, "moe_gemm2", *L.e2[e], mid + e * mid_stride, o.ld4h, n_e[e], BEPI_F32_BIAS, e2);
+            e2.bias = zero; e2.out = y; e2.ld_out = (int)o.ldy; e2.n_valid = h;
+            e2.Wtab = (const half_t* const*)L.wtab2.p; e2.rows_tab = counts; e2.x_estride = mid_stride; e2.out_estride = y_stride;
+            run_big_gemm(m, "moe_gemm2", *L.e2[0], mid, o.ld4h, n_max, BEPI_F32_BIAS, e2, E);
+        } else {
+            for (int e = 0; e < E; ++e) {
+                if (n_e[e] == 0) continue;
+                BigArgs e1; std::memset(&e1, 0, sizeof(e1));
+                e1.bias = zero; e1.out16 = mid + e * mid_stride; e1.ld16 = (int)o.ld4h; e1.act = c.act; e1.gated = 0; e1.n_valid = 4 * h;
+                run_big_gemm(m, "moe_gemm1", *L.e1[e], xg + e * xg_stride, m->ldh, n_e[e], BEPI_ACT16, e1);
+                BigArgs e2; std::memset(&e2, 0, sizeof(e2));
+                e2.bias = zero; e2.out = y + e * y_stride; e2.ld_out = (int)o.ldy; e2.n_valid = h;
+                run_big_gemm(m, "moe_gemm2", *L.e2[e], mid + e * mid_stride, o.ld4h, n_e[e], BEPI_F32_BIAS, e2);
+            }
         }
     } else if (m->f16) {
         half_t* xg = (half_t*)(base + o.xg); half_t* mid = (half_t*)(base + o.mid);

@@ -568,6 +568,10 @@ struct BigArgs {
     // [sequence][kv_hkv heads][kv_max_len x kv_D]; only the query columns are stored to `out`.  kcache null: off.
     half_t* kcache; half_t* vcache; long kv_max_len; int kv_col0, kv_gd, kv_D, kv_hkv, kv_Tq, kv_pos0;
     const float* rope_cos; const float* rope_sin;
+    // Several independent problems in one launch of the LDS-tiled kernel (the experts of a MoE layer at prefill): problem
+    // e = blockIdx.x / blocks_per_problem takes its weights from Wtab[e], its row count from rows_tab[e] (read on the
+    // device; blocks beyond it leave at once) and its activations / outputs at fixed strides.  0: one problem.
+    int blocks_per_problem; const half_t* const* Wtab; const int* rows_tab; long x_estride, out_estride, out16_estride;
 };
 
 template <int EPI>
@@ -1171,8 +1175,18 @@ __global__ __launch_bounds__(512) void big_gemm3_f16_kernel(BigArgs a) {
     constexpr int STAGE = 2 * FR * 512;                  // halfs per stage: weight fragments, then activation fragments
     const int t = threadIdx.x, lane = t & 63, w = __builtin_amdgcn_readfirstlane(t >> 6);
     const int wr = w >> 1, wn = w & 1;                   // 4 x 2 wavefronts
+    unsigned bid = blockIdx.x;
+    int rot = 0;
+    if (a.blocks_per_problem) {
+        const int e = (int)(bid / (unsigned)a.blocks_per_problem);
+        bid -= (unsigned)e * (unsigned)a.blocks_per_problem;
+        a.R = a.rows_tab[e]; a.W = a.Wtab[e]; a.X += e * a.x_estride;
+        if (a.out) a.out += e * a.out_estride;
+        if (a.out16) a.out16 += e * a.out16_estride;
+        rot = e;      // a problem with fewer than eight patches would leave XCDs idle: problem e starts on XCD e % 8
+    }
     const int CT = (a.NT + 7) / 8, RT = (int)((a.R + 255) / 256), PC = (CT + 3) / 4;
-    const int xcd = blockIdx.x & 7, seq = blockIdx.x >> 3;
+    const int xcd = (int)((bid - (unsigned)rot) & 7), seq = (int)(bid >> 3);
     const int patch = (seq >> 5) * 8 + xcd, q = seq & 31;
     const int ctile = (patch % PC) * 4 + (q & 3), rtile = (patch / PC) * 8 + (q >> 2);
     if (ctile >= CT || rtile >= RT) return;

@@ -603,3 +603,22 @@ def test_argument_errors(G):
     with pytest.raises(TSHipError, match="shape"):
         G.HipGpt(cfg, bad, max_batch=2, max_seq_len=12)
     gpu.close()
+
+
+def test_moe_prefill_one_launch_for_all_experts_equals_one_per_expert(G, monkeypatch):
+    """From 512 rows per expert on, the prefill runs each projection of all experts as one launch of the LDS-tiled kernel
+    (weights by pointer table, row counts read on the device).  Same logits, bit for bit, as one launch per expert
+    (TSHIP_NO_MOE_BATCH=1), also when an expert holds far fewer rows than the largest one."""
+    cfg = synth.tiny_config(n_layers=3, n_experts=4, experts_per_token=1, norm_type=synth.LAYERNORM, act=synth.RELU, dtype="f16",
+                            batch=5, prompt=520, vocab=300)
+    w = synth.make_weights(cfg, 62, random_bias=True)
+    seqs = synth.make_prompts(cfg, 162)
+    gpu = G.HipGpt(cfg, w, max_batch=5, max_seq_len=530)
+    gpu.prefill(seqs)
+    one = gpu.logits()
+    monkeypatch.setenv("TSHIP_NO_MOE_BATCH", "1")
+    gpu.reset()
+    gpu.prefill(seqs)
+    monkeypatch.delenv("TSHIP_NO_MOE_BATCH")
+    assert np.array_equal(one, gpu.logits())
+    gpu.close()
