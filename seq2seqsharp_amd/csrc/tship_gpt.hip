@@ -445,8 +445,18 @@ static void run_big_gemm(TSHipGpt* m, const char* name, const GemmW& w, const vo
         constexpr int CK = 4;
         const unsigned shm = 2u * 2u * 8u * CK * 1024u;
         // one-dimensional grid of 8-row x 4-column tile patches, 32 blocks each, rounded up to whole rounds of 8 patches
-        const long CT = ceil_div(w.NT, 8), RT = ceil_div(R, 256), patches = ceil_div(CT, 4) * ceil_div(RT, 8);
+        const long CT = ceil_div(w.NT, 8), RT = ceil_div(R, 256);
+        long patches = ceil_div(CT, 4) * ceil_div(RT, 8);
         dim3 grid((unsigned)(round_up(patches, 8) * 32));
+        if (w.KT % 2 == 0 && n_problems == 1) {
+            // fewer than eight patches would leave XCDs without work: flatter patches (4, 2 or 1 row tiles)
+            int ph = 8;
+            while (ph > 1 && ceil_div(CT, 4) * ceil_div(RT, ph) < 8) ph /= 2;
+            if (const char* v = std::getenv("TSHIP_PATCH_ROWS")) ph = std::max(1, std::min(8, std::atoi(v)));      // (tests: 1, 2, 4 or 8)
+            patches = ceil_div(CT, 4) * ceil_div(RT, ph);
+            e.patch_rows = ph;
+            grid.x = (unsigned)(round_up(patches, 8) * 4 * ph);
+        }
         if (n_problems > 1) { e.blocks_per_problem = (int)grid.x; grid.x *= (unsigned)n_problems; }
         if (w.KT % 2 == 0) {      // asynchronous staging: four stages of two k-tiles, eight wavefronts
             if (epi == BEPI_F32_BIAS) launch_shm(m, name, big_gemm3_f16_kernel<BEPI_F32_BIAS>, grid, dim3(512), shm, e);

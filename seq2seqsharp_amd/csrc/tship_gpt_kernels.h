@@ -572,6 +572,9 @@ struct BigArgs {
     // e = blockIdx.x / blocks_per_problem takes its weights from Wtab[e], its row count from rows_tab[e] (read on the
     // device; blocks beyond it leave at once) and its activations / outputs at fixed strides.  0: one problem.
     int blocks_per_problem; const half_t* const* Wtab; const int* rows_tab; long x_estride, out_estride, out16_estride;
+    // LDS-tiled asynchronous kernel: row tiles per XCD patch (8, or fewer for launches that would otherwise fill fewer
+    // than eight patches and leave XCDs idle); 0 means 8
+    int patch_rows;
 };
 
 template <int EPI>
@@ -1187,8 +1190,9 @@ __global__ __launch_bounds__(512) void big_gemm3_f16_kernel(BigArgs a) {
     }
     const int CT = (a.NT + 7) / 8, RT = (int)((a.R + 255) / 256), PC = (CT + 3) / 4;
     const int xcd = (int)((bid - (unsigned)rot) & 7), seq = (int)(bid >> 3);
-    const int patch = (seq >> 5) * 8 + xcd, q = seq & 31;
-    const int ctile = (patch % PC) * 4 + (q & 3), rtile = (patch / PC) * 8 + (q >> 2);
+    const int PH = a.patch_rows ? a.patch_rows : 8;          // a patch: PH row tiles x 4 column tiles
+    const int patch = (seq / (4 * PH)) * 8 + xcd, q = seq % (4 * PH);
+    const int ctile = (patch % PC) * 4 + (q & 3), rtile = (patch / PC) * PH + (q >> 2);
     if (ctile >= CT || rtile >= RT) return;
     const int nt0 = ctile * 8;
     const long row0 = (long)rtile * 256;
