@@ -35,6 +35,27 @@ __device__ __forceinline__ void rope_pair(float x0, float x1, float c, float s, 
     y1 = x1 * c + x0 * s;
 }
 
+// op(v[l], v[l ^ 16]) and op(v[l], v[l ^ 32]) in every lane with v_permlane16_swap / v_permlane32_swap (gfx950): the swap
+// of a register with its own copy leaves the lower partner's value in one result and the upper partner's in the other, in
+// all lanes, so the reduction needs no trip through LDS (ds_bpermute: two dependent LDS round trips per softmax step) and
+// adds the two partners in the same order in both lanes.
+__device__ __forceinline__ float max_xor16(float v) {
+    const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float max_xor32(float v) {
+    const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float sum_xor16(float v) {
+    const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+__device__ __forceinline__ float sum_xor32(float v) {
+    const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+
 // GEMM inputs of the fp16 decode path are stored "fragment packed": for every k-tile of 16 the 32 rows form the
 // 1 KiB B-operand fragment of v_mfma_f32_32x32x16_f16 (lane l holds row l%32, k = kt*16 + 8*(l/32) .. +7), so a
 // wavefront fetches it with one coalesced 16-byte load per lane.  Index of element (row b, column k):
@@ -2272,8 +2293,7 @@ __global__ __launch_bounds__(D == 128 ? 256 : 512) void attn_mfma_kernel(AttnArg
         float cm = -INFINITY;
 #pragma unroll
         for (int j = 0; j < 8; ++j) cm = fmaxf(cm, s[j]);
-        cm = fmaxf(cm, __shfl_xor(cm, 16, 64));
-        cm = fmaxf(cm, __shfl_xor(cm, 32, 64));
+        cm = max_xor32(max_xor16(cm));
         // (a chunk that is processed has a visible position, so m_new is finite; exp2(-inf) = 0 covers hidden positions
         // and the first chunk's m_run)
         const float m_new = fmaxf(m_run, cm);
@@ -2336,8 +2356,7 @@ __global__ __launch_bounds__(D == 128 ? 256 : 512) void attn_mfma_kernel(AttnArg
     };
     if (n_own >= 1) chain(chain, std::integral_constant<int, 0>{}, kfA, vfA);
     // the four lane groups of a column saw different positions: add their sums (the maximum is already common)
-    l_run += __shfl_xor(l_run, 16, 64);
-    l_run += __shfl_xor(l_run, 32, 64);
+    l_run = sum_xor32(sum_xor16(l_run));
     if (q == 0) { sM[w][r16] = m_run; sL[w][r16] = l_run; }
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt)
@@ -2432,9 +2451,10 @@ __global__ __launch_bounds__(D == 128 ? 256 : 512) void attn_mfma_prefill_kernel
     constexpr int NF = 2 * KD + DT;          // 1 KiB fragments per chunk: keys (tile, kd), then values (dt)
     constexpr int FPW = NF / NW;             // fragments a wavefront brings per chunk
     static_assert(NF % NW == 0, "fragments must divide among the wavefronts");
-    __shared__ float sbuf[NW][D * 16];       // per wavefront: Q staging [16 columns][D], later the outputs [D][16 columns]
+    __shared__ __attribute__((aligned(16))) float sbuf[NW][D * 16];       // per wavefront: Q staging [16 columns][D], later the outputs [D][16 columns]
     __shared__ float sl[NW][16];
     __shared__ __attribute__((aligned(16))) half_t schunk[2][NF * 512];
+    static_assert(sizeof(sbuf) >= NF * 1024, "the third chunk stage lives in the query / output staging area");
     const int lane = threadIdx.x & 63, w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int r16 = lane & 15, q = lane >> 4;
     const int kvh = blockIdx.y, b = blockIdx.z;
@@ -2450,15 +2470,20 @@ __global__ __launch_bounds__(D == 128 ? 256 : 512) void attn_mfma_prefill_kernel
     const half_t* Vt = (const half_t*)a.vcache + ((long)b * a.Hkv + kvh) * (long)D * a.max_len;
     typedef const void __attribute__((address_space(1)))* gptr_t;
     typedef void __attribute__((address_space(3)))* lptr_t;
-    auto fetch = [&](int c) {                // this wavefront's fragments of chunk c -> stage c % 2
+    // Three chunk stages: two of their own and, while the chunks are walked, the first NF KiB of the staging area (free
+    // between the query prologue and the output epilogue; the barriers of the first and behind the last chunk fence it).
+    auto stage_of = [&](int c) -> half_t* { const int st = c % 3; return st == 2 ? (half_t*)&sbuf[0][0] : schunk[st]; };
+    auto fetch = [&](int c) {                // this wavefront's fragments of chunk c -> stage c % 3
+        half_t* dst = stage_of(c);
 #pragma unroll
         for (int i = 0; i < FPW; ++i) {
             const int f = w + i * NW;
             const half_t* src = (f < 2 * KD ? Kb + (long)c * (32 * D) + f * 512 : Vt + (long)c * (32 * D) + (f - 2 * KD) * 512) + lane * 8;
-            __builtin_amdgcn_global_load_lds((gptr_t)src, (lptr_t)(&schunk[c & 1][f * 512]), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds((gptr_t)src, (lptr_t)(dst + f * 512), 16, 0, 0);
         }
     };
     fetch(0);
+    if (nchunks > 1) fetch(1);
 
     // queries: projection + bias, rotary embedding, 1 / sqrt(d); columns beyond the prompt stay zero.  A lane takes
     // four consecutive elements (two rotary pairs) of a column at a time; the requests of four such pieces go out
@@ -2539,8 +2564,7 @@ __global__ __launch_bounds__(D == 128 ? 256 : 512) void attn_mfma_prefill_kernel
             if (MASKED && t0 + 8 * q + j > tmax) s[j] = -INFINITY;       // causal mask (adding -30000 gives exactly 0 after exp in fp32 too)
             cm = fmaxf(cm, s[j]);
         }
-        cm = fmaxf(cm, __shfl_xor(cm, 16, 64));
-        cm = fmaxf(cm, __shfl_xor(cm, 32, 64));
+        cm = max_xor32(max_xor16(cm));
         const float m_new = fmaxf(m_run, cm);
         // (unmasked chunks have finite scores, so m_new is finite and exp2(-inf - m_new) = 0 covers the first chunk)
         const float corr = (MASKED && m_new == -INFINITY) ? 1.0f : __builtin_amdgcn_exp2f(m_run - m_new);
@@ -2570,24 +2594,30 @@ __global__ __launch_bounds__(D == 128 ? 256 : 512) void attn_mfma_prefill_kernel
     // One loop per kind of chunk (unmasked, masked, not this wavefront's): with the kinds as branches of one loop the
     // compiler copies the running outputs between registers around every branch, a third of the loop's instructions.
     // Every wavefront passes the same nchunks barriers whatever its split.
+    // Chunks are requested two ahead.  The fragment reads and their waits are written out: the compiler cannot tell which
+    // LDS bytes a load in flight will write and would wait for all of them before any LDS read.
     auto step = [&](auto mode_c, int c) {
         constexpr int MODE = decltype(mode_c)::value;         // 0: unmasked, 1: masked, 2: only the block's fetch and barrier
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");      // this wavefront's share of chunk c has landed
-        __syncthreads();                                      // ... and everybody's; chunk c - 1 is consumed
-        if (MODE == 2) { if (c + 1 < nchunks) fetch(c + 1); return; }
+        // this wavefront's share of chunk c has landed once only the requests of chunk c + 1 are outstanding
+        if (c + 1 < nchunks) asm volatile("s_waitcnt vmcnt(%0)" :: "n"(FPW) : "memory");
+        else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __builtin_amdgcn_s_barrier();                         // ... and everybody's; chunk c - 1 is consumed
+        if (MODE == 2) { if (c + 2 < nchunks) fetch(c + 2); return; }
         half8 kf[2][KD], vf[DT];
-        const half_t* st = schunk[c & 1] + lane * 8;
+        const unsigned sa = (unsigned)(size_t)(lptr_t)stage_of(c) + lane * 16;
 #pragma unroll
         for (int tile = 0; tile < 2; ++tile)
 #pragma unroll
-            for (int kd = 0; kd < KD; ++kd) kf[tile][kd] = *(const half8*)(st + (tile * KD + kd) * 512);
+            for (int kd = 0; kd < KD; ++kd) asm volatile("ds_read_b128 %0, %1 offset:%2" : "=&v"(kf[tile][kd]) : "v"(sa), "n"((tile * KD + kd) * 1024) : "memory");
 #pragma unroll
-        for (int dt = 0; dt < DT; ++dt) vf[dt] = *(const half8*)(st + (2 * KD + dt) * 512);
-        // the operands are in registers before the next chunk is requested into the other stage, so the wait the
-        // compiler puts ahead of LDS reads (they might alias the LDS destination of a load in flight) costs nothing
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        for (int dt = 0; dt < DT; ++dt) asm volatile("ds_read_b128 %0, %1 offset:%2" : "=&v"(vf[dt]) : "v"(sa), "n"((2 * KD + dt) * 1024) : "memory");
+        if (c + 2 < nchunks) fetch(c + 2);                    // into the stage of chunk c - 1
+        if constexpr (D == 64)
+            asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(kf[0][0]), "+v"(kf[0][1]), "+v"(kf[1][0]), "+v"(kf[1][1]), "+v"(vf[0]), "+v"(vf[1]), "+v"(vf[2]), "+v"(vf[3]) :: "memory");
+        else
+            asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(kf[0][0]), "+v"(kf[0][1]), "+v"(kf[0][2]), "+v"(kf[0][3]), "+v"(kf[1][0]), "+v"(kf[1][1]), "+v"(kf[1][2]), "+v"(kf[1][3]),
+                         "+v"(vf[0]), "+v"(vf[1]), "+v"(vf[2]), "+v"(vf[3]), "+v"(vf[4]), "+v"(vf[5]), "+v"(vf[6]), "+v"(vf[7]) :: "memory");
         __builtin_amdgcn_sched_barrier(0);
-        if (c + 1 < nchunks) fetch(c + 1);
         if (MODE == 0) do_chunk(plain, c, kf, vf); else do_chunk(masked, c, kf, vf);
     };
     {
@@ -2596,10 +2626,9 @@ __global__ __launch_bounds__(D == 128 ? 256 : 512) void attn_mfma_prefill_kernel
         for (; c < n_own; ++c) step(std::integral_constant<int, 1>{}, c);
         for (; c < nchunks; ++c) step(std::integral_constant<int, 2>{}, c);
     }
-    l_run += __shfl_xor(l_run, 16, 64);
-    l_run += __shfl_xor(l_run, 32, 64);
+    l_run = sum_xor32(sum_xor16(l_run));
     // outputs through this wavefront's LDS slice so that rows go out contiguously: O^T[d][col] -> out[row(col)][d]
-    __builtin_amdgcn_wave_barrier();          // the Q staging has been consumed
+    __builtin_amdgcn_s_barrier();             // every wavefront has read its last chunk (the third stage shares this memory)
     if (q == 0) sl[w][r16] = l_run;
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt)
