@@ -127,6 +127,7 @@ struct TSHipGpt {
     static constexpr int MAX_ATTN_SPLITS = 16;
     DevBuf attn_xchg, attn_count;  // decode attention with several blocks per (row, KV head): partial sums and one counter per pair
     bool any_blocked = false;
+    bool embed_done = false;       // the sampling kernel of this step has already done the next step's embedding (greedy_embed_kernel)
     DevBuf blocked;                // one byte per token, non-zero = DecodingOptions.BlockedTokens (allocated with the model: graphs keep its address)
     int cur_batch = 0;
     std::vector<std::string> last_symbols;      // launched symbols of the last profiled step, in launch order
@@ -571,7 +572,8 @@ static void run_moe_ffn(TSHipGpt* m, LayerW& L, int rows, const ResidNormArgs& p
 static void run_moe_ffn_prefill(TSHipGpt* m, LayerW& L, int rows, const ResidNormArgs& pre, const int* last_rows, int n_last);
 static void moe_alloc(TSHipGpt* m);
 static void moe_get_routing(TSHipGpt* m, int layer, float* top_idx, float* top_val, float* probs);
-static void sample_tokens(TSHipGpt* m, int mode, float top_p, float temperature, const float* host_uniforms, const float* dev_uniforms, int B, int* gen_out, const int* d_step, bool record);
+static void sample_tokens(TSHipGpt* m, int mode, float top_p, float temperature, const float* host_uniforms, const float* dev_uniforms, int B, int* gen_out, const int* d_step, bool record,
+                          bool embed_next = false);
 // tokens `d_ids` [rows][Tq] enter the sequences at indices pos0 ..: remember where each token occurred last
 static void record_history(TSHipGpt* m, const int* d_ids, int rows, int Tq, int pos0) {
     if (!m->last_pos.p) return;
@@ -591,6 +593,14 @@ static void record_history(TSHipGpt* m, const int* d_ids, int rows, int Tq, int 
 // rinv = 1 / sqrt(mean(x^2) + eps) is rebuilt by every consumer from the tile sums, so no launch exists only to
 // normalise (RMSNormalization.Norm, Seq2SeqSharp/Layers/RMSNormalization.cs:33-37, folded into its neighbours).
 // ------------------------------------------------------------------------------------------------
+// first kernel of a decode step on the fused-norm path: embedding row x sqrt(h), the first layer's normalisation input, sums of squares
+static FnPrepArgs embed_prepare_args(TSHipGpt* m, const int* d_ids) {
+    const int h = m->c.hidden;
+    FnPrepArgs a; std::memset(&a, 0, sizeof(a));
+    a.x = m->x.as<float>(); a.ldx = h; a.h = h; a.ids = d_ids; a.emb = m->emb.p; a.emb_f16 = 1; a.emb_scale = (float)std::sqrt((double)h);
+    a.gamma = m->L[0]->n1_g.as<float>(); a.xg16 = m->xn.as<half_t>(); a.xg_kt = (int)(m->ldh / 16); a.ssq_out = m->ssq.as<float>(); a.ssq_ld = m->Bpad;
+    return a;
+}
 static void decode_step_fn(TSHipGpt* m, const int* d_ids, int B) {
     auto& c = m->c;
     const int h = c.hidden, F = c.ffn_dim;
@@ -603,10 +613,10 @@ static void decode_step_fn(TSHipGpt* m, const int* d_ids, int B) {
         e.bias = bias; e.n_valid = h; e.x = m->x.as<float>(); e.ldx_res = h; e.gamma = gamma;
         e.xg16 = m->xn.as<half_t>(); e.xg_kt = xkt; e.ssq_out = ssq; e.ssq_out_ld = m->Bpad;
     };
-    {
-        FnPrepArgs a; std::memset(&a, 0, sizeof(a));
-        a.x = m->x.as<float>(); a.ldx = h; a.h = h; a.ids = d_ids; a.emb = m->emb.p; a.emb_f16 = 1; a.emb_scale = (float)std::sqrt((double)h);
-        a.gamma = m->L[0]->n1_g.as<float>(); a.xg16 = m->xn.as<half_t>(); a.xg_kt = xkt; a.ssq_out = ssq; a.ssq_ld = m->Bpad;
+    if (m->embed_done) {
+        m->embed_done = false;        // (the greedy sampling kernel went on to embed the tokens it chose)
+    } else {
+        FnPrepArgs a = embed_prepare_args(m, d_ids);
         if (h <= 2048) launch(m, "embed_prepare", fn_prepare_kernel<8>, dim3(B), dim3(256), a);
         else if (h <= 4096) launch(m, "embed_prepare", fn_prepare_kernel<16>, dim3(B), dim3(256), a);
         else launch(m, "embed_prepare", fn_prepare_kernel<32>, dim3(B), dim3(256), a);
@@ -1203,6 +1213,7 @@ TSHIP_API int TSHip_GptDecode(TSHipGpt* m, const int32_t* host_ids, int batch) {
     for (int i = 0; i < batch; ++i) TSHIP_REQUIRE(host_ids[i] >= 0 && host_ids[i] < m->c.vocab, "TSHip_GptDecode: token id out of range");
     TSHIP_CHECK_HIP(hipMemcpyAsync(m->ids.p, host_ids, batch * sizeof(int), hipMemcpyHostToDevice, stream()));
     TSHIP_CHECK_HIP(hipStreamSynchronize(stream()));
+    m->embed_done = false;          // (set only between a sampling kernel and the decode step that follows it at once)
     record_history(m, m->ids.as<int>(), batch, 1, m->pos);
     decode_step(m, m->ids.as<int>(), batch);
     TSHIP_CHECK_HIP(hipStreamSynchronize(stream()));
@@ -1230,6 +1241,7 @@ static int generate_impl(TSHipGpt* m, int n_steps, int mode, float top_p, float 
     TSHIP_REQUIRE(m->cur_batch > 0, "TSHip_GptGenerate: no logits yet; prefill first");
     TSHIP_REQUIRE(n_steps >= 1, "TSHip_GptGenerate: n_steps must be positive");
     TSHIP_REQUIRE(m->pos + n_steps <= m->c.max_seq_len, "TSHip_GptGenerate: KV cache too small for n_steps (max_seq_len)");
+    m->embed_done = false;
     TSHIP_REQUIRE(mode == TSHIP_GREEDY || (mode == TSHIP_TOPP && host_uniforms), "TSHip_GptGenerate: top-p needs the uniform stream");
     const int B = m->cur_batch;
     // token and uniform buffers live in the model so that the captured step graph stays valid across calls
@@ -1266,9 +1278,9 @@ static int generate_impl(TSHipGpt* m, int n_steps, int mode, float top_p, float 
             TSHIP_CHECK_HIP(hipStreamBeginCapture(stream(), hipStreamCaptureModeThreadLocal));
             const int saved_pos = m->pos;
             try {
-                sample_tokens(m, mode, top_p, temperature, nullptr, uni_base, B, gen.as<int>(), d_step, true);
+                sample_tokens(m, mode, top_p, temperature, nullptr, uni_base, B, gen.as<int>(), d_step, true, true);
                 decode_step(m, m->ids.as<int>(), B);
-            } catch (...) { hipGraph_t g2 = nullptr; (void)hipStreamEndCapture(stream(), &g2); if (g2) (void)hipGraphDestroy(g2); m->pos = saved_pos; throw; }
+            } catch (...) { hipGraph_t g2 = nullptr; (void)hipStreamEndCapture(stream(), &g2); if (g2) (void)hipGraphDestroy(g2); m->pos = saved_pos; m->embed_done = false; throw; }
             m->pos = saved_pos;                    // capturing launched nothing
             TSHIP_CHECK_HIP(hipStreamEndCapture(stream(), &graph));
             hipError_t ge = hipGraphInstantiate(&m->step_graph, graph, nullptr, nullptr, 0);
@@ -1287,7 +1299,7 @@ static int generate_impl(TSHipGpt* m, int n_steps, int mode, float top_p, float 
     for (int s = 0; s < n_steps; ++s) {
         if (use_graph) { TSHIP_CHECK_HIP(hipGraphLaunch(m->step_graph, stream())); m->pos += 1; }
         else {
-            sample_tokens(m, mode, top_p, temperature, nullptr, uni_base, B, gen.as<int>(), d_step, true);
+            sample_tokens(m, mode, top_p, temperature, nullptr, uni_base, B, gen.as<int>(), d_step, true, true);
             decode_step(m, m->ids.as<int>(), B);
         }
         done = s + 1;
@@ -1537,6 +1549,7 @@ TSHIP_API int TSHip_GptProfileDecode(TSHipGpt* m, const int32_t* host_ids, int b
     TSHIP_CHECK_HIP(hipStreamSynchronize(stream()));
     Profiler prof;
     m->prof = &prof;
+    m->embed_done = false;          // (set only between a sampling kernel and the decode step that follows it at once)
     record_history(m, m->ids.as<int>(), batch, 1, m->pos);
     try { decode_step(m, m->ids.as<int>(), batch); } catch (...) { m->prof = nullptr; throw; }
     m->prof = nullptr;

@@ -195,14 +195,26 @@ static void run_moe_ffn_prefill(TSHipGpt* m, LayerW& L, int rows, const ResidNor
 // next tokens from the logits on the device -> m->ids (and gen_out); greedy or top-p.
 // With d_step set, gen_out and dev_uniforms are bases indexed by the device step counter (graph replays).
 // record: the chosen tokens are about to be appended (generate loop), so their position enters the token history.
+// embed_next: a decode step on these tokens follows at once (the generate loop): on the fused-norm path the greedy kernel
+// then also does that step's first kernel for its row and sets m->embed_done.
 static void sample_tokens(TSHipGpt* m, int mode, float top_p, float temperature, const float* host_uniforms, const float* dev_uniforms, int B,
-                          int* gen_out, const int* d_step, bool record) {
+                          int* gen_out, const int* d_step, bool record, bool embed_next) {
     const long Vp = round_up(m->c.vocab, 32);
     int* last = m->last_pos.as<int>();           // null unless a repeat penalty was set
     if (last) TSHIP_REQUIRE((size_t)B * m->last_ld * sizeof(int) <= m->last_pos.bytes && m->last_ld >= m->c.vocab, "internal: token history table too small");
     if (mode == TSHIP_GREEDY) {
-        launch(m, "greedy", greedy_kernel, dim3(B), dim3(1024), (const float*)m->logits.as<float>(), Vp, m->c.vocab, m->ids.as<int>(), gen_out, d_step,
-               record ? last : (int*)nullptr, m->last_ld, (const int*)m->d_pos.as<int>(), m->any_blocked ? (const unsigned char*)m->blocked.p : (const unsigned char*)nullptr);
+        const float* lg = m->logits.as<float>(); int* ids = m->ids.as<int>(); int* lastp = record ? last : (int*)nullptr;
+        const int* dpos = m->d_pos.as<int>(); const unsigned char* bl = m->any_blocked ? (const unsigned char*)m->blocked.p : (const unsigned char*)nullptr;
+        if (embed_next && m->fused_norm && m->c.hidden <= 8192) {
+            const FnPrepArgs pa = embed_prepare_args(m, ids);
+            const int h = m->c.hidden;
+            if (h <= 2048) launch(m, "greedy_embed", greedy_embed_kernel<2>, dim3(B), dim3(1024), lg, Vp, m->c.vocab, ids, gen_out, d_step, lastp, m->last_ld, dpos, bl, pa);
+            else if (h <= 4096) launch(m, "greedy_embed", greedy_embed_kernel<4>, dim3(B), dim3(1024), lg, Vp, m->c.vocab, ids, gen_out, d_step, lastp, m->last_ld, dpos, bl, pa);
+            else launch(m, "greedy_embed", greedy_embed_kernel<8>, dim3(B), dim3(1024), lg, Vp, m->c.vocab, ids, gen_out, d_step, lastp, m->last_ld, dpos, bl, pa);
+            m->embed_done = true;
+            return;
+        }
+        launch(m, "greedy", greedy_kernel, dim3(B), dim3(1024), lg, Vp, m->c.vocab, ids, gen_out, d_step, lastp, m->last_ld, dpos, bl);
         return;
     }
     TSHIP_REQUIRE(mode == TSHIP_TOPP, "unknown sampling mode");

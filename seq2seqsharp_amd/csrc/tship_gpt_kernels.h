@@ -1740,23 +1740,22 @@ struct FnPrepArgs {
     const float* gamma; half_t* xg16; int xg_kt; float* ssq_out; long ssq_ld;
     long xg_ld;             // xg_kt == 0: xg16 is row-major with this leading dimension
 };
-template <int NPT>
-__global__ __launch_bounds__(256) void fn_prepare_kernel(FnPrepArgs a) {
-    const int r = blockIdx.x, t = threadIdx.x;
-    const long erow = a.ids ? (long)a.ids[r] : 0;
+// (row r of the launch; erow: embedding row when a.ids is set; NT threads, NPT elements each)
+template <int NPT, int NT>
+__device__ __forceinline__ void fn_prepare_row(const FnPrepArgs& a, int r, long erow, int t) {
     const long srow = a.row_map ? a.row_map[r] : r;
     // all requests first (unconditional, the column clamped), then the arithmetic and the stores
     float vin[NPT], gmv[NPT];
 #pragma unroll
     for (int i = 0; i < NPT; ++i) {
-        const int c = min(t + i * 256, a.h - 1);
+        const int c = min(t + i * NT, a.h - 1);
         if (a.ids) vin[i] = a.emb_f16 ? (float)((const half_t*)a.emb)[erow * a.h + c] : ((const float*)a.emb)[erow * a.h + c];
         else vin[i] = a.src[srow * a.ld_src + c];
         gmv[i] = a.gamma[c];
     }
 #pragma unroll
     for (int i = 0; i < NPT; ++i) {
-        const int c = t + i * 256;
+        const int c = t + i * NT;
         float v = 0.0f;
         if (c < a.h) {
             v = a.ids ? vin[i] * a.emb_scale : vin[i];
@@ -1769,6 +1768,11 @@ __global__ __launch_bounds__(256) void fn_prepare_kernel(FnPrepArgs a) {
         for (int o = 16; o > 0; o >>= 1) q += __shfl_xor(q, o, 64);
         if ((t & 31) == 0 && c < a.h) a.ssq_out[(long)(c >> 5) * a.ssq_ld + r] = q;
     }
+}
+template <int NPT>
+__global__ __launch_bounds__(256) void fn_prepare_kernel(FnPrepArgs a) {
+    const int r = blockIdx.x;
+    fn_prepare_row<NPT, 256>(a, r, a.ids ? (long)a.ids[r] : 0, threadIdx.x);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -2664,12 +2668,14 @@ __global__ __launch_bounds__(D == 128 ? 256 : 512) void attn_mfma_prefill_kernel
 // blocked (optional): one byte per token; the reference adds -1 to the probabilities of blocked tokens
 // (Decoder.cs:745-753), which puts them below every other token: they are left out here.  (A blocked token could
 // only win there if every other probability had underflowed to zero.)
-__global__ __launch_bounds__(1024) void greedy_kernel(const float* __restrict__ logits, long ld, int V, int* __restrict__ next_ids,
-                                                      int* __restrict__ gen_out, const int* __restrict__ d_step,
-                                                      int* __restrict__ last_pos, long last_ld, const int* __restrict__ d_len,
-                                                      const unsigned char* __restrict__ blocked) {
+// (1024 threads; the chosen token is returned to every thread)
+__device__ __forceinline__ int greedy_row(const float* __restrict__ logits, long ld, int V, int* __restrict__ next_ids,
+                                          int* __restrict__ gen_out, const int* __restrict__ d_step,
+                                          int* __restrict__ last_pos, long last_ld, const int* __restrict__ d_len,
+                                          const unsigned char* __restrict__ blocked) {
     __shared__ float sv[16];
     __shared__ int si[16];
+    __shared__ int s_tok;
     const int b = blockIdx.x, t = threadIdx.x;
     const float* row = logits + (long)b * ld;
     float best = -INFINITY; int bi = 0x7fffffff;
@@ -2703,7 +2709,27 @@ __global__ __launch_bounds__(1024) void greedy_kernel(const float* __restrict__ 
         next_ids[b] = bi;
         if (gen_out) gen_out[(d_step ? (long)*d_step * gridDim.x : 0) + b] = bi;
         if (last_pos) last_pos[(long)b * last_ld + bi] = *d_len;
+        s_tok = bi;
     }
+    __syncthreads();
+    return s_tok;
+}
+__global__ __launch_bounds__(1024) void greedy_kernel(const float* __restrict__ logits, long ld, int V, int* __restrict__ next_ids,
+                                                      int* __restrict__ gen_out, const int* __restrict__ d_step,
+                                                      int* __restrict__ last_pos, long last_ld, const int* __restrict__ d_len,
+                                                      const unsigned char* __restrict__ blocked) {
+    greedy_row(logits, ld, V, next_ids, gen_out, d_step, last_pos, last_ld, d_len, blocked);
+}
+// The same, and the block goes on with what the next decode step would do first for its row: the embedding of the chosen
+// token times sqrt(h), the first layer's normalisation input and its sums of squares (fn_prepare_kernel): one launch and
+// one trip through memory for the token less per generated token.
+template <int NPT>
+__global__ __launch_bounds__(1024) void greedy_embed_kernel(const float* __restrict__ logits, long ld, int V, int* __restrict__ next_ids,
+                                                            int* __restrict__ gen_out, const int* __restrict__ d_step,
+                                                            int* __restrict__ last_pos, long last_ld, const int* __restrict__ d_len,
+                                                            const unsigned char* __restrict__ blocked, FnPrepArgs pa) {
+    const int tok = greedy_row(logits, ld, V, next_ids, gen_out, d_step, last_pos, last_ld, d_len, blocked);
+    fn_prepare_row<NPT, 1024>(pa, blockIdx.x, tok, threadIdx.x);
 }
 
 }  // namespace tship
