@@ -358,3 +358,23 @@ def test_projection_writes_the_cache_like_the_separate_kernel(G, oracle, monkeyp
     _, lg = orc.step(np.concatenate([seqs, more], 1), use_cache=True)
     assert np.abs(gpu.logits() - lg).max() <= FP16_ABS
     gpu.close()
+
+
+@pytest.mark.parametrize("patch_rows", ["1", "2", "4", "8"])
+def test_prefill_tile_patch_heights_give_the_same_bits(G, monkeypatch, patch_rows):
+    """The LDS-tiled prefill GEMM maps its blocks to tiles in patches of (8, 4, 2 or 1) x 4 tiles per XCD, chosen from the
+    launch size; the mapping must not change any result.  1536 rows x 512 columns: 6 x 2 tiles, fewer than eight patches at
+    every height, against the height the launch code picks."""
+    cfg = synth._cfg(n_layers=2, hidden=512, n_heads=8, n_kv_heads=2, ffn_dim=1024, vocab=157, attn_type=synth.GQA,
+                     norm_type=synth.RMSNORM, act=synth.SWIGLU, batch=3, prompt=512, steps=1, dtype="f16")
+    w = synth.make_weights(cfg, 91, random_bias=True)
+    seqs = synth.make_prompts(cfg, 92)
+    gpu = G.HipGpt(cfg, w, max_batch=3, max_seq_len=520)
+    gpu.prefill(seqs)
+    want = gpu.logits()
+    monkeypatch.setenv("TSHIP_PATCH_ROWS", patch_rows)
+    gpu.reset()
+    gpu.prefill(seqs)
+    monkeypatch.delenv("TSHIP_PATCH_ROWS")
+    assert np.array_equal(want, gpu.logits())
+    gpu.close()
