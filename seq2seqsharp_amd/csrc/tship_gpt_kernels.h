@@ -56,6 +56,24 @@ __device__ __forceinline__ float sum_xor32(float v) {
     return __uint_as_float(r[0]) + __uint_as_float(r[1]);
 }
 
+// The same with the activation fixed at compile time: the epilogues of the LDS-tiled GEMM apply it to 64-128 values per lane,
+// and a run-time switch per value is a chain of scalar compares and branches around each of them.
+template <int ACT>
+__device__ __forceinline__ float act_apply_c(float w) {
+    if constexpr (ACT == 0) return w < 0.0f ? 0.0f : w;
+    else if constexpr (ACT == 1 || ACT == 4) return w / (1.0f + __expf(-w));
+    else if constexpr (ACT == 2) return w < 0.0f ? 0.01f * w : w;
+    else return w;
+}
+// calls f(std::integral_constant<int, act>) for the run-time activation code
+template <typename F>
+__device__ __forceinline__ void with_act(int act, F&& f) {
+    if (act == 0) f(std::integral_constant<int, 0>{});
+    else if (act == 1 || act == 4) f(std::integral_constant<int, 1>{});
+    else if (act == 2) f(std::integral_constant<int, 2>{});
+    else f(std::integral_constant<int, 3>{});
+}
+
 // GEMM inputs of the fp16 decode path are stored "fragment packed": for every k-tile of 16 the 32 rows form the
 // 1 KiB B-operand fragment of v_mfma_f32_32x32x16_f16 (lane l holds row l%32, k = kt*16 + 8*(l/32) .. +7), so a
 // wavefront fetches it with one coalesced 16-byte load per lane.  Index of element (row b, column k):
@@ -651,6 +669,7 @@ __global__ __launch_bounds__(256) void big_gemm_f16_kernel(BigArgs a) {
 // that rows leave as whole 128-byte lines (eight lanes x 16 bytes per row, eight rows per store instruction) instead of
 // 32 pieces of 16 bytes per instruction: the fragmented form takes four times the store requests.  `stage`: 64 rows x 72
 // halfs of LDS owned by this wavefront (row stride 144 bytes: 16-byte aligned pieces, rows spread over the banks).  Whole tiles only.
+template <int ACT>
 __device__ __forceinline__ void gated_store_lines(const BigArgs& a, floatx16 (&acc)[4][2], int nt_first, long row_first, int lane, half_t* stage,
                                                   const float (&rinv2)[2]) {
     constexpr int LDSROW = 72;
@@ -669,7 +688,7 @@ __device__ __forceinline__ void gated_store_lines(const BigArgs& a, floatx16 (&a
             for (int g = 0; g < 2; ++g) {
                 half4v o;
 #pragma unroll
-                for (int e = 0; e < 4; ++e) o[e] = (half_t)(act_apply(a.act, acc[j][i][4 * g + e] * rinv2[i] + b1[4 * g + e]) * (acc[j][i][4 * g + e + 8] * rinv2[i] + b2[4 * g + e]));
+                for (int e = 0; e < 4; ++e) o[e] = (half_t)(act_apply_c<ACT>(acc[j][i][4 * g + e] * rinv2[i] + b1[4 * g + e]) * (acc[j][i][4 * g + e + 8] * rinv2[i] + b2[4 * g + e]));
                 *(half4v*)(stage + (32 * i + r) * LDSROW + 16 * j + 8 * g + 4 * lh) = o;
             }
         }
@@ -738,6 +757,7 @@ __device__ __forceinline__ void resid_store_lines(const BigArgs& a, const floatx
 
 // Ungated activation output (ReLU / SiLU / LeakyReLU feed-forward, MoE experts): a wavefront's 64 rows x 128 columns go
 // out in two halves of 64 columns (one 128-byte line per row each) through the same 64 x 72 halfs of LDS.
+template <int ACT>
 __device__ __forceinline__ void act_store_lines(const BigArgs& a, floatx16 (&acc)[4][2], int nt_first, long row_first, int lane, half_t* stage,
                                                 const float (&rinv2)[2]) {
     constexpr int LDSROW = 72;
@@ -756,7 +776,7 @@ __device__ __forceinline__ void act_store_lines(const BigArgs& a, floatx16 (&acc
                 for (int g = 0; g < 4; ++g) {
                     half4v o;
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) o[e] = (half_t)act_apply(a.act, acc[j][i][4 * g + e] * rinv2[i] + bb[4 * g + e]);
+                    for (int e = 0; e < 4; ++e) o[e] = (half_t)act_apply_c<ACT>(acc[j][i][4 * g + e] * rinv2[i] + bb[4 * g + e]);
                     *(half4v*)(stage + (32 * i + r) * LDSROW + 32 * jj + 8 * g + 4 * lh) = o;
                 }
         }
@@ -893,12 +913,12 @@ __device__ __forceinline__ void big_gemm_store(const BigArgs& a, floatx16 (&acc)
         const int ntf = nt0 + 4 * wn;
         if (stage && a.gated && rf + 64 <= a.R && ntf + 4 <= a.NT && (ntf + 4) * 16 <= a.n_valid && (a.ld16 & 7) == 0) {
             const float r2[2] = {rinv4[0], rinv4[1]};
-            gated_store_lines(a, acc, ntf, rf, lane, stage, r2);
+            with_act(a.act, [&](auto A) { gated_store_lines<decltype(A)::value>(a, acc, ntf, rf, lane, stage, r2); });
             return;
         }
         if (stage && !a.gated && rf + 64 <= a.R && ntf + 4 <= a.NT && (ntf + 4) * 32 <= a.n_valid && (a.ld16 & 7) == 0) {
             const float r2[2] = {rinv4[0], rinv4[1]};
-            act_store_lines(a, acc, ntf, rf, lane, stage, r2);
+            with_act(a.act, [&](auto A) { act_store_lines<decltype(A)::value>(a, acc, ntf, rf, lane, stage, r2); });
             return;
         }
     }
