@@ -63,7 +63,10 @@ def test_padded_batch_fp32(G, oracle, kw):
     gpu.close()
 
 
-@pytest.mark.parametrize("hidden,heads,kv_heads,lens", [(256, 4, 2, [70, 33, 1, 64, 2]), (512, 4, 1, [40, 9, 31]), (256, 4, 4, [130, 129, 5, 64])])
+@pytest.mark.parametrize("hidden,heads,kv_heads,lens", [(256, 4, 2, [70, 33, 1, 64, 2]), (512, 4, 1, [40, 9, 31]), (256, 4, 4, [130, 129, 5, 64]),
+                                                        # 9 x 64 = 576 padded rows in whole 32-position chunks: the LDS-tiled GEMMs, and the QKV
+                                                        # projection writes the cache (padding positions included) from its epilogue
+                                                        (512, 8, 4, [64, 17, 1, 33, 64, 50, 2, 31, 48]), (512, 4, 2, [64, 3, 40, 64, 20, 9, 33, 1, 60])])
 def test_padded_batch_fp16_mfma_attention(G, oracle, hidden, heads, kv_heads, lens):
     """head_dim 64 and 128 (the MFMA prefill attention): lengths on both sides of 32-position chunk boundaries, a row of
     length 1, rows of full length."""
