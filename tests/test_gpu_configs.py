@@ -336,7 +336,7 @@ def test_projection_writes_the_cache_like_the_separate_kernel(G, oracle, monkeyp
                      norm_type=synth.RMSNORM, act=synth.SWIGLU, batch=batch, prompt=prompt, steps=2, dtype="f16")
     w = synth.make_weights(cfg, 77, random_bias=True)
     seqs = synth.make_prompts(cfg, 78)
-    gpu = G.HipGpt(cfg, w, max_batch=batch, max_seq_len=prompt + 40)
+    gpu = G.HipGpt(cfg, w, max_batch=batch, max_seq_len=prompt + 136)
     gpu.prefill(seqs)
     fused = [(gpu.get_kv(l, 0), gpu.get_kv(l, 1)) for l in range(2)]
     lg_fused = gpu.logits()
@@ -349,14 +349,23 @@ def test_projection_writes_the_cache_like_the_separate_kernel(G, oracle, monkeyp
         assert np.array_equal(fused[l][0], k), "keys of layer %d" % l
         assert np.array_equal(fused[l][1], v), "values of layer %d" % l
     assert np.array_equal(lg_fused, gpu.logits())
-    # appended tokens behind the fused prefill (fewer than 512 rows: the separate kernel) continue the same cache
-    more = synth.make_prompts(dict(cfg, prompt=32), 79)
+    # appended tokens behind the fused prefill continue the same cache: 128 more per sequence (with three or five sequences
+    # again 512 rows or more, written by the projection at a cache offset; with one sequence by the separate kernel)
+    more = synth.make_prompts(dict(cfg, prompt=128), 79)
     gpu.reset()
     gpu.prefill(seqs)
     gpu.prefill(more)
+    lg_app = gpu.logits()
+    k_app = gpu.get_kv(1, 0)
     orc = oracle.OracleGpt(cfg, w)
     _, lg = orc.step(np.concatenate([seqs, more], 1), use_cache=True)
-    assert np.abs(gpu.logits() - lg).max() <= FP16_ABS
+    assert np.abs(lg_app - lg).max() <= FP16_ABS
+    monkeypatch.setenv("TSHIP_NO_KV_FUSE", "1")
+    gpu.reset()
+    gpu.prefill(seqs)
+    gpu.prefill(more)
+    monkeypatch.delenv("TSHIP_NO_KV_FUSE")
+    assert np.array_equal(lg_app, gpu.logits()) and np.array_equal(k_app, gpu.get_kv(1, 0))
     gpu.close()
 
 
