@@ -195,6 +195,13 @@ static void run_moe_ffn_prefill(TSHipGpt* m, LayerW& L, int rows, const ResidNor
 // next tokens from the logits on the device -> m->ids (and gen_out); greedy or top-p.
 // With d_step set, gen_out and dev_uniforms are bases indexed by the device step counter (graph replays).
 // record: the chosen tokens are about to be appended (generate loop), so their position enters the token history.
+// top-p pick whose block goes on with the next decode step's first kernel for its row (as greedy_embed_kernel does)
+template <int NPT>
+__global__ __launch_bounds__(PICK_THREADS) void topp_pick_embed_kernel(TopPArgs a, FnPrepArgs pa) {
+    const int tok = topp_pick_scan_row(a);
+    fn_prepare_row<NPT, PICK_THREADS>(pa, blockIdx.x, tok, threadIdx.x);
+}
+
 // embed_next: a decode step on these tokens follows at once (the generate loop): on the fused-norm path the greedy kernel
 // then also does that step's first kernel for its row and sets m->embed_done.
 static void sample_tokens(TSHipGpt* m, int mode, float top_p, float temperature, const float* host_uniforms, const float* dev_uniforms, int B,
@@ -239,7 +246,18 @@ static void sample_tokens(TSHipGpt* m, int mode, float top_p, float temperature,
     // of cached positions
     a.blocked = m->any_blocked ? (const unsigned char*)m->blocked.p : nullptr;
     a.repeat_penalty = m->repeat_penalty; a.last_pos = last; a.last_ld = m->last_ld; a.d_len = m->d_pos.as<int>(); a.record = record ? 1 : 0;
-    topp_run(a, B, [&](const char* name, void (*kernel)(TopPArgs), dim3 grid, dim3 block, const TopPArgs& args) { launch(m, name, kernel, grid, block, args); });
+    auto run = [&](const char* name, void (*kernel)(TopPArgs), dim3 grid, dim3 block, const TopPArgs& args) { launch(m, name, kernel, grid, block, args); };
+    if (embed_next && m->fused_norm && m->c.hidden <= 8192) {
+        const TopPArgs pick = topp_run(a, B, run, false);
+        const FnPrepArgs pa = embed_prepare_args(m, m->ids.as<int>());
+        const int h = m->c.hidden;
+        if (h <= 2048) launch(m, "topp_pick_embed", topp_pick_embed_kernel<4>, dim3(B), dim3(PICK_THREADS), pick, pa);
+        else if (h <= 4096) launch(m, "topp_pick_embed", topp_pick_embed_kernel<8>, dim3(B), dim3(PICK_THREADS), pick, pa);
+        else launch(m, "topp_pick_embed", topp_pick_embed_kernel<16>, dim3(B), dim3(PICK_THREADS), pick, pa);
+        m->embed_done = true;
+        return;
+    }
+    topp_run(a, B, run);
 }
 
 }  // namespace tship

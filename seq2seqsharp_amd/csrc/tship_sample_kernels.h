@@ -30,6 +30,7 @@ struct TopPArgs {
     long Vs;
     int* hist; int nseg;                   // scratch [rows][nseg][256]
     int shift;                             // digit of the current sort pass
+    int scan_in_scatter;                   // the scatter kernel turns the digit counts into offsets itself (rows of up to 64 segments)
     int* next_ids; int* gen_out; float* out_f32;   // any of them may be null
     const int* d_step;                             // optional: uniforms and gen_out are indexed by *d_step * rows + row
     // repeat penalty (0: none).  last_pos [rows][last_ld]; the row's sequence length is row_lens[row], else *d_len,
@@ -270,7 +271,37 @@ static __global__ __launch_bounds__(256) void topp_scatter_kernel(TopPArgs a) {
     }
     __syncthreads();
     {
-        int run = a.hist[((long)r * a.nseg + seg) * 256 + t];
+        int run;
+        if (a.scan_in_scatter) {
+            // offset of (segment, digit t) in (digit major, segment minor) order from the row's raw counts: the digit's counts in
+            // the segments before this one, plus the totals of all smaller digits (what topp_scan_kernel leaves in `hist`;
+            // every block of the row repeats the sums, which costs less than a launch of its own between histogram and scatter)
+            __shared__ int tot[256];
+            const int* h = a.hist + (long)r * a.nseg * 256;
+            int before = 0, total = 0;
+            for (int s0 = 0; s0 < a.nseg; s0 += 8) {
+                int v[8];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) v[u] = s0 + u < a.nseg ? h[(s0 + u) * 256 + t] : 0;
+#pragma unroll
+                for (int u = 0; u < 8; ++u) { total += v[u]; if (s0 + u < seg) before += v[u]; }
+            }
+            tot[t] = total;
+            __syncthreads();
+            if (t < 64) {       // one wavefront: 4 digits per lane, then a shuffle scan over the lane sums
+                const int v0 = tot[4 * t], v1 = tot[4 * t + 1], v2 = tot[4 * t + 2], v3 = tot[4 * t + 3];
+                const int mine = v0 + v1 + v2 + v3;
+                int inc = mine;
+#pragma unroll
+                for (int o = 1; o < 64; o <<= 1) { const int n = __shfl_up(inc, o, 64); if (t >= o) inc += n; }
+                const int base = inc - mine;
+                tot[4 * t] = base; tot[4 * t + 1] = base + v0; tot[4 * t + 2] = base + v0 + v1; tot[4 * t + 3] = base + v0 + v1 + v2;
+            }
+            __syncthreads();
+            run = tot[t] + before;
+        } else {
+            run = a.hist[((long)r * a.nseg + seg) * 256 + t];
+        }
 #pragma unroll
         for (int s = 0; s < 16; ++s) { const int v = wh[s][t]; wh[s][t] = run; run += v; }
     }
@@ -335,8 +366,10 @@ __device__ __forceinline__ unsigned pick_map_below(unsigned long long isc, unsig
 // block barrier that orders LDS traffic only (outstanding global stores are not waited for)
 __device__ __forceinline__ void pick_lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
-static __global__ __launch_bounds__(PICK_THREADS) void topp_pick_scan_kernel(TopPArgs a) {
+// (the chosen token is returned to every thread of the block)
+__device__ __forceinline__ int topp_pick_scan_row(const TopPArgs& a) {
     __shared__ unsigned s_wmap[PICK_WAVES], s_wsum[PICK_WAVES];
+    __shared__ int s_id;
     __shared__ int s_event[PICK_WAVES];
     __shared__ float s_acc;
     __shared__ int s_j0, s_n, s_state, s_pick[PICK_WAVES];
@@ -536,27 +569,35 @@ static __global__ __launch_bounds__(PICK_THREADS) void topp_pick_scan_kernel(Top
         if (a.gen_out) a.gen_out[slot] = id;
         if (a.out_f32) a.out_f32[r] = (float)id;
         if (a.record && a.last_pos) a.last_pos[(long)r * a.last_ld + id] = topp_seq_len(a, r);     // the new token's index
+        s_id = id;
     }
+    __syncthreads();
+    return s_id;
 }
+static __global__ __launch_bounds__(PICK_THREADS) void topp_pick_scan_kernel(TopPArgs a) { topp_pick_scan_row(a); }
 
 // the whole pipeline; `launch_fn(name, kernel, grid, block, args)` puts one kernel on the library stream
+// with_pick = false: everything but the last kernel; returns the arguments that kernel takes (the caller launches a pick
+// kernel of its own, see topp_pick_embed_kernel)
 template <typename LaunchFn>
-inline void topp_run(TopPArgs a, int rows, LaunchFn&& launch_fn) {
+inline TopPArgs topp_run(TopPArgs a, int rows, LaunchFn&& launch_fn, bool with_pick = true) {
     const dim3 segs((unsigned)a.nseg, (unsigned)rows);
     if (a.in_is_logits) {
         launch_fn("topp_rowmax", topp_rowmax_kernel, segs, dim3(256), a);
         launch_fn("topp_rowsum", topp_rowsum_kernel, segs, dim3(256), a);
     }
+    a.scan_in_scatter = a.nseg <= 64 ? 1 : 0;      // (beyond that every block of a row would re-read too many counts)
     launch_fn("topp_keys", topp_keys_kernel, segs, dim3(256), a);          // also the digit counts of pass 0
     for (int pass = 0; pass < 4; ++pass) {
         a.shift = pass * 8;
         if (pass > 0) launch_fn("topp_hist", topp_hist_kernel, dim3((unsigned)a.nseg, (unsigned)rows), dim3(256), a);
-        launch_fn("topp_scan", topp_scan_kernel, dim3((unsigned)rows), dim3(256), a);
+        if (!a.scan_in_scatter) launch_fn("topp_scan", topp_scan_kernel, dim3((unsigned)rows), dim3(256), a);
         launch_fn("topp_scatter", topp_scatter_kernel, dim3((unsigned)a.nseg, (unsigned)rows), dim3(256), a);
         unsigned* tk = a.keysA; a.keysA = a.keysB; a.keysB = tk;
         int* ti = a.idxA; a.idxA = a.idxB; a.idxB = ti;
     }
-    launch_fn("topp_pick", topp_pick_scan_kernel, dim3((unsigned)rows), dim3(PICK_THREADS), a);
+    if (with_pick) launch_fn("topp_pick", topp_pick_scan_kernel, dim3((unsigned)rows), dim3(PICK_THREADS), a);
+    return a;
 }
 
 }  // namespace tship
