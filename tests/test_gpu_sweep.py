@@ -105,3 +105,41 @@ def test_moe_expert_counts_beyond_eight(oracle, experts, k, batch, dtype):
                 assert same.all()
             assert np.abs(gl[same] - lg[same]).max() <= 3e-2
     gpu.close()
+
+
+def _big_prefill_cfg(seed):
+    """512 to 1700 prompt rows in whole 32-position chunks, key and value widths multiples of 128: the shapes where the
+    LDS-tiled prefill kernels, their adaptive tile patches and the cache write from the QKV projection are in use."""
+    rng = np.random.default_rng(3000 + seed)
+    while True:
+        d = int(rng.choice([64, 128]))
+        g = int(rng.choice([1, 2, 4, 8]))
+        kv = int(rng.choice([2, 4, 8])) if d == 64 else int(rng.choice([1, 2, 4]))
+        hidden = kv * g * d
+        tp = int(rng.choice([32, 64, 96, 160, 256, 544]))
+        batch = max(1, int(np.ceil(rng.integers(512, 1400) / tp)))
+        if hidden <= 2048 and batch <= 32:
+            break
+    return synth._cfg(n_layers=2, hidden=hidden, n_heads=kv * g, n_kv_heads=kv, ffn_dim=int(rng.choice([1, 2, 3])) * hidden, vocab=211,
+                      attn_type=synth.GQA, norm_type=synth.RMSNORM, act=int(rng.choice([synth.SWIGLU, synth.RELU, synth.SILU])),
+                      batch=batch, prompt=tp, steps=1, use_rope=int(rng.integers(0, 4) != 0), dtype="f16")
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_large_prefill_paths_agree_bit_for_bit(monkeypatch, seed):
+    """The cache written by the QKV projection's epilogue and the tile patches chosen from the launch size, against the
+    separate cache-write kernel and fixed 8 x 4 patches: same logits, keys and values."""
+    from seq2seqsharp_amd import gpt as G
+    cfg = _big_prefill_cfg(seed)
+    w = synth.make_weights(cfg, 100 + seed, random_bias=True)
+    seqs = synth.make_prompts(cfg, 200 + seed)
+    gpu = G.HipGpt(cfg, w, max_batch=cfg["batch"], max_seq_len=cfg["prompt"] + 8)
+    gpu.prefill(seqs)
+    lg, k, v = gpu.logits(), gpu.get_kv(1, 0), gpu.get_kv(1, 1)
+    assert np.isfinite(lg).all()
+    monkeypatch.setenv("TSHIP_NO_KV_FUSE", "1")
+    monkeypatch.setenv("TSHIP_PATCH_ROWS", "8")
+    gpu.reset()
+    gpu.prefill(seqs)
+    assert np.array_equal(lg, gpu.logits()) and np.array_equal(k, gpu.get_kv(1, 0)) and np.array_equal(v, gpu.get_kv(1, 1))
+    gpu.close()
