@@ -898,8 +898,8 @@ static void prefill(TSHipGpt* m, const int32_t* host_ids, int B, int Tp, const i
             launch(m, "p_kv_write", pick_kvw(m), dim3(Tp, B), dim3(256), aa);
         }
         if (m->vt) {      // a wavefront per 16 / G query positions, 8 (head_dim 64) or 4 (head_dim 128) wavefronts per block
-            const int per_block = (16 / m->G) * (m->D == 128 ? 4 : 8);
-            launch(m, "p_attn", pick_attn(m, true, false, host_lens != nullptr), dim3((unsigned)ceil_div(Tp, per_block), c.n_kv_heads, B), dim3(m->D == 128 ? 256 : 512), aa);
+            const int per_block = (16 / m->G) * 8;
+            launch(m, "p_attn", pick_attn(m, true, false, host_lens != nullptr), dim3((unsigned)ceil_div(Tp, per_block), c.n_kv_heads, B), dim3(512), aa);
         }
         else launch(m, "p_attn", pick_attn(m, true), dim3(Tp, c.n_kv_heads, B), dim3(256), aa);
         ResidNormArgs a2 = rn;

@@ -2469,8 +2469,8 @@ __global__ __launch_bounds__(D == 128 ? 256 : 512) void attn_mfma_kernel(AttnArg
 // column of the padded sequence with scores rounded as the float32 addition of -30000 rounds them; every chunk then
 // takes the masked path and a block that holds such a row walks all chunks.
 template <int D, int G, bool RAGGED = false>
-__global__ __launch_bounds__(D == 128 ? 256 : 512) void attn_mfma_prefill_kernel(AttnArgs a) {
-    constexpr int NW = D == 128 ? 4 : 8;
+__global__ __launch_bounds__(512) void attn_mfma_prefill_kernel(AttnArgs a) {
+    constexpr int NW = 8;
     constexpr int QB = 16 / G, KD = D / 32, DT = D / 16;
     constexpr int NF = 2 * KD + DT;          // 1 KiB fragments per chunk: keys (tile, kd), then values (dt)
     constexpr int FPW = NF / NW;             // fragments a wavefront brings per chunk
