@@ -552,6 +552,56 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(float* __restrict__ x,
 #pragma clang fp contract(off)
     const int i = blockIdx.x;
     if (clear_counts && i == 0 && (int)threadIdx.x < E) clear_counts[threadIdx.x] = 0;       // for the next router launch
+    if (k <= 8 && h % 4 == 0 && ldx % 4 == 0 && ldy % 4 == 0 && estride % 4 == 0) {
+        // The token's picks in expert-major order (equal experts in pick order), found once per thread instead of once
+        // per element and expert; then the same products and sums in that order, four columns per thread and request.
+        int ex[8], sl[8]; float pr[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const int jj = min(j, k - 1);
+            ex[j] = j < k ? (int)top_idx[i * k + jj] : 0x7fffffff;
+            sl[j] = slot[i * k + jj];
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) pr[j] = j < k ? probs[i * E + min(max(ex[j], 0), E - 1)] : 0.0f;
+        int ord[8];          // ord[r] = pick with rank r
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            int rank = 0;
+#pragma unroll
+            for (int o = 0; o < 8; ++o) rank += (ex[o] < ex[j] || (ex[o] == ex[j] && o < j)) ? 1 : 0;
+#pragma unroll
+            for (int r = 0; r < 8; ++r) if (r == rank) ord[r] = j;
+        }
+        for (int c = 4 * threadIdx.x; c < h; c += 1024) {
+            floatx4 yv[8];
+#pragma unroll
+            for (int r = 0; r < 8; ++r) {
+                // (pick number ord[r], selected without dynamic register indexing)
+                int e = 0, s_ = 0;
+#pragma unroll
+                for (int j = 0; j < 8; ++j) if (ord[r] == j) { e = ex[j]; s_ = sl[j]; }
+                const bool on = r < k && e >= 0 && e < E;
+                yv[r] = on ? *(const floatx4*)(y + (long)e * estride + (long)s_ * ldy + c) : floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+            }
+            floatx4 xv = *(const floatx4*)(x + (long)i * ldx + c);
+            floatx4 out = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+            for (int r = 0; r < 8; ++r) {
+                float p = 0.0f; int e = -1;
+#pragma unroll
+                for (int j = 0; j < 8; ++j) if (ord[r] == j) { p = pr[j]; e = ex[j]; }
+                if (r < k && e >= 0 && e < E) {
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) { const float sc = yv[r][q] * p; out[q] += sc; }
+                }
+            }
+#pragma unroll
+            for (int q = 0; q < 4; ++q) xv[q] = xv[q] + out[q];
+            *(floatx4*)(x + (long)i * ldx + c) = xv;
+        }
+        return;
+    }
     for (int c = threadIdx.x; c < h; c += 256) {
         float out = 0.0f;
         for (int e = 0; e < E; ++e)
