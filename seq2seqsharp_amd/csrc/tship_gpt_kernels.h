@@ -2468,7 +2468,7 @@ __global__ __launch_bounds__(D == 128 ? 256 : 512) void attn_mfma_kernel(AttnArg
 // RAGGED: sequences padded to one length (a.lens).  A query row at or beyond its sequence's length attends to every
 // column of the padded sequence with scores rounded as the float32 addition of -30000 rounds them; every chunk then
 // takes the masked path and a block that holds such a row walks all chunks.
-template <int D, int G, bool RAGGED = false>
+template <int D, int G, bool RAGGED = false, int PIPE = 1>
 __global__ __launch_bounds__(512) void attn_mfma_prefill_kernel(AttnArgs a) {
     constexpr int NW = 8;
     constexpr int QB = 16 / G, KD = D / 32, DT = D / 16;
@@ -2477,7 +2477,8 @@ __global__ __launch_bounds__(512) void attn_mfma_prefill_kernel(AttnArgs a) {
     static_assert(NF % NW == 0, "fragments must divide among the wavefronts");
     __shared__ __attribute__((aligned(16))) float sbuf[NW][D * 16];       // per wavefront: Q staging [16 columns][D], later the outputs [D][16 columns]
     __shared__ float sl[NW][16];
-    __shared__ __attribute__((aligned(16))) half_t schunk[2][NF * 512];
+    __shared__ __attribute__((aligned(16))) half_t schunk[(PIPE != 0 && PIPE != 2) ? 1 : 2][(PIPE != 0 && PIPE != 2) ? 8 : NF * 512];
+    __shared__ __attribute__((aligned(16))) half_t sstage[(PIPE != 0 && PIPE != 2) ? 4 * NF * 512 : 8];
     static_assert(sizeof(sbuf) >= NF * 1024, "the third chunk stage lives in the query / output staging area");
     const int lane = threadIdx.x & 63, w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int r16 = lane & 15, q = lane >> 4;
@@ -2496,7 +2497,12 @@ __global__ __launch_bounds__(512) void attn_mfma_prefill_kernel(AttnArgs a) {
     typedef void __attribute__((address_space(3)))* lptr_t;
     // Three chunk stages: two of their own and, while the chunks are walked, the first NF KiB of the staging area (free
     // between the query prologue and the output epilogue; the barriers of the first and behind the last chunk fence it).
-    auto stage_of = [&](int c) -> half_t* { const int st = c % 3; return st == 2 ? (half_t*)&sbuf[0][0] : schunk[st]; };
+    static_assert(sizeof(sbuf) >= 2 * NF * 1024, "the third and fourth chunk stages live in the query / output staging area");
+    auto stage_of = [&](int c) -> half_t* {
+        if constexpr (PIPE == 2) { const int st = c & 3; return st >= 2 ? (half_t*)&sbuf[0][0] + (st - 2) * (NF * 512) : schunk[st]; }
+        else if constexpr (PIPE) { return sstage + (c & 3) * (NF * 512); }
+        else { const int st = c % 3; return st == 2 ? (half_t*)&sbuf[0][0] : schunk[st]; }
+    };
     auto fetch = [&](int c) {                // this wavefront's fragments of chunk c -> stage c % 3
         half_t* dst = stage_of(c);
 #pragma unroll
@@ -2506,8 +2512,18 @@ __global__ __launch_bounds__(512) void attn_mfma_prefill_kernel(AttnArgs a) {
             __builtin_amdgcn_global_load_lds((gptr_t)src, (lptr_t)(dst + f * 512), 16, 0, 0);
         }
     };
+    auto fetch_to = [&](int c, int slot) {   // chunk c -> the stage of chunk `slot`
+        half_t* dst = stage_of(slot);
+#pragma unroll
+        for (int i = 0; i < FPW; ++i) {
+            const int f = w + i * NW;
+            const half_t* src = (f < 2 * KD ? Kb + (long)c * (32 * D) + f * 512 : Vt + (long)c * (32 * D) + (f - 2 * KD) * 512) + lane * 8;
+            __builtin_amdgcn_global_load_lds((gptr_t)src, (lptr_t)(dst + f * 512), 16, 0, 0);
+        }
+    };
     fetch(0);
-    if (nchunks > 1) fetch(1);
+    if (PIPE) fetch_to(min(1, nchunks - 1), 1);
+    else if (nchunks > 1) fetch(1);
 
     // queries: projection + bias, rotary embedding, 1 / sqrt(d); columns beyond the prompt stay zero.  A lane takes
     // four consecutive elements (two rotary pairs) of a column at a time; the requests of four such pieces go out
@@ -2644,15 +2660,199 @@ __global__ __launch_bounds__(512) void attn_mfma_prefill_kernel(AttnArgs a) {
         __builtin_amdgcn_sched_barrier(0);
         if (MODE == 0) do_chunk(plain, c, kf, vf); else do_chunk(masked, c, kf, vf);
     };
-    {
+    // Pipelined walk (PIPE): iteration c holds the scores of chunk c (their MFMAs were issued in iteration c - 1) and
+    // the value fragments and probabilities of chunk c - 1.  It requests the key fragments of chunk c + 1 and the
+    // value fragments of chunk c from LDS, issues the value MFMAs of chunk c - 1 and the score MFMAs of chunk c + 1,
+    // and meanwhile runs the exponentials of chunk c on the vector ALU: the matrix pipe and the LDS reads work under
+    // the scalar-per-score arithmetic instead of in turns with it.  Same operations on the same values in the same
+    // order as the plain walk.  Barrier j (one per chunk): chunk j has landed for everybody and nobody reads chunk
+    // j - 2 any more, whose stage the request for chunk j + 2 then overwrites (four stages).
+    // (no branches: behind the last chunk the last chunk is requested again, into a stage nobody reads any more, so
+    // that the count of outstanding requests is the same at every barrier)
+    auto wait_barrier = [&](int j) {
+        asm volatile("s_waitcnt vmcnt(%0)" :: "n"(FPW) : "memory");
+        __builtin_amdgcn_s_barrier();
+        fetch_to(min(j + 2, nchunks - 1), j + 2);
+    };
+    if constexpr (!PIPE) {
         int c = 0;
         for (; c < n_full; ++c) step(std::integral_constant<int, 0>{}, c);
         for (; c < n_own; ++c) step(std::integral_constant<int, 1>{}, c);
         for (; c < nchunks; ++c) step(std::integral_constant<int, 2>{}, c);
+    } else {
+        half8 kf[2][KD], vf[DT];
+        floatx4 sA = floatx4{0.0f, 0.0f, 0.0f, 0.0f}, sB = sA;
+        auto read_k = [&](int c) {
+            const unsigned sa = (unsigned)(size_t)(lptr_t)stage_of(c) + lane * 16;
+#pragma unroll
+            for (int tile = 0; tile < 2; ++tile)
+#pragma unroll
+                for (int kd = 0; kd < KD; ++kd) asm volatile("ds_read_b128 %0, %1 offset:%2" : "=&v"(kf[tile][kd]) : "v"(sa), "n"((tile * KD + kd) * 1024) : "memory");
+        };
+        auto read_v = [&](int c, half8 (&vf)[DT]) {
+            const unsigned sa = (unsigned)(size_t)(lptr_t)stage_of(c) + lane * 16;
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) asm volatile("ds_read_b128 %0, %1 offset:%2" : "=&v"(vf[dt]) : "v"(sa), "n"((2 * KD + dt) * 1024) : "memory");
+        };
+        // The key fragments have arrived once only the reads issued behind them are outstanding.  (A count that lets
+        // a read land late hands its registers to the compiler while the LDS still writes them: an address kept there
+        // is then overwritten.)
+        auto k_landed = [&]() {              // in a chunk's iteration: the DT value reads follow the key reads
+            if constexpr (KD == 2)
+                asm volatile("s_waitcnt lgkmcnt(%4)" : "+v"(kf[0][0]), "+v"(kf[0][1]), "+v"(kf[1][0]), "+v"(kf[1][1]) : "n"(DT) : "memory");
+            else
+                asm volatile("s_waitcnt lgkmcnt(%8)" : "+v"(kf[0][0]), "+v"(kf[0][1]), "+v"(kf[0][2]), "+v"(kf[0][3]), "+v"(kf[1][0]), "+v"(kf[1][1]), "+v"(kf[1][2]), "+v"(kf[1][3]) : "n"(DT) : "memory");
+        };
+        auto k_landed_alone = [&]() {        // before the first chunk: nothing follows the key reads
+            if constexpr (KD == 2)
+                asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(kf[0][0]), "+v"(kf[0][1]), "+v"(kf[1][0]), "+v"(kf[1][1]) :: "memory");
+            else
+                asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(kf[0][0]), "+v"(kf[0][1]), "+v"(kf[0][2]), "+v"(kf[0][3]), "+v"(kf[1][0]), "+v"(kf[1][1]), "+v"(kf[1][2]), "+v"(kf[1][3]) :: "memory");
+        };
+        auto v_landed = [&](half8 (&vf)[DT]) {
+            if constexpr (D == 64)
+                asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(vf[0]), "+v"(vf[1]), "+v"(vf[2]), "+v"(vf[3]) :: "memory");
+            else
+                asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(vf[0]), "+v"(vf[1]), "+v"(vf[2]), "+v"(vf[3]), "+v"(vf[4]), "+v"(vf[5]), "+v"(vf[6]), "+v"(vf[7]) :: "memory");
+        };
+        // Scores are kept relative to a reference m_ref per column (units of log 2): the score MFMAs start from
+        // -m_ref, so that their outputs are s - m_ref and the probabilities are bare exponentials of them.  The
+        // reference is the column's running maximum as of the last time it was moved; it is moved (and the running
+        // outputs and sums rescaled) only in a chunk where some score exceeds it by more than SLACK: probabilities
+        // then lie in (0, 2^SLACK], well inside fp16 and fp32 range, and the quotient of output and sum does not
+        // depend on the reference.  Most chunks therefore take neither the cross-lane maximum nor the 4 DT
+        // multiplications of the running outputs.
+        constexpr float SLACK = 8.0f;
+        float m_ref = 0.0f;
+        floatx4 nmq = floatx4{0.0f, 0.0f, 0.0f, 0.0f};       // -m_ref four times: the score MFMAs' starting accumulator
+        auto scores = [&]() {
+#pragma unroll
+            for (int kd = 0; kd < KD; ++kd) {
+                sA = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf[0][kd], qf[kd], kd == 0 ? nmq : sA, 0, 0, 0);
+                sB = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf[1][kd], qf[kd], kd == 0 ? nmq : sB, 0, 0, 0);
+            }
+        };
+        // A row beyond its sequence's length: round the new scores (units of log 2) as s + (-30000) rounds them in
+        // natural units.  (A per-lane branch: it sits where no LDS read is in flight.)
+        auto round_scores = [&]() {
+            if (RAGGED && fully) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const float an = (sA[j] + m_ref) * 0.69314718f + (-30000.0f), bn = (sB[j] + m_ref) * 0.69314718f + (-30000.0f);
+                    sA[j] = (an - (-30000.0f)) * 1.44269504f - m_ref; sB[j] = (bn - (-30000.0f)) * 1.44269504f - m_ref;
+                }
+            }
+        };
+        auto mask_scores = [&](int c) {
+            const int t0 = c * 32;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                if (t0 + 8 * q + j > tmax) sA[j] = -INFINITY;
+                if (t0 + 8 * q + 4 + j > tmax) sB[j] = -INFINITY;
+            }
+        };
+        // Moves the reference of every column to its maximum in the chunk at hand where that is larger, and rescales
+        // what has been accumulated.  Inside the loop this is a rarely taken branch, and the updates are written as
+        // instructions on the registers in place: left to the compiler, the join behind the branch costs a copy of
+        // every running output in every chunk.  The compiler inserts no wait states between an MFMA and an
+        // instruction it cannot see, so the idle instructions in front (tied to the outputs, hence behind the MFMAs
+        // that produce them) provide the distance the hardware requires between the two.
+        auto move_reference = [&]() {
+            float cm = sA[0];
+#pragma unroll
+            for (int j = 1; j < 8; ++j) cm = fmaxf(cm, j < 4 ? sA[j] : sB[j - 4]);
+            cm = max_xor32(max_xor16(cm));
+            float d = fmaxf(cm, 0.0f);
+            float corr = __builtin_amdgcn_exp2f(-d);
+            // (tied to the factor as well: an exponential's result also needs a distance the compiler only keeps for
+            // instructions it can see)
+            if constexpr (DT == 4)
+                asm volatile("s_nop 15\n\ts_nop 15" : "+v"(d), "+v"(corr), "+v"(acc_o[0]), "+v"(acc_o[1]), "+v"(acc_o[2]), "+v"(acc_o[3]));
+            else
+                asm volatile("s_nop 15\n\ts_nop 15" : "+v"(d), "+v"(corr), "+v"(acc_o[0]), "+v"(acc_o[1]), "+v"(acc_o[2]), "+v"(acc_o[3]), "+v"(acc_o[4]), "+v"(acc_o[5]), "+v"(acc_o[6]), "+v"(acc_o[7]));
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) asm volatile("v_mul_f32 %0, %0, %1" : "+v"(acc_o[dt][i]) : "v"(corr));
+            asm volatile("v_mul_f32 %0, %0, %1" : "+v"(l_run) : "v"(corr));
+            asm volatile("v_add_f32 %0, %0, %1" : "+v"(m_ref) : "v"(d));
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                asm volatile("v_sub_f32 %0, %0, %1" : "+v"(sA[j]) : "v"(d));
+                asm volatile("v_sub_f32 %0, %0, %1" : "+v"(sB[j]) : "v"(d));
+                asm volatile("v_sub_f32 %0, %0, %1" : "+v"(nmq[j]) : "v"(d));
+            }
+        };
+        // One chunk.  Its value MFMAs are issued last and run under the next chunk's comparisons and its wait at the
+        // barrier.  They are written as instructions that accumulate in place: the register allocator otherwise
+        // writes results over dead fragments and copies them back, one copy per running output per chunk.  Nothing
+        // reads the running outputs before the same place one chunk later except the rescaling and the epilogue,
+        // which keep their own distance; the idle instruction in front covers the probabilities just converted.
+        auto iter = [&](auto masked_c, int c) {
+            constexpr bool MASKED = decltype(masked_c)::value;
+            if (MASKED) mask_scores(c);
+            {   // any score more than SLACK above its column's reference?  (no LDS read is in flight here)
+                float lm = sA[0];
+#pragma unroll
+                for (int j = 1; j < 8; ++j) lm = fmaxf(lm, j < 4 ? sA[j] : sB[j - 4]);
+                if (__builtin_amdgcn_ballot_w64(lm > SLACK) != 0) move_reference();
+            }
+            wait_barrier(c + 1);
+            read_k(c + 1);                   // (behind the wavefront's last chunk: any stage, the scores are not used)
+            read_v(c, vf);
+            float psum = 0.0f;
+            half8 pf;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const float p = __builtin_amdgcn_exp2f(j < 4 ? sA[j] : sB[j - 4]);
+                psum += p;
+                pf[j] = (half_t)p;
+            }
+            l_run += psum;
+            k_landed();
+            scores();                        // (the next chunk's scores, into the registers the exponentials have just read)
+            // The value fragments are tied in the basic block that requested them, behind everything above (by now
+            // they have long arrived).  Tied across a branch, the compiler may copy the registers on the edge, before
+            // the wait: a copy of a register whose read is still in flight.
+            __builtin_amdgcn_sched_barrier(0);
+            v_landed(vf);
+            asm volatile("s_nop 4" : "+v"(pf));
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+                asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+v"(acc_o[dt]) : "v"(vf[dt]), "v"(pf));
+            round_scores();
+        };
+        // barrier 0, the first chunk's scores and every column's first reference
+        wait_barrier(0);
+        if (n_own > 0) {
+            read_k(0);
+            k_landed_alone();
+            scores();
+            round_scores();
+            if (n_full == 0) mask_scores(0);
+            {   // every column's first reference: its maximum in the first chunk (finite: position 0 is visible to all)
+                float cm = sA[0];
+#pragma unroll
+                for (int j = 1; j < 8; ++j) cm = fmaxf(cm, j < 4 ? sA[j] : sB[j - 4]);
+                m_ref = max_xor32(max_xor16(cm));
+#pragma unroll
+                for (int j = 0; j < 4; ++j) { sA[j] -= m_ref; sB[j] -= m_ref; nmq[j] = -m_ref; }
+            }
+        }
+        int c = 0;
+        for (; c < n_full; ++c) iter(plain, c);
+        for (; c < n_own; ++c) iter(masked, c);
+        // (the epilogue reads the running outputs with instructions the compiler places without knowing of the MFMAs above)
+        if constexpr (DT == 4)
+            asm volatile("s_nop 15\n\ts_nop 15" : "+v"(acc_o[0]), "+v"(acc_o[1]), "+v"(acc_o[2]), "+v"(acc_o[3]));
+        else
+            asm volatile("s_nop 15\n\ts_nop 15" : "+v"(acc_o[0]), "+v"(acc_o[1]), "+v"(acc_o[2]), "+v"(acc_o[3]), "+v"(acc_o[4]), "+v"(acc_o[5]), "+v"(acc_o[6]), "+v"(acc_o[7]));
+        for (int j = n_own + 1; j <= nchunks; ++j) wait_barrier(j);      // every wavefront passes barriers 0 ... nchunks
     }
     l_run = sum_xor32(sum_xor16(l_run));
     // outputs through this wavefront's LDS slice so that rows go out contiguously: O^T[d][col] -> out[row(col)][d]
-    __builtin_amdgcn_s_barrier();             // every wavefront has read its last chunk (the third stage shares this memory)
+    if (PIPE) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");      // the repeated requests behind the last chunk land in the staging area too
+    __builtin_amdgcn_s_barrier();             // every wavefront has read its last chunk (the later stages share this memory)
     if (q == 0) sl[w][r16] = l_run;
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt)
