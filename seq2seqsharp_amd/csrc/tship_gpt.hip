@@ -511,7 +511,7 @@ static AttnKernel pick_attn_mfma(int G, bool prefill, bool split, bool ragged) {
     switch (G) {
         case 1: return prefill ? attn_mfma_prefill_kernel<D, 1> : split ? attn_mfma_kernel<D, 1, true> : attn_mfma_kernel<D, 1, false>;
         case 2: return prefill ? attn_mfma_prefill_kernel<D, 2> : split ? attn_mfma_kernel<D, 2, true> : attn_mfma_kernel<D, 2, false>;
-        case 4: return prefill ? (getenv("TSHIP_ATTN_OLD") ? attn_mfma_prefill_kernel<D, 4, false, 0> : attn_mfma_prefill_kernel<D, 4>) : split ? attn_mfma_kernel<D, 4, true> : attn_mfma_kernel<D, 4, false>;
+        case 4: return prefill ? attn_mfma_prefill_kernel<D, 4> : split ? attn_mfma_kernel<D, 4, true> : attn_mfma_kernel<D, 4, false>;
         case 8: return prefill ? attn_mfma_prefill_kernel<D, 8> : split ? attn_mfma_kernel<D, 8, true> : attn_mfma_kernel<D, 8, false>;
         default: throw Error("query heads per KV head must be 1, 2, 4 or 8");
     }

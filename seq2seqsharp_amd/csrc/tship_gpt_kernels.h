@@ -2293,7 +2293,7 @@ __global__ __launch_bounds__(D == 128 ? 256 : 512) void attn_mfma_kernel(AttnArg
     // last position the columns may attend to (the same for all: one query position per sequence)
     const int tmax = T - 1;
 
-    float m_run = -INFINITY, l_run = 0.0f;
+    float l_run = 0.0f;
     floatx4 acc_o[DT];
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) acc_o[dt] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
@@ -2462,13 +2462,13 @@ __global__ __launch_bounds__(D == 128 ? 256 : 512) void attn_mfma_kernel(AttnArg
 // Prefill variant: a wavefront owns QB = 16 / G consecutive query positions (the 16 MFMA columns are its positions x
 // the G query heads of the group), so there is no merge across wavefronts.  The NW wavefronts of a block sit at
 // neighbouring positions and need the same chunks: the block fetches every 32-position chunk of its causal prefix once,
-// straight into LDS (two stages; wavefront w brings fragments w, w + NW, ...), and all wavefronts read their MFMA
-// operands from there.  (With every wavefront streaming its own prefix the kernel was bound by L2: the L1 holds two
-// chunks and the wavefronts drift apart.)  grid (ceil(Tq / (QB NW)), Hkv, batch).
+// straight into LDS (four stages, requested two chunks ahead; wavefront w brings fragments w, w + NW, ...), and all
+// wavefronts read their MFMA operands from there.  (With every wavefront streaming its own prefix the kernel was bound
+// by L2: the L1 holds two chunks and the wavefronts drift apart.)  grid (ceil(Tq / (QB NW)), Hkv, batch).
 // RAGGED: sequences padded to one length (a.lens).  A query row at or beyond its sequence's length attends to every
 // column of the padded sequence with scores rounded as the float32 addition of -30000 rounds them; every chunk then
 // takes the masked path and a block that holds such a row walks all chunks.
-template <int D, int G, bool RAGGED = false, int PIPE = 1>
+template <int D, int G, bool RAGGED = false>
 __global__ __launch_bounds__(512) void attn_mfma_prefill_kernel(AttnArgs a) {
     constexpr int NW = 8;
     constexpr int QB = 16 / G, KD = D / 32, DT = D / 16;
@@ -2477,9 +2477,7 @@ __global__ __launch_bounds__(512) void attn_mfma_prefill_kernel(AttnArgs a) {
     static_assert(NF % NW == 0, "fragments must divide among the wavefronts");
     __shared__ __attribute__((aligned(16))) float sbuf[NW][D * 16];       // per wavefront: Q staging [16 columns][D], later the outputs [D][16 columns]
     __shared__ float sl[NW][16];
-    __shared__ __attribute__((aligned(16))) half_t schunk[(PIPE != 0 && PIPE != 2) ? 1 : 2][(PIPE != 0 && PIPE != 2) ? 8 : NF * 512];
-    __shared__ __attribute__((aligned(16))) half_t sstage[(PIPE != 0 && PIPE != 2) ? 4 * NF * 512 : 8];
-    static_assert(sizeof(sbuf) >= NF * 1024, "the third chunk stage lives in the query / output staging area");
+    __shared__ __attribute__((aligned(16))) half_t sstage[4 * NF * 512];     // four chunk stages
     const int lane = threadIdx.x & 63, w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int r16 = lane & 15, q = lane >> 4;
     const int kvh = blockIdx.y, b = blockIdx.z;
@@ -2495,24 +2493,8 @@ __global__ __launch_bounds__(512) void attn_mfma_prefill_kernel(AttnArgs a) {
     const half_t* Vt = (const half_t*)a.vcache + ((long)b * a.Hkv + kvh) * (long)D * a.max_len;
     typedef const void __attribute__((address_space(1)))* gptr_t;
     typedef void __attribute__((address_space(3)))* lptr_t;
-    // Three chunk stages: two of their own and, while the chunks are walked, the first NF KiB of the staging area (free
-    // between the query prologue and the output epilogue; the barriers of the first and behind the last chunk fence it).
-    static_assert(sizeof(sbuf) >= 2 * NF * 1024, "the third and fourth chunk stages live in the query / output staging area");
-    auto stage_of = [&](int c) -> half_t* {
-        if constexpr (PIPE == 2) { const int st = c & 3; return st >= 2 ? (half_t*)&sbuf[0][0] + (st - 2) * (NF * 512) : schunk[st]; }
-        else if constexpr (PIPE) { return sstage + (c & 3) * (NF * 512); }
-        else { const int st = c % 3; return st == 2 ? (half_t*)&sbuf[0][0] : schunk[st]; }
-    };
-    auto fetch = [&](int c) {                // this wavefront's fragments of chunk c -> stage c % 3
-        half_t* dst = stage_of(c);
-#pragma unroll
-        for (int i = 0; i < FPW; ++i) {
-            const int f = w + i * NW;
-            const half_t* src = (f < 2 * KD ? Kb + (long)c * (32 * D) + f * 512 : Vt + (long)c * (32 * D) + (f - 2 * KD) * 512) + lane * 8;
-            __builtin_amdgcn_global_load_lds((gptr_t)src, (lptr_t)(dst + f * 512), 16, 0, 0);
-        }
-    };
-    auto fetch_to = [&](int c, int slot) {   // chunk c -> the stage of chunk `slot`
+    auto stage_of = [&](int c) -> half_t* { return sstage + (c & 3) * (NF * 512); };
+    auto fetch_to = [&](int c, int slot) {   // this wavefront's fragments of chunk c -> the stage of chunk `slot`
         half_t* dst = stage_of(slot);
 #pragma unroll
         for (int i = 0; i < FPW; ++i) {
@@ -2521,9 +2503,8 @@ __global__ __launch_bounds__(512) void attn_mfma_prefill_kernel(AttnArgs a) {
             __builtin_amdgcn_global_load_lds((gptr_t)src, (lptr_t)(dst + f * 512), 16, 0, 0);
         }
     };
-    fetch(0);
-    if (PIPE) fetch_to(min(1, nchunks - 1), 1);
-    else if (nchunks > 1) fetch(1);
+    fetch_to(0, 0);
+    fetch_to(min(1, nchunks - 1), 1);
 
     // queries: projection + bias, rotary embedding, 1 / sqrt(d); columns beyond the prompt stay zero.  A lane takes
     // four consecutive elements (two rotary pairs) of a column at a time; the requests of four such pieces go out
@@ -2577,109 +2558,32 @@ __global__ __launch_bounds__(512) void attn_mfma_prefill_kernel(AttnArgs a) {
     const bool fully = RAGGED && tq0 + r16 / G >= len_b;                    // this lane's query row has every column masked
     const int tmax = fully ? Ttot - 1 : pos_base + r16 / G;                 // last position this lane's column may attend to
 
-    float m_run = -INFINITY, l_run = 0.0f;
+    float l_run = 0.0f;
     floatx4 acc_o[DT];
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) acc_o[dt] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
-    // masked = false: every position of the chunk is visible to every column (all chunks but the last one or two)
-    auto do_chunk = [&](auto masked_c, int c, half8 (&kf)[2][KD], half8 (&vf)[DT]) {
-        constexpr bool MASKED = decltype(masked_c)::value;
-        const int t0 = c * 32;
-        floatx4 sA = floatx4{0.0f, 0.0f, 0.0f, 0.0f}, sB = sA;
-#pragma unroll
-        for (int kd = 0; kd < KD; ++kd) {
-            sA = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf[0][kd], qf[kd], sA, 0, 0, 0);
-            sB = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf[1][kd], qf[kd], sB, 0, 0, 0);
-        }
-        float s[8];
-#pragma unroll
-        for (int j = 0; j < 4; ++j) { s[j] = sA[j]; s[4 + j] = sB[j]; }
-        float cm = -INFINITY;
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            if (RAGGED && fully) {      // scores are in units of log 2 here: round in natural units as s + (-30000) does, and back
-                const float sn = s[j] * 0.69314718f + (-30000.0f);
-                s[j] = (sn - (-30000.0f)) * 1.44269504f;
-            }
-            if (MASKED && t0 + 8 * q + j > tmax) s[j] = -INFINITY;       // causal mask (adding -30000 gives exactly 0 after exp in fp32 too)
-            cm = fmaxf(cm, s[j]);
-        }
-        cm = max_xor32(max_xor16(cm));
-        const float m_new = fmaxf(m_run, cm);
-        // (unmasked chunks have finite scores, so m_new is finite and exp2(-inf - m_new) = 0 covers the first chunk)
-        const float corr = (MASKED && m_new == -INFINITY) ? 1.0f : __builtin_amdgcn_exp2f(m_run - m_new);
-        half8 pf;
-        float psum = 0.0f;
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            const float p = (MASKED && s[j] == -INFINITY) ? 0.0f : __builtin_amdgcn_exp2f(s[j] - m_new);
-            psum += p;
-            pf[j] = (half_t)p;
-        }
-        l_run = l_run * corr + psum;
-        m_run = m_new;
-#pragma unroll
-        for (int dt = 0; dt < DT; ++dt) {
-#pragma unroll
-            for (int i = 0; i < 4; ++i) acc_o[dt][i] *= corr;
-            acc_o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vf[dt], pf, acc_o[dt], 0, 0, 0);
-        }
-    };
     // Chunks [0, n_full) lie entirely at or below this wavefront's first query position; chunks from n_own on lie
     // entirely behind its last one (the block's later wavefronts still need them).
     const std::integral_constant<bool, false> plain; const std::integral_constant<bool, true> masked;
     const bool wave_fully = RAGGED && active && min(tq0 + QB, a.Tq) > len_b;      // its last query row lies beyond the sequence's length
     const int n_own = active ? (wave_fully ? (Ttot + 31) / 32 : (T + 31) / 32) : 0;
     const int n_full = RAGGED ? 0 : min(n_own, (pos_base + 1) / 32);
-    // One loop per kind of chunk (unmasked, masked, not this wavefront's): with the kinds as branches of one loop the
-    // compiler copies the running outputs between registers around every branch, a third of the loop's instructions.
-    // Every wavefront passes the same nchunks barriers whatever its split.
-    // Chunks are requested two ahead.  The fragment reads and their waits are written out: the compiler cannot tell which
-    // LDS bytes a load in flight will write and would wait for all of them before any LDS read.
-    auto step = [&](auto mode_c, int c) {
-        constexpr int MODE = decltype(mode_c)::value;         // 0: unmasked, 1: masked, 2: only the block's fetch and barrier
-        // this wavefront's share of chunk c has landed once only the requests of chunk c + 1 are outstanding
-        if (c + 1 < nchunks) asm volatile("s_waitcnt vmcnt(%0)" :: "n"(FPW) : "memory");
-        else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        __builtin_amdgcn_s_barrier();                         // ... and everybody's; chunk c - 1 is consumed
-        if (MODE == 2) { if (c + 2 < nchunks) fetch(c + 2); return; }
-        half8 kf[2][KD], vf[DT];
-        const unsigned sa = (unsigned)(size_t)(lptr_t)stage_of(c) + lane * 16;
-#pragma unroll
-        for (int tile = 0; tile < 2; ++tile)
-#pragma unroll
-            for (int kd = 0; kd < KD; ++kd) asm volatile("ds_read_b128 %0, %1 offset:%2" : "=&v"(kf[tile][kd]) : "v"(sa), "n"((tile * KD + kd) * 1024) : "memory");
-#pragma unroll
-        for (int dt = 0; dt < DT; ++dt) asm volatile("ds_read_b128 %0, %1 offset:%2" : "=&v"(vf[dt]) : "v"(sa), "n"((2 * KD + dt) * 1024) : "memory");
-        if (c + 2 < nchunks) fetch(c + 2);                    // into the stage of chunk c - 1
-        if constexpr (D == 64)
-            asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(kf[0][0]), "+v"(kf[0][1]), "+v"(kf[1][0]), "+v"(kf[1][1]), "+v"(vf[0]), "+v"(vf[1]), "+v"(vf[2]), "+v"(vf[3]) :: "memory");
-        else
-            asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(kf[0][0]), "+v"(kf[0][1]), "+v"(kf[0][2]), "+v"(kf[0][3]), "+v"(kf[1][0]), "+v"(kf[1][1]), "+v"(kf[1][2]), "+v"(kf[1][3]),
-                         "+v"(vf[0]), "+v"(vf[1]), "+v"(vf[2]), "+v"(vf[3]), "+v"(vf[4]), "+v"(vf[5]), "+v"(vf[6]), "+v"(vf[7]) :: "memory");
-        __builtin_amdgcn_sched_barrier(0);
-        if (MODE == 0) do_chunk(plain, c, kf, vf); else do_chunk(masked, c, kf, vf);
-    };
-    // Pipelined walk (PIPE): iteration c holds the scores of chunk c (their MFMAs were issued in iteration c - 1) and
-    // the value fragments and probabilities of chunk c - 1.  It requests the key fragments of chunk c + 1 and the
-    // value fragments of chunk c from LDS, issues the value MFMAs of chunk c - 1 and the score MFMAs of chunk c + 1,
-    // and meanwhile runs the exponentials of chunk c on the vector ALU: the matrix pipe and the LDS reads work under
-    // the scalar-per-score arithmetic instead of in turns with it.  Same operations on the same values in the same
-    // order as the plain walk.  Barrier j (one per chunk): chunk j has landed for everybody and nobody reads chunk
-    // j - 2 any more, whose stage the request for chunk j + 2 then overwrites (four stages).
-    // (no branches: behind the last chunk the last chunk is requested again, into a stage nobody reads any more, so
-    // that the count of outstanding requests is the same at every barrier)
+    // The walk over the chunks.  An iteration holds the scores of its chunk (their MFMAs were issued in the iteration
+    // before).  It requests the key fragments of the next chunk and the value fragments of its own from LDS, runs the
+    // exponentials of its scores, issues the next chunk's score MFMAs and, last, its own value MFMAs: the matrix pipe
+    // and the LDS reads work under the per-score arithmetic instead of in turns with it.
+    // Barrier j (one per chunk, and one more): chunk j has landed for everybody and nobody reads chunk j - 2 any
+    // more, whose stage the request for chunk j + 2 then overwrites.  No branches: behind the last chunk the last
+    // chunk is requested again, into a stage nobody reads any more, so that the count of outstanding requests is the
+    // same at every barrier.  Every wavefront passes barriers 0 ... nchunks whatever its own number of chunks.
+    // The fragment reads and their waits are written out: the compiler cannot tell which LDS bytes a request in
+    // flight will write and would wait for all of them before any LDS read.
     auto wait_barrier = [&](int j) {
         asm volatile("s_waitcnt vmcnt(%0)" :: "n"(FPW) : "memory");
         __builtin_amdgcn_s_barrier();
         fetch_to(min(j + 2, nchunks - 1), j + 2);
     };
-    if constexpr (!PIPE) {
-        int c = 0;
-        for (; c < n_full; ++c) step(std::integral_constant<int, 0>{}, c);
-        for (; c < n_own; ++c) step(std::integral_constant<int, 1>{}, c);
-        for (; c < nchunks; ++c) step(std::integral_constant<int, 2>{}, c);
-    } else {
+    {
         half8 kf[2][KD], vf[DT];
         floatx4 sA = floatx4{0.0f, 0.0f, 0.0f, 0.0f}, sB = sA;
         auto read_k = [&](int c) {
@@ -2851,8 +2755,8 @@ __global__ __launch_bounds__(512) void attn_mfma_prefill_kernel(AttnArgs a) {
     }
     l_run = sum_xor32(sum_xor16(l_run));
     // outputs through this wavefront's LDS slice so that rows go out contiguously: O^T[d][col] -> out[row(col)][d]
-    if (PIPE) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");      // the repeated requests behind the last chunk land in the staging area too
-    __builtin_amdgcn_s_barrier();             // every wavefront has read its last chunk (the later stages share this memory)
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");      // (no request of this block outlives it)
+    __builtin_amdgcn_s_barrier();
     if (q == 0) sl[w][r16] = l_run;
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt)
