@@ -498,7 +498,25 @@ static AttnKernel pick_attn_d(int D, int G, bool prefill) {
     }
 }
 template <int D>
-static AttnKernel pick_attn_mfma(int G, bool prefill, bool split, bool ragged) {
+static AttnKernel pick_attn_mfma(int G, bool prefill, bool split, bool ragged, int nq = 1) {
+    if (prefill && nq == 2) {
+        if (ragged) {
+            switch (G) {
+                case 1: return attn_mfma_prefill_kernel<D, 1, true, 2>;
+                case 2: return attn_mfma_prefill_kernel<D, 2, true, 2>;
+                case 4: return attn_mfma_prefill_kernel<D, 4, true, 2>;
+                case 8: return attn_mfma_prefill_kernel<D, 8, true, 2>;
+                default: throw Error("query heads per KV head must be 1, 2, 4 or 8");
+            }
+        }
+        switch (G) {
+            case 1: return attn_mfma_prefill_kernel<D, 1, false, 2>;
+            case 2: return attn_mfma_prefill_kernel<D, 2, false, 2>;
+            case 4: return attn_mfma_prefill_kernel<D, 4, false, 2>;
+            case 8: return attn_mfma_prefill_kernel<D, 8, false, 2>;
+            default: throw Error("query heads per KV head must be 1, 2, 4 or 8");
+        }
+    }
     if (prefill && ragged) {
         switch (G) {
             case 1: return attn_mfma_prefill_kernel<D, 1, true>;
@@ -516,8 +534,8 @@ static AttnKernel pick_attn_mfma(int G, bool prefill, bool split, bool ragged) {
         default: throw Error("query heads per KV head must be 1, 2, 4 or 8");
     }
 }
-static AttnKernel pick_attn(TSHipGpt* m, bool prefill, bool split = false, bool ragged = false) {
-    if (m->vt) return m->D == 64 ? pick_attn_mfma<64>(m->G, prefill, split, ragged) : pick_attn_mfma<128>(m->G, prefill, split, ragged);
+static AttnKernel pick_attn(TSHipGpt* m, bool prefill, bool split = false, bool ragged = false, int nq = 1) {
+    if (m->vt) return m->D == 64 ? pick_attn_mfma<64>(m->G, prefill, split, ragged, nq) : pick_attn_mfma<128>(m->G, prefill, split, ragged, nq);
     return m->f16 ? pick_attn_d<half_t, half_t>(m->D, m->G, prefill) : pick_attn_d<float, float>(m->D, m->G, prefill);
 }
 template <typename CT>
@@ -898,8 +916,13 @@ static void prefill(TSHipGpt* m, const int32_t* host_ids, int B, int Tp, const i
             launch(m, "p_kv_write", pick_kvw(m), dim3(Tp, B), dim3(256), aa);
         }
         if (m->vt) {      // a wavefront per 16 / G query positions, 8 (head_dim 64) or 4 (head_dim 128) wavefronts per block
-            const int per_block = (16 / m->G) * 8;
-            launch(m, "p_attn", pick_attn(m, true, false, host_lens != nullptr), dim3((unsigned)ceil_div(Tp, per_block), c.n_kv_heads, B), dim3(512), aa);
+            // Two groups of 16 MFMA columns per wavefront (half the LDS fragment reads per score) at head size 128,
+            // once the prompt is long enough for the coarser blocks to fill the chip.  (At head size 64 the second
+            // group costs the second block per compute unit its registers and measured the same.)
+            int nq = (m->D == 128 && (long)ceil_div(Tp, (16 / m->G) * 16) * c.n_kv_heads * B >= 2048) ? 2 : 1;
+            if (const char* e = std::getenv("TSHIP_ATTN_NQ")) nq = std::atoi(e) == 2 ? 2 : 1;
+            const int per_block = (16 / m->G) * 8 * nq;
+            launch(m, "p_attn", pick_attn(m, true, false, host_lens != nullptr, nq), dim3((unsigned)ceil_div(Tp, per_block), c.n_kv_heads, B), dim3(512), aa);
         }
         else launch(m, "p_attn", pick_attn(m, true), dim3(Tp, c.n_kv_heads, B), dim3(256), aa);
         ResidNormArgs a2 = rn;

@@ -2293,7 +2293,7 @@ __global__ __launch_bounds__(D == 128 ? 256 : 512) void attn_mfma_kernel(AttnArg
     // last position the columns may attend to (the same for all: one query position per sequence)
     const int tmax = T - 1;
 
-    float l_run = 0.0f;
+    float m_run = -INFINITY, l_run = 0.0f;
     floatx4 acc_o[DT];
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) acc_o[dt] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
@@ -2468,8 +2468,10 @@ __global__ __launch_bounds__(D == 128 ? 256 : 512) void attn_mfma_kernel(AttnArg
 // RAGGED: sequences padded to one length (a.lens).  A query row at or beyond its sequence's length attends to every
 // column of the padded sequence with scores rounded as the float32 addition of -30000 rounds them; every chunk then
 // takes the masked path and a block that holds such a row walks all chunks.
-template <int D, int G, bool RAGGED = false>
-__global__ __launch_bounds__(512) void attn_mfma_prefill_kernel(AttnArgs a) {
+// NQ: groups of 16 MFMA columns per wavefront (NQ QB consecutive positions): every key and value fragment read from
+// LDS then serves NQ MFMAs.
+template <int D, int G, bool RAGGED = false, int NQ = 1>
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(D == 64 ? 4 : 2))) void attn_mfma_prefill_kernel(AttnArgs a) {
     constexpr int NW = 8;
     constexpr int QB = 16 / G, KD = D / 32, DT = D / 16;
     constexpr int NF = 2 * KD + DT;          // 1 KiB fragments per chunk: keys (tile, kd), then values (dt)
@@ -2481,11 +2483,11 @@ __global__ __launch_bounds__(512) void attn_mfma_prefill_kernel(AttnArgs a) {
     const int lane = threadIdx.x & 63, w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int r16 = lane & 15, q = lane >> 4;
     const int kvh = blockIdx.y, b = blockIdx.z;
-    const int tq0 = (blockIdx.x * NW + w) * QB;
+    const int tq0 = (blockIdx.x * NW + w) * (QB * NQ);
     const bool active = tq0 < a.Tq;          // wavefronts beyond the prompt still fetch their share of every chunk
-    const int pos_base = a.pos0 + tq0, T = min(pos_base + QB, a.pos0 + a.Tq);
+    const int pos_base = a.pos0 + tq0, T = min(pos_base + QB * NQ, a.pos0 + a.Tq);
     // chunks of the block: up to the last position of its last active wavefront
-    const int tq_last = min(a.Tq, (int)(blockIdx.x + 1) * NW * QB);
+    const int tq_last = min(a.Tq, (int)(blockIdx.x + 1) * NW * QB * NQ);
     const int len_b = RAGGED ? a.lens[b] : 0x7fffffff;
     const int Ttot = a.pos0 + a.Tq;
     const int nchunks = (RAGGED && tq_last > len_b) ? (Ttot + 31) / 32 : (a.pos0 + tq_last + 31) / 32;
@@ -2510,7 +2512,9 @@ __global__ __launch_bounds__(512) void attn_mfma_prefill_kernel(AttnArgs a) {
     // four consecutive elements (two rotary pairs) of a column at a time; the requests of four such pieces go out
     // together (one memory round trip per batch: piece by piece the block spent longer here than in its chunks)
     float* sq = sbuf[w];
-    {
+    half8 qf[NQ][KD];
+#pragma unroll
+    for (int g2 = 0; g2 < NQ; ++g2) {
         constexpr int PIECES = 16 * D / 4 / 64, BATCH = 4;       // pieces per lane, pieces requested together
         static_assert(PIECES % BATCH == 0, "whole batches");
         const float qs = a.scale * 1.44269504f;                  // (scores are kept in units of log 2, so that the exponentials below are bare v_exp_f32)
@@ -2522,9 +2526,9 @@ __global__ __launch_bounds__(512) void attn_mfma_prefill_kernel(AttnArgs a) {
                 const int p = lane + 64 * (b0 + u);
                 const int col = p / (D / 4), i4 = p % (D / 4);
                 const int qi = col / G, g = col % G;
-                ok[u] = active && tq0 + qi < a.Tq;
-                const int qic = ok[u] ? qi : 0;                  // (a valid address either way; the value is dropped)
-                const long row = (long)b * a.Tq + min(tq0, a.Tq - 1) + (ok[u] ? qic : 0);
+                ok[u] = active && tq0 + g2 * QB + qi < a.Tq;
+                const int qic = ok[u] ? g2 * QB + qi : 0;        // (a valid address either way; the value is dropped)
+                const long row = (long)b * a.Tq + min(tq0, a.Tq - 1) + qic;
                 const int c0 = (kvh * G + g) * D + 4 * i4;
                 xv[u] = *(const floatx4*)(a.qkv + row * a.ldq + c0);
                 bv[u] = *(const floatx4*)(a.bias + c0);
@@ -2548,24 +2552,28 @@ __global__ __launch_bounds__(512) void attn_mfma_prefill_kernel(AttnArgs a) {
                 *(floatx4*)(sq + col * D + 4 * i4) = y;
             }
         }
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int kd = 0; kd < KD; ++kd)
+#pragma unroll
+            for (int j = 0; j < 8; ++j) qf[g2][kd][j] = (half_t)sq[r16 * D + kd * 32 + 8 * q + j];
+        __builtin_amdgcn_wave_barrier();
     }
-    __builtin_amdgcn_wave_barrier();
-    half8 qf[KD];
+    bool fully[NQ]; int tmax[NQ];
+    float l_run[NQ];
+    floatx4 acc_o[NQ][DT];
 #pragma unroll
-    for (int kd = 0; kd < KD; ++kd)
+    for (int g2 = 0; g2 < NQ; ++g2) {
+        fully[g2] = RAGGED && tq0 + g2 * QB + r16 / G >= len_b;              // this lane's query row has every column masked
+        tmax[g2] = fully[g2] ? Ttot - 1 : pos_base + g2 * QB + r16 / G;      // last position this lane's column may attend to
+        l_run[g2] = 0.0f;
 #pragma unroll
-        for (int j = 0; j < 8; ++j) qf[kd][j] = (half_t)sq[r16 * D + kd * 32 + 8 * q + j];
-    const bool fully = RAGGED && tq0 + r16 / G >= len_b;                    // this lane's query row has every column masked
-    const int tmax = fully ? Ttot - 1 : pos_base + r16 / G;                 // last position this lane's column may attend to
-
-    float l_run = 0.0f;
-    floatx4 acc_o[DT];
-#pragma unroll
-    for (int dt = 0; dt < DT; ++dt) acc_o[dt] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+        for (int dt = 0; dt < DT; ++dt) acc_o[g2][dt] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+    }
     // Chunks [0, n_full) lie entirely at or below this wavefront's first query position; chunks from n_own on lie
     // entirely behind its last one (the block's later wavefronts still need them).
     const std::integral_constant<bool, false> plain; const std::integral_constant<bool, true> masked;
-    const bool wave_fully = RAGGED && active && min(tq0 + QB, a.Tq) > len_b;      // its last query row lies beyond the sequence's length
+    const bool wave_fully = RAGGED && active && min(tq0 + QB * NQ, a.Tq) > len_b;      // its last query row lies beyond the sequence's length
     const int n_own = active ? (wave_fully ? (Ttot + 31) / 32 : (T + 31) / 32) : 0;
     const int n_full = RAGGED ? 0 : min(n_own, (pos_base + 1) / 32);
     // The walk over the chunks.  An iteration holds the scores of its chunk (their MFMAs were issued in the iteration
@@ -2585,7 +2593,7 @@ __global__ __launch_bounds__(512) void attn_mfma_prefill_kernel(AttnArgs a) {
     };
     {
         half8 kf[2][KD], vf[DT];
-        floatx4 sA = floatx4{0.0f, 0.0f, 0.0f, 0.0f}, sB = sA;
+        floatx4 sA[NQ], sB[NQ];
         auto read_k = [&](int c) {
             const unsigned sa = (unsigned)(size_t)(lptr_t)stage_of(c) + lane * 16;
 #pragma unroll
@@ -2627,33 +2635,47 @@ __global__ __launch_bounds__(512) void attn_mfma_prefill_kernel(AttnArgs a) {
         // depend on the reference.  Most chunks therefore take neither the cross-lane maximum nor the 4 DT
         // multiplications of the running outputs.
         constexpr float SLACK = 8.0f;
-        float m_ref = 0.0f;
-        floatx4 nmq = floatx4{0.0f, 0.0f, 0.0f, 0.0f};       // -m_ref four times: the score MFMAs' starting accumulator
+        float m_ref[NQ];
+        floatx4 nmq[NQ];                                     // -m_ref four times: the score MFMAs' starting accumulator
+#pragma unroll
+        for (int g2 = 0; g2 < NQ; ++g2) { m_ref[g2] = 0.0f; nmq[g2] = floatx4{0.0f, 0.0f, 0.0f, 0.0f}; sA[g2] = nmq[g2]; sB[g2] = nmq[g2]; }
         auto scores = [&]() {
 #pragma unroll
-            for (int kd = 0; kd < KD; ++kd) {
-                sA = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf[0][kd], qf[kd], kd == 0 ? nmq : sA, 0, 0, 0);
-                sB = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf[1][kd], qf[kd], kd == 0 ? nmq : sB, 0, 0, 0);
-            }
+            for (int kd = 0; kd < KD; ++kd)
+#pragma unroll
+                for (int g2 = 0; g2 < NQ; ++g2) {
+                    sA[g2] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf[0][kd], qf[g2][kd], kd == 0 ? nmq[g2] : sA[g2], 0, 0, 0);
+                    sB[g2] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf[1][kd], qf[g2][kd], kd == 0 ? nmq[g2] : sB[g2], 0, 0, 0);
+                }
         };
         // A row beyond its sequence's length: round the new scores (units of log 2) as s + (-30000) rounds them in
         // natural units.  (A per-lane branch: it sits where no LDS read is in flight.)
         auto round_scores = [&]() {
-            if (RAGGED && fully) {
 #pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const float an = (sA[j] + m_ref) * 0.69314718f + (-30000.0f), bn = (sB[j] + m_ref) * 0.69314718f + (-30000.0f);
-                    sA[j] = (an - (-30000.0f)) * 1.44269504f - m_ref; sB[j] = (bn - (-30000.0f)) * 1.44269504f - m_ref;
+            for (int g2 = 0; g2 < NQ; ++g2)
+                if (RAGGED && fully[g2]) {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        const float an = (sA[g2][j] + m_ref[g2]) * 0.69314718f + (-30000.0f), bn = (sB[g2][j] + m_ref[g2]) * 0.69314718f + (-30000.0f);
+                        sA[g2][j] = (an - (-30000.0f)) * 1.44269504f - m_ref[g2]; sB[g2][j] = (bn - (-30000.0f)) * 1.44269504f - m_ref[g2];
+                    }
                 }
-            }
         };
         auto mask_scores = [&](int c) {
             const int t0 = c * 32;
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                if (t0 + 8 * q + j > tmax) sA[j] = -INFINITY;
-                if (t0 + 8 * q + 4 + j > tmax) sB[j] = -INFINITY;
-            }
+            for (int g2 = 0; g2 < NQ; ++g2)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    if (t0 + 8 * q + j > tmax[g2]) sA[g2][j] = -INFINITY;
+                    if (t0 + 8 * q + 4 + j > tmax[g2]) sB[g2][j] = -INFINITY;
+                }
+        };
+        auto local_max = [&](int g2) {
+            float lm = sA[g2][0];
+#pragma unroll
+            for (int j = 1; j < 8; ++j) lm = fmaxf(lm, j < 4 ? sA[g2][j] : sB[g2][j - 4]);
+            return lm;
         };
         // Moves the reference of every column to its maximum in the chunk at hand where that is larger, and rescales
         // what has been accumulated.  Inside the loop this is a rarely taken branch, and the updates are written as
@@ -2662,29 +2684,29 @@ __global__ __launch_bounds__(512) void attn_mfma_prefill_kernel(AttnArgs a) {
         // instruction it cannot see, so the idle instructions in front (tied to the outputs, hence behind the MFMAs
         // that produce them) provide the distance the hardware requires between the two.
         auto move_reference = [&]() {
-            float cm = sA[0];
 #pragma unroll
-            for (int j = 1; j < 8; ++j) cm = fmaxf(cm, j < 4 ? sA[j] : sB[j - 4]);
-            cm = max_xor32(max_xor16(cm));
-            float d = fmaxf(cm, 0.0f);
-            float corr = __builtin_amdgcn_exp2f(-d);
-            // (tied to the factor as well: an exponential's result also needs a distance the compiler only keeps for
-            // instructions it can see)
-            if constexpr (DT == 4)
-                asm volatile("s_nop 15\n\ts_nop 15" : "+v"(d), "+v"(corr), "+v"(acc_o[0]), "+v"(acc_o[1]), "+v"(acc_o[2]), "+v"(acc_o[3]));
-            else
-                asm volatile("s_nop 15\n\ts_nop 15" : "+v"(d), "+v"(corr), "+v"(acc_o[0]), "+v"(acc_o[1]), "+v"(acc_o[2]), "+v"(acc_o[3]), "+v"(acc_o[4]), "+v"(acc_o[5]), "+v"(acc_o[6]), "+v"(acc_o[7]));
+            for (int g2 = 0; g2 < NQ; ++g2) {
+                const float cm = max_xor32(max_xor16(local_max(g2)));
+                float d = fmaxf(cm, 0.0f);
+                float corr = __builtin_amdgcn_exp2f(-d);
+                // (tied to the factor as well: an exponential's result also needs a distance the compiler only keeps
+                // for instructions it can see)
+                if constexpr (DT == 4)
+                    asm volatile("s_nop 15\n\ts_nop 15" : "+v"(d), "+v"(corr), "+v"(acc_o[g2][0]), "+v"(acc_o[g2][1]), "+v"(acc_o[g2][2]), "+v"(acc_o[g2][3]));
+                else
+                    asm volatile("s_nop 15\n\ts_nop 15" : "+v"(d), "+v"(corr), "+v"(acc_o[g2][0]), "+v"(acc_o[g2][1]), "+v"(acc_o[g2][2]), "+v"(acc_o[g2][3]), "+v"(acc_o[g2][4]), "+v"(acc_o[g2][5]), "+v"(acc_o[g2][6]), "+v"(acc_o[g2][7]));
 #pragma unroll
-            for (int dt = 0; dt < DT; ++dt)
+                for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-                for (int i = 0; i < 4; ++i) asm volatile("v_mul_f32 %0, %0, %1" : "+v"(acc_o[dt][i]) : "v"(corr));
-            asm volatile("v_mul_f32 %0, %0, %1" : "+v"(l_run) : "v"(corr));
-            asm volatile("v_add_f32 %0, %0, %1" : "+v"(m_ref) : "v"(d));
+                    for (int i = 0; i < 4; ++i) asm volatile("v_mul_f32 %0, %0, %1" : "+v"(acc_o[g2][dt][i]) : "v"(corr));
+                asm volatile("v_mul_f32 %0, %0, %1" : "+v"(l_run[g2]) : "v"(corr));
+                asm volatile("v_add_f32 %0, %0, %1" : "+v"(m_ref[g2]) : "v"(d));
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                asm volatile("v_sub_f32 %0, %0, %1" : "+v"(sA[j]) : "v"(d));
-                asm volatile("v_sub_f32 %0, %0, %1" : "+v"(sB[j]) : "v"(d));
-                asm volatile("v_sub_f32 %0, %0, %1" : "+v"(nmq[j]) : "v"(d));
+                for (int j = 0; j < 4; ++j) {
+                    asm volatile("v_sub_f32 %0, %0, %1" : "+v"(sA[g2][j]) : "v"(d));
+                    asm volatile("v_sub_f32 %0, %0, %1" : "+v"(sB[g2][j]) : "v"(d));
+                    asm volatile("v_sub_f32 %0, %0, %1" : "+v"(nmq[g2][j]) : "v"(d));
+                }
             }
         };
         // One chunk.  Its value MFMAs are issued last and run under the next chunk's comparisons and its wait at the
@@ -2696,23 +2718,26 @@ __global__ __launch_bounds__(512) void attn_mfma_prefill_kernel(AttnArgs a) {
             constexpr bool MASKED = decltype(masked_c)::value;
             if (MASKED) mask_scores(c);
             {   // any score more than SLACK above its column's reference?  (no LDS read is in flight here)
-                float lm = sA[0];
+                float lm = local_max(0);
 #pragma unroll
-                for (int j = 1; j < 8; ++j) lm = fmaxf(lm, j < 4 ? sA[j] : sB[j - 4]);
+                for (int g2 = 1; g2 < NQ; ++g2) lm = fmaxf(lm, local_max(g2));
                 if (__builtin_amdgcn_ballot_w64(lm > SLACK) != 0) move_reference();
             }
             wait_barrier(c + 1);
             read_k(c + 1);                   // (behind the wavefront's last chunk: any stage, the scores are not used)
             read_v(c, vf);
-            float psum = 0.0f;
-            half8 pf;
+            half8 pf[NQ];
 #pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                const float p = __builtin_amdgcn_exp2f(j < 4 ? sA[j] : sB[j - 4]);
-                psum += p;
-                pf[j] = (half_t)p;
+            for (int g2 = 0; g2 < NQ; ++g2) {
+                float psum = 0.0f;
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const float p = __builtin_amdgcn_exp2f(j < 4 ? sA[g2][j] : sB[g2][j - 4]);
+                    psum += p;
+                    pf[g2][j] = (half_t)p;
+                }
+                l_run[g2] += psum;
             }
-            l_run += psum;
             k_landed();
             scores();                        // (the next chunk's scores, into the registers the exponentials have just read)
             // The value fragments are tied in the basic block that requested them, behind everything above (by now
@@ -2720,10 +2745,13 @@ __global__ __launch_bounds__(512) void attn_mfma_prefill_kernel(AttnArgs a) {
             // the wait: a copy of a register whose read is still in flight.
             __builtin_amdgcn_sched_barrier(0);
             v_landed(vf);
-            asm volatile("s_nop 4" : "+v"(pf));
+            if constexpr (NQ == 1) asm volatile("s_nop 4" : "+v"(pf[0]));
+            else asm volatile("s_nop 4" : "+v"(pf[0]), "+v"(pf[NQ - 1]));
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt)
-                asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+v"(acc_o[dt]) : "v"(vf[dt]), "v"(pf));
+#pragma unroll
+                for (int g2 = 0; g2 < NQ; ++g2)
+                    asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+v"(acc_o[g2][dt]) : "v"(vf[dt]), "v"(pf[g2]));
             round_scores();
         };
         // barrier 0, the first chunk's scores and every column's first reference
@@ -2734,40 +2762,38 @@ __global__ __launch_bounds__(512) void attn_mfma_prefill_kernel(AttnArgs a) {
             scores();
             round_scores();
             if (n_full == 0) mask_scores(0);
-            {   // every column's first reference: its maximum in the first chunk (finite: position 0 is visible to all)
-                float cm = sA[0];
 #pragma unroll
-                for (int j = 1; j < 8; ++j) cm = fmaxf(cm, j < 4 ? sA[j] : sB[j - 4]);
-                m_ref = max_xor32(max_xor16(cm));
+            for (int g2 = 0; g2 < NQ; ++g2) {   // every column's first reference: its maximum in the first chunk (finite: position 0 is visible to all)
+                m_ref[g2] = max_xor32(max_xor16(local_max(g2)));
 #pragma unroll
-                for (int j = 0; j < 4; ++j) { sA[j] -= m_ref; sB[j] -= m_ref; nmq[j] = -m_ref; }
+                for (int j = 0; j < 4; ++j) { sA[g2][j] -= m_ref[g2]; sB[g2][j] -= m_ref[g2]; nmq[g2][j] = -m_ref[g2]; }
             }
         }
         int c = 0;
         for (; c < n_full; ++c) iter(plain, c);
         for (; c < n_own; ++c) iter(masked, c);
         // (the epilogue reads the running outputs with instructions the compiler places without knowing of the MFMAs above)
-        if constexpr (DT == 4)
-            asm volatile("s_nop 15\n\ts_nop 15" : "+v"(acc_o[0]), "+v"(acc_o[1]), "+v"(acc_o[2]), "+v"(acc_o[3]));
-        else
-            asm volatile("s_nop 15\n\ts_nop 15" : "+v"(acc_o[0]), "+v"(acc_o[1]), "+v"(acc_o[2]), "+v"(acc_o[3]), "+v"(acc_o[4]), "+v"(acc_o[5]), "+v"(acc_o[6]), "+v"(acc_o[7]));
+        // (every variable once: for an operand listed twice the compiler makes a copy in front, itself such an instruction)
+        if constexpr (NQ == 1) asm volatile("s_nop 15\n\ts_nop 15" : "+v"(acc_o[0][DT - 1]));
+        else asm volatile("s_nop 15\n\ts_nop 15" : "+v"(acc_o[0][DT - 1]), "+v"(acc_o[1][DT - 1]));
         for (int j = n_own + 1; j <= nchunks; ++j) wait_barrier(j);      // every wavefront passes barriers 0 ... nchunks
     }
-    l_run = sum_xor32(sum_xor16(l_run));
     // outputs through this wavefront's LDS slice so that rows go out contiguously: O^T[d][col] -> out[row(col)][d]
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");      // (no request of this block outlives it)
     __builtin_amdgcn_s_barrier();
-    if (q == 0) sl[w][r16] = l_run;
-#pragma unroll
-    for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) sq[(dt * 16 + 4 * q + i) * 16 + r16] = acc_o[dt][i];
-    __builtin_amdgcn_wave_barrier();
     if (!active) return;
-    // four lanes per column: lane (col, part) divides once and writes D / 4 consecutive outputs of its column as 16-byte pieces
-    {
+#pragma unroll
+    for (int g2 = 0; g2 < NQ; ++g2) {
+        const float l_col = sum_xor32(sum_xor16(l_run[g2]));
+        if (q == 0) sl[w][r16] = l_col;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) sq[(dt * 16 + 4 * q + i) * 16 + r16] = acc_o[g2][dt][i];
+        __builtin_amdgcn_wave_barrier();
+        // four lanes per column: lane (col, part) divides once and writes D / 4 consecutive outputs of its column as 16-byte pieces
         const int col = lane >> 2, part = lane & 3;
-        const int qi = col / G, g = col % G;
+        const int qi = g2 * QB + col / G, g = col % G;
         if (tq0 + qi < a.Tq) {
             half_t* out = (half_t*)a.out + ((long)b * a.Tq + tq0 + qi) * a.ld_out + (kvh * G + g) * D + part * (D / 4);
             const float inv = 1.0f / sl[w][col];
@@ -2779,6 +2805,7 @@ __global__ __launch_bounds__(512) void attn_mfma_prefill_kernel(AttnArgs a) {
                 *(half8*)(out + d8) = o;
             }
         }
+        __builtin_amdgcn_wave_barrier();
     }
 }
 

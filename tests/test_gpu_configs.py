@@ -387,3 +387,32 @@ def test_prefill_tile_patch_heights_give_the_same_bits(G, monkeypatch, patch_row
     monkeypatch.delenv("TSHIP_PATCH_ROWS")
     assert np.array_equal(want, gpu.logits())
     gpu.close()
+
+
+@pytest.mark.parametrize("head_dim", [64, 128])
+def test_prefill_attention_column_groups_agree(G, monkeypatch, head_dim):
+    """The prefill attention gives a wavefront one or two groups of 16 MFMA columns (4 or 8 query positions at four query
+    heads per KV head), chosen from the head size and the launch size.  The grouping changes which chunks move a column's
+    reference, hence the rounding, not the result: logits and the second layer's cache must agree within the fp16 bar,
+    for a plain and for a padded batch, and large scores (which move the reference often) must not overflow."""
+    cfg = synth._cfg(n_layers=2, hidden=8 * head_dim, n_heads=8, n_kv_heads=2, ffn_dim=1024, vocab=157, attn_type=synth.GQA,
+                     norm_type=synth.RMSNORM, act=synth.SWIGLU, batch=3, prompt=200, steps=1, dtype="f16")
+    w = synth.make_weights(cfg, 93, random_bias=True)
+    for name in w:
+        if name.endswith(".Q") or name.endswith(".K"):
+            w[name] = w[name] * 6.0          # peaked attention: scores far apart, so that the reference moves often
+    seqs = synth.make_prompts(cfg, 94)
+    lens = np.array([200, 37, 129], np.int32)
+    out = {}
+    for nq in ("1", "2"):
+        monkeypatch.setenv("TSHIP_ATTN_NQ", nq)
+        for padded in (False, True):
+            gpu = G.HipGpt(cfg, w, max_batch=3, max_seq_len=224)
+            gpu.prefill(seqs, lens if padded else None)
+            out[nq, padded] = (gpu.logits(), gpu.get_kv(1, 0), gpu.get_kv(1, 1))
+            gpu.close()
+    monkeypatch.delenv("TSHIP_ATTN_NQ")
+    for padded in (False, True):
+        for a, b in zip(out["1", padded], out["2", padded]):
+            assert np.isfinite(a).all() and np.isfinite(b).all()
+            assert np.abs(a - b).max() <= FP16_ABS
