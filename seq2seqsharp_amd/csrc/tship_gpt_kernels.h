@@ -2479,7 +2479,9 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(D == 64 ? 4
     static_assert(NF % NW == 0, "fragments must divide among the wavefronts");
     __shared__ __attribute__((aligned(16))) float sbuf[NW][D * 16];       // per wavefront: Q staging [16 columns][D], later the outputs [D][16 columns]
     __shared__ float sl[NW][16];
-    __shared__ __attribute__((aligned(16))) half_t sstage[4 * NF * 512];     // four chunk stages
+    // four chunk stages, of their own: with two of them in the query / output staging area (16 KiB less, a third block
+    // per compute unit at head size 64) single rows of the wavefronts that own that area came out wrong now and then
+    __shared__ __attribute__((aligned(16))) half_t sstage[4 * NF * 512];
     const int lane = threadIdx.x & 63, w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int r16 = lane & 15, q = lane >> 4;
     const int kvh = blockIdx.y, b = blockIdx.z;
@@ -2700,7 +2702,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(D == 64 ? 4
 #pragma unroll
                     for (int i = 0; i < 4; ++i) asm volatile("v_mul_f32 %0, %0, %1" : "+v"(acc_o[g2][dt][i]) : "v"(corr));
                 asm volatile("v_mul_f32 %0, %0, %1" : "+v"(l_run[g2]) : "v"(corr));
-                asm volatile("v_add_f32 %0, %0, %1" : "+v"(m_ref[g2]) : "v"(d));
+                if (RAGGED) asm volatile("v_add_f32 %0, %0, %1" : "+v"(m_ref[g2]) : "v"(d));       // (only the rounding of rows beyond their length reads it)
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
                     asm volatile("v_sub_f32 %0, %0, %1" : "+v"(sA[g2][j]) : "v"(d));
