@@ -2471,13 +2471,15 @@ __global__ __launch_bounds__(D == 128 ? 256 : 512) void attn_mfma_kernel(AttnArg
 // NQ: groups of 16 MFMA columns per wavefront (NQ QB consecutive positions): every key and value fragment read from
 // LDS then serves NQ MFMAs.
 template <int D, int G, bool RAGGED = false, int NQ = 1>
-__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(D == 64 ? 4 : 2))) void attn_mfma_prefill_kernel(AttnArgs a) {
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(D == 64 ? (NQ == 1 ? 6 : 4) : 2))) void attn_mfma_prefill_kernel(AttnArgs a) {
     constexpr int NW = 8;
     constexpr int QB = 16 / G, KD = D / 32, DT = D / 16;
     constexpr int NF = 2 * KD + DT;          // 1 KiB fragments per chunk: keys (tile, kd), then values (dt)
     constexpr int FPW = NF / NW;             // fragments a wavefront brings per chunk
     static_assert(NF % NW == 0, "fragments must divide among the wavefronts");
-    __shared__ __attribute__((aligned(16))) float sbuf[NW][D * 16];       // per wavefront: Q staging [16 columns][D], later the outputs [D][16 columns]
+    // per wavefront: the queries [16 columns][D] as fp16, later the outputs [D / 2][16 columns] as fp32, half of them at a
+    // time (2 KiB at head size 64: with the stages 48.5 KiB per block, three blocks per compute unit)
+    __shared__ __attribute__((aligned(16))) half_t sbuf[NW][D * 16];
     __shared__ float sl[NW][16];
     // four chunk stages, of their own: with two of them in the query / output staging area (16 KiB less, a third block
     // per compute unit at head size 64) single rows of the wavefronts that own that area came out wrong now and then
@@ -2513,7 +2515,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(D == 64 ? 4
     // queries: projection + bias, rotary embedding, 1 / sqrt(d); columns beyond the prompt stay zero.  A lane takes
     // four consecutive elements (two rotary pairs) of a column at a time; the requests of four such pieces go out
     // together (one memory round trip per batch: piece by piece the block spent longer here than in its chunks)
-    float* sq = sbuf[w];
+    half_t* sq = sbuf[w];
     half8 qf[NQ][KD];
 #pragma unroll
     for (int g2 = 0; g2 < NQ; ++g2) {
@@ -2551,14 +2553,17 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(D == 64 ? 4
                     if (a.rope_cos) rope_pair(x0, x1, cv[u][pr], sv[u][pr], y0, y1);
                     y[2 * pr] = ok[u] ? qs * y0 : 0.0f; y[2 * pr + 1] = ok[u] ? qs * y1 : 0.0f;
                 }
-                *(floatx4*)(sq + col * D + 4 * i4) = y;
+                half4 yh;
+#pragma unroll
+                for (int e4 = 0; e4 < 4; ++e4) yh[e4] = (half_t)y[e4];
+                *(half4*)(sq + col * D + 4 * i4) = yh;
             }
         }
         __builtin_amdgcn_wave_barrier();
 #pragma unroll
         for (int kd = 0; kd < KD; ++kd)
 #pragma unroll
-            for (int j = 0; j < 8; ++j) qf[g2][kd][j] = (half_t)sq[r16 * D + kd * 32 + 8 * q + j];
+            for (int j = 0; j < 8; ++j) qf[g2][kd][j] = sq[r16 * D + kd * 32 + 8 * q + j];
         __builtin_amdgcn_wave_barrier();
     }
     bool fully[NQ]; int tmax[NQ];
@@ -2784,30 +2789,34 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(D == 64 ? 4
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");      // (no request of this block outlives it)
     __builtin_amdgcn_s_barrier();
     if (!active) return;
+    float* so = (float*)sbuf[w];              // [D / 2][16 columns]
 #pragma unroll
     for (int g2 = 0; g2 < NQ; ++g2) {
         const float l_col = sum_xor32(sum_xor16(l_run[g2]));
         if (q == 0) sl[w][r16] = l_col;
 #pragma unroll
-        for (int dt = 0; dt < DT; ++dt)
+        for (int hf = 0; hf < 2; ++hf) {
 #pragma unroll
-            for (int i = 0; i < 4; ++i) sq[(dt * 16 + 4 * q + i) * 16 + r16] = acc_o[g2][dt][i];
-        __builtin_amdgcn_wave_barrier();
-        // four lanes per column: lane (col, part) divides once and writes D / 4 consecutive outputs of its column as 16-byte pieces
-        const int col = lane >> 2, part = lane & 3;
-        const int qi = g2 * QB + col / G, g = col % G;
-        if (tq0 + qi < a.Tq) {
-            half_t* out = (half_t*)a.out + ((long)b * a.Tq + tq0 + qi) * a.ld_out + (kvh * G + g) * D + part * (D / 4);
-            const float inv = 1.0f / sl[w][col];
+            for (int dt = 0; dt < DT / 2; ++dt)
 #pragma unroll
-            for (int d8 = 0; d8 < D / 4; d8 += 8) {
-                half8 o;
+                for (int i = 0; i < 4; ++i) so[(dt * 16 + 4 * q + i) * 16 + r16] = acc_o[g2][hf * (DT / 2) + dt][i];
+            __builtin_amdgcn_wave_barrier();
+            // four lanes per column: lane (col, part) divides and writes D / 8 consecutive outputs of its column as 16-byte pieces
+            const int col = lane >> 2, part = lane & 3;
+            const int qi = g2 * QB + col / G, g = col % G;
+            if (tq0 + qi < a.Tq) {
+                half_t* out = (half_t*)a.out + ((long)b * a.Tq + tq0 + qi) * a.ld_out + (kvh * G + g) * D + hf * (D / 2) + part * (D / 8);
+                const float inv = 1.0f / sl[w][col];
 #pragma unroll
-                for (int j = 0; j < 8; ++j) o[j] = (half_t)(sq[(part * (D / 4) + d8 + j) * 16 + col] * inv);
-                *(half8*)(out + d8) = o;
+                for (int d8 = 0; d8 < D / 8; d8 += 8) {
+                    half8 o;
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) o[j] = (half_t)(so[(part * (D / 8) + d8 + j) * 16 + col] * inv);
+                    *(half8*)(out + d8) = o;
+                }
             }
+            __builtin_amdgcn_wave_barrier();
         }
-        __builtin_amdgcn_wave_barrier();
     }
 }
 
