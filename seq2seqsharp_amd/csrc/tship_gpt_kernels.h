@@ -2471,7 +2471,7 @@ __global__ __launch_bounds__(D == 128 ? 256 : 512) void attn_mfma_kernel(AttnArg
 // NQ: groups of 16 MFMA columns per wavefront (NQ QB consecutive positions): every key and value fragment read from
 // LDS then serves NQ MFMAs.
 template <int D, int G, bool RAGGED = false, int NQ = 1>
-__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(D == 64 ? (NQ == 1 ? 6 : 4) : 2))) void attn_mfma_prefill_kernel(AttnArgs a) {
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(D == 64 ? (NQ == 1 && !RAGGED ? 6 : 4) : 2))) void attn_mfma_prefill_kernel(AttnArgs a) {
     constexpr int NW = 8;
     constexpr int QB = 16 / G, KD = D / 32, DT = D / 16;
     constexpr int NF = 2 * KD + DT;          // 1 KiB fragments per chunk: keys (tile, kd), then values (dt)
