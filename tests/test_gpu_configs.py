@@ -416,3 +416,25 @@ def test_prefill_attention_column_groups_agree(G, monkeypatch, head_dim):
         for a, b in zip(out["1", padded], out["2", padded]):
             assert np.isfinite(a).all() and np.isfinite(b).all()
             assert np.abs(a - b).max() <= FP16_ABS
+
+
+def test_full_size_prefill_repeats_bit_for_bit(G):
+    """The benchmark configuration's prefill (16 layers, 32 x 1024 tokens, 8192 attention blocks per layer) six times on
+    one model: finite and the same bits every time.  The prefill kernels hand data between wavefronts through LDS under
+    hand-counted waits; a wait that is one short shows as a row that differs in some launches, not in all."""
+    cfg = dict(synth.CONFIGS["cfg2_1b_gqa_f16"])
+    B, Tp, last = cfg["batch"], cfg["prompt"], cfg["n_layers"] - 1
+    w = synth.make_weights(cfg, 0)
+    seqs = synth.make_prompts(cfg, 1, length=Tp)
+    gpu = G.HipGpt(cfg, w, max_batch=B, max_seq_len=Tp + 16)
+    first = None
+    for _ in range(6):
+        gpu.reset()
+        gpu.prefill(seqs)
+        cur = (gpu.logits().copy(), gpu.get_kv(last, 0).copy(), gpu.get_kv(last, 1).copy())
+        assert all(np.isfinite(x).all() for x in cur)
+        if first is None:
+            first = cur
+        else:
+            assert all(np.array_equal(a, b) for a, b in zip(first, cur))
+    gpu.close()
