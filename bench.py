@@ -74,7 +74,6 @@ def main():
     ap.add_argument("--no-topp", action="store_true")
     ap.add_argument("--prompt", type=int, default=0, help="override the prompt length")
     ap.add_argument("--prefill-runs", type=int, default=3, help="timed prefill calls (the fastest is reported; many of them keep the chip under load long enough to sample its clock)")
-    ap.add_argument("--structure-probe", action="store_true", help="also time the step's launch structure with pure streaming reads of the same bytes")
     ap.add_argument("--no-copy-calibration", action="store_true",
                     help="skip the 256 MiB plain copy that gives rocprofv3 counter runs a kernel of known traffic")
     args = ap.parse_args()
@@ -193,31 +192,6 @@ def main():
         traffic_kv_len = tj.get("kv_len")                    # attention: the KV length of the counter run (its bytes grow with it)
         traffic_source = "profiles/" + os.path.basename(tpath)
 
-    structure = None
-    if args.structure_probe:
-        # the step's launch structure with pure streaming reads of the same bytes (see TSHip_StreamStructureProbe)
-        from seq2seqsharp_amd.gpt import stream_structure_probe
-        per_layer = [("gemm_qkv", 64), ("attn_decode", 4), ("gemm_wo", 32), ("gemm_ffn13", 128), ("gemm_ffn2", 90)]
-        pb, ak = [], []
-        for _ in range(cfg["n_layers"]):
-            for name, kib in per_layer:
-                pb.append(launch_bytes[name])
-                ak.append(kib)
-        pb.append(launch_bytes["gemm_head"])
-        ak.append(128)
-        # half-layer fusion: the output projection with the FFN up projection, the FFN down projection with what follows
-        fuse = [1 if name in ("gemm_wo", "gemm_ffn2") else 0 for _ in range(cfg["n_layers"]) for name, _k in per_layer] + [0]
-        ms3 = stream_structure_probe(pb, ak, repeats=6, fuse_with_next=fuse)
-        ms3_noact = stream_structure_probe(pb, [0] * len(ak), repeats=6, fuse_with_next=fuse)
-        structure = {"phases": len(pb), "bytes": float(sum(pb)),
-                     "one_launch_per_phase_ms": round(ms3[0], 4), "persistent_grid_barrier_ms": round(ms3[1], 4), "persistent_prefetch_before_barrier_ms": round(ms3[2], 4),
-                     "one_launch_per_phase_cache_resident_ms": round(ms3[3], 4),
-                     "half_layer_fusion_ms": round(ms3[4], 4),
-                     "without_shared_activation_reads": {"one_launch_per_phase_ms": round(ms3_noact[0], 4), "persistent_grid_barrier_ms": round(ms3_noact[1], 4),
-                                                         "persistent_prefetch_before_barrier_ms": round(ms3_noact[2], 4),
-                                                         "one_launch_per_phase_cache_resident_ms": round(ms3_noact[3], 4),
-                                                         "half_layer_fusion_ms": round(ms3_noact[4], 4)}}
-
     out = {
         "metric": "decode tokens/s on 1 GPU (1B GQA fp16, batch 32)" if args.config == "cfg2_1b_gqa_f16" else "decode tokens/s on 1 GPU",
         "value": round(tok_s, 1), "unit": "tokens/s", "n_gpus": 1, "steps": K, "warmup": W,
@@ -237,7 +211,6 @@ def main():
                     "algorithmic_TFLOPs": round(prefill_tflops, 2),
                     "frac_of_fp16_mfma_peak": round(prefill_tflops / MFMA_FP16_PEAK_TFLOPS, 4) if cfg["dtype"] == "f16" else None},
         "kernel_ms_per_step": kernel_ms,
-        "launch_structure_probe": structure,
         "load_seconds": round(t_load, 1),
     }
     if not args.no_topp:

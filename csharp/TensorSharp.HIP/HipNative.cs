@@ -133,7 +133,6 @@ namespace TensorSharp.HIP
         [DllImport(Dll, CallingConvention = CC)] internal static extern int TSHip_GptStepBytes(IntPtr model, int batch, out double weightBytes, out double kvBytes);
 
         // ---- measurement aid ----
-        [DllImport(Dll, CallingConvention = CC)] internal static extern int TSHip_StreamStructureProbe(int nPhases, double[] phaseBytes, int[] actKib, int[] fuseWithNextOrNull, int repeats, float[] msOut);
 
         internal static string LastError() => Marshal.PtrToStringAnsi(TSHip_GetLastError()) ?? string.Empty;
 

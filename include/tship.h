@@ -244,16 +244,6 @@ TSHIP_API int TSHip_GptProfileSymbols(TSHipGpt* m, char* symbols, int stride, in
 /* algorithmic bytes one decode step moves at the current sequence length (weights once, compact KV once) */
 TSHIP_API int TSHip_GptStepBytes(TSHipGpt* m, int batch, double* weight_bytes, double* kv_bytes);
 
-/* Measurement aid (no counterpart in the reference): the cost of a decode step's launch structure on this machine with
- * every kernel replaced by a pure streaming read.  phase_bytes[i] bytes are read once in phase i, every block also reads
- * act_kib[i] KiB shared by all blocks, and every phase depends on the one before.  ms_out[0]: one launch per phase;
- * ms_out[1]: one persistent kernel with a grid-wide barrier between phases (bounded polling); ms_out[2]: the same with
- * the next phase's first loads requested before the barrier; ms_out[3]: one launch per phase with every phase reading
- * the same region (cache resident where it fits); ms_out[4] (0 when fuse_with_next is null): one launch per phase except
- * that every phase i with fuse_with_next[i] != 0 shares a resident launch with phase i + 1, one grid barrier between
- * them and the second phase's first loads requested before it.  Best of `repeats` runs each; ms_out holds five floats. */
-TSHIP_API int TSHip_StreamStructureProbe(int n_phases, const double* phase_bytes, const int* act_kib, const int* fuse_with_next, int repeats,
-                                         float* ms_out);
 
 #ifdef __cplusplus
 }

@@ -12,11 +12,14 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(HERE, "build")
 LIB = os.path.join(HERE, "libtship.so")
-SOURCES = ["tship_runtime.hip", "tship_gpt.hip", "tship_ops.hip", "tship_probe.hip"]
+SOURCES = ["tship_runtime.hip", "tship_gpt.hip", "tship_ops.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 # -packed-fp32-ops off: keep the compiler from forming packed fp32 instructions out of scalar float code
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden",
-         "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-result", "-Wno-pass-failed"]
+         "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-result", "-Wno-pass-failed",
+         # leading scalar kernel arguments arrive in scalar registers when a wavefront starts (no load from the argument
+         # segment in front of the first memory requests); arguments inside by-value structs are not affected
+         "-mllvm", "-amdgpu-kernarg-preload-count=16"]
 
 
 def _deps():

@@ -179,6 +179,13 @@ static void launch_shm(TSHipGpt* m, const char* name, void (*kernel)(KArgs...), 
     TSHIP_CHECK_HIP(hipGetLastError());
 }
 
+// decode GEMM launch: the scalars that the kernel's first requests depend on travel as leading arguments of their own
+// (preloaded into scalar registers at wavefront start), the rest in the struct
+template <typename... KArgs>
+static void launch_skinny(TSHipGpt* m, const char* name, void (*kernel)(KArgs...), dim3 grid, dim3 block, const SkinnyArgs& e) {
+    launch(m, name, kernel, grid, block, e.W, e.X, e.KT, e.NT, e.KS, e.rows_valid, e.ssq, e.ssq_nt, e.ssq_ld, e);
+}
+
 // decode GEMM split-K: a block has NW wavefronts of 8 k-tiles each in flight; split K across blocks until one
 // pass covers the block's range (keeps partial-sum traffic small: K = 2048 needs no split at batch <= 32)
 static int pick_ks_f16(int NT, int KT, int BT) {
@@ -400,18 +407,34 @@ static void run_skinny(TSHipGpt* m, const char* name, const GemmW& w, const void
             if (cost < best_cost) { best = 10 * nj; best_cost = cost; }
         }
         if (const char* v = std::getenv("TSHIP_FFN_TILES")) best = std::atoi(v);      // (tests: 10, 15, 20, 30 or 40)
-        if (best == 15) { launch(m, name, skinny_gemm_f16_kernel<1, EPI_ACT16, 8, 8, 2, true>, dim3((unsigned)hb), dim3(512), e); return; }
-        if (best == 20) { launch(m, name, skinny_gemm_f16_kernel<1, EPI_ACT16, 8, 8, 2>, dim3((unsigned)ceil_div(w.NT, 2)), dim3(512), e); return; }
-        if (best == 30) { launch(m, name, skinny_gemm_f16_kernel<1, EPI_ACT16, 8, 4, 3>, dim3((unsigned)ceil_div(w.NT, 3)), dim3(512), e); return; }
-        if (best == 40) { launch(m, name, skinny_gemm_f16_kernel<1, EPI_ACT16, 8, 4, 4>, dim3((unsigned)ceil_div(w.NT, 4)), dim3(512), e); return; }
+        if (best == 15) { launch_skinny(m, name, skinny_gemm_f16_kernel<1, EPI_ACT16, 8, 8, 2, true>, dim3((unsigned)hb), dim3(512), e); return; }
+        if (best == 20) { launch_skinny(m, name, skinny_gemm_f16_kernel<1, EPI_ACT16, 8, 8, 2>, dim3((unsigned)ceil_div(w.NT, 2)), dim3(512), e); return; }
+        if (best == 30) { launch_skinny(m, name, skinny_gemm_f16_kernel<1, EPI_ACT16, 8, 4, 3>, dim3((unsigned)ceil_div(w.NT, 3)), dim3(512), e); return; }
+        if (best == 40) { launch_skinny(m, name, skinny_gemm_f16_kernel<1, EPI_ACT16, 8, 4, 4>, dim3((unsigned)ceil_div(w.NT, 4)), dim3(512), e); return; }
         TSHIP_REQUIRE(best == 10, "TSHIP_FFN_TILES: 10, 15, 20, 30 or 40");
     }
+    TSHIP_REQUIRE(!e.Wtab, "internal: batched problems go through the kernel's BATCHED instantiations");
+    if (BT == 1 && (epi == EPI_PARTIAL || epi == EPI_SPLIT_TAIL)) {
+        // the first batch of a wavefront is requested whole (fragments beyond its k range are clamped duplicates): a batch as
+        // long as the range keeps the requested bytes at the needed ones
+        const long pw = ceil_div(ceil_div(w.KT, e.KS), 8);
+        if (pw <= 2) {
+            if (epi == EPI_PARTIAL) launch_skinny(m, name, skinny_gemm_f16_kernel<1, EPI_PARTIAL, 8, 2>, grid, dim3(512), e);
+            else launch_skinny(m, name, skinny_gemm_f16_kernel<1, EPI_SPLIT_TAIL, 8, 2>, grid, dim3(512), e);
+            return;
+        }
+        if (pw <= 4) {
+            if (epi == EPI_PARTIAL) launch_skinny(m, name, skinny_gemm_f16_kernel<1, EPI_PARTIAL, 8, 4>, grid, dim3(512), e);
+            else launch_skinny(m, name, skinny_gemm_f16_kernel<1, EPI_SPLIT_TAIL, 8, 4>, grid, dim3(512), e);
+            return;
+        }
+    }
 #define TSHIP_SK(BTV, NWV)                                                                                                  \
-    if (epi == EPI_PARTIAL) launch(m, name, skinny_gemm_f16_kernel<BTV, EPI_PARTIAL, NWV>, grid, dim3(NWV * 64), e);        \
-    else if (epi == EPI_F32_BIAS) launch(m, name, skinny_gemm_f16_kernel<BTV, EPI_F32_BIAS, NWV>, grid, dim3(NWV * 64), e); \
-    else if (epi == EPI_RESID_TAIL) launch(m, name, skinny_gemm_f16_kernel<BTV, EPI_RESID_TAIL, NWV, (BTV == 1 ? 16 : 8)>, grid, dim3(NWV * 64), e); \
-    else if (epi == EPI_SPLIT_TAIL) launch(m, name, skinny_gemm_f16_kernel<BTV, EPI_SPLIT_TAIL, NWV>, grid, dim3(NWV * 64), e); \
-    else launch(m, name, skinny_gemm_f16_kernel<BTV, EPI_ACT16, NWV>, grid, dim3(NWV * 64), e);
+    if (epi == EPI_PARTIAL) launch_skinny(m, name, skinny_gemm_f16_kernel<BTV, EPI_PARTIAL, NWV>, grid, dim3(NWV * 64), e);        \
+    else if (epi == EPI_F32_BIAS) launch_skinny(m, name, skinny_gemm_f16_kernel<BTV, EPI_F32_BIAS, NWV>, grid, dim3(NWV * 64), e); \
+    else if (epi == EPI_RESID_TAIL) launch_skinny(m, name, skinny_gemm_f16_kernel<BTV, EPI_RESID_TAIL, NWV, (BTV == 1 ? 16 : 8)>, grid, dim3(NWV * 64), e); \
+    else if (epi == EPI_SPLIT_TAIL) launch_skinny(m, name, skinny_gemm_f16_kernel<BTV, EPI_SPLIT_TAIL, NWV>, grid, dim3(NWV * 64), e); \
+    else launch_skinny(m, name, skinny_gemm_f16_kernel<BTV, EPI_ACT16, NWV>, grid, dim3(NWV * 64), e);
     if (BT == 1) { TSHIP_SK(1, 8) } else if (BT == 2) { TSHIP_SK(2, 8) } else { TSHIP_SK(4, 4) }
 #undef TSHIP_SK
 }
@@ -526,11 +549,25 @@ static AttnKernel pick_attn_mfma(int G, bool prefill, bool split, bool ragged, i
             default: throw Error("query heads per KV head must be 1, 2, 4 or 8");
         }
     }
+    TSHIP_REQUIRE(prefill, "internal: the MFMA decode kernels are picked by pick_attn_mfma_decode");
+    (void)split;
     switch (G) {
-        case 1: return prefill ? attn_mfma_prefill_kernel<D, 1> : split ? attn_mfma_kernel<D, 1, true> : attn_mfma_kernel<D, 1, false>;
-        case 2: return prefill ? attn_mfma_prefill_kernel<D, 2> : split ? attn_mfma_kernel<D, 2, true> : attn_mfma_kernel<D, 2, false>;
-        case 4: return prefill ? attn_mfma_prefill_kernel<D, 4> : split ? attn_mfma_kernel<D, 4, true> : attn_mfma_kernel<D, 4, false>;
-        case 8: return prefill ? attn_mfma_prefill_kernel<D, 8> : split ? attn_mfma_kernel<D, 8, true> : attn_mfma_kernel<D, 8, false>;
+        case 1: return attn_mfma_prefill_kernel<D, 1>;
+        case 2: return attn_mfma_prefill_kernel<D, 2>;
+        case 4: return attn_mfma_prefill_kernel<D, 4>;
+        case 8: return attn_mfma_prefill_kernel<D, 8>;
+        default: throw Error("query heads per KV head must be 1, 2, 4 or 8");
+    }
+}
+// MFMA decode attention: leading scalar arguments (preloaded at wavefront start) in front of the struct
+typedef void (*AttnDecodeKernel)(void*, void*, const float*, const int*, int, int, int, int, int, int, AttnArgs);
+template <int D>
+static AttnDecodeKernel pick_attn_mfma_decode(int G, bool split) {
+    switch (G) {
+        case 1: return split ? attn_mfma_kernel<D, 1, true> : attn_mfma_kernel<D, 1, false>;
+        case 2: return split ? attn_mfma_kernel<D, 2, true> : attn_mfma_kernel<D, 2, false>;
+        case 4: return split ? attn_mfma_kernel<D, 4, true> : attn_mfma_kernel<D, 4, false>;
+        case 8: return split ? attn_mfma_kernel<D, 8, true> : attn_mfma_kernel<D, 8, false>;
         default: throw Error("query heads per KV head must be 1, 2, 4 or 8");
     }
 }
@@ -573,14 +610,20 @@ static int attn_splits(TSHipGpt* m, int B) {
     return (int)std::max<long>(1, std::min<long>(S, TSHipGpt::MAX_ATTN_SPLITS));
 }
 static void launch_attn_decode(TSHipGpt* m, AttnArgs a, int B) {
+    if (!m->vt) { launch(m, "attn_decode", pick_attn(m, false), dim3(m->c.n_kv_heads, B), dim3(1024), a); return; }
     const int S = attn_splits(m, B);
-    const unsigned threads = m->vt ? (m->D == 128 ? 256 : 512) : 1024;
-    if (S == 1) { launch(m, "attn_decode", pick_attn(m, false), dim3(m->c.n_kv_heads, B), dim3(threads), a); return; }
-    const long pairs = (long)B * m->c.n_kv_heads, per = (long)m->G * m->D + 2 * m->G;
-    TSHIP_REQUIRE((size_t)(pairs * S * per) * sizeof(float) <= m->attn_xchg.bytes && (size_t)pairs * sizeof(int) <= m->attn_count.bytes,
-                  "internal: attention exchange area too small");
-    a.S = S; a.xchg = m->attn_xchg.as<float>(); a.xcount = m->attn_count.as<int>();
-    launch(m, "attn_decode", pick_attn(m, false, true), dim3(m->c.n_kv_heads, B, S), dim3(threads), a);
+    const unsigned threads = m->D == 128 ? 256 : 512;
+    dim3 grid(m->c.n_kv_heads, B);
+    if (S > 1) {
+        const long pairs = (long)B * m->c.n_kv_heads, per = (long)m->G * m->D + 2 * m->G;
+        TSHIP_REQUIRE((size_t)(pairs * S * per) * sizeof(float) <= m->attn_xchg.bytes && (size_t)pairs * sizeof(int) <= m->attn_count.bytes,
+                      "internal: attention exchange area too small");
+        a.S = S; a.xchg = m->attn_xchg.as<float>(); a.xcount = m->attn_count.as<int>();
+        grid.z = (unsigned)S;
+    }
+    TSHIP_REQUIRE(a.max_len < (1L << 31) && a.ldq < (1L << 31) && a.split_stride < (1L << 31), "internal: attention strides beyond 32 bits");
+    AttnDecodeKernel k = m->D == 64 ? pick_attn_mfma_decode<64>(m->G, S > 1) : pick_attn_mfma_decode<128>(m->G, S > 1);
+    launch(m, "attn_decode", k, grid, dim3(threads), a.kcache, a.vcache, a.qkv, a.d_pos, (int)a.max_len, a.Hkv, a.H, a.KS, (int)a.ldq, (int)a.split_stride, a);
 }
 
 // ------------------------------------------------------------------------------------------------

@@ -143,11 +143,11 @@ static void run_moe_ffn_impl(TSHipGpt* m, LayerW& L, int rows, const ResidNormAr
         // Measured and not used: 2 or 4 column tiles per block with one copy of the activations (20 and 23 us), and the same
         // split for the down projection (19.1 against 17.9 us: its 256 blocks are one round either way).
         e1.row_tiles_z = 1;
-        launch(m, "moe_gemm1", skinny_gemm_f16_kernel<1, EPI_ACT16, 8>, dim3(e1.NT, E, (unsigned)m->BT), dim3(512), e1);
+        launch_skinny(m, "moe_gemm1", skinny_gemm_f16_kernel<1, EPI_ACT16, 8, 8, 1, false, true>, dim3(e1.NT, E, (unsigned)m->BT), dim3(512), e1);
         dim3 g2(e2.NT, E);
-        if (m->BT == 1) launch(m, "moe_gemm2", skinny_gemm_f16_kernel<1, EPI_F32_BIAS, 8>, g2, dim3(512), e2);
-        else if (m->BT == 2) launch(m, "moe_gemm2", skinny_gemm_f16_kernel<2, EPI_F32_BIAS, 8>, g2, dim3(512), e2);
-        else launch(m, "moe_gemm2", skinny_gemm_f16_kernel<4, EPI_F32_BIAS, 4>, g2, dim3(256), e2);
+        if (m->BT == 1) launch_skinny(m, "moe_gemm2", skinny_gemm_f16_kernel<1, EPI_F32_BIAS, 8, 8, 1, false, true>, g2, dim3(512), e2);
+        else if (m->BT == 2) launch_skinny(m, "moe_gemm2", skinny_gemm_f16_kernel<2, EPI_F32_BIAS, 8, 8, 1, false, true>, g2, dim3(512), e2);
+        else launch_skinny(m, "moe_gemm2", skinny_gemm_f16_kernel<4, EPI_F32_BIAS, 4, 8, 1, false, true>, g2, dim3(256), e2);
     } else {
         float* xg = (float*)(base + o.xg); float* mid = (float*)(base + o.mid);
         if (fused_lists) launch(m, "moe_gather", moe_gather_lists_kernel<float>, dim3(rows, E), dim3(256), (const float*)top_idx, rows, k, (const float*)xn32, h,

@@ -167,8 +167,17 @@ struct SkinnyArgs {
 // tile, or 8-15 and 24-31: whole 128-byte runs of a weight fragment, and both factors of a gated pair (n, n + 16).
 // The lanes of the other columns fetch their neighbours' bytes again (same cache lines, no further request) and
 // compute sums that are never stored.
-template <int BT, int EPI, int NW, int U = 8, int NJ = 1, bool HALF = false>
-__global__ __launch_bounds__(NW * 64) void skinny_gemm_f16_kernel(SkinnyArgs a) {
+// The leading scalar arguments are the ones the first weight and activation requests depend on.  They are preloaded into
+// scalar registers when the wavefront is created (the translation unit is compiled with a kernel-argument preload count;
+// a struct passed by value is never preloaded), so those requests go out without a round trip to the argument segment;
+// everything else arrives from the struct while they are in flight.  The struct's own copies of these fields are ignored.
+// BATCHED: the launch covers several problems (MoE experts, a.Wtab / a.rows_tab); a template argument, because the branch
+// would otherwise put a wait for the struct in front of every launch's first requests.
+template <int BT, int EPI, int NW, int U = 8, int NJ = 1, bool HALF = false, bool BATCHED = false>
+__global__ __launch_bounds__(NW * 64) void skinny_gemm_f16_kernel(const half_t* __restrict__ W_, const half_t* __restrict__ X_, int KT_, int NT_, int KS_,
+                                                                  int rows_valid_, const float* __restrict__ ssq_, int ssq_nt_, int ssq_ld_,
+                                                                  SkinnyArgs a) {
+    a.W = W_; a.X = X_; a.KT = KT_; a.NT = NT_; a.KS = KS_; a.rows_valid = rows_valid_; a.ssq = ssq_; a.ssq_nt = ssq_nt_; a.ssq_ld = ssq_ld_;
     static_assert(!HALF || NJ == 2, "tile-and-a-half blocks are two-tile blocks with one tile half masked");
     static_assert(NJ == 1 || (EPI == EPI_ACT16 && BT == 1 && NW == 8), "several column tiles per block: one-round activation epilogue only");
     // one batch tile and eight wavefronts: every wavefront stores its accumulator once and the epilogue adds the eight
@@ -178,7 +187,7 @@ __global__ __launch_bounds__(NW * 64) void skinny_gemm_f16_kernel(SkinnyArgs a) 
     __shared__ float smem[RED > FIN ? RED : FIN];      // the tree buffers are dead when the transpose buffer is written
     float (*red)[BT][16][64] = (float (*)[BT][16][64])smem;
     float (*fin)[BT * 32][33] = (float (*)[BT * 32][33])smem;
-    if (a.Wtab) {
+    if constexpr (BATCHED) {
         const int e = blockIdx.y;
         a.rows_valid = a.rows_tab[e];
         if (a.row_tiles_z) {
@@ -231,52 +240,22 @@ __global__ __launch_bounds__(NW * 64) void skinny_gemm_f16_kernel(SkinnyArgs a) 
     __shared__ float srinv[BT * 32];
     constexpr int NCH = (NW * 64) / (BT * 32);
     __shared__ float schunk[NCH][BT * 32];
-    // (a chunk's tail beyond four tiles is added here, one dependent load after the other; its first four sums stay in
-    // registers until the weight stream has been requested, so that their latency hides behind it)
-    float ssq_part = 0.0f, ssq_v[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    // (the first eight tile sums of a chunk are requested here and stay in registers until the weight stream has been
+    // requested, so that their latency hides behind it; a chunk's tail beyond eight tiles is added behind the stream)
+    float ssq_v[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
     if (a.ssq) {
         const int b = threadIdx.x % (BT * 32), ch = threadIdx.x / (BT * 32);
         const int per_ch = (a.ssq_nt + NCH - 1) / NCH;
         const int t0 = ch * per_ch, t1 = min(a.ssq_nt, t0 + per_ch);
-#pragma unroll
-        for (int i = 0; i < 4; ++i) if (t0 + i < t1) ssq_v[i] = a.ssq[(long)(t0 + i) * a.ssq_ld + b];
+        // (unconditional requests at clamped tiles; what lies beyond the chunk is dropped)
+        // (the values stay untouched until they are added behind the stream: any arithmetic on them here would wait for them)
+        (void)t1;
         if (per_ch > 4) {
-            ssq_part = ((ssq_v[0] + ssq_v[1]) + ssq_v[2]) + ssq_v[3];
-            ssq_v[0] = ssq_v[1] = ssq_v[2] = ssq_v[3] = 0.0f;
-            for (int t = t0 + 4; t < t1; ++t) ssq_part += a.ssq[(long)t * a.ssq_ld + b];
-        }
-    }
-    // bias of this thread's outputs in the one-round activation epilogue
-    float eb1[NJ], eb2[NJ];
 #pragma unroll
-    for (int j = 0; j < NJ; ++j) {
-        eb1[j] = 0.0f; eb2[j] = 0.0f;
-        if (ONE_ROUND && EPI == EPI_ACT16) {
-            const int n1 = 8 * (w >> 2) + 4 * (lane >> 5) + (w & 3);
-            if (a.gated) {
-                const int f = tile_of[j] * 16 + n1;
-                if (f < a.n_valid) { eb1[j] = a.bias[f]; eb2[j] = a.bias2[f]; }
-            } else {
-                const int f = tile_of[j] * 32 + n1;
-                if (f < a.n_valid) eb1[j] = a.bias[f];
-                if (f + 16 < a.n_valid) eb2[j] = a.bias[f + 16];
-            }
-        }
-    }
-    // residual tail: the old residual, bias and gamma of this thread's outputs do not depend on the product
-    constexpr int ITER = BT * 1024 / (NW * 64);
-    float tail_x[ITER], tail_b[ITER], tail_g[ITER];
-    if (EPI == EPI_RESID_TAIL || EPI == EPI_SPLIT_TAIL) {
+            for (int i = 0; i < 8; ++i) ssq_v[i] = a.ssq[(long)min(t0 + i, a.ssq_nt - 1) * a.ssq_ld + b];
+        } else {
 #pragma unroll
-        for (int it = 0; it < ITER; ++it) {
-            const int idx = threadIdx.x + it * NW * 64;
-            // (one-round epilogue: outputs (lane % 32, n1) and (lane % 32, n1 + 16); otherwise row-major over the tile)
-            const int col = nt * 32 + (ONE_ROUND ? 8 * (w >> 2) + 4 * (lane >> 5) + (w & 3) + 16 * it : (idx & 31));
-            const int b = ONE_ROUND ? (lane & 31) : (idx >> 5);
-            const bool ok = b < a.rows_valid && col < a.n_valid;
-            tail_x[it] = ok ? a.x[(long)b * a.ldx_res + col] : 0.0f;
-            tail_b[it] = ok ? a.bias[col] : 0.0f;
-            tail_g[it] = ok ? a.gamma[col] : 0.0f;
+            for (int i = 0; i < 4; ++i) ssq_v[i] = a.ssq[(long)min(t0 + i, a.ssq_nt - 1) * a.ssq_ld + b];
         }
     }
     // (a tile beyond the last one reads the last one again; nothing of it is stored)
@@ -301,6 +280,80 @@ __global__ __launch_bounds__(NW * 64) void skinny_gemm_f16_kernel(SkinnyArgs a) 
     // Full batches of U k-tiles run without conditions: a request under a condition of its own would make every
     // later wait cover all requests, and the products could not start while the batch is still arriving.
     int kt = wk0;
+    // The first batch is requested before anything that needs the argument struct: its addresses come from preloaded
+    // arguments only.  Its requests are unconditional (k-tiles beyond the wavefront's range are clamped into the matrix and
+    // their fragments dropped), so that the waits stay exact.
+    half8 wf0[U][NJ];
+    half8 xf0[U][BT];
+    {
+        const int klast = max(min(wk1, a.KT) - 1, 0);
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int kk = min(kt + u, klast);
+#pragma unroll
+            for (int j = 0; j < NJ; ++j) wf0[u][j] = *(const half8*)(wp[j] + (long)kk * 512);
+#pragma unroll
+            for (int bt = 0; bt < BT; ++bt) xf0[u][bt] = *(const half8*)(xp[bt] + (long)kk * 512);
+        }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    // bias of this thread's outputs in the one-round activation epilogue
+    float eb1[NJ], eb2[NJ];
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+        eb1[j] = 0.0f; eb2[j] = 0.0f;
+        if (ONE_ROUND && EPI == EPI_ACT16) {
+            const int n1 = 8 * (w >> 2) + 4 * (lane >> 5) + (w & 3);
+            // (unconditional requests at clamped indices: a request under a condition of its own, issued between the first
+            // batch's requests and its products, would make the waits for the batch inexact)
+            const int nlast = max(a.n_valid, 1) - 1;
+            if (a.gated) {
+                const int f = tile_of[j] * 16 + n1;
+                eb1[j] = a.bias[min(f, nlast)]; eb2[j] = a.bias2[min(f, nlast)];      // (used only where f < n_valid)
+            } else {
+                const int f = tile_of[j] * 32 + n1;
+                eb1[j] = a.bias[min(f, nlast)]; eb2[j] = a.bias[min(f + 16, nlast)];  // (used only where the column is valid)
+            }
+        }
+    }
+    // residual tail: the old residual, bias and gamma of this thread's outputs do not depend on the product
+    constexpr int ITER = BT * 1024 / (NW * 64);
+    float tail_x[ITER], tail_b[ITER], tail_g[ITER];
+    if (EPI == EPI_RESID_TAIL || EPI == EPI_SPLIT_TAIL) {
+#pragma unroll
+        for (int it = 0; it < ITER; ++it) {
+            const int idx = threadIdx.x + it * NW * 64;
+            // (one-round epilogue: outputs (lane % 32, n1) and (lane % 32, n1 + 16); otherwise row-major over the tile)
+            const int col = nt * 32 + (ONE_ROUND ? 8 * (w >> 2) + 4 * (lane >> 5) + (w & 3) + 16 * it : (idx & 31));
+            const int b = ONE_ROUND ? (lane & 31) : (idx >> 5);
+            // (unconditional requests at clamped indices, see above; the values are used only for valid rows and columns)
+            const int bc = min(b, max(a.rows_valid, 1) - 1), cc = min(col, max(a.n_valid, 1) - 1);
+            tail_x[it] = a.x[(long)bc * a.ldx_res + cc];
+            tail_b[it] = a.bias[cc];
+            tail_g[it] = a.gamma[cc];
+        }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    if (kt + U <= wk1) {
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+            for (int j = 0; j < NJ; ++j)
+#pragma unroll
+                for (int bt = 0; bt < BT; ++bt) acc[j][bt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf0[u][j], xf0[u][bt], acc[j][bt], 0, 0, 0);
+    } else {
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            if (kt + u < wk1) {
+#pragma unroll
+                for (int j = 0; j < NJ; ++j)
+#pragma unroll
+                    for (int bt = 0; bt < BT; ++bt) acc[j][bt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf0[u][j], xf0[u][bt], acc[j][bt], 0, 0, 0);
+            }
+        }
+    }
+    kt = min(kt + U, max(wk1, wk0));
+    __builtin_amdgcn_sched_barrier(0);
     for (; kt + U <= wk1; kt += U) {
         half8 wf[U][NJ];
         half8 xf[U][BT];
@@ -345,7 +398,21 @@ __global__ __launch_bounds__(NW * 64) void skinny_gemm_f16_kernel(SkinnyArgs a) 
     // rinv per row from the tile sums: NCH chunks of tiles are added in parallel (loads issued before the weight
     // stream, see above), then the chunk sums in order
     if (a.ssq) {
-        ssq_part = (((ssq_part + ssq_v[0]) + ssq_v[1]) + ssq_v[2]) + ssq_v[3];
+        float ssq_part = 0.0f;
+        {
+            const int b = threadIdx.x % (BT * 32), ch = threadIdx.x / (BT * 32);
+            const int per_ch = (a.ssq_nt + NCH - 1) / NCH;
+            const int t0 = ch * per_ch, t1 = min(a.ssq_nt, t0 + per_ch);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) ssq_part += (i < (per_ch > 4 ? 8 : 4) && t0 + i < t1) ? ssq_v[i] : 0.0f;
+            for (int t = t0 + 8; t < t1; t += 8) {       // (wide models at batches above 32: eight independent requests at a time)
+                float v[8];
+#pragma unroll
+                for (int i = 0; i < 8; ++i) v[i] = a.ssq[(long)min(t + i, a.ssq_nt - 1) * a.ssq_ld + b];
+#pragma unroll
+                for (int i = 0; i < 8; ++i) ssq_part += t + i < t1 ? v[i] : 0.0f;
+            }
+        }
         schunk[threadIdx.x / (BT * 32)][threadIdx.x % (BT * 32)] = ssq_part;
         __syncthreads();
         if (threadIdx.x < BT * 32) {
@@ -2161,8 +2228,14 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(AttnArgs a) {
 // block leaves its unnormalised sums in an exchange area and the block that arrives last merges them in block order
 // (same publication protocol as the split-K projections: agent-scope atomic stores, wait, counter; no spinning).
 // For launches with fewer (row, head) pairs than CUs.
+// The leading scalar arguments are what the first requests (projection partial sums, first cache chunk, position) depend
+// on; they are preloaded into scalar registers at wavefront start (see skinny_gemm_f16_kernel), the struct arrives while
+// those requests are in flight.  The struct's own copies of these fields are ignored.
 template <int D, int G, bool SPLIT>
-__global__ __launch_bounds__(D == 128 ? 256 : 512) void attn_mfma_kernel(AttnArgs a) {
+__global__ __launch_bounds__(D == 128 ? 256 : 512) void attn_mfma_kernel(void* kcache_, void* vcache_, const float* __restrict__ qkv_, const int* __restrict__ d_pos_,
+                                                                       int max_len_, int Hkv_, int H_, int KS_, int ldq_, int split_stride_, AttnArgs a) {
+    a.kcache = kcache_; a.vcache = vcache_; a.qkv = qkv_; a.d_pos = d_pos_; a.max_len = max_len_; a.Hkv = Hkv_; a.H = H_; a.KS = KS_;
+    a.ldq = ldq_; a.split_stride = split_stride_;
     constexpr int NW = D == 128 ? 4 : 8, NTH = NW * 64;
     constexpr int NCOL = G;                   // MFMA columns in use: the G query heads of the group
     constexpr int KD = D / 32, DT = D / 16;
@@ -2204,20 +2277,16 @@ __global__ __launch_bounds__(D == 128 ? 256 : 512) void attn_mfma_kernel(AttnArg
     {
         constexpr int CPT = ((G + 2) * D + NTH - 1) / NTH;        // projection columns per thread
         constexpr int PPT = ((G + 1) * D / 2 + NTH - 1) / NTH;    // rotary pairs per thread
-        // every global load of the prologue is issued before the first use
-        // (the first four tile sums of a lane are requested without a wait of their own: a load-and-add loop would cost a
-        // memory round trip ahead of every other request; they are added below in the same order)
-        float ssq_part = 0.0f, ssq_v[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-        if (a.ssq) {      // (unconditional requests at clamped indices; the values beyond the last tile are dropped below)
-#pragma unroll
-            for (int u = 0; u < 4; ++u) ssq_v[u] = a.ssq[(long)min(lane + 64 * u, a.ssq_nt - 1) * a.ssq_ld + b];
-        }
+        // Every global load of the prologue is issued before the first use.  Order: what needs preloaded arguments only
+        // (the projection's partial sums, then the first chunk of keys and values, whose address does not depend on the
+        // position), then what needs the argument struct or the position (bias, tile sums, rotation), requested while the
+        // first are in flight.
         float part[CPT][8], bias[CPT];
         int pcol[CPT];
 #pragma unroll
         for (int ci = 0; ci < CPT; ++ci) {
             const int idx = t + ci * NTH;
-            bias[ci] = 0.0f; pcol[ci] = 0;
+            pcol[ci] = 0;
 #pragma unroll
             for (int k = 0; k < 8; ++k) part[ci][k] = 0.0f;
             if (idx < (G + 2) * D) {
@@ -2228,10 +2297,20 @@ __global__ __launch_bounds__(D == 128 ? 256 : 512) void attn_mfma_kernel(AttnArg
                 pcol[ci] = col;
 #pragma unroll
                 for (int k = 0; k < 8; ++k) if (k < a.KS) part[ci][k] = a.qkv[k * a.split_stride + (long)b * a.ldq + col];
-                bias[ci] = a.bias[col];
             }
         }
         __builtin_amdgcn_sched_barrier(0);
+        load_chunk(min(gw, (int)(a.max_len >> 5) - 1), kfA, vfA);
+        __builtin_amdgcn_sched_barrier(0);
+        // (the first four tile sums of a lane are requested without a wait of their own: a load-and-add loop would cost a
+        // memory round trip ahead of every other request; they are added below in the same order)
+        float ssq_part = 0.0f, ssq_v[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+        if (a.ssq) {      // (unconditional requests at clamped indices; the values beyond the last tile are dropped below)
+#pragma unroll
+            for (int u = 0; u < 4; ++u) ssq_v[u] = a.ssq[(long)min(lane + 64 * u, a.ssq_nt - 1) * a.ssq_ld + b];
+        }
+#pragma unroll
+        for (int ci = 0; ci < CPT; ++ci) bias[ci] = a.bias[pcol[ci]];
         const int pos = pos_base;
         T = pos_base + 1; nchunks = (T + 31) / 32;
         n_own = nchunks > gw ? (nchunks - gw + GS - 1) / GS : 0;
@@ -2243,9 +2322,6 @@ __global__ __launch_bounds__(D == 128 ? 256 : 512) void attn_mfma_kernel(AttnArg
             rc[pi] = 1.0f; rs[pi] = 0.0f;
             if (p < (G + 1) * D / 2 && a.rope_cos) { rc[pi] = a.rope_cos[(long)pos * (D / 2) + p % (D / 2)]; rs[pi] = a.rope_sin[(long)pos * (D / 2) + p % (D / 2)]; }
         }
-        // the stream starts behind the prologue's own requests (its address does not depend on the position)
-        __builtin_amdgcn_sched_barrier(0);
-        load_chunk(min(gw, (int)(a.max_len >> 5) - 1), kfA, vfA);
         __builtin_amdgcn_sched_barrier(0);
         float rinv = 1.0f;
         if (a.ssq) {

@@ -48,7 +48,6 @@ def _protos():
     L.TSHip_GptGetMoeRouting.argtypes = [vp, C.c_int, vp, vp, vp]
     L.TSHip_GptProfileDecode.argtypes = [vp, vp, C.c_int, vp, vp, C.c_int, C.POINTER(C.c_int)]
     L.TSHip_GptProfileSymbols.argtypes = [vp, vp, C.c_int, C.c_int, C.POINTER(C.c_int)]
-    L.TSHip_StreamStructureProbe.argtypes = [C.c_int, vp, vp, vp, C.c_int, vp]
     L.TSHip_GptStepBytes.argtypes = [vp, C.c_int, C.POINTER(C.c_double), C.POINTER(C.c_double)]
     L.TSHip_Synchronize.argtypes = []
     _proto_done = True
@@ -307,19 +306,3 @@ class HipGpt:
         check(lib().TSHip_GptStepBytes(self.h, batch or self.batch, C.byref(w), C.byref(k)))
         return w.value, k.value
 
-
-def stream_structure_probe(phase_bytes, act_kib, repeats=5, fuse_with_next=None):
-    """TSHip_StreamStructureProbe: milliseconds of (one launch per phase, persistent kernel with grid barriers, the same with
-    the next phase's first loads requested before the barrier, one launch per phase with every phase reading the same
-    cache-resident region, one launch per phase with the phases marked in `fuse_with_next` sharing a resident launch with
-    their successor) for a chain of pure streaming phases."""
-    _protos()
-    pb = np.ascontiguousarray(phase_bytes, dtype=np.float64)
-    ak = np.ascontiguousarray(act_kib, dtype=np.int32)
-    assert pb.size == ak.size
-    fz = None if fuse_with_next is None else np.ascontiguousarray(fuse_with_next, dtype=np.int32)
-    assert fz is None or fz.size == pb.size
-    out = np.zeros((5,), np.float32)
-    check(lib().TSHip_Init(0))
-    check(lib().TSHip_StreamStructureProbe(int(pb.size), _ptr(pb), _ptr(ak), _ptr(fz), int(repeats), _ptr(out)))
-    return [float(x) for x in out]

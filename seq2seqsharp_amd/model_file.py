@@ -200,6 +200,13 @@ def gpt_config(m, dtype=None):
         raise ValueError("model file: DecoderType %d is not GPTDecoder" % m["DecoderType"])
     if m["PEType"] == PE_APE:
         raise ValueError("model file: absolute position embeddings (PEType APE) are outside the decode path built here (RoPE and NoPE are supported)")
+    if m["EnableSegmentEmbeddings"]:
+        # CreateTokensEmbeddings adds SegmentEmbedding[segment index] to every token embedding (Utils/TensorUtils.cs:147-152,
+        # table built by Misc.CreateAuxEmbeddings, Utils/Misc.cs:164-168); the fused path has no such table
+        raise ValueError("model file: segment embeddings (EnableSegmentEmbeddings, MaxSegmentNum %d) are not built into this decode path; "
+                         "its logits would differ from the reference's" % m["MaxSegmentNum"])
+    # EnableTagEmbeddings does not change GPTDecoder's results: Decoder.GPTDecode calls CreateTokensEmbeddings without
+    # enableTagEmbedding (Applications/Decoder.cs:673,695; only Encoder.cs:102 passes it), so the flag is accepted
     vocab = len(m["TgtVocab"]["index_to_word"]) if m["TgtVocab"] else 0
     heads = m["MultiHeadNum"]
     gqa = m["MultiHeadAttentionType"] == GQA
@@ -224,6 +231,12 @@ def load_gpt(path_or_bytes, dtype=None):
         if flat.size != int(np.prod(shape)):
             raise ValueError("model file: weight '%s' holds %d values, the configuration needs %s" % (name, flat.size, list(shape)))
         weights[name] = flat.reshape(shape)
+    # a parameter in the file that the decode path would not consume (a segment or position embedding table, another
+    # network's layers) means the file describes a model this path does not compute: refuse rather than ignore it
+    stored = set(m["Name2Weights"]) | set(m["Name2WeightsHalf"]) | set(m["Name2WeightsVQ"])
+    extra = sorted(stored - set(weights))
+    if extra:
+        raise ValueError("model file: %d parameter(s) that the GPTDecoder path does not use: %s" % (len(extra), ", ".join(extra[:8])))
     return cfg, weights, m["TgtVocab"]
 
 

@@ -154,13 +154,3 @@ def test_profile_reports_the_launched_symbols():
     assert "attn" in syms[names.index("attn_decode")] and all("tship::" in s or "kernel" in s for s in syms)
     gpu.close()
 
-
-def test_stream_structure_probe_runs_and_orders_sensibly():
-    """The measurement aid: five timings for a small chain; every block of the persistent variants leaves its bounded
-    barrier (the call fails otherwise)."""
-    from seq2seqsharp_amd.gpt import stream_structure_probe
-    ms = stream_structure_probe([4e6, 1e6, 8e6, 2e6] * 3, [16, 4, 32, 8] * 3, repeats=2, fuse_with_next=[0, 1, 0, 1] * 3)
-    assert len(ms) == 5 and all(0 < m < 50 for m in ms)
-    assert stream_structure_probe([4e6, 1e6], [0, 0], repeats=1)[4] == 0.0          # no fusion asked for
-    with pytest.raises(Exception):
-        stream_structure_probe([1e6] * 200, [0] * 200)          # more phases than the probe's plan holds

@@ -170,6 +170,29 @@ def test_loader_refuses_what_the_path_does_not_cover():
         mf.load_gpt(mf.write_model(m))
 
 
+def test_loader_refuses_segment_embeddings_and_unused_parameters():
+    """A file whose reference decode adds segment embeddings (Utils/TensorUtils.cs:147-152) must not load silently; neither
+    must one that stores parameters the path would ignore.  EnableTagEmbeddings is accepted: GPTDecode never passes it on."""
+    cfg = synth.tiny_config()
+    blob = mf.save_gpt(cfg, synth.make_weights(cfg, 1))
+    m = mf.read_model(blob)
+    m["EnableSegmentEmbeddings"], m["MaxSegmentNum"] = 1, 16
+    with pytest.raises(ValueError, match="segment embeddings"):
+        mf.load_gpt(mf.write_model(m))
+    with pytest.raises(ValueError, match="segment embeddings"):
+        mf.gpt_config(mf.read_model(mf.write_model(m)))
+    m = mf.read_model(blob)
+    m["MaxSegmentNum"] = 16          # the number alone changes nothing in the reference either
+    m["EnableTagEmbeddings"] = 1
+    cfg2, w2, _ = mf.load_gpt(mf.write_model(m))
+    assert cfg2["hidden"] == cfg["hidden"] and "TgtEmbeddings" in w2
+    for extra in ("SegmentEmbedding", "PosEmbedding", "GPTDecoder.SelfAttn_99.W0"):
+        m = mf.read_model(blob)
+        m["Name2Weights"][extra] = np.zeros((16 * cfg["hidden"],), np.float32)
+        with pytest.raises(ValueError, match="does not use.*" + extra.replace(".", r"\.")):
+            mf.load_gpt(mf.write_model(m))
+
+
 def test_oracle_runs_a_loaded_model(oracle, tmp_path):
     """A model written as Float16, read back and fed to the oracle gives the logits of the fp16-rounded weights."""
     cfg = synth.tiny_config()
