@@ -560,7 +560,25 @@ static AttnKernel pick_attn_mfma(int G, bool prefill, bool split, bool ragged, i
     }
 }
 // MFMA decode attention: leading scalar arguments (preloaded at wavefront start) in front of the struct
-typedef void (*AttnDecodeKernel)(void*, void*, const float*, const int*, int, int, int, int, int, int, AttnArgs);
+typedef void (*AttnDecodeKernel)(void*, int, int, int, int, int, int, int, int, unsigned, int, int, unsigned, AttnArgs);
+// the decode kernel's leading arguments: one base pointer and 256-byte offsets from it (see AttnPacked)
+static AttnPacked attn_pack_args(const AttnArgs& a) {
+    auto off = [&](const void* p, const char* what) {
+        if (!p) return 0;
+        const long d = (const char*)p - (const char*)a.kcache;
+        TSHIP_REQUIRE((d & 255) == 0 && (d >> 8) >= INT32_MIN && (d >> 8) <= INT32_MAX, std::string("internal: attention operand not at a 256-byte offset in reach of the key cache: ") + what);
+        return (int)(d >> 8);
+    };
+    TSHIP_REQUIRE(a.max_len < (1L << 31) && a.ldq < (1L << 31) && a.split_stride < (1L << 31), "internal: attention strides beyond 32 bits");
+    TSHIP_REQUIRE(a.H < 256 && a.Hkv < 256 && a.KS < 256 && a.ssq_nt < 65536 && a.ssq_ld < 65536, "internal: attention counts beyond their packed fields");
+    AttnPacked p;
+    p.kcache = a.kcache; p.d_vcache = off(a.vcache, "values"); p.d_qkv = off(a.qkv, "projection"); p.d_pos = off(a.d_pos, "position");
+    p.d_bias = off(a.bias, "bias"); p.d_ssq = off(a.ssq, "tile sums"); p.d_rope_cos = off(a.rope_cos, "cosines"); p.d_rope_sin = off(a.rope_sin, "sines");
+    p.max_len = (int)a.max_len;
+    p.counts = (unsigned)a.H | ((unsigned)a.Hkv << 8) | ((unsigned)a.KS << 16) | (a.ssq ? 1u << 24 : 0u) | (a.rope_cos ? 1u << 25 : 0u);
+    p.ldq = (int)a.ldq; p.split_stride = (int)a.split_stride; p.ssq_dims = (unsigned)a.ssq_nt | ((unsigned)a.ssq_ld << 16);
+    return p;
+}
 template <int D>
 static AttnDecodeKernel pick_attn_mfma_decode(int G, bool split) {
     switch (G) {
@@ -621,9 +639,10 @@ static void launch_attn_decode(TSHipGpt* m, AttnArgs a, int B) {
         a.S = S; a.xchg = m->attn_xchg.as<float>(); a.xcount = m->attn_count.as<int>();
         grid.z = (unsigned)S;
     }
-    TSHIP_REQUIRE(a.max_len < (1L << 31) && a.ldq < (1L << 31) && a.split_stride < (1L << 31), "internal: attention strides beyond 32 bits");
     AttnDecodeKernel k = m->D == 64 ? pick_attn_mfma_decode<64>(m->G, S > 1) : pick_attn_mfma_decode<128>(m->G, S > 1);
-    launch(m, "attn_decode", k, grid, dim3(threads), a.kcache, a.vcache, a.qkv, a.d_pos, (int)a.max_len, a.Hkv, a.H, a.KS, (int)a.ldq, (int)a.split_stride, a);
+    const AttnPacked p = attn_pack_args(a);
+    launch(m, "attn_decode", k, grid, dim3(threads), p.kcache, p.d_vcache, p.d_qkv, p.d_pos, p.d_bias, p.d_ssq, p.d_rope_cos, p.d_rope_sin, p.max_len, p.counts,
+           p.ldq, p.split_stride, p.ssq_dims, a);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -1356,9 +1375,13 @@ static int generate_impl(TSHipGpt* m, int n_steps, int mode, float top_p, float 
             m->graph_uniforms = uni_base; m->graph_gen = gen.as<int>(); m->graph_penalty = m->repeat_penalty;
         }
     }
-    hipEvent_t e0, e1;
-    TSHIP_CHECK_HIP(hipEventCreate(&e0));
-    TSHIP_CHECK_HIP(hipEventCreate(&e1));
+    struct EventPair {      // destroyed on every path out of the function
+        hipEvent_t a = nullptr, b = nullptr;
+        ~EventPair() { if (a) (void)hipEventDestroy(a); if (b) (void)hipEventDestroy(b); }
+    } ev;
+    TSHIP_CHECK_HIP(hipEventCreate(&ev.a));
+    TSHIP_CHECK_HIP(hipEventCreate(&ev.b));
+    const hipEvent_t e0 = ev.a, e1 = ev.b;
     TSHIP_CHECK_HIP(hipStreamSynchronize(stream()));
     TSHIP_CHECK_HIP(hipEventRecord(e0, stream()));
     int done = 0;
@@ -1382,7 +1405,6 @@ static int generate_impl(TSHipGpt* m, int n_steps, int mode, float top_p, float 
     TSHIP_CHECK_HIP(hipStreamSynchronize(stream()));
     float ms = 0.0f;
     TSHIP_CHECK_HIP(hipEventElapsedTime(&ms, e0, e1));
-    (void)hipEventDestroy(e0); (void)hipEventDestroy(e1);
     if (elapsed_ms) *elapsed_ms = ms;
     if (steps_done) *steps_done = done;
     if (eos_id < 0) TSHIP_CHECK_HIP(hipMemcpy(host_ids_out, gen.p, (size_t)n_steps * B * sizeof(int), hipMemcpyDeviceToHost));

@@ -2228,14 +2228,29 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(AttnArgs a) {
 // block leaves its unnormalised sums in an exchange area and the block that arrives last merges them in block order
 // (same publication protocol as the split-K projections: agent-scope atomic stores, wait, counter; no spinning).
 // For launches with fewer (row, head) pairs than CUs.
-// The leading scalar arguments are what the first requests (projection partial sums, first cache chunk, position) depend
-// on; they are preloaded into scalar registers at wavefront start (see skinny_gemm_f16_kernel), the struct arrives while
-// those requests are in flight.  The struct's own copies of these fields are ignored.
+// The leading scalar arguments are everything the prologue's requests depend on: they are preloaded into scalar registers
+// at wavefront start (see skinny_gemm_f16_kernel; at most 14 of them), so that no request waits for the argument struct.
+// To fit, the pointers travel as one base (the key cache) and offsets from it in units of 256 bytes (every one of them is
+// the start of a device allocation), and the small integers share words; attn_pack_args (host) builds them.  The struct's
+// own copies of these fields are ignored.
+struct AttnPacked {
+    void* kcache; int d_vcache, d_qkv, d_pos, d_bias, d_ssq, d_rope_cos, d_rope_sin;   // offsets from kcache, 256-byte units
+    int max_len; unsigned counts;     // H | Hkv << 8 | KS << 16 | (ssq ? 1 : 0) << 24 | (rope ? 1 : 0) << 25
+    int ldq, split_stride; unsigned ssq_dims;   // ssq_nt | ssq_ld << 16
+};
 template <int D, int G, bool SPLIT>
-__global__ __launch_bounds__(D == 128 ? 256 : 512) void attn_mfma_kernel(void* kcache_, void* vcache_, const float* __restrict__ qkv_, const int* __restrict__ d_pos_,
-                                                                       int max_len_, int Hkv_, int H_, int KS_, int ldq_, int split_stride_, AttnArgs a) {
-    a.kcache = kcache_; a.vcache = vcache_; a.qkv = qkv_; a.d_pos = d_pos_; a.max_len = max_len_; a.Hkv = Hkv_; a.H = H_; a.KS = KS_;
-    a.ldq = ldq_; a.split_stride = split_stride_;
+__global__ __launch_bounds__(D == 128 ? 256 : 512) void attn_mfma_kernel(void* kcache_, int d_vcache, int d_qkv, int d_pos, int d_bias, int d_ssq, int d_rope_cos,
+                                                                       int d_rope_sin, int max_len_, unsigned counts, int ldq_, int split_stride_,
+                                                                       unsigned ssq_dims, AttnArgs a) {
+    {
+        char* base = (char*)kcache_;
+        auto at = [&](int d) { return (void*)(base + ((long)d << 8)); };
+        a.kcache = kcache_; a.vcache = at(d_vcache); a.qkv = (const float*)at(d_qkv); a.d_pos = (const int*)at(d_pos); a.bias = (const float*)at(d_bias);
+        a.ssq = (counts >> 24) & 1 ? (const float*)at(d_ssq) : nullptr;
+        a.rope_cos = (counts >> 25) & 1 ? (const float*)at(d_rope_cos) : nullptr; a.rope_sin = (counts >> 25) & 1 ? (const float*)at(d_rope_sin) : nullptr;
+        a.max_len = max_len_; a.H = counts & 255; a.Hkv = (counts >> 8) & 255; a.KS = (counts >> 16) & 255;
+        a.ldq = ldq_; a.split_stride = split_stride_; a.ssq_nt = ssq_dims & 0xffff; a.ssq_ld = ssq_dims >> 16;
+    }
     constexpr int NW = D == 128 ? 4 : 8, NTH = NW * 64;
     constexpr int NCOL = G;                   // MFMA columns in use: the G query heads of the group
     constexpr int KD = D / 32, DT = D / 16;
@@ -2277,10 +2292,17 @@ __global__ __launch_bounds__(D == 128 ? 256 : 512) void attn_mfma_kernel(void* k
     {
         constexpr int CPT = ((G + 2) * D + NTH - 1) / NTH;        // projection columns per thread
         constexpr int PPT = ((G + 1) * D / 2 + NTH - 1) / NTH;    // rotary pairs per thread
-        // Every global load of the prologue is issued before the first use.  Order: what needs preloaded arguments only
-        // (the projection's partial sums, then the first chunk of keys and values, whose address does not depend on the
-        // position), then what needs the argument struct or the position (bias, tile sums, rotation), requested while the
-        // first are in flight.
+        // Every global load of the prologue is issued before the first use, and none of them waits for the argument
+        // struct.  Order: the tile sums, the projection's partial sums and the bias (the first phase of the prologue needs
+        // them; loads return in order), then the first chunk of keys and values, whose address does not depend on the
+        // position, then the rotation of the position, which the second phase needs.
+        // (the first four tile sums of a lane are requested without a wait of their own: a load-and-add loop would cost a
+        // memory round trip ahead of every other request; they are added below in the same order)
+        float ssq_part = 0.0f, ssq_v[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+        if (a.ssq) {      // (unconditional requests at clamped indices; the values beyond the last tile are dropped below)
+#pragma unroll
+            for (int u = 0; u < 4; ++u) ssq_v[u] = a.ssq[(long)min(lane + 64 * u, a.ssq_nt - 1) * a.ssq_ld + b];
+        }
         float part[CPT][8], bias[CPT];
         int pcol[CPT];
 #pragma unroll
@@ -2298,19 +2320,11 @@ __global__ __launch_bounds__(D == 128 ? 256 : 512) void attn_mfma_kernel(void* k
 #pragma unroll
                 for (int k = 0; k < 8; ++k) if (k < a.KS) part[ci][k] = a.qkv[k * a.split_stride + (long)b * a.ldq + col];
             }
+            bias[ci] = a.bias[pcol[ci]];
         }
         __builtin_amdgcn_sched_barrier(0);
         load_chunk(min(gw, (int)(a.max_len >> 5) - 1), kfA, vfA);
         __builtin_amdgcn_sched_barrier(0);
-        // (the first four tile sums of a lane are requested without a wait of their own: a load-and-add loop would cost a
-        // memory round trip ahead of every other request; they are added below in the same order)
-        float ssq_part = 0.0f, ssq_v[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-        if (a.ssq) {      // (unconditional requests at clamped indices; the values beyond the last tile are dropped below)
-#pragma unroll
-            for (int u = 0; u < 4; ++u) ssq_v[u] = a.ssq[(long)min(lane + 64 * u, a.ssq_nt - 1) * a.ssq_ld + b];
-        }
-#pragma unroll
-        for (int ci = 0; ci < CPT; ++ci) bias[ci] = a.bias[pcol[ci]];
         const int pos = pos_base;
         T = pos_base + 1; nchunks = (T + 31) / 32;
         n_own = nchunks > gw ? (nchunks - gw + GS - 1) / GS : 0;
