@@ -37,10 +37,34 @@ def _log(msg):
     print("[bench] " + msg, file=sys.stderr, flush=True)
 
 
-def cpu_baseline(cfg, gpu, weights, next_ids, budget_note):
-    """One decode step of the CPU oracle (kind "port": a restatement of the reference's CPU path), single
-    thread, at the benchmark's shape, on the KV cache the GPU prefill produced.  Also returns the logit
-    difference between that step and the GPU's, a full-size parity number."""
+def _cpu_model():
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.lower().startswith("model name"):
+                return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def _oracle_flags():
+    """The compiler line of the oracle's build recipe (oracle/Makefile), as text."""
+    cxx, flags = "g++", ""
+    try:
+        for line in open(os.path.join(ROOT, "oracle", "Makefile")):
+            if line.startswith("CXXFLAGS"):
+                flags = line.split("=", 1)[1].strip()
+            elif line.startswith("CXX "):
+                cxx = line.split("=", 1)[1].strip()
+    except OSError:
+        pass
+    return (cxx + " " + flags + " -fopenmp").strip()
+
+
+def cpu_baseline(cfg, gpu, weights, next_ids, budget_note, n_steps=4):
+    """n_steps decode steps of the CPU oracle (kind "port": a restatement of the reference's CPU path), single
+    thread, at the benchmark's shape, on the KV cache the GPU prefill produced; the mean is reported.  Also returns
+    the logits of the first of those steps, for a full-size parity number against the GPU's."""
     from oracle import ts_oracle as O
     O.set_threads(1)
     B = gpu.batch
@@ -57,11 +81,21 @@ def cpu_baseline(cfg, gpu, weights, next_ids, budget_note):
         orc.set_cache(l, 0, ke, B * H, T, d)
         orc.set_cache(l, 1, ve, B * H, T, d)
     seqs = np.ascontiguousarray(next_ids.reshape(B, 1), dtype=np.int32)
-    t0 = time.perf_counter()
-    _, lg = orc.step(seqs, use_cache=True)
-    dt = time.perf_counter() - t0
-    return {"value": B / dt, "unit": "tokens/s", "cores": 1, "kind": "port",
-            "sample": "1 decode step of the whole batch at KV length %d (%s), %.1f s" % (T, budget_note, dt)}, lg
+    times, first_logits = [], None
+    for i in range(max(1, n_steps)):
+        t0 = time.perf_counter()
+        probs, lg = orc.step(seqs, use_cache=True)       # (a cached step looks at the last token of every sequence only)
+        times.append(time.perf_counter() - t0)
+        _log("CPU oracle step %d of %d: %.1f s" % (i + 1, n_steps, times[-1]))
+        if first_logits is None:
+            first_logits = lg
+        seqs = np.concatenate([seqs, O.argmax(probs).astype(np.int32).reshape(B, 1)], 1)
+    dt = float(np.mean(times))
+    return {"value": B / dt, "unit": "tokens/s", "cores": 1, "threads": 1, "kind": "port",
+            "cpu_model": _cpu_model(), "nproc": os.cpu_count(), "compiler": _oracle_flags(),
+            "seconds_per_step": [round(t, 2) for t in times],
+            "sample": "%d decode steps of the whole batch from KV length %d (%s), mean %.1f s per step; the full run of %d steps "
+                      "would take about %.0f s at that rate (extrapolated)" % (len(times), T, budget_note, dt, cfg.get("steps", 0), dt * cfg.get("steps", 0))}, first_logits
 
 
 def main():
@@ -71,6 +105,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=8)
     ap.add_argument("--config", default="cfg2_1b_gqa_f16")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-steps", type=int, default=4, help="decode steps of the CPU oracle to time (their mean is the reported baseline)")
     ap.add_argument("--no-topp", action="store_true")
     ap.add_argument("--prompt", type=int, default=0, help="override the prompt length")
     ap.add_argument("--prefill-runs", type=int, default=3, help="timed prefill calls (the fastest is reported; many of them keep the chip under load long enough to sample its clock)")
@@ -184,12 +219,14 @@ def main():
     # HBM traffic per launch of the dominant kernel comes from hardware counters, which a separate rocprofv3 --pmc run of this
     # script collects; the figure printed here is the one from the committed summary of that run (named beside it), never
     # a value measured in this process
-    traffic, traffic_source, traffic_kv_len = None, None, None
+    traffic, traffic_source, traffic_kv_len, traffic_ratio, traffic_alg = None, None, None, None, None
     tpath = os.path.join(ROOT, "profiles", "decode_%s_%s_traffic.json" % (args.config, dom))
     if os.path.exists(tpath):
         tj = json.load(open(tpath))
         traffic = tj.get("traffic_bytes_per_launch")
         traffic_kv_len = tj.get("kv_len")                    # attention: the KV length of the counter run (its bytes grow with it)
+        traffic_alg = tj.get("algorithmic_bytes_per_launch")  # algorithmic bytes at that same KV length
+        traffic_ratio = tj.get("traffic_over_algorithmic")    # the comparable figure: both byte counts at the counter run's KV length
         traffic_source = "profiles/" + os.path.basename(tpath)
 
     out = {
@@ -200,7 +237,8 @@ def main():
         "config": {"workload": args.config, "batch": B, "prompt_len": Tp, "kv_len_start": T_start, "kv_len_end": T_end,
                    "sampling": "greedy", "rope_base": cfg["rope_base"]},
         "roofline": {"bound": "hbm", "achieved": dom_r["achieved_GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": dom_r["frac"],
-                     "traffic": traffic, "traffic_source": traffic_source, "traffic_kv_len": traffic_kv_len, "kernel": dom_r["kernel"], "launch": dom,
+                     "traffic": traffic, "traffic_over_algorithmic": traffic_ratio, "traffic_algorithmic_bytes_same_run": traffic_alg,
+                     "traffic_source": traffic_source, "traffic_kv_len": traffic_kv_len, "kernel": dom_r["kernel"], "launch": dom,
                      "bytes_per_launch": dom_r["bytes_per_launch"], "avg_launch_ms": round(dom_r["avg_launch_us"] / 1e3, 5),
                      "timing": "device events attached to each dispatch of 5 profiled steps (a rocprofv3 kernel trace of the graph replays reads about 5 % longer)",
                      "kv_len": t_attn if dom == "attn_decode" else None, "share_of_step": dom_r["share_of_step"]},
@@ -219,9 +257,9 @@ def main():
         _, ms_p = gpu.generate(K, mode=TOPP, top_p=0.9, temperature=1.0, uniforms=u)
         out["topp"] = {"top_p": 0.9, "repeat_penalty": 2.0, "tokens_per_s": round(B * K / (ms_p / 1e3), 1), "ms_per_step": round(ms_p / K, 4)}
     if not args.no_cpu_baseline:
-        _log("CPU baseline (one decode step of the oracle, single thread)")
+        _log("CPU baseline (%d decode steps of the oracle, single thread)" % args.cpu_steps)
         nxt = gpu.sample()
-        base, lg = cpu_baseline(cfg, gpu, weights, nxt, "cache from the GPU prefill")
+        base, lg = cpu_baseline(cfg, gpu, weights, nxt, "cache from the GPU prefill", n_steps=args.cpu_steps)
         gpu.decode(nxt)
         out["cpu_baseline"] = base
         gl = gpu.logits()

@@ -14,6 +14,7 @@
 #pragma once
 
 #include "tship_internal.h"
+#include <cstddef>
 #include <type_traits>
 
 namespace tship {
@@ -2567,13 +2568,39 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(D == 64 ? (
     constexpr int NF = 2 * KD + DT;          // 1 KiB fragments per chunk: keys (tile, kd), then values (dt)
     constexpr int FPW = NF / NW;             // fragments a wavefront brings per chunk
     static_assert(NF % NW == 0, "fragments must divide among the wavefronts");
-    // per wavefront: the queries [16 columns][D] as fp16, later the outputs [D / 2][16 columns] as fp32, half of them at a
-    // time (2 KiB at head size 64: with the stages 48.5 KiB per block, three blocks per compute unit)
-    __shared__ __attribute__((aligned(16))) half_t sbuf[NW][D * 16];
-    __shared__ float sl[NW][16];
-    // four chunk stages, of their own: with two of them in the query / output staging area (16 KiB less, a third block
-    // per compute unit at head size 64) single rows of the wavefronts that own that area came out wrong now and then
-    __shared__ __attribute__((aligned(16))) half_t sstage[4 * NF * 512];
+    // LDS layout, as one struct so that the compiler lays the regions out and the assertions below are about what it did.
+    // The invariant they state: a direct-to-LDS request may land at any time between its issue and the wait at the barrier
+    // two chunks later, so the bytes it targets (one stage) must belong to nothing that any wavefront reads or writes in
+    // that window: the stages are an array of their own, apart from the per-wavefront staging of queries and outputs (which
+    // is written right behind barriers), and a request issued at barrier j targets the stage of chunk j + AHEAD, while
+    // the wavefronts between barriers j and j + 1 read the stages of chunks j (values) and j + 1 (keys) and older
+    // requests are still landing in the stage of chunk j + 1.
+    constexpr int STAGES = 4, AHEAD = 2;
+    struct PrefillLds {
+        // per wavefront: the queries [16 columns][D] as fp16, later the outputs [D / 2][16 columns] as fp32, half of them
+        // at a time (2 KiB at head size 64: with the stages 48.5 KiB per block, three blocks per compute unit)
+        __attribute__((aligned(16))) half_t sbuf[NW][D * 16];
+        float sl[NW][16];
+        // the chunk stages, of their own: with two of them in the query / output staging area (16 KiB less, a third block
+        // per compute unit at head size 64) single rows of the wavefronts that own that area came out wrong now and then
+        __attribute__((aligned(16))) half_t sstage[STAGES][NF * 512];
+    };
+    static_assert((STAGES & (STAGES - 1)) == 0, "stage_of() masks the chunk number");
+    static_assert(AHEAD + 2 <= STAGES, "the stage a request lands in (chunk j + AHEAD) must differ from the stages read between barriers j and j + 1 "
+                                       "(chunks j, j + 1) and from the one the wavefronts that have not yet passed barrier j still read (chunk j - 1)");
+    static_assert(sizeof(float) * (D / 2) * 16 <= sizeof(half_t) * D * 16, "half of a wavefront's outputs [D / 2][16] as fp32 must fit its query staging slice");
+    static_assert(offsetof(PrefillLds, sstage) >= offsetof(PrefillLds, sl) + sizeof(float) * NW * 16 &&
+                  offsetof(PrefillLds, sl) >= offsetof(PrefillLds, sbuf) + sizeof(half_t) * NW * D * 16, "staging, sums and stages do not overlap");
+    static_assert(offsetof(PrefillLds, sstage) % 16 == 0 && (NF * 1024) % 16 == 0, "16-byte fragment reads and direct-to-LDS writes are aligned");
+    static_assert((NF - 1) * 1024 + 63 * 16 + 16 <= NF * 1024, "the last fragment read of a stage (offset (NF - 1) KiB, lane 63) ends inside the stage");
+    static_assert(FPW * NW == NF, "the wavefronts' requests cover a stage exactly: fragments w, w + NW, ...");
+    // blocks per compute unit the launch bounds ask for (waves per SIMD x 4 SIMDs / 8 wavefronts per block): their LDS must fit
+    constexpr int BLOCKS_PER_CU = (D == 64 ? (NQ == 1 && !RAGGED ? 6 : 4) : 2) * 4 / NW;
+    static_assert(sizeof(PrefillLds) * BLOCKS_PER_CU <= 160 * 1024, "the resident blocks' LDS fits the 160 KiB of a compute unit");
+    __shared__ PrefillLds lds;
+    half_t (&sbuf)[NW][D * 16] = lds.sbuf;
+    float (&sl)[NW][16] = lds.sl;
+    half_t* const sstage = &lds.sstage[0][0];
     const int lane = threadIdx.x & 63, w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int r16 = lane & 15, q = lane >> 4;
     const int kvh = blockIdx.y, b = blockIdx.z;
@@ -2589,7 +2616,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(D == 64 ? (
     const half_t* Vt = (const half_t*)a.vcache + ((long)b * a.Hkv + kvh) * (long)D * a.max_len;
     typedef const void __attribute__((address_space(1)))* gptr_t;
     typedef void __attribute__((address_space(3)))* lptr_t;
-    auto stage_of = [&](int c) -> half_t* { return sstage + (c & 3) * (NF * 512); };
+    auto stage_of = [&](int c) -> half_t* { return sstage + (c & (STAGES - 1)) * (NF * 512); };
     auto fetch_to = [&](int c, int slot) {   // this wavefront's fragments of chunk c -> the stage of chunk `slot`
         half_t* dst = stage_of(slot);
 #pragma unroll
@@ -2599,6 +2626,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(D == 64 ? (
             __builtin_amdgcn_global_load_lds((gptr_t)src, (lptr_t)(dst + f * 512), 16, 0, 0);
         }
     };
+    static_assert(AHEAD == 2, "the two requests below are the AHEAD chunks in flight before barrier 0");
     fetch_to(0, 0);
     fetch_to(min(1, nchunks - 1), 1);
 
@@ -2686,11 +2714,14 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(D == 64 ? (
     auto wait_barrier = [&](int j) {
         asm volatile("s_waitcnt vmcnt(%0)" :: "n"(FPW) : "memory");
         __builtin_amdgcn_s_barrier();
-        fetch_to(min(j + 2, nchunks - 1), j + 2);
+        fetch_to(min(j + AHEAD, nchunks - 1), j + AHEAD);
     };
     {
         half8 kf[2][KD], vf[DT];
         floatx4 sA[NQ], sB[NQ];
+        // (hand-written reads: the compiler takes their results as present once issued.  Every read_k is tied by k_landed /
+        // k_landed_alone and every read_v by v_landed, in the basic block that issues it, before anything uses or reuses
+        // the registers; tests/test_asm_hazards.py scans the generated code for a read without such a wait.)
         auto read_k = [&](int c) {
             const unsigned sa = (unsigned)(size_t)(lptr_t)stage_of(c) + lane * 16;
 #pragma unroll
