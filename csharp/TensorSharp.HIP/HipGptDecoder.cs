@@ -130,6 +130,44 @@ namespace TensorSharp.HIP
             return Enumerable.Range(0, B).Select(b => hyp.Select(beam => beam[b]).ToList()).ToList();
         }
 
+        // ---- parked conversations: what GPT.cs keeps in its MemoryCache keyed by the generated text (GPT.cs:153-173, 236-247,
+        //      312-328), as device snapshots: no host round trip, the cache's own layout ----
+        private readonly Dictionary<string, (IntPtr snapshot, DateTime lastUse)> parked = new Dictionary<string, (IntPtr, DateTime)>();
+        public TimeSpan ParkedExpiry { get; set; } = TimeSpan.FromMinutes(10);      // the reference's sliding expiration
+
+        private void DropExpired()
+        {
+            DateTime now = DateTime.UtcNow;
+            foreach (string key in parked.Where(kv => now - kv.Value.lastUse > ParkedExpiry).Select(kv => kv.Key).ToList())
+            {
+                HipNative.TSHip_GptFreeSnapshot(parked[key].snapshot);
+                parked.Remove(key);
+            }
+        }
+
+        /// <summary>Park the current sequences under `key` (the generated text so far, as the reference keys its cache).</summary>
+        public void Park(string key)
+        {
+            DropExpired();
+            HipNative.Check(HipNative.TSHip_GptSaveRows(handle, out IntPtr snap), "GptSaveRows");
+            if (parked.TryGetValue(key, out var old)) HipNative.TSHip_GptFreeSnapshot(old.snapshot);
+            parked[key] = (snap, DateTime.UtcNow);
+        }
+
+        /// <summary>Make the sequences parked under `key` current again; false when nothing (or nothing fresh enough) is parked there.</summary>
+        public bool Resume(string key)
+        {
+            DropExpired();
+            if (!parked.TryGetValue(key, out var hit)) return false;
+            HipNative.Check(HipNative.TSHip_GptRestoreRows(handle, hit.snapshot), "GptRestoreRows");
+            HipNative.Check(HipNative.TSHip_GptSnapshotInfo(hit.snapshot, out int rows, out int _, out long _), "GptSnapshotInfo");
+            batch = rows;
+            parked[key] = (hit.snapshot, DateTime.UtcNow);
+            return true;
+        }
+
+        public int ParkedCount { get { DropExpired(); return parked.Count; } }
+
         // ---- inspection (parity tests, benchmarks) ----
         public float[] Logits() { float[] o = new float[batch * config.Vocab]; HipNative.Check(HipNative.TSHip_GptGetLogits(handle, o), "GptGetLogits"); return o; }
         public float[] Hidden() { float[] o = new float[batch * config.Hidden]; HipNative.Check(HipNative.TSHip_GptGetHidden(handle, o), "GptGetHidden"); return o; }
@@ -171,6 +209,8 @@ namespace TensorSharp.HIP
 
         public void Dispose()
         {
+            foreach (var kv in parked) HipNative.TSHip_GptFreeSnapshot(kv.Value.snapshot);
+            parked.Clear();
             if (handle != IntPtr.Zero) { HipNative.TSHip_GptDestroy(handle); handle = IntPtr.Zero; }
         }
     }

@@ -127,6 +127,10 @@ namespace TensorSharp.HIP
         [DllImport(Dll, CallingConvention = CC)] internal static extern int TSHip_GptGetKV(IntPtr model, int layer, int which, float[] hostOut);
         [DllImport(Dll, CallingConvention = CC)] internal static extern int TSHip_GptSetKV(IntPtr model, int layer, int which, float[] hostIn, int batch, int len);
         [DllImport(Dll, CallingConvention = CC)] internal static extern int TSHip_GptSetSeqLen(IntPtr model, int batch, int len);
+        [DllImport(Dll, CallingConvention = CC)] internal static extern int TSHip_GptSaveRows(IntPtr model, out IntPtr snapshot);
+        [DllImport(Dll, CallingConvention = CC)] internal static extern int TSHip_GptRestoreRows(IntPtr model, IntPtr snapshot);
+        [DllImport(Dll, CallingConvention = CC)] internal static extern int TSHip_GptSnapshotInfo(IntPtr snapshot, out int batch, out int len, out long deviceBytes);
+        [DllImport(Dll, CallingConvention = CC)] internal static extern int TSHip_GptFreeSnapshot(IntPtr snapshot);
         [DllImport(Dll, CallingConvention = CC)] internal static extern int TSHip_GptGetMoeRouting(IntPtr model, int layer, float[] topIdx, float[] topVal, float[] probs);
         [DllImport(Dll, CallingConvention = CC)] internal static extern int TSHip_GptProfileDecode(IntPtr model, int[] hostIds, int batch, byte[] names, float[] ms, int nMax, out int n);
         [DllImport(Dll, CallingConvention = CC)] internal static extern int TSHip_GptProfileSymbols(IntPtr model, byte[] symbols, int stride, int nMax, out int n);

@@ -233,6 +233,22 @@ TSHIP_API int TSHip_GptGetKV(TSHipGpt* m, int layer, int which, float* host_out)
 /* install cache contents (same layout) and the sequence length: lets a benchmark start at a given context length */
 TSHIP_API int TSHip_GptSetKV(TSHipGpt* m, int layer, int which, const float* host_in, int batch, int len);
 TSHIP_API int TSHip_GptSetSeqLen(TSHipGpt* m, int batch, int len);
+
+/* Saved sequence sets, device to device.  The reference parks the KV tensors of a finished request in a MemoryCache keyed by
+ * the generated text (sliding expiry of ten minutes) and takes them out again when a later request continues that text
+ * (Seq2SeqSharp/Applications/GPT.cs:153-173, 236-247, 312-328); several conversations are parked at a time.  Here
+ * TSHip_GptSaveRows copies the used prefix of every layer's cache regions of the current sequences (in the cache's own
+ * layout and type: no host round trip, no float32 expansion), the logits of the last step and the token history into a
+ * snapshot that lives in device memory until TSHip_GptFreeSnapshot; TSHip_GptRestoreRows puts a snapshot back as the
+ * model's current sequences (rows 0 .. batch-1, length as saved), after which TSHip_GptSample / TSHip_GptDecode /
+ * TSHip_GptPrefill (append) continue bit for bit as if nothing had run in between.  The model may serve other sequences
+ * between the two calls; the dictionary keyed by text, and its expiry, belong to the caller (HipGptDecoder.cs).  A snapshot
+ * fits any model object of the same shape and type whose cache is long enough. */
+typedef struct TSHipGptSnapshot TSHipGptSnapshot;
+TSHIP_API int TSHip_GptSaveRows(TSHipGpt* m, TSHipGptSnapshot** out);
+TSHIP_API int TSHip_GptRestoreRows(TSHipGpt* m, const TSHipGptSnapshot* snapshot);
+TSHIP_API int TSHip_GptSnapshotInfo(const TSHipGptSnapshot* snapshot, int* batch, int* len, int64_t* device_bytes);
+TSHIP_API int TSHip_GptFreeSnapshot(TSHipGptSnapshot* snapshot);
 /* routing of MoE layer `layer` at the last step: top_idx/top_val [rows, k], probs [rows, E] (host, float32) */
 TSHIP_API int TSHip_GptGetMoeRouting(TSHipGpt* m, int layer, float* top_idx, float* top_val, float* probs);
 /* per-kernel device times of one decode step (events around every launch on the library stream).

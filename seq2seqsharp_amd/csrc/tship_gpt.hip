@@ -137,6 +137,18 @@ struct TSHipGpt {
     size_t esz() const { return f16 ? 2 : 4; }
 };
 
+// A saved set of sequences: the used prefix of every (sequence, KV head) cache region of every layer, in the cache's own
+// layout and element type, plus what a decode step afterwards needs (logits of the last step, token history).  Device
+// memory only; TSHip_GptSaveRows fills it and TSHip_GptRestoreRows copies it back, device to device.
+struct TSHipGptSnapshot {
+    int batch = 0, len = 0;
+    int n_layers = 0, n_kv_heads = 0, D = 0, vocab = 0; bool f16 = false, vt = false;
+    size_t region_bytes = 0;                       // saved bytes per (sequence, KV head) region
+    std::vector<std::unique_ptr<tship::DevBuf>> k, v;
+    tship::DevBuf logits, last_pos; long last_ld = 0;
+    size_t total_bytes = 0;
+};
+
 namespace tship {
 
 template <typename... KArgs, typename... Args>
@@ -1617,6 +1629,91 @@ TSHIP_API int TSHip_GptSetKV(TSHipGpt* m, int layer, int which, const float* hos
         }
         TSHIP_CHECK_HIP(hipMemcpy(base + ((size_t)b * G + g) * ML * D * m->esz(), tmp.data(), tmp.size(), hipMemcpyHostToDevice));
     }
+    TSHIP_END
+}
+
+// ------------------------------------------------------------------------------------------------
+// Saved sequence sets.  The reference keeps the KV tensors of finished requests in a MemoryCache keyed by the generated
+// text (10 minutes sliding expiry) and puts them back when a request continues that text
+// (Seq2SeqSharp/Applications/GPT.cs:153-173, 236-247, 312-328).  Here the cache rows stay on the device: a snapshot holds
+// the used prefix of the model's cache regions; the text-keyed dictionary lives with the caller.
+// ------------------------------------------------------------------------------------------------
+static size_t used_region_bytes(const TSHipGpt* m, int len) {
+    // fragment-major layout: whole 32-position chunks; row-major: whole positions
+    const long rows = m->vt ? round_up(len, 32) : len;
+    return (size_t)rows * m->D * m->esz();
+}
+
+TSHIP_API int TSHip_GptSaveRows(TSHipGpt* m, TSHipGptSnapshot** out) {
+    TSHIP_BEGIN
+    TSHIP_REQUIRE(m && out, "TSHip_GptSaveRows: null argument");
+    TSHIP_REQUIRE(m->finalized && m->cur_batch > 0, "TSHip_GptSaveRows: no sequences in the cache (prefill first)");
+    std::unique_ptr<TSHipGptSnapshot> sn(new TSHipGptSnapshot());
+    const int B = m->cur_batch, G = m->c.n_kv_heads;
+    sn->batch = B; sn->len = m->pos; sn->n_layers = m->c.n_layers; sn->n_kv_heads = G; sn->D = m->D; sn->vocab = m->c.vocab;
+    sn->f16 = m->f16; sn->vt = m->vt;
+    sn->region_bytes = used_region_bytes(m, m->pos);
+    const size_t pitch = (size_t)m->ML * m->D * m->esz();
+    for (int l = 0; l < m->c.n_layers; ++l) {
+        sn->k.emplace_back(new DevBuf()); sn->v.emplace_back(new DevBuf());
+        if (sn->region_bytes == 0) continue;
+        sn->k[l]->alloc(sn->region_bytes * B * G); sn->v[l]->alloc(sn->region_bytes * B * G);
+        TSHIP_CHECK_HIP(hipMemcpy2DAsync(sn->k[l]->p, sn->region_bytes, m->L[l]->kc.p, pitch, sn->region_bytes, (size_t)B * G, hipMemcpyDeviceToDevice, stream()));
+        TSHIP_CHECK_HIP(hipMemcpy2DAsync(sn->v[l]->p, sn->region_bytes, m->L[l]->vc.p, pitch, sn->region_bytes, (size_t)B * G, hipMemcpyDeviceToDevice, stream()));
+        sn->total_bytes += 2 * sn->region_bytes * B * G;
+    }
+    const size_t lbytes = (size_t)B * round_up(m->c.vocab, 32) * sizeof(float);
+    sn->logits.alloc(lbytes);
+    TSHIP_CHECK_HIP(hipMemcpyAsync(sn->logits.p, m->logits.p, lbytes, hipMemcpyDeviceToDevice, stream()));
+    sn->total_bytes += lbytes;
+    if (m->last_pos.p) {
+        sn->last_ld = m->last_ld;
+        const size_t hbytes = (size_t)B * m->last_ld * sizeof(int);
+        sn->last_pos.alloc(hbytes);
+        TSHIP_CHECK_HIP(hipMemcpyAsync(sn->last_pos.p, m->last_pos.p, hbytes, hipMemcpyDeviceToDevice, stream()));
+        sn->total_bytes += hbytes;
+    }
+    TSHIP_CHECK_HIP(hipStreamSynchronize(stream()));
+    *out = sn.release();
+    TSHIP_END
+}
+
+TSHIP_API int TSHip_GptRestoreRows(TSHipGpt* m, const TSHipGptSnapshot* sn) {
+    TSHIP_BEGIN
+    TSHIP_REQUIRE(m && sn, "TSHip_GptRestoreRows: null argument");
+    TSHIP_REQUIRE(m->finalized, "TSHip_GptRestoreRows: the model is not finalised");
+    TSHIP_REQUIRE(sn->n_layers == m->c.n_layers && sn->n_kv_heads == m->c.n_kv_heads && sn->D == m->D && sn->vocab == m->c.vocab &&
+                  sn->f16 == m->f16 && sn->vt == m->vt, "TSHip_GptRestoreRows: the snapshot was taken from a model of another shape or type");
+    TSHIP_REQUIRE(sn->batch <= m->c.max_batch && sn->len < m->c.max_seq_len, "TSHip_GptRestoreRows: the snapshot does not fit this model's cache");
+    TSHIP_REQUIRE(!m->last_pos.p || (sn->last_pos.p && sn->last_ld == m->last_ld),
+                  "TSHip_GptRestoreRows: the model keeps a token history (repeat penalty) and the snapshot holds none");
+    const int B = sn->batch, G = sn->n_kv_heads;
+    const size_t pitch = (size_t)m->ML * m->D * m->esz();
+    TSHIP_REQUIRE(sn->region_bytes <= pitch, "TSHip_GptRestoreRows: the snapshot's regions are longer than this model's");
+    for (int l = 0; l < m->c.n_layers && sn->region_bytes; ++l) {
+        TSHIP_CHECK_HIP(hipMemcpy2DAsync(m->L[l]->kc.p, pitch, sn->k[l]->p, sn->region_bytes, sn->region_bytes, (size_t)B * G, hipMemcpyDeviceToDevice, stream()));
+        TSHIP_CHECK_HIP(hipMemcpy2DAsync(m->L[l]->vc.p, pitch, sn->v[l]->p, sn->region_bytes, sn->region_bytes, (size_t)B * G, hipMemcpyDeviceToDevice, stream()));
+    }
+    TSHIP_CHECK_HIP(hipMemcpyAsync(m->logits.p, sn->logits.p, sn->logits.bytes, hipMemcpyDeviceToDevice, stream()));
+    if (m->last_pos.p) TSHIP_CHECK_HIP(hipMemcpyAsync(m->last_pos.p, sn->last_pos.p, (size_t)B * m->last_ld * sizeof(int), hipMemcpyDeviceToDevice, stream()));
+    m->pos = sn->len; m->cur_batch = B; m->embed_done = false;
+    TSHIP_CHECK_HIP(hipMemcpyAsync(m->d_pos.p, &m->pos, sizeof(int), hipMemcpyHostToDevice, stream()));
+    TSHIP_CHECK_HIP(hipStreamSynchronize(stream()));
+    TSHIP_END
+}
+
+TSHIP_API int TSHip_GptSnapshotInfo(const TSHipGptSnapshot* sn, int* batch, int* len, int64_t* device_bytes) {
+    TSHIP_BEGIN
+    TSHIP_REQUIRE(sn, "TSHip_GptSnapshotInfo: null snapshot");
+    if (batch) *batch = sn->batch;
+    if (len) *len = sn->len;
+    if (device_bytes) *device_bytes = (int64_t)sn->total_bytes;
+    TSHIP_END
+}
+
+TSHIP_API int TSHip_GptFreeSnapshot(TSHipGptSnapshot* sn) {
+    TSHIP_BEGIN
+    delete sn;
     TSHIP_END
 }
 

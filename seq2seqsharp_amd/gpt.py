@@ -45,6 +45,10 @@ def _protos():
     L.TSHip_GptGetKV.argtypes = [vp, C.c_int, C.c_int, vp]
     L.TSHip_GptSetKV.argtypes = [vp, C.c_int, C.c_int, vp, C.c_int, C.c_int]
     L.TSHip_GptSetSeqLen.argtypes = [vp, C.c_int, C.c_int]
+    L.TSHip_GptSaveRows.argtypes = [vp, C.POINTER(vp)]
+    L.TSHip_GptRestoreRows.argtypes = [vp, vp]
+    L.TSHip_GptSnapshotInfo.argtypes = [vp, C.POINTER(C.c_int), C.POINTER(C.c_int), C.POINTER(C.c_int64)]
+    L.TSHip_GptFreeSnapshot.argtypes = [vp]
     L.TSHip_GptGetMoeRouting.argtypes = [vp, C.c_int, vp, vp, vp]
     L.TSHip_GptProfileDecode.argtypes = [vp, vp, C.c_int, vp, vp, C.c_int, C.POINTER(C.c_int)]
     L.TSHip_GptProfileSymbols.argtypes = [vp, vp, C.c_int, C.c_int, C.POINTER(C.c_int)]
@@ -55,6 +59,68 @@ def _protos():
 
 def _ptr(a):
     return None if a is None else a.ctypes.data_as(C.c_void_p)
+
+
+class KvSnapshot:
+    """Handle of a TSHipGptSnapshot (device memory, freed by close())."""
+
+    def __init__(self, h):
+        self.h = h
+
+    def info(self):
+        b, n, nb = C.c_int(0), C.c_int(0), C.c_int64(0)
+        check(lib().TSHip_GptSnapshotInfo(self.h, C.byref(b), C.byref(n), C.byref(nb)))
+        return b.value, n.value, nb.value
+
+    def close(self):
+        if getattr(self, "h", None):
+            lib().TSHip_GptFreeSnapshot(self.h)
+            self.h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+class KvStore:
+    """The reference's text-keyed cache of parked conversations (GPT.cs:153-173: MemoryCache, sliding expiry of ten
+    minutes), holding device snapshots instead of host tensors.  `clock` is injectable for tests."""
+
+    def __init__(self, ttl_seconds=600.0, clock=None):
+        import time
+        self.ttl, self.clock, self.items = float(ttl_seconds), clock or time.monotonic, {}
+
+    def _expire(self):
+        now = self.clock()
+        for key in [k for k, (_, t) in self.items.items() if now - t > self.ttl]:
+            self.items.pop(key)[0].close()
+
+    def put(self, key, snap):
+        self._expire()
+        old = self.items.pop(key, None)
+        if old:
+            old[0].close()
+        self.items[key] = (snap, self.clock())
+
+    def get(self, key):
+        """The snapshot parked under `key` (its expiry slides), or None."""
+        self._expire()
+        hit = self.items.get(key)
+        if hit is None:
+            return None
+        self.items[key] = (hit[0], self.clock())
+        return hit[0]
+
+    def remove(self, key):
+        hit = self.items.pop(key, None)
+        if hit:
+            hit[0].close()
+
+    def __len__(self):
+        self._expire()
+        return len(self.items)
 
 
 class HipGpt:
@@ -271,6 +337,17 @@ class HipGpt:
     def set_seq_len(self, batch, length):
         check(lib().TSHip_GptSetSeqLen(self.h, batch, length))
         self.batch = batch
+
+    def save_rows(self):
+        """TSHip_GptSaveRows: the current sequences' cache rows, last logits and token history, copied device to device."""
+        h = C.c_void_p()
+        check(lib().TSHip_GptSaveRows(self.h, C.byref(h)))
+        return KvSnapshot(h)
+
+    def restore_rows(self, snap):
+        """TSHip_GptRestoreRows: make a saved set the current sequences again; decoding continues bit for bit."""
+        check(lib().TSHip_GptRestoreRows(self.h, snap.h))
+        self.batch = snap.info()[0]
 
     def moe_routing(self, layer):
         k, E = self.cfg["experts_per_token"], self.cfg["n_experts"]
