@@ -261,6 +261,17 @@ TSHIP_API int TSHip_GptProfileSymbols(TSHipGpt* m, char* symbols, int stride, in
 TSHIP_API int TSHip_GptStepBytes(TSHipGpt* m, int batch, double* weight_bytes, double* kv_bytes);
 
 
+/* Environment switches (test hooks, read once at the start of every TSHip_GptPrefill*, TSHip_GptDecode,
+ * TSHip_GptGenerate*, TSHip_GptProfileDecode call; a value outside the listed ones makes the call fail).  None of them
+ * changes results beyond what the tests that use them state; production runs set none.
+ *   TSHIP_NO_GRAPH=1          the generate loop launches its kernels one by one instead of replaying a captured HIP graph
+ *   TSHIP_ATTN_SPLITS=n       decode attention: n blocks per (sequence, KV head) pair (default: chosen from the batch and context)
+ *   TSHIP_FFN_TILES=10|15|20|30|40   decode FFN up projection: column tiles per block x 10 (15 = a tile and a half)
+ *   TSHIP_PATCH_ROWS=1|2|4|8  prefill GEMM: row tiles per tile patch of an XCD
+ *   TSHIP_ATTN_NQ=1|2         prefill attention: groups of 16 MFMA columns per wavefront
+ *   TSHIP_NO_KV_FUSE=1        prefill: the QKV projection leaves the cache write to a kernel of its own
+ *   TSHIP_NO_MOE_BATCH=1      prefill of MoE layers: one GEMM launch per expert instead of one per projection */
+
 #ifdef __cplusplus
 }
 #endif

@@ -31,11 +31,7 @@ struct DevBuf {
     void alloc(size_t b) {
         release();
         if (b == 0) b = 256;
-        hipError_t e = hipMalloc(&p, b);
-        if (e != hipSuccess) {
-            (void)hipGetLastError(); p = nullptr;
-            throw Error("out of device memory: hipMalloc(" + std::to_string(b) + " bytes) failed");
-        }
+        p = device_malloc_retry(b);      // (throws when the memory is not there even after the pool's cached blocks went back)
         bytes = b;
         TSHIP_CHECK_HIP(hipMemsetAsync(p, 0, b, stream()));
     }
@@ -150,6 +146,36 @@ struct TSHipGptSnapshot {
 };
 
 namespace tship {
+
+// Test hooks (environment variables, listed in include/tship.h).  They are read once per call of an entry point that runs
+// the model (refresh_test_hooks), never inside the per-layer code.
+struct TestHooks {
+    int ffn_tiles = 0;        // TSHIP_FFN_TILES: 10, 15, 20, 30 or 40 = column tiles x 10 per block of the decode FFN up projection
+    int patch_rows = 0;       // TSHIP_PATCH_ROWS: 1, 2, 4 or 8 row tiles per tile patch of the prefill GEMM
+    long attn_splits = 0;     // TSHIP_ATTN_SPLITS: blocks per (sequence, KV head) pair in decode attention
+    int attn_nq = 0;          // TSHIP_ATTN_NQ: 1 or 2 groups of 16 MFMA columns per wavefront in prefill attention
+    bool no_kv_fuse = false;  // TSHIP_NO_KV_FUSE: the QKV projection of a prefill does not write the cache itself
+    bool no_moe_batch = false;// TSHIP_NO_MOE_BATCH: one prefill GEMM launch per expert
+    bool no_graph = false;    // TSHIP_NO_GRAPH: the generate loop launches its kernels one by one
+};
+static TestHooks g_hooks;
+static void refresh_test_hooks() {
+    TestHooks h;
+    if (const char* v = std::getenv("TSHIP_FFN_TILES")) {
+        h.ffn_tiles = std::atoi(v);
+        TSHIP_REQUIRE(h.ffn_tiles == 10 || h.ffn_tiles == 15 || h.ffn_tiles == 20 || h.ffn_tiles == 30 || h.ffn_tiles == 40, "TSHIP_FFN_TILES: 10, 15, 20, 30 or 40");
+    }
+    if (const char* v = std::getenv("TSHIP_PATCH_ROWS")) {
+        h.patch_rows = std::atoi(v);
+        TSHIP_REQUIRE(h.patch_rows == 1 || h.patch_rows == 2 || h.patch_rows == 4 || h.patch_rows == 8, "TSHIP_PATCH_ROWS: 1, 2, 4 or 8");
+    }
+    if (const char* v = std::getenv("TSHIP_ATTN_SPLITS")) { h.attn_splits = std::atol(v); TSHIP_REQUIRE(h.attn_splits >= 1, "TSHIP_ATTN_SPLITS: a positive number"); }
+    if (const char* v = std::getenv("TSHIP_ATTN_NQ")) { h.attn_nq = std::atoi(v); TSHIP_REQUIRE(h.attn_nq == 1 || h.attn_nq == 2, "TSHIP_ATTN_NQ: 1 or 2"); }
+    h.no_kv_fuse = std::getenv("TSHIP_NO_KV_FUSE") != nullptr;
+    h.no_moe_batch = std::getenv("TSHIP_NO_MOE_BATCH") != nullptr;
+    h.no_graph = std::getenv("TSHIP_NO_GRAPH") != nullptr;
+    g_hooks = h;
+}
 
 template <typename... KArgs, typename... Args>
 static void launch(TSHipGpt* m, const char* name, void (*kernel)(KArgs...), dim3 grid, dim3 block, Args... args) {
@@ -418,12 +444,12 @@ static void run_skinny(TSHipGpt* m, const char* name, const GemmW& w, const void
             const long cost = ceil_div(ceil_div(w.NT, nj), ncu) * (2 * nj + 2);
             if (cost < best_cost) { best = 10 * nj; best_cost = cost; }
         }
-        if (const char* v = std::getenv("TSHIP_FFN_TILES")) best = std::atoi(v);      // (tests: 10, 15, 20, 30 or 40)
+        if (g_hooks.ffn_tiles) best = g_hooks.ffn_tiles;
         if (best == 15) { launch_skinny(m, name, skinny_gemm_f16_kernel<1, EPI_ACT16, 8, 8, 2, true>, dim3((unsigned)hb), dim3(512), e); return; }
         if (best == 20) { launch_skinny(m, name, skinny_gemm_f16_kernel<1, EPI_ACT16, 8, 8, 2>, dim3((unsigned)ceil_div(w.NT, 2)), dim3(512), e); return; }
         if (best == 30) { launch_skinny(m, name, skinny_gemm_f16_kernel<1, EPI_ACT16, 8, 4, 3>, dim3((unsigned)ceil_div(w.NT, 3)), dim3(512), e); return; }
         if (best == 40) { launch_skinny(m, name, skinny_gemm_f16_kernel<1, EPI_ACT16, 8, 4, 4>, dim3((unsigned)ceil_div(w.NT, 4)), dim3(512), e); return; }
-        TSHIP_REQUIRE(best == 10, "TSHIP_FFN_TILES: 10, 15, 20, 30 or 40");
+        TSHIP_REQUIRE(best == 10, "internal: column tiles per block");
     }
     TSHIP_REQUIRE(!e.Wtab, "internal: batched problems go through the kernel's BATCHED instantiations");
     if (BT == 1 && (epi == EPI_PARTIAL || epi == EPI_SPLIT_TAIL)) {
@@ -488,7 +514,7 @@ static void run_big_gemm(TSHipGpt* m, const char* name, const GemmW& w, const vo
             // fewer than eight patches would leave XCDs without work: flatter patches (4, 2 or 1 row tiles)
             int ph = 8;
             while (ph > 1 && ceil_div(CT, 4) * ceil_div(RT, ph) < 8) ph /= 2;
-            if (const char* v = std::getenv("TSHIP_PATCH_ROWS")) ph = std::max(1, std::min(8, std::atoi(v)));      // (tests: 1, 2, 4 or 8)
+            if (g_hooks.patch_rows) ph = g_hooks.patch_rows;
             patches = ceil_div(CT, 4) * ceil_div(RT, ph);
             e.patch_rows = ph;
             grid.x = (unsigned)(round_up(patches, 8) * 4 * ph);
@@ -636,7 +662,7 @@ static int attn_splits(TSHipGpt* m, int B) {
     // Splitting pays when a wavefront still walks many chunks: at a context of 1 k the launch is bound by its fixed
     // costs and the exchange adds 0.7 us (measured: 16.8 vs 15.9 us at 4 rows); at 8 k it gains 2.5 %.
     S = std::min<long>(S, (m->ML / 32) / (NW * 8L));
-    if (const char* e = std::getenv("TSHIP_ATTN_SPLITS")) S = std::atol(e);  // testing: force the number of blocks per pair
+    if (g_hooks.attn_splits) S = g_hooks.attn_splits;      // (testing: force the number of blocks per pair)
     return (int)std::max<long>(1, std::min<long>(S, TSHipGpt::MAX_ATTN_SPLITS));
 }
 static void launch_attn_decode(TSHipGpt* m, AttnArgs a, int B) {
@@ -964,7 +990,7 @@ static void prefill(TSHipGpt* m, const int32_t* host_ids, int B, int Tp, const i
         // when its wavefronts' 64 x 128 tiles are whole chunks of whole heads; otherwise a kernel of its own does.
         const int HD = c.n_heads * m->D, GD = c.n_kv_heads * m->D;
         const bool fuse_kv = m->f16 && m->vt && pos0 % 32 == 0 && Tp % 32 == 0 && HD % 128 == 0 && GD % 128 == 0 && R >= 512 && L.qkv.KT % 2 == 0 &&
-                             (m->D == 64 || m->D == 128) && !std::getenv("TSHIP_NO_KV_FUSE");
+                             (m->D == 64 || m->D == 128) && !g_hooks.no_kv_fuse;
         if (m->f16) {
             BigArgs e; std::memset(&e, 0, sizeof(e));
             e.out = pqkv.as<float>(); e.ld_out = (int)qp; e.bias = L.bqkv.as<float>(); e.n_valid = m->Nqkv;
@@ -994,7 +1020,7 @@ static void prefill(TSHipGpt* m, const int32_t* host_ids, int B, int Tp, const i
             // once the prompt is long enough for the coarser blocks to fill the chip.  (At head size 64 the second
             // group costs the second block per compute unit its registers and measured the same.)
             int nq = (m->D == 128 && (long)ceil_div(Tp, (16 / m->G) * 16) * c.n_kv_heads * B >= 2048) ? 2 : 1;
-            if (const char* e = std::getenv("TSHIP_ATTN_NQ")) nq = std::atoi(e) == 2 ? 2 : 1;
+            if (g_hooks.attn_nq) nq = g_hooks.attn_nq;
             const int per_block = (16 / m->G) * 8 * nq;
             launch(m, "p_attn", pick_attn(m, true, false, host_lens != nullptr, nq), dim3((unsigned)ceil_div(Tp, per_block), c.n_kv_heads, B), dim3(512), aa);
         }
@@ -1279,6 +1305,7 @@ TSHIP_API int TSHip_GptSetRepeatPenalty(TSHipGpt* m, float repeat_penalty) {
 
 TSHIP_API int TSHip_GptPrefill(TSHipGpt* m, const int32_t* host_ids, int batch, int prompt_len) {
     TSHIP_BEGIN
+    refresh_test_hooks();
     TSHIP_REQUIRE(m && host_ids, "TSHip_GptPrefill: null argument");
     TSHIP_REQUIRE(m->finalized, "TSHip_GptPrefill: call TSHip_GptFinalize first");
     TSHIP_REQUIRE(batch >= 1 && batch <= m->c.max_batch, "TSHip_GptPrefill: batch out of range");
@@ -1290,6 +1317,7 @@ TSHIP_API int TSHip_GptPrefill(TSHipGpt* m, const int32_t* host_ids, int batch, 
 
 TSHIP_API int TSHip_GptPrefillPadded(TSHipGpt* m, const int32_t* host_ids, const int32_t* host_lens, int batch, int padded_len) {
     TSHIP_BEGIN
+    refresh_test_hooks();
     TSHIP_REQUIRE(m && host_ids && host_lens, "TSHip_GptPrefillPadded: null argument");
     TSHIP_REQUIRE(m->finalized, "TSHip_GptPrefillPadded: call TSHip_GptFinalize first");
     TSHIP_REQUIRE(batch >= 1 && batch <= m->c.max_batch, "TSHip_GptPrefillPadded: batch out of range");
@@ -1302,6 +1330,7 @@ TSHIP_API int TSHip_GptPrefillPadded(TSHipGpt* m, const int32_t* host_ids, const
 
 TSHIP_API int TSHip_GptDecode(TSHipGpt* m, const int32_t* host_ids, int batch) {
     TSHIP_BEGIN
+    refresh_test_hooks();
     TSHIP_REQUIRE(m && host_ids, "TSHip_GptDecode: null argument");
     TSHIP_REQUIRE(m->finalized, "TSHip_GptDecode: call TSHip_GptFinalize first");
     TSHIP_REQUIRE(batch >= 1 && batch <= m->c.max_batch, "TSHip_GptDecode: batch out of range");
@@ -1334,6 +1363,7 @@ TSHIP_API int TSHip_GptSample(TSHipGpt* m, int mode, float top_p, float temperat
 static int generate_impl(TSHipGpt* m, int n_steps, int mode, float top_p, float temperature, const float* host_uniforms, int32_t* host_ids_out,
                          float* elapsed_ms, int eos_id, int* steps_done) {
     TSHIP_BEGIN
+    refresh_test_hooks();
     TSHIP_REQUIRE(m && host_ids_out, "TSHip_GptGenerate: null argument");
     TSHIP_REQUIRE(m->cur_batch > 0, "TSHip_GptGenerate: no logits yet; prefill first");
     TSHIP_REQUIRE(n_steps >= 1, "TSHip_GptGenerate: n_steps must be positive");
@@ -1353,7 +1383,7 @@ static int generate_impl(TSHipGpt* m, int n_steps, int mode, float top_p, float 
     TSHIP_CHECK_HIP(hipMemsetAsync(m->d_pos.as<int>() + 1, 0, sizeof(int), stream()));
     const int* d_step = m->d_pos.as<int>() + 1;
     const float* uni_base = mode == TSHIP_TOPP ? uni.as<float>() : nullptr;
-    const bool use_graph = std::getenv("TSHIP_NO_GRAPH") == nullptr;
+    const bool use_graph = !g_hooks.no_graph;
     if (mode == TSHIP_TOPP) {      // scratch must exist before capture (no allocation inside a graph)
         const size_t need = topp_scratch_bytes(m->Bpad, m->c.vocab);
         if (m->topp_scratch.bytes < need) m->topp_scratch.alloc(need);
@@ -1727,6 +1757,7 @@ TSHIP_API int TSHip_GptGetMoeRouting(TSHipGpt* m, int layer, float* top_idx, flo
 
 TSHIP_API int TSHip_GptProfileDecode(TSHipGpt* m, const int32_t* host_ids, int batch, char* names, float* ms, int n_max, int* n) {
     TSHIP_BEGIN
+    refresh_test_hooks();
     TSHIP_REQUIRE(m && host_ids && names && ms && n, "TSHip_GptProfileDecode: null argument");
     TSHIP_REQUIRE(m->finalized && batch >= 1 && batch <= m->c.max_batch, "TSHip_GptProfileDecode: bad state or batch");
     TSHIP_REQUIRE(m->pos + 1 <= m->c.max_seq_len, "TSHip_GptProfileDecode: KV cache is full");

@@ -98,7 +98,7 @@ static void run_moe_ffn_impl(TSHipGpt* m, LayerW& L, int rows, const ResidNormAr
         launch(m, "moe_gather", moe_gather_kernel<half_t>, dim3(rows, E), dim3(256), (const float*)xn32, h, (const int*)counts, (const int*)lists, (int)Bp, xg,
                m->ldh, xg_stride, 0);
         const int n_max = *std::max_element(n_e.begin(), n_e.end());
-        if (big_gemm_batched_ok(*L.e1[0], n_max) && big_gemm_batched_ok(*L.e2[0], n_max) && L.wtab1.p && L.wtab2.p && !std::getenv("TSHIP_NO_MOE_BATCH")) {
+        if (big_gemm_batched_ok(*L.e1[0], n_max) && big_gemm_batched_ok(*L.e2[0], n_max) && L.wtab1.p && L.wtab2.p && !g_hooks.no_moe_batch) {
             // all experts in one launch per projection (row counts read on the device): the down projection of one expert
             // is 64 tiles at 8 x 4096 rows, a quarter of the compute units
             BigArgs e1; std::memset(&e1, 0, sizeof(e1));

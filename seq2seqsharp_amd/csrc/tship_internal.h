@@ -61,6 +61,11 @@ void ensure_init();
 int current_device();          // device the library was initialised on, -1 before TSHip_Init
 void noalloc_device_setup(int device);   // tship_ops.hip: address of the fixed scratch array, once per device
 int n_compute_units();
+// device memory for the library's own use: blocks of the size-class pool behind TSHip_Malloc / TSHip_Free (no driver call
+// when a cached block fits), and a plain allocation that, on failure, releases what the pool only caches and tries again
+void* pool_alloc(size_t bytes);
+void pool_release(void* p);
+void* device_malloc_retry(size_t bytes);
 
 typedef _Float16 half_t;
 #if defined(__HIP_DEVICE_COMPILE__) && !defined(__gfx950__)

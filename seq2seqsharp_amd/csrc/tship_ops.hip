@@ -729,14 +729,13 @@ TSHIP_API int TSHip_BuildSelfTriMask(const TSHipTensor* result, const TSHipTenso
 
 // shared by gather and scatter_fill: a device flag for indices outside the dimension, read back after the kernel
 static void run_indexed(const char* what, const std::function<void(int*)>& launch_fn) {
-    int* flag = nullptr;
-    TSHIP_CHECK_HIP(hipMalloc(&flag, sizeof(int)));
+    int* flag = (int*)pool_alloc(sizeof(int));        // (a cached block after the first call: no driver call per pick of a beam loop)
     int host = 0;
     hipError_t e = hipMemsetAsync(flag, 0, sizeof(int), stream());
     if (e == hipSuccess) { launch_fn(flag); e = hipGetLastError(); }
     if (e == hipSuccess) e = hipMemcpyAsync(&host, flag, sizeof(int), hipMemcpyDeviceToHost, stream());
     if (e == hipSuccess) e = hipStreamSynchronize(stream());
-    (void)hipFree(flag);
+    pool_release(flag);
     TSHIP_CHECK_HIP(e);
     if (host) throw Error(std::string(what) + ": an index lies outside the dimension");
 }
@@ -779,13 +778,12 @@ TSHIP_API int TSHip_IsCorrupted(const TSHipTensor* src, int* corrupted) {
     long n = count(s);
     *corrupted = 0;
     if (n == 0) return 1;
-    int* flag = nullptr;
-    TSHIP_CHECK_HIP(hipMalloc(&flag, sizeof(int)));
+    int* flag = (int*)pool_alloc(sizeof(int));
     hipError_t e = hipMemsetAsync(flag, 0, sizeof(int), stream());
     if (e == hipSuccess) { hipLaunchKernelGGL(iscorrupted_kernel, grid1(n), dim3(256), 0, stream(), s, n, flag); e = hipGetLastError(); }
     if (e == hipSuccess) e = hipMemcpyAsync(corrupted, flag, sizeof(int), hipMemcpyDeviceToHost, stream());
     if (e == hipSuccess) e = hipStreamSynchronize(stream());
-    (void)hipFree(flag);
+    pool_release(flag);
     TSHIP_CHECK_HIP(e);
     TSHIP_END
 }
@@ -811,8 +809,7 @@ static int topp_sample_op(const char* who, const TSHipTensor* result, const TSHi
     const size_t sort_bytes = round_up((long)topp_scratch_bytes(rows, K), 256);
     const size_t last_bytes = decay ? (size_t)rows * last_ld * sizeof(int) : 0;
     const size_t seq_bytes = decay ? round_up((long)((size_t)rows * seq_ld * sizeof(int)), 256) : 0, len_bytes = decay ? round_up(rows * (long)sizeof(int), 256) : 0;
-    char* scratch = nullptr;
-    TSHIP_CHECK_HIP(hipMalloc((void**)&scratch, sort_bytes + last_bytes + seq_bytes + len_bytes));
+    char* scratch = (char*)pool_alloc(sort_bytes + last_bytes + seq_bytes + len_bytes);
     TopPArgs a; std::memset(&a, 0, sizeof(a));
     a.in = (const float*)p.p; a.ld = p.st[0]; a.V = (int)K; a.in_is_logits = 0; a.temperature = 1.0f;
     a.uniforms = (const float*)u.p; a.top_p = top_p;
@@ -841,7 +838,7 @@ static int topp_sample_op(const char* who, const TSHipTensor* result, const TSHi
     // (the host arrays must stay valid until the copies are done: synchronise before returning in every case)
     hipError_t es = hipStreamSynchronize(stream());
     if (e == hipSuccess) e = es;
-    (void)hipFree(scratch);
+    pool_release(scratch);
     TSHIP_CHECK_HIP(e);
     TSHIP_END
 }

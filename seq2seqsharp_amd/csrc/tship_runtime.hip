@@ -63,7 +63,7 @@ void ensure_init() {
 // allocation failure release them).  A freed block may be handed out again at once without waiting for the GPU: every
 // kernel and copy of this library runs on the one library stream, so whatever still reads the block was enqueued before
 // whatever the next owner enqueues.
-// Size classes: multiples of 256 bytes up to 4 KiB, then four classes per power of two (at most 19 % slack).
+// Size classes: multiples of 256 bytes up to 4 KiB, then four classes per power of two (a request just above a power of two rounds up by a quarter: at most 25 % slack).
 // ------------------------------------------------------------------------------------------------
 static std::mutex g_pool_mutex;
 static std::unordered_map<void*, size_t> g_pool_live;                 // block -> class size
@@ -121,6 +121,26 @@ static void pool_free(void* p) {
     g_pool_live.erase(it);
     g_pool_free[cls].push_back(p);
     g_pool_bytes_live -= cls; g_pool_bytes_cached += cls;
+}
+
+// for the library's own temporaries and long-lived buffers (declared in tship_internal.h)
+void* pool_alloc(size_t bytes) { return pool_malloc(bytes); }
+void pool_release(void* p) { pool_free(p); }
+void* device_malloc_retry(size_t bytes) {
+    void* p = nullptr;
+    hipError_t e = hipMalloc(&p, bytes);
+    if (e != hipSuccess) {
+        // memory that is only cached by the pool is not lost: wait for the GPU, give the cached blocks back, try once more
+        (void)hipGetLastError();
+        (void)hipStreamSynchronize(stream());
+        { std::lock_guard<std::mutex> lk(g_pool_mutex); pool_release_cached_locked(); }
+        e = hipMalloc(&p, bytes);
+    }
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        throw Error("out of device memory: hipMalloc(" + std::to_string(bytes) + " bytes) failed: " + hipGetErrorString(e));
+    }
+    return p;
 }
 
 }  // namespace tship
