@@ -109,7 +109,11 @@ def test_cfg3_moe_layer_shape(G, oracle, dtype):
     bit-exact and logits within 1e-4.  fp16 model: the router sees activations that differ from the oracle's by the fp16
     path's rounding, so a token whose k-th and (k+1)-th expert probabilities are closer than that can be routed to the
     other expert; such rows (few, and only with a margin below 2e-3 in the oracle's own probabilities) are checked for
-    that margin instead of the logit bar, every other row meets the fp16 bars."""
+    that margin instead of the logit bar, every other row meets the fp16 bars.  The margin: the reference adds -65000 to the
+    router's logits (MoEFeedForward.cs:83), which rounds them to multiples of 2^-8, the float32 spacing there; an input
+    difference far below one such step can move a logit across a rounding boundary, by one step.  The choice may differ from
+    the oracle's only where the oracle's own two logits are one step (2^-8) apart or tied (measured here: 1 row of 256,
+    at exactly one step).  The logit gap is the log of the probability ratio."""
     cfg = dict(synth.CONFIGS["cfg3_moe_f16"], n_layers=3, vocab=2048, prompt=6, dtype=dtype)
     B, k = cfg["batch"], cfg["experts_per_token"]
     w = synth.make_weights(cfg, 5, random_bias=True)
@@ -118,7 +122,7 @@ def test_cfg3_moe_layer_shape(G, oracle, dtype):
     cur = synth.make_prompts(cfg, 105)
     gpu.prefill(cur)
     hit = set()
-    agree, flipped = [], 0
+    agree, flipped, worst_gap = [], 0, 0.0
     for step in range(4):
         p, lg = orc.step(cur, use_cache=True)
         gl = gpu.logits()
@@ -136,9 +140,11 @@ def test_cfg3_moe_layer_shape(G, oracle, dtype):
         else:
             same = np.array([set(ti[r]) == set(oi[r]) for r in range(B)])
             srt = -np.sort(-op, axis=1)
-            margin = srt[:, k - 1] - srt[:, k]              # the oracle's own gap between the last expert in and the first out
-            assert (margin[~same] < 2e-3).all()
+            # the oracle's own gap between the last expert in and the first out, in steps of the -65000 quantisation
+            gap_steps = (np.log(srt[:, k - 1].astype(np.float64)) - np.log(srt[:, k].astype(np.float64))) / 2.0 ** -8
+            assert (gap_steps[~same] <= 1.0 + 0.05).all(), gap_steps[~same]
             flipped += int((~same).sum())
+            worst_gap = max(worst_gap, float(gap_steps[~same].max()) if (~same).any() else 0.0)
             assert np.abs(gl[same] - lg[same]).max() <= FP16_ABS
             assert np.abs(pr - op).max() <= 2e-3
             agree.append(top1_agreement(gl[same], lg[same])[0])
@@ -147,6 +153,8 @@ def test_cfg3_moe_layer_shape(G, oracle, dtype):
         gpu.decode(nxt)
     assert hit == set(range(8))                             # every expert is hit at batch 64
     if dtype == "f16":
+        print("fp16 MoE routing at cfg3's layer shape: %d of %d rows routed differently from the fp32 oracle, largest oracle gap among them %.2f steps of 2^-8"
+              % (flipped, 4 * B, worst_gap))
         assert np.mean(agree) >= 0.99 and flipped <= 0.05 * 4 * B
     gpu.close()
 
