@@ -61,6 +61,9 @@ struct LayerW {
     GemmW qkv, wo, w13, w2;
     DevBuf bqkv, bo, b1, b3, b2;
     DevBuf kc, vc;
+    // deferred LayerNorm: per packed output column the folded constants d (norm's beta through the weights, plus the bias)
+    // followed by c (norm's gamma through the weights); see SkinnyArgs.  qkv: [2][round_up(Nqkv, 32)], w13: [2][NT * 32]
+    DevBuf ln_qkv, ln_13;
     bool moe = false;
     // MoE (Seq2SeqSharp/Layers/MoEFeedForward.cs:49-55)
     DevBuf router, router_b;               // fp32 [h][E], [E]
@@ -110,7 +113,9 @@ struct TSHipGpt {
     DevBuf moe_ws, topp_scratch, topp_uni, gen_buf, uni_buf, tile_count;
     DevBuf pw_lens, pw_ids, pw_x, pw_xn, pw_qkv, pw_o, pw_a, pw_f, pw_rowmap, pw_ssq, pw_rinv, pw_zero_bias, pw_moe;     // prefill workspace
     DevBuf ssq;                    // deferred-norm path: per-column-tile sums of squares [h/32][Bpad]
-    bool fused_norm = false;       // fp16 + RMSNorm + dense layers: residual/norm folded into the GEMM tails
+    bool fused_norm = false;       // fp16 + dense layers (RMSNorm; LayerNorm up to 32 rows): residual/norm folded into the GEMM tails
+    bool ln = false;               // that path with LayerNorm: tile sums of x beside the sums of squares, folded constants per consumer
+    DevBuf ln_head;                // [2][round_up(vocab, 32)]: d then c of the vocabulary projection behind the final norm
     bool vt = false;               // fp16 cache with head_dim 64/128: keys and values stored fragment-major for the MFMA attention kernels
     long ML = 0;                   // cache rows per (sequence, KV head): max_seq_len rounded up to 32
     // one decode step (sample + decode) captured as a HIP graph; valid for one (batch, sampling mode) at a time
@@ -221,7 +226,7 @@ static void launch_shm(TSHipGpt* m, const char* name, void (*kernel)(KArgs...), 
 // (preloaded into scalar registers at wavefront start), the rest in the struct
 template <typename... KArgs>
 static void launch_skinny(TSHipGpt* m, const char* name, void (*kernel)(KArgs...), dim3 grid, dim3 block, const SkinnyArgs& e) {
-    launch(m, name, kernel, grid, block, e.W, e.X, e.KT, e.NT, e.KS, e.rows_valid, e.ssq, e.ssq_nt, e.ssq_ld, e);
+    launch(m, name, kernel, grid, block, e.W, e.X, e.KT, e.NT, e.KS, e.rows_valid, e.ssq, e.ssq_nt, e.ssq_ld, e.ln, e);
 }
 
 // decode GEMM split-K: a block has NW wavefronts of 8 k-tiles each in flight; split K across blocks until one
@@ -613,7 +618,7 @@ static AttnPacked attn_pack_args(const AttnArgs& a) {
     p.kcache = a.kcache; p.d_vcache = off(a.vcache, "values"); p.d_qkv = off(a.qkv, "projection"); p.d_pos = off(a.d_pos, "position");
     p.d_bias = off(a.bias, "bias"); p.d_ssq = off(a.ssq, "tile sums"); p.d_rope_cos = off(a.rope_cos, "cosines"); p.d_rope_sin = off(a.rope_sin, "sines");
     p.max_len = (int)a.max_len;
-    p.counts = (unsigned)a.H | ((unsigned)a.Hkv << 8) | ((unsigned)a.KS << 16) | (a.ssq ? 1u << 24 : 0u) | (a.rope_cos ? 1u << 25 : 0u);
+    p.counts = (unsigned)a.H | ((unsigned)a.Hkv << 8) | ((unsigned)a.KS << 16) | (a.ssq ? 1u << 24 : 0u) | (a.rope_cos ? 1u << 25 : 0u) | (a.ln ? 1u << 26 : 0u);
     p.ldq = (int)a.ldq; p.split_stride = (int)a.split_stride; p.ssq_dims = (unsigned)a.ssq_nt | ((unsigned)a.ssq_ld << 16);
     return p;
 }
@@ -717,6 +722,7 @@ static FnPrepArgs embed_prepare_args(TSHipGpt* m, const int* d_ids) {
     FnPrepArgs a; std::memset(&a, 0, sizeof(a));
     a.x = m->x.as<float>(); a.ldx = h; a.h = h; a.ids = d_ids; a.emb = m->emb.p; a.emb_f16 = 1; a.emb_scale = (float)std::sqrt((double)h);
     a.gamma = m->L[0]->n1_g.as<float>(); a.xg16 = m->xn.as<half_t>(); a.xg_kt = (int)(m->ldh / 16); a.ssq_out = m->ssq.as<float>(); a.ssq_ld = m->Bpad;
+    a.ln = m->ln ? 1 : 0;
     return a;
 }
 static void decode_step_fn(TSHipGpt* m, const int* d_ids, int B) {
@@ -725,11 +731,12 @@ static void decode_step_fn(TSHipGpt* m, const int* d_ids, int B) {
     const long hp = round_up(h, 32), qp = round_up(m->Nqkv, 32), Vp = round_up(c.vocab, 32);
     const int NTh = (int)(hp / 32), xkt = (int)(m->ldh / 16);
     float* ssq = m->ssq.as<float>();
-    auto with_ssq = [&](SkinnyArgs& e) { e.ssq = ssq; e.ssq_nt = NTh; e.ssq_ld = m->Bpad; e.inv_h = 1.0f / (float)h; e.eps = c.norm_eps; };
+    auto with_ssq = [&](SkinnyArgs& e) { e.ssq = ssq; e.ssq_nt = NTh; e.ssq_ld = m->Bpad; e.inv_h = 1.0f / (float)h; e.eps = c.norm_eps; e.ln = m->ln ? 1 : 0; };
     auto tail = [&](SkinnyArgs& e, const float* bias, const float* gamma) {
         e.out = m->part_h.as<float>(); e.ld_out = (int)hp; e.split_stride = (long)m->Bpad * hp;
         e.bias = bias; e.n_valid = h; e.x = m->x.as<float>(); e.ldx_res = h; e.gamma = gamma;
         e.xg16 = m->xn.as<half_t>(); e.xg_kt = xkt; e.ssq_out = ssq; e.ssq_out_ld = m->Bpad;
+        e.ln = m->ln ? 1 : 0;      // (LayerNorm: the tails also store the tiles' plain sums)
     };
     if (m->embed_done) {
         m->embed_done = false;        // (the greedy sampling kernel went on to embed the tokens it chose)
@@ -752,6 +759,7 @@ static void decode_step_fn(TSHipGpt* m, const int* d_ids, int B) {
             a.qkv = m->part_qkv.as<float>(); a.KS = L.qkv.KS; a.split_stride = qstride; a.ldq = qp;
             a.out = m->o.p; a.ld_out = m->ldh; a.out_kt = xkt;
             a.ssq = ssq; a.ssq_nt = NTh; a.ssq_ld = m->Bpad; a.inv_h = 1.0f / (float)h; a.eps = c.norm_eps;
+            if (m->ln) { a.ln = 1; a.bias = L.ln_qkv.as<float>(); TSHIP_REQUIRE(a.ldq == qp, "internal: folded LayerNorm constants are laid out by the projection's leading dimension"); }
             launch_attn_decode(m, a, B);
         }
         {
@@ -769,6 +777,7 @@ static void decode_step_fn(TSHipGpt* m, const int* d_ids, int B) {
             e.bias = L.b1.as<float>(); e.bias2 = L.b3.as<float>(); e.out16 = m->a.as<half_t>(); e.ld16 = (int)m->ldF;
             e.act = c.act; e.gated = m->gated; e.n_valid = F; e.out16_kt = L.w2.KT;
             with_ssq(e);
+            if (m->ln) { e.ln_d = L.ln_13.as<float>(); e.ln_c = L.ln_13.as<float>() + (long)L.w13.NT * 32; }
             run_skinny(m, "gemm_ffn13", L.w13, m->xn.p, m->ldh, B, EPI_ACT16, e);
         }
         const float* next_gamma = l + 1 < c.n_layers ? m->L[l + 1]->n1_g.as<float>() : m->fn_g.as<float>();
@@ -802,6 +811,7 @@ static void decode_step_fn(TSHipGpt* m, const int* d_ids, int B) {
         SkinnyArgs e; std::memset(&e, 0, sizeof(e));
         e.out = m->logits.as<float>(); e.ld_out = (int)Vp; e.bias = m->head_b.as<float>(); e.n_valid = c.vocab;
         with_ssq(e);
+        if (m->ln) { e.ln_d = m->ln_head.as<float>(); e.ln_c = m->ln_head.as<float>() + Vp; }
         e.advance_pos = m->d_pos.as<int>();
         run_skinny(m, "gemm_head", m->head, m->xn.p, m->ldh, B, EPI_F32_BIAS, e);
     }
@@ -951,7 +961,7 @@ static void prefill(TSHipGpt* m, const int32_t* host_ids, int B, int Tp, const i
     // Deferred RMSNorm (fp16 RMSNorm models, LDS-tiled GEMMs): no norm kernels.  The producer of the residual stream
     // stores half(gamma * x) and per-(32-column tile, row) sums of squares, a one-thread-per-row kernel turns those into
     // 1 / rms, and the consuming GEMMs scale their output rows by it.
-    const bool deferred = m->fused_norm && R >= 512;
+    const bool deferred = m->fused_norm && !m->ln && R >= 512;
     const int NTh = (int)(round_up(h, 32) / 32);
     DevBuf &pssq = m->pw_ssq, &prinv = m->pw_rinv;
     auto make_rinv = [&](const char* name) {
@@ -1069,7 +1079,7 @@ static void prefill(TSHipGpt* m, const int32_t* host_ids, int B, int Tp, const i
         else if (l + 1 < c.n_layers || !m->f16) run_resid_norm(m, "p_norm_attn", (int)R, a3);
     }
     // last position of every sequence (Decoder.cs:705-716) -> final norm -> vocabulary projection
-    if (m->fused_norm) {
+    if (m->fused_norm && !m->ln) {
         FnPrepArgs a; std::memset(&a, 0, sizeof(a));
         a.x = m->x.as<float>(); a.ldx = h; a.h = h; a.src = px.as<float>(); a.ld_src = h; a.row_map = rowmap.as<int>();
         a.gamma = m->fn_g.as<float>(); a.xg16 = m->xn.as<half_t>(); a.xg_kt = (int)(m->ldh / 16); a.ssq_out = m->ssq.as<float>(); a.ssq_ld = m->Bpad;
@@ -1086,7 +1096,7 @@ static void prefill(TSHipGpt* m, const int32_t* host_ids, int B, int Tp, const i
     if (m->f16) {
         SkinnyArgs e; std::memset(&e, 0, sizeof(e));
         e.out = m->logits.as<float>(); e.ld_out = (int)Vp; e.bias = m->head_b.as<float>(); e.n_valid = c.vocab;
-        if (m->fused_norm) { e.ssq = m->ssq.as<float>(); e.ssq_nt = (int)(round_up(h, 32) / 32); e.ssq_ld = m->Bpad; e.inv_h = 1.0f / (float)h; e.eps = c.norm_eps; }
+        if (m->fused_norm && !m->ln) { e.ssq = m->ssq.as<float>(); e.ssq_nt = (int)(round_up(h, 32) / 32); e.ssq_ld = m->Bpad; e.inv_h = 1.0f / (float)h; e.eps = c.norm_eps; }
         run_skinny(m, "gemm_head", m->head, m->xn.p, m->ldh, B, EPI_F32_BIAS, e);
     } else {
         run_gemm_f32(m, "gemm_head", m->head, m->xn.as<float>(), m->ldh, B, m->logits.as<float>(), Vp, 0, 1, m->head_b.as<float>());
@@ -1193,9 +1203,11 @@ TSHIP_API int TSHip_GptCreate(const TSHipGptConfig* cfg, TSHipGpt** out) {
     TSHIP_CHECK_HIP(hipMemset(m->blocked.p, 0, m->blocked.bytes));
     m->hidden.alloc((size_t)m->Bpad * h * sizeof(float));
     if (c.n_experts > 1) moe_alloc(m.get());
-    m->fused_norm = m->f16 && c.norm_type == 0 && c.n_experts <= 1;
+    // (LayerNorm: batches of up to 32 rows; the tails of larger batches do not store the tiles' plain sums)
+    m->fused_norm = m->f16 && c.n_experts <= 1 && (c.norm_type == 0 || m->BT == 1);
+    m->ln = m->fused_norm && c.norm_type == 1;
     if (m->fused_norm) {
-        m->ssq.alloc((size_t)(hp / 32) * m->Bpad * sizeof(float));
+        m->ssq.alloc((size_t)(m->ln ? 2 : 1) * (hp / 32) * m->Bpad * sizeof(float));
         m->tile_count.alloc((size_t)(std::max<long>(hp, round_up(m->F13, 32)) / 32) * sizeof(int));     // zero-filled; every use returns it to zero
     }
     TSHIP_CHECK_HIP(hipStreamSynchronize(stream()));
@@ -1242,6 +1254,26 @@ TSHIP_API int TSHip_GptFinalize(TSHipGpt* m) {
             L->wo.KS = tail_ks(L->wo);
             L->w2.KS = m->BT == 1 ? tail_ks(L->w2) : (L->w2.KS <= 2 ? 1 : L->w2.KS);
         }
+    }
+    if (m->ln) {
+        // deferred LayerNorm: every consumer of a normalised row gets the norm's gamma and beta folded through its weights
+        // (LayerNormalization.Norm feeds Q/K/V or QKV, feedForwardLayer1/3 and the vocabulary projection)
+        auto fold = [&](DevBuf& dst, const GemmW& w, const DevBuf& gamma, const DevBuf& beta, const float* b1, const float* b2, int mode, int n_logical) {
+            const long n_packed = (long)w.NT * 32;
+            dst.alloc((size_t)2 * n_packed * sizeof(float));
+            ln_fold_kernel<<<(unsigned)ceil_div(n_packed, 64), 64, 0, stream()>>>(w.buf.as<half_t>(), w.KT, w.NT, w.K, gamma.as<float>(), beta.as<float>(), b1, b2, mode, n_logical,
+                                                                                   dst.as<float>() + n_packed, dst.as<float>());
+            TSHIP_CHECK_HIP(hipGetLastError());
+        };
+        const int F = m->c.ffn_dim;
+        for (int l = 0; l < m->c.n_layers; ++l) {
+            LayerW& L = *m->L[l];
+            TSHIP_REQUIRE((long)L.qkv.NT * 32 == round_up(m->Nqkv, 32), "internal: QKV tile count");
+            fold(L.ln_qkv, L.qkv, L.n1_g, L.n1_b, L.bqkv.as<float>(), nullptr, 0, m->Nqkv);
+            fold(L.ln_13, L.w13, L.n2_g, L.n2_b, L.b1.as<float>(), L.b3.as<float>(), m->gated ? 1 : 0, F);
+        }
+        fold(m->ln_head, m->head, m->fn_g, m->fn_b, m->head_b.as<float>(), nullptr, 0, m->c.vocab);
+        TSHIP_CHECK_HIP(hipStreamSynchronize(stream()));
     }
     for (auto& L : m->L) {
         if (!L->moe) continue;
@@ -1581,9 +1613,19 @@ TSHIP_API int TSHip_GptGetHidden(TSHipGpt* m, float* host_out) {
         std::vector<float> xs((size_t)B * h), gm(h);
         TSHIP_CHECK_HIP(hipMemcpy(xs.data(), m->x.p, xs.size() * sizeof(float), hipMemcpyDeviceToHost));
         TSHIP_CHECK_HIP(hipMemcpy(gm.data(), m->fn_g.p, gm.size() * sizeof(float), hipMemcpyDeviceToHost));
+        std::vector<float> bt(h, 0.0f);
+        if (m->ln) TSHIP_CHECK_HIP(hipMemcpy(bt.data(), m->fn_b.p, bt.size() * sizeof(float), hipMemcpyDeviceToHost));
         for (int b = 0; b < B; ++b) {
-            double sq = 0.0;
-            for (int i = 0; i < h; ++i) sq += (double)xs[(size_t)b * h + i] * xs[(size_t)b * h + i];
+            double sq = 0.0, sm = 0.0;
+            for (int i = 0; i < h; ++i) { sq += (double)xs[(size_t)b * h + i] * xs[(size_t)b * h + i]; sm += xs[(size_t)b * h + i]; }
+            if (m->ln) {
+                const double mean = sm / h;
+                double d2 = 0.0;
+                for (int i = 0; i < h; ++i) { const double d = xs[(size_t)b * h + i] - mean; d2 += d * d; }
+                const float sigma = (float)std::sqrt(m->c.norm_eps + d2 / h);
+                for (int i = 0; i < h; ++i) host_out[(size_t)b * h + i] = gm[i] * ((xs[(size_t)b * h + i] - (float)mean) / sigma) + bt[i];
+                continue;
+            }
             float rms = (float)std::sqrt(sq / h + m->c.norm_eps);
             for (int i = 0; i < h; ++i) host_out[(size_t)b * h + i] = gm[i] * (xs[(size_t)b * h + i] / rms);
         }

@@ -113,6 +113,35 @@ __global__ void pack_w_kernel(const float* __restrict__ src, long ld, int K, int
 }
 
 // fp32 -> T copy of a [rows][cols] matrix into a wider destination at a column offset
+// Deferred LayerNorm: fold the norm's gamma and beta into per-column constants of a packed weight matrix (once, when the
+// model is finalised).  For packed column n:  c[n] = sum_k gamma[k] W[k][n],  d[n] = sum_k beta[k] W[k][n] + bias(n),
+// W being the fp16 values the GEMM multiplies with; sums in double, k ascending.  bias_mode 0: bias[n] (plain layout);
+// 1: the gated interleave (packed column 32 g + j stands for column 16 g + j of W1 when j < 16, of W3 otherwise: bias1 /
+// bias2); a null bias counts as zero.  One thread per packed column.
+__global__ void ln_fold_kernel(const half_t* __restrict__ W, int KT, int NT, int K, const float* __restrict__ gamma, const float* __restrict__ beta,
+                               const float* __restrict__ bias1, const float* __restrict__ bias2, int bias_mode, int n_logical,
+                               float* __restrict__ c_out, float* __restrict__ d_out) {
+    const int n = blockIdx.x * blockDim.x + threadIdx.x;
+    if (n >= NT * 32) return;
+    const int nt = n >> 5, nl = n & 31;
+    double c = 0.0, d = 0.0;
+    for (int k = 0; k < K; ++k) {
+        const int kt = k >> 4, kl = k & 15, lane = nl + 32 * (kl >> 3), j = kl & 7;
+        const double w = (double)(float)W[(((long)nt * KT + kt) * 64 + lane) * 8 + j];
+        c += (double)gamma[k] * w;
+        if (beta) d += (double)beta[k] * w;
+    }
+    float b = 0.0f;
+    if (bias_mode == 0) { if (bias1 && n < n_logical) b = bias1[n]; }
+    else {
+        const int f = (n >> 5) * 16 + (n & 15);
+        const float* src = (n & 16) ? bias2 : bias1;
+        if (src && f < n_logical) b = src[f];
+    }
+    c_out[n] = (float)c;
+    d_out[n] = (float)(d + (double)b);
+}
+
 template <typename T>
 __global__ void copy_cols_kernel(const float* __restrict__ src, long ld_src, long rows, long cols, T* __restrict__ dst, long ld_dst,
                                  long col_off) {
@@ -145,6 +174,13 @@ struct SkinnyArgs {
     // deferred RMSNorm: the input rows were stored as half(gamma * x); the epilogue multiplies row b by
     // 1 / sqrt(sum_t ssq[t][b] / h + eps), the factor the norm would have applied (exact up to rounding)
     const float* ssq; int ssq_nt; int ssq_ld; float inv_h; float eps;
+    // deferred LayerNorm (ln != 0; LayerNormalization.Norm, kernel TensorSharp/TensorApplyCPU.cs:1360-1447): the producers
+    // also store the tiles' plain sums, behind the sums of squares (ssq + ssq_nt * ssq_ld); a consumer rebuilds the
+    // row's mean and 1 / sigma = 1 / sqrt(E[x^2] - mean^2 + eps) and computes
+    //     Y = ((half(gamma x) W) - mean * c) / sigma + d,   c[n] = sum_k gamma[k] W[k][n],   d[n] = sum_k beta[k] W[k][n] + bias[n]
+    // with c and d per packed output column (ln_c, ln_d; folded once, when the model is finalised), which is the
+    // product of the normalised row with W.  The bias pointers are not read then.
+    int ln; const float* ln_c; const float* ln_d;
     // EPI_RESID_TAIL (KS == 1: the block holds the complete sums of its column tile): adds bias and residual, stores
     // x, the next GEMM's packed input half(gamma * x) and the tile's per-row sum of squares
     float* x; int ldx_res; const float* gamma; half_t* xg16; int xg_kt; float* ssq_out; int ssq_out_ld;
@@ -176,9 +212,9 @@ struct SkinnyArgs {
 // would otherwise put a wait for the struct in front of every launch's first requests.
 template <int BT, int EPI, int NW, int U = 8, int NJ = 1, bool HALF = false, bool BATCHED = false>
 __global__ __launch_bounds__(NW * 64) void skinny_gemm_f16_kernel(const half_t* __restrict__ W_, const half_t* __restrict__ X_, int KT_, int NT_, int KS_,
-                                                                  int rows_valid_, const float* __restrict__ ssq_, int ssq_nt_, int ssq_ld_,
+                                                                  int rows_valid_, const float* __restrict__ ssq_, int ssq_nt_, int ssq_ld_, int ln_,
                                                                   SkinnyArgs a) {
-    a.W = W_; a.X = X_; a.KT = KT_; a.NT = NT_; a.KS = KS_; a.rows_valid = rows_valid_; a.ssq = ssq_; a.ssq_nt = ssq_nt_; a.ssq_ld = ssq_ld_;
+    a.W = W_; a.X = X_; a.KT = KT_; a.NT = NT_; a.KS = KS_; a.rows_valid = rows_valid_; a.ssq = ssq_; a.ssq_nt = ssq_nt_; a.ssq_ld = ssq_ld_; a.ln = ln_;
     static_assert(!HALF || NJ == 2, "tile-and-a-half blocks are two-tile blocks with one tile half masked");
     static_assert(NJ == 1 || (EPI == EPI_ACT16 && BT == 1 && NW == 8), "several column tiles per block: one-round activation epilogue only");
     // one batch tile and eight wavefronts: every wavefront stores its accumulator once and the epilogue adds the eight
@@ -241,9 +277,12 @@ __global__ __launch_bounds__(NW * 64) void skinny_gemm_f16_kernel(const half_t* 
     __shared__ float srinv[BT * 32];
     constexpr int NCH = (NW * 64) / (BT * 32);
     __shared__ float schunk[NCH][BT * 32];
+    __shared__ float schunk2[NCH][BT * 32];      // LayerNorm: the plain sums' chunks
+    __shared__ float smean[BT * 32];
     // (the first eight tile sums of a chunk are requested here and stay in registers until the weight stream has been
     // requested, so that their latency hides behind it; a chunk's tail beyond eight tiles is added behind the stream)
     float ssq_v[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+    float ssum_v[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};      // (LayerNorm: the tiles' plain sums)
     if (a.ssq) {
         const int b = threadIdx.x % (BT * 32), ch = threadIdx.x / (BT * 32);
         const int per_ch = (a.ssq_nt + NCH - 1) / NCH;
@@ -251,12 +290,21 @@ __global__ __launch_bounds__(NW * 64) void skinny_gemm_f16_kernel(const half_t* 
         // (unconditional requests at clamped tiles; what lies beyond the chunk is dropped)
         // (the values stay untouched until they are added behind the stream: any arithmetic on them here would wait for them)
         (void)t1;
+        const long sum_off = (long)a.ssq_nt * a.ssq_ld;
         if (per_ch > 4) {
 #pragma unroll
             for (int i = 0; i < 8; ++i) ssq_v[i] = a.ssq[(long)min(t0 + i, a.ssq_nt - 1) * a.ssq_ld + b];
+            if (a.ln) {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) ssum_v[i] = a.ssq[sum_off + (long)min(t0 + i, a.ssq_nt - 1) * a.ssq_ld + b];
+            }
         } else {
 #pragma unroll
             for (int i = 0; i < 4; ++i) ssq_v[i] = a.ssq[(long)min(t0 + i, a.ssq_nt - 1) * a.ssq_ld + b];
+            if (a.ln) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) ssum_v[i] = a.ssq[sum_off + (long)min(t0 + i, a.ssq_nt - 1) * a.ssq_ld + b];
+            }
         }
     }
     // (a tile beyond the last one reads the last one again; nothing of it is stored)
@@ -299,16 +347,20 @@ __global__ __launch_bounds__(NW * 64) void skinny_gemm_f16_kernel(const half_t* 
     }
     __builtin_amdgcn_sched_barrier(0);
     // bias of this thread's outputs in the one-round activation epilogue
-    float eb1[NJ], eb2[NJ];
+    float eb1[NJ], eb2[NJ], ec1[NJ], ec2[NJ];      // (ec: LayerNorm's column sums c of the thread's outputs, 0 otherwise)
 #pragma unroll
     for (int j = 0; j < NJ; ++j) {
-        eb1[j] = 0.0f; eb2[j] = 0.0f;
+        eb1[j] = 0.0f; eb2[j] = 0.0f; ec1[j] = 0.0f; ec2[j] = 0.0f;
         if (ONE_ROUND && EPI == EPI_ACT16) {
             const int n1 = 8 * (w >> 2) + 4 * (lane >> 5) + (w & 3);
             // (unconditional requests at clamped indices: a request under a condition of its own, issued between the first
             // batch's requests and its products, would make the waits for the batch inexact)
             const int nlast = max(a.n_valid, 1) - 1;
-            if (a.gated) {
+            if (a.ln) {
+                // per packed column (the tile's columns n1 and n1 + 16, whatever they stand for)
+                const int pc = min(tile_of[j], a.NT - 1) * 32 + n1;
+                eb1[j] = a.ln_d[pc]; eb2[j] = a.ln_d[pc + 16]; ec1[j] = a.ln_c[pc]; ec2[j] = a.ln_c[pc + 16];
+            } else if (a.gated) {
                 const int f = tile_of[j] * 16 + n1;
                 eb1[j] = a.bias[min(f, nlast)]; eb2[j] = a.bias2[min(f, nlast)];      // (used only where f < n_valid)
             } else {
@@ -415,12 +467,33 @@ __global__ __launch_bounds__(NW * 64) void skinny_gemm_f16_kernel(const half_t* 
             }
         }
         schunk[threadIdx.x / (BT * 32)][threadIdx.x % (BT * 32)] = ssq_part;
+        if (a.ln) {
+            float ssum_part = 0.0f;
+            const int b = threadIdx.x % (BT * 32), ch = threadIdx.x / (BT * 32);
+            const int per_ch = (a.ssq_nt + NCH - 1) / NCH;
+            const int t0 = ch * per_ch, t1 = min(a.ssq_nt, t0 + per_ch);
+            const long sum_off = (long)a.ssq_nt * a.ssq_ld;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) ssum_part += (i < (per_ch > 4 ? 8 : 4) && t0 + i < t1) ? ssum_v[i] : 0.0f;
+            for (int t = t0 + 8; t < t1; ++t) ssum_part += a.ssq[sum_off + (long)t * a.ssq_ld + b];
+            schunk2[threadIdx.x / (BT * 32)][threadIdx.x % (BT * 32)] = ssum_part;
+        }
         __syncthreads();
         if (threadIdx.x < BT * 32) {
             float tot = 0.0f;
 #pragma unroll
             for (int c = 0; c < NCH; ++c) tot += schunk[c][threadIdx.x];
-            srinv[threadIdx.x] = 1.0f / sqrtf(tot * a.inv_h + a.eps);
+            if (a.ln) {
+                float tots = 0.0f;
+#pragma unroll
+                for (int c = 0; c < NCH; ++c) tots += schunk2[c][threadIdx.x];
+                const float mean = tots * a.inv_h;
+                srinv[threadIdx.x] = 1.0f / sqrtf(fmaxf(tot * a.inv_h - mean * mean, 0.0f) + a.eps);
+                smean[threadIdx.x] = mean;
+            } else {
+                srinv[threadIdx.x] = 1.0f / sqrtf(tot * a.inv_h + a.eps);
+                smean[threadIdx.x] = 0.0f;
+            }
         }
     }
     if (a.advance_pos && blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) { a.advance_pos[0] += 1; a.advance_pos[1] += 1; }
@@ -438,7 +511,8 @@ __global__ __launch_bounds__(NW * 64) void skinny_gemm_f16_kernel(const half_t* 
             float s1 = red[0][0][w][lane], s2 = red[0][0][w + 8][lane];
 #pragma unroll
             for (int i = 1; i < NW; ++i) { s1 += red[i][0][w][lane]; s2 += red[i][0][w + 8][lane]; }
-            const float rinv = a.ssq ? srinv[b] : 1.0f;
+            const float rinv = a.ssq ? srinv[b] : 1.0f, mean = a.ssq ? smean[b] : 0.0f;
+            s1 -= mean * ec1[j]; s2 -= mean * ec2[j];       // (LayerNorm: the mean's share of the product; 0 otherwise)
             // (outputs n1 and n1 + 16 belong to the first half of a tile when n1 < 8)
             const bool mine = half_of[j] == 0 || (half_of[j] == 1) == (n1 < 8);
             if (a.gated) {
@@ -472,7 +546,8 @@ __global__ __launch_bounds__(NW * 64) void skinny_gemm_f16_kernel(const half_t* 
         for (int i = 1; i < NW; ++i) { s1 += red[i][0][w][lane]; s2 += red[i][0][w + 8][lane]; }
         const int b = lane & 31, n1 = 8 * (w >> 2) + 4 * (lane >> 5) + (w & 3);
         const bool rok = b < a.rows_valid;
-        const float rinv = a.ssq ? srinv[b] : 1.0f;
+        const float rinv = a.ssq ? srinv[b] : 1.0f, mean = a.ssq ? smean[b] : 0.0f;
+        if (EPI == EPI_ACT16) { s1 -= mean * ec1[0]; s2 -= mean * ec2[0]; }      // (LayerNorm: the mean's share of the product; 0 otherwise)
         if (EPI == EPI_SPLIT_TAIL) {
             // publish this block's partial sums, then find out whether it is the last of its column tile
             //
@@ -525,8 +600,13 @@ __global__ __launch_bounds__(NW * 64) void skinny_gemm_f16_kernel(const half_t* 
             }
         } else if (EPI == EPI_F32_BIAS) {
             const int c1 = nt * 32 + n1, c2 = c1 + 16;
+            if (a.ln) {
+                if (rok && c1 < a.n_valid) a.out[(long)b * a.ld_out + c1] = (s1 - mean * a.ln_c[c1]) * rinv + a.ln_d[c1];
+                if (rok && c2 < a.n_valid) a.out[(long)b * a.ld_out + c2] = (s2 - mean * a.ln_c[c2]) * rinv + a.ln_d[c2];
+            } else {
             if (rok && c1 < a.n_valid) a.out[(long)b * a.ld_out + c1] = s1 * rinv + a.bias[c1];
             if (rok && c2 < a.n_valid) a.out[(long)b * a.ld_out + c2] = s2 * rinv + a.bias[c2];
+            }
         } else if (EPI == EPI_ACT16) {
             if (a.gated) {
                 const int f = nt * 16 + n1;
@@ -548,7 +628,8 @@ __global__ __launch_bounds__(NW * 64) void skinny_gemm_f16_kernel(const half_t* 
             }
         } else {      // EPI_RESID_TAIL, EPI_SPLIT_TAIL
             __shared__ float sq[NW][32];
-            float q = 0.0f;
+            __shared__ float ssm[NW][32];
+            float q = 0.0f, sv = 0.0f;
 #pragma unroll
             for (int h2 = 0; h2 < 2; ++h2) {
                 const int col = nt * 32 + n1 + 16 * h2;
@@ -556,17 +637,24 @@ __global__ __launch_bounds__(NW * 64) void skinny_gemm_f16_kernel(const half_t* 
                     const float v = ((h2 ? s2 : s1) + tail_b[h2]) + tail_x[h2];
                     a.x[(long)b * a.ldx_res + col] = v;
                     a.xg16[xpack_index(b, col, a.xg_kt)] = (half_t)(tail_g[h2] * v);
-                    q += v * v;
+                    q += v * v; sv += v;
                 }
             }
             q += __shfl_xor(q, 32, 64);           // the two lane halves hold different columns of the same row
             if (lane < 32) sq[w][lane] = q;
+            if (a.ln) { sv += __shfl_xor(sv, 32, 64); if (lane < 32) ssm[w][lane] = sv; }
             __syncthreads();
             if (threadIdx.x < 32 && threadIdx.x < a.rows_valid) {
                 float tot = sq[0][threadIdx.x];
 #pragma unroll
                 for (int i = 1; i < NW; ++i) tot += sq[i][threadIdx.x];
                 a.ssq_out[(long)nt * a.ssq_out_ld + threadIdx.x] = tot;
+                if (a.ln) {      // the tile's plain sum, behind the NT tiles of sums of squares
+                    float tots = ssm[0][threadIdx.x];
+#pragma unroll
+                    for (int i = 1; i < NW; ++i) tots += ssm[i][threadIdx.x];
+                    a.ssq_out[((long)a.NT + nt) * a.ssq_out_ld + threadIdx.x] = tots;
+                }
             }
         }
         return;
@@ -612,7 +700,7 @@ __global__ __launch_bounds__(NW * 64) void skinny_gemm_f16_kernel(const half_t* 
             keep[it] = s;
         } else if (EPI == EPI_F32_BIAS) {
             const int col = nt * 32 + n;
-            if (col < a.n_valid) a.out[(long)b * a.ld_out + col] = s * rinv + a.bias[col];
+            if (col < a.n_valid) a.out[(long)b * a.ld_out + col] = a.ln ? (s - smean[b] * a.ln_c[col]) * rinv + a.ln_d[col] : s * rinv + a.bias[col];
         } else {
             float val; int f; bool ok;
             if (a.gated) {
@@ -1827,6 +1915,7 @@ struct FnPrepArgs {
     const float* src; long ld_src; const int* row_map;
     const float* gamma; half_t* xg16; int xg_kt; float* ssq_out; long ssq_ld;
     long xg_ld;             // xg_kt == 0: xg16 is row-major with this leading dimension
+    int ln;                 // deferred LayerNorm: also store the tiles' plain sums, behind the ceil(h / 32) tiles of sums of squares
 };
 // (row r of the launch; erow: embedding row when a.ids is set; NT threads, NPT elements each)
 template <int NPT, int NT>
@@ -1855,6 +1944,12 @@ __device__ __forceinline__ void fn_prepare_row(const FnPrepArgs& a, int r, long 
 #pragma unroll
         for (int o = 16; o > 0; o >>= 1) q += __shfl_xor(q, o, 64);
         if ((t & 31) == 0 && c < a.h) a.ssq_out[(long)(c >> 5) * a.ssq_ld + r] = q;
+        if (a.ln) {
+            float sv = v;
+#pragma unroll
+            for (int o = 16; o > 0; o >>= 1) sv += __shfl_xor(sv, o, 64);
+            if ((t & 31) == 0 && c < a.h) a.ssq_out[(long)(((a.h + 31) >> 5) + (c >> 5)) * a.ssq_ld + r] = sv;
+        }
     }
 }
 template <int NPT>
@@ -1879,6 +1974,7 @@ struct AttnArgs {
     int out_kt;                                    // > 0: out is fragment packed with this many k-tiles
     float scale;
     const float* ssq; int ssq_nt; int ssq_ld; float inv_h; float eps;   // deferred RMSNorm of the projection input (see SkinnyArgs)
+    int ln;      // deferred LayerNorm (see SkinnyArgs): plain sums behind the sums of squares, `bias` holds d[ldq] followed by c[ldq]
     int vt;      // 1: keys and values are stored fragment-major (kfrag_index / vfrag_index) for the MFMA attention kernels
     // decode with several blocks per (row, KV head): their number, the exchange area [pairs][S][G D + 2 G] floats and one counter per pair
     int S; float* xchg; int* xcount;
@@ -2049,12 +2145,19 @@ __global__ __launch_bounds__(1024) void attn_decode_kernel(AttnArgs a) {
     const int kvh = blockIdx.x, b = blockIdx.y, t = threadIdx.x;
     const int pos = *a.d_pos;
     const int HD = a.H * D, GD = a.Hkv * D;
-    float rinv = 1.0f;
+    float rinv = 1.0f, mean = 0.0f;
     if (a.ssq) {
         float s = 0.0f;
         for (int tt = (t & 63); tt < a.ssq_nt; tt += 64) s += a.ssq[(long)tt * a.ssq_ld + b];
         s = wave_sum(s);                                   // same butterfly in every wavefront: identical result
-        rinv = 1.0f / sqrtf(s * a.inv_h + a.eps);
+        if (a.ln) {
+            float sv = 0.0f;
+            for (int tt = (t & 63); tt < a.ssq_nt; tt += 64) sv += a.ssq[(long)(a.ssq_nt + tt) * a.ssq_ld + b];
+            mean = wave_sum(sv) * a.inv_h;
+            rinv = 1.0f / sqrtf(fmaxf(s * a.inv_h - mean * mean, 0.0f) + a.eps);
+        } else {
+            rinv = 1.0f / sqrtf(s * a.inv_h + a.eps);
+        }
     }
     for (int idx = t; idx < (G + 2) * D; idx += NTH) {
         int col;
@@ -2070,7 +2173,7 @@ __global__ __launch_bounds__(1024) void attn_decode_kernel(AttnArgs a) {
 #pragma unroll
             for (int j = 0; j < 8; ++j) if (k + j < a.KS) s += pk[j];
         }
-        sm.in[idx] = s * rinv + a.bias[col];
+        sm.in[idx] = a.ln ? (s - mean * a.bias[a.ldq + col]) * rinv + a.bias[col] : s * rinv + a.bias[col];
     }
     __syncthreads();
     CT* Kb = (CT*)a.kcache + ((long)b * a.Hkv + kvh) * a.max_len * D;
@@ -2236,7 +2339,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(AttnArgs a) {
 // own copies of these fields are ignored.
 struct AttnPacked {
     void* kcache; int d_vcache, d_qkv, d_pos, d_bias, d_ssq, d_rope_cos, d_rope_sin;   // offsets from kcache, 256-byte units
-    int max_len; unsigned counts;     // H | Hkv << 8 | KS << 16 | (ssq ? 1 : 0) << 24 | (rope ? 1 : 0) << 25
+    int max_len; unsigned counts;     // H | Hkv << 8 | KS << 16 | (ssq ? 1 : 0) << 24 | (rope ? 1 : 0) << 25 | (ln ? 1 : 0) << 26
     int ldq, split_stride; unsigned ssq_dims;   // ssq_nt | ssq_ld << 16
 };
 template <int D, int G, bool SPLIT>
@@ -2247,7 +2350,7 @@ __global__ __launch_bounds__(D == 128 ? 256 : 512) void attn_mfma_kernel(void* k
         char* base = (char*)kcache_;
         auto at = [&](int d) { return (void*)(base + ((long)d << 8)); };
         a.kcache = kcache_; a.vcache = at(d_vcache); a.qkv = (const float*)at(d_qkv); a.d_pos = (const int*)at(d_pos); a.bias = (const float*)at(d_bias);
-        a.ssq = (counts >> 24) & 1 ? (const float*)at(d_ssq) : nullptr;
+        a.ssq = (counts >> 24) & 1 ? (const float*)at(d_ssq) : nullptr; a.ln = (counts >> 26) & 1;
         a.rope_cos = (counts >> 25) & 1 ? (const float*)at(d_rope_cos) : nullptr; a.rope_sin = (counts >> 25) & 1 ? (const float*)at(d_rope_sin) : nullptr;
         a.max_len = max_len_; a.H = counts & 255; a.Hkv = (counts >> 8) & 255; a.KS = (counts >> 16) & 255;
         a.ldq = ldq_; a.split_stride = split_stride_; a.ssq_nt = ssq_dims & 0xffff; a.ssq_ld = ssq_dims >> 16;
@@ -2299,12 +2402,16 @@ __global__ __launch_bounds__(D == 128 ? 256 : 512) void attn_mfma_kernel(void* k
         // position, then the rotation of the position, which the second phase needs.
         // (the first four tile sums of a lane are requested without a wait of their own: a load-and-add loop would cost a
         // memory round trip ahead of every other request; they are added below in the same order)
-        float ssq_part = 0.0f, ssq_v[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+        float ssq_part = 0.0f, ssq_v[4] = {0.0f, 0.0f, 0.0f, 0.0f}, ssum_v[4] = {0.0f, 0.0f, 0.0f, 0.0f};
         if (a.ssq) {      // (unconditional requests at clamped indices; the values beyond the last tile are dropped below)
 #pragma unroll
             for (int u = 0; u < 4; ++u) ssq_v[u] = a.ssq[(long)min(lane + 64 * u, a.ssq_nt - 1) * a.ssq_ld + b];
+            if (a.ln) {
+#pragma unroll
+                for (int u = 0; u < 4; ++u) ssum_v[u] = a.ssq[(long)(a.ssq_nt + min(lane + 64 * u, a.ssq_nt - 1)) * a.ssq_ld + b];
+            }
         }
-        float part[CPT][8], bias[CPT];
+        float part[CPT][8], bias[CPT], lnc[CPT];
         int pcol[CPT];
 #pragma unroll
         for (int ci = 0; ci < CPT; ++ci) {
@@ -2322,6 +2429,7 @@ __global__ __launch_bounds__(D == 128 ? 256 : 512) void attn_mfma_kernel(void* k
                 for (int k = 0; k < 8; ++k) if (k < a.KS) part[ci][k] = a.qkv[k * a.split_stride + (long)b * a.ldq + col];
             }
             bias[ci] = a.bias[pcol[ci]];
+            lnc[ci] = a.ln ? a.bias[a.ldq + pcol[ci]] : 0.0f;
         }
         __builtin_amdgcn_sched_barrier(0);
         load_chunk(min(gw, (int)(a.max_len >> 5) - 1), kfA, vfA);
@@ -2338,13 +2446,22 @@ __global__ __launch_bounds__(D == 128 ? 256 : 512) void attn_mfma_kernel(void* k
             if (p < (G + 1) * D / 2 && a.rope_cos) { rc[pi] = a.rope_cos[(long)pos * (D / 2) + p % (D / 2)]; rs[pi] = a.rope_sin[(long)pos * (D / 2) + p % (D / 2)]; }
         }
         __builtin_amdgcn_sched_barrier(0);
-        float rinv = 1.0f;
+        float rinv = 1.0f, mean = 0.0f;
         if (a.ssq) {
 #pragma unroll
             for (int u = 0; u < 4; ++u) if (lane + 64 * u >= a.ssq_nt) ssq_v[u] = 0.0f;
             ssq_part = ((ssq_v[0] + ssq_v[1]) + ssq_v[2]) + ssq_v[3];
             for (int tt = lane + 256; tt < a.ssq_nt; tt += 64) ssq_part += a.ssq[(long)tt * a.ssq_ld + b];
-            rinv = 1.0f / sqrtf(wave_sum(ssq_part) * a.inv_h + a.eps);
+            if (a.ln) {
+#pragma unroll
+                for (int u = 0; u < 4; ++u) if (lane + 64 * u >= a.ssq_nt) ssum_v[u] = 0.0f;
+                float ssum_part = ((ssum_v[0] + ssum_v[1]) + ssum_v[2]) + ssum_v[3];
+                for (int tt = lane + 256; tt < a.ssq_nt; tt += 64) ssum_part += a.ssq[(long)(a.ssq_nt + tt) * a.ssq_ld + b];
+                mean = wave_sum(ssum_part) * a.inv_h;
+                rinv = 1.0f / sqrtf(fmaxf(wave_sum(ssq_part) * a.inv_h - mean * mean, 0.0f) + a.eps);
+            } else {
+                rinv = 1.0f / sqrtf(wave_sum(ssq_part) * a.inv_h + a.eps);
+            }
         }
 #pragma unroll
         for (int ci = 0; ci < CPT; ++ci) {
@@ -2354,7 +2471,7 @@ __global__ __launch_bounds__(D == 128 ? 256 : 512) void attn_mfma_kernel(void* k
 #pragma unroll
                 for (int k = 1; k < 8; ++k) if (k < a.KS) s += part[ci][k];
                 for (int k = 8; k < a.KS; ++k) s += a.qkv[k * a.split_stride + (long)b * a.ldq + pcol[ci]];     // (more than eight splits: wide models at batches above 64)
-                sIn[idx] = s * rinv + bias[ci];
+                sIn[idx] = (s - mean * lnc[ci]) * rinv + bias[ci];      // (LayerNorm: the mean's share of the product; 0 otherwise)
             }
         }
         __syncthreads();

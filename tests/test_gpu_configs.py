@@ -102,6 +102,54 @@ def test_cfg1_fp16_full_width(G, oracle):
     gpu.close()
 
 
+@pytest.mark.parametrize("kw", [dict(), dict(hidden=128, n_heads=2, n_kv_heads=2, ffn_dim=320), dict(act=synth.SWIGLU, attn_type=synth.GQA, n_kv_heads=2)])
+def test_deferred_layernorm_with_a_large_row_mean(G, oracle, kw):
+    """fp16 LayerNorm models take the five-launch decode step: the producers of the residual stream store half(gamma x) and
+    the tiles' sums of x and x^2, the consumers rebuild mean and 1 / sigma and take the mean's share out of their products
+    (folded constants c, d per output column).  Here every embedding carries an offset of about twice its spread and gamma,
+    beta and the biases are random, so that a wrong mean term, a dropped beta or a transposed fold would move the logits far
+    beyond the bar; the generate loop (sampling kernel + embedding in one launch) must give the step-wise tokens."""
+    cfg = synth.tiny_config(dtype="f16", norm_type=synth.LAYERNORM, **{**dict(attn_type=synth.MHA, n_kv_heads=4, act=synth.RELU), **kw})
+    w = synth.make_weights(cfg, 21, random_bias=True)
+    rng = np.random.default_rng(5)
+    w = {k: np.array(v, np.float32) for k, v in w.items()}
+    w["TgtEmbeddings"] = w["TgtEmbeddings"] + np.float32(0.04)
+    for k in w:
+        if k.endswith("m_alpha"):
+            w[k] = (1.0 + 0.3 * rng.standard_normal(w[k].shape)).astype(np.float32)
+        elif k.endswith("m_beta"):
+            w[k] = (0.2 * rng.standard_normal(w[k].shape)).astype(np.float32)
+    orc = oracle.OracleGpt(cfg, w)
+    gpu = G.HipGpt(cfg, w, max_batch=cfg["batch"], max_seq_len=cfg["prompt"] + 12)
+    seqs = synth.make_prompts(cfg, 3)
+    p, lg = orc.step(seqs, use_cache=True)
+    gpu.prefill(seqs)
+    assert np.abs(gpu.logits() - lg).max() <= FP16_ABS
+    cur, agree = seqs, []
+    for _ in range(5):
+        nxt = oracle.argmax(p).astype(np.int32)
+        cur = np.concatenate([cur, nxt[:, None]], 1)
+        p, lg = orc.step(cur, use_cache=True)
+        gpu.decode(nxt)
+        gl = gpu.logits()
+        assert np.abs(gl - lg).max() <= FP16_ABS
+        agree.append(top1_agreement(gl, lg)[0])
+    hid = gpu.hidden()
+    assert np.isfinite(hid).all()
+    assert np.mean(agree) >= 0.99
+    # the graph-captured loop against step-by-step decoding from the same state
+    gpu.reset()
+    gpu.prefill(seqs)
+    ids, _ = gpu.generate(4)
+    gpu.reset()
+    gpu.prefill(seqs)
+    for s in range(4):
+        nxt = gpu.sample()
+        assert np.array_equal(nxt, ids[s])
+        gpu.decode(nxt)
+    gpu.close()
+
+
 @pytest.mark.parametrize("dtype", ["f32", "f16"])
 def test_cfg3_moe_layer_shape(G, oracle, dtype):
     """Configuration 3's layer shape: hidden 1024, 16 / 4 heads, 8 experts of width 4096 with 2 per token, batch 64, at
