@@ -40,6 +40,8 @@ namespace TensorSharp.HIP
         public int UseRope;
         public int DType;
         public int MaxBatch, MaxSeqLen;
+        public int MaxSegments;                   // IModel.MaxSegmentNum when EnableSegmentEmbeddings, else 0 (table "SegmentEmbedding")
+        public int SepTokenId;                    // the vocabulary's index of BuildInTokens.SEP ("[SEP]")
     }
 
     internal static class HipNative

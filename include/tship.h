@@ -156,6 +156,14 @@ typedef struct TSHipGptConfig {
     int32_t dtype;              /* TSHIP_F32 or TSHIP_F16: storage type of weights and KV cache */
     int32_t max_batch;
     int32_t max_seq_len;        /* KV cache capacity per sequence (prompt + generated) */
+    /* Segment embeddings (IModel.EnableSegmentEmbeddings / MaxSegmentNum; table "SegmentEmbedding" [max_segments, hidden] built by
+     * Misc.CreateAuxEmbeddings, Utils/Misc.cs:164-168): 0 = none.  TensorUtils.CreateTokensEmbeddings (Utils/TensorUtils.cs:60-72,
+     * 147-152) adds row s of the table to the scaled embedding of a token, s = number of sep_token_id tokens ("[SEP]",
+     * SENTTAGS.SEP = 3 in the reference's vocabularies) that come BEFORE it in the token list of the call: a prefill counts
+     * through its own tokens from 0, and a cached decode step feeds one token per sequence, which therefore always gets
+     * segment 0 (Applications/Decoder.cs:661-673).  This library counts the same way. */
+    int32_t max_segments;
+    int32_t sep_token_id;
 } TSHipGptConfig;
 
 typedef struct TSHipGpt TSHipGpt;

@@ -533,6 +533,8 @@ struct Config {
     float norm_eps;
     float rope_base;    // the reference hard-codes 500000
     int use_rope;
+    int max_segments;   // > 0: segment embeddings ("SegmentEmbedding" [max_segments, hidden], Utils/Misc.cs:164-168)
+    int sep_token_id;   // vocabulary index of BuildInTokens.SEP
 };
 
 struct Model {
@@ -739,6 +741,22 @@ static Tensor gpt_step(const Model& m, const int* seqs, long B, long len, Cache*
     Tensor x = indexselect_t(E, idx);
     float scale = (float)std::sqrt((double)E.sz[1]);
     if (scale != 1.0f) { float* p = x.p(); long n = x.count(); for (long i = 0; i < n; ++i) p[i] = p[i] * scale; }
+    if (m.c.max_segments > 0) {
+        // TensorUtils.cs:60-72, 147-152: the segment index of a token is the number of SEP tokens before it in the list that is
+        // fed (the whole sequence, or only its last token on a cached step: then always 0); embeddingRst = Add(embeddingRst,
+        // IndexSelect(segmentEmbedding, segIdxs))
+        std::vector<float> seg(ids.size());
+        for (long b = 0; b < B; ++b) {
+            int s_idx = 0;
+            for (long j = 0; j < Tq; ++j) {
+                seg[b * Tq + j] = (float)s_idx;
+                if ((int)ids[b * Tq + j] == m.c.sep_token_id) ++s_idx;
+            }
+        }
+        Tensor sx = indexselect_t(m.W("SegmentEmbedding"), Tensor::from(seg.data(), {(long)seg.size(), 1}));
+        float* p = x.p(); const float* q = sx.p(); long n = x.count();
+        for (long i = 0; i < n; ++i) p[i] = p[i] + q[i];
+    }
     Tensor out = decoder(m, x, haveMask ? &mask : nullptr, B, cache, traces);
     std::vector<float> last(B);
     for (long i = 0; i < B; ++i) last[i] = (float)(Tq * (i + 1) - 1);

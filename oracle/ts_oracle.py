@@ -32,6 +32,7 @@ class OrcConfig(C.Structure):
         ("ffn_dim", C.c_int), ("vocab", C.c_int), ("attn_type", C.c_int), ("norm_type", C.c_int),
         ("act", C.c_int), ("n_experts", C.c_int), ("experts_per_token", C.c_int),
         ("norm_eps", C.c_float), ("rope_base", C.c_float), ("use_rope", C.c_int),
+        ("max_segments", C.c_int), ("sep_token_id", C.c_int),
     ]
 
 
@@ -279,7 +280,8 @@ class OracleGpt:
         self.cfg = dict(cfg)
         c = OrcConfig(cfg["n_layers"], cfg["hidden"], cfg["n_heads"], cfg["n_kv_heads"], cfg["ffn_dim"], cfg["vocab"],
                       cfg["attn_type"], cfg["norm_type"], cfg["act"], cfg.get("n_experts", 1), cfg.get("experts_per_token", 1),
-                      cfg.get("norm_eps", 1e-6), cfg.get("rope_base", 500000.0), cfg.get("use_rope", 1))
+                      cfg.get("norm_eps", 1e-6), cfg.get("rope_base", 500000.0), cfg.get("use_rope", 1),
+                      cfg.get("max_segments", 0), cfg.get("sep_token_id", 3))
         self.h = L.orc_gpt_create(C.byref(c))
         for name, w in weights.items():
             w = _f(w)

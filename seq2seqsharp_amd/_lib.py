@@ -24,7 +24,8 @@ class TSHipGptConfig(C.Structure):
                 ("ffn_dim", C.c_int32), ("vocab", C.c_int32), ("attn_type", C.c_int32), ("norm_type", C.c_int32),
                 ("act", C.c_int32), ("n_experts", C.c_int32), ("experts_per_token", C.c_int32),
                 ("norm_eps", C.c_float), ("rope_base", C.c_float), ("use_rope", C.c_int32), ("dtype", C.c_int32),
-                ("max_batch", C.c_int32), ("max_seq_len", C.c_int32)]
+                ("max_batch", C.c_int32), ("max_seq_len", C.c_int32),
+                ("max_segments", C.c_int32), ("sep_token_id", C.c_int32)]
 
 
 _lib = None

@@ -102,6 +102,8 @@ struct TSHipGpt {
     bool gated;
     std::vector<std::unique_ptr<LayerW>> L;
     DevBuf emb;                    // [V][h] model dtype
+    DevBuf seg;                    // segment embeddings, fp32 [max_segments][h] (null without them); pw_seg: a prefill's segment of every row
+    DevBuf pw_seg;
     DevBuf fn_g, fn_b;             // final norm
     GemmW head; DevBuf head_b;
     DevBuf rope_cos, rope_sin;
@@ -303,6 +305,7 @@ static void build_expected(TSHipGpt* m) {
     bool ln = c.norm_type == 1;
     auto norm = [&](const std::string& p) { e.insert(p + ".m_alpha"); if (ln) e.insert(p + ".m_beta"); };
     e.insert("TgtEmbeddings");
+    if (c.max_segments > 0) e.insert("SegmentEmbedding");
     for (int i = 0; i < c.n_layers; ++i) {
         std::string a = "GPTDecoder.SelfAttn_" + std::to_string(i);
         norm(a + ".layerNormQ");
@@ -345,6 +348,9 @@ static void set_weight(TSHipGpt* m, const std::string& name, const float* host, 
         else copy_cols_kernel<float><<<(unsigned)ceil_div(total, 256), 256, 0, stream()>>>(tmp.as<float>(), h, V, h, m->emb.as<float>(), h, 0);
         TSHIP_CHECK_HIP(hipGetLastError());
         TSHIP_CHECK_HIP(hipStreamSynchronize(stream()));
+    } else if (name == "SegmentEmbedding") {
+        expect_shape(name.c_str(), ndim, sizes, {c.max_segments, h});
+        upload_f32(m->seg, host, (size_t)c.max_segments * h);
     } else if (name == "GPTDecoder.layerNorm.m_alpha") vec(m->fn_g, h);
     else if (name == "GPTDecoder.layerNorm.m_beta") vec(m->fn_b, h);
     else if (name == "FeedForward_Decoder_0.m_Whd") {
@@ -721,6 +727,7 @@ static FnPrepArgs embed_prepare_args(TSHipGpt* m, const int* d_ids) {
     const int h = m->c.hidden;
     FnPrepArgs a; std::memset(&a, 0, sizeof(a));
     a.x = m->x.as<float>(); a.ldx = h; a.h = h; a.ids = d_ids; a.emb = m->emb.p; a.emb_f16 = 1; a.emb_scale = (float)std::sqrt((double)h);
+    a.seg = m->seg.as<float>();      // (a cached decode step feeds one token per sequence: segment 0, Decoder.cs:661-673)
     a.gamma = m->L[0]->n1_g.as<float>(); a.xg16 = m->xn.as<half_t>(); a.xg_kt = (int)(m->ldh / 16); a.ssq_out = m->ssq.as<float>(); a.ssq_ld = m->Bpad;
     a.ln = m->ln ? 1 : 0;
     return a;
@@ -834,6 +841,7 @@ static void decode_step(TSHipGpt* m, const int* d_ids, int B) {
     {
         ResidNormArgs a = rn;
         a.ids = d_ids; a.emb = m->emb.p; a.emb_f16 = m->f16; a.emb_scale = (float)std::sqrt((double)h);
+        a.seg = m->seg.as<float>();      // (a cached decode step feeds one token per sequence: segment 0, Decoder.cs:661-673)
         a.gamma = m->L[0]->n1_g.as<float>(); a.beta = m->L[0]->n1_b.as<float>();
         run_resid_norm(m, "embed_norm", B, a);
     }
@@ -937,6 +945,21 @@ static void prefill(TSHipGpt* m, const int32_t* host_ids, int B, int Tp, const i
     ids.reserve(R * sizeof(int));
     TSHIP_CHECK_HIP(hipMemcpyAsync(ids.p, host_ids, R * sizeof(int), hipMemcpyHostToDevice, stream()));
     record_history(m, ids.as<int>(), B, Tp, pos0);
+    if (m->seg.p) {
+        // the segment of a token = the separators before it in this call's token list of its sequence (TensorUtils.cs:60-72)
+        std::vector<int> sg((size_t)R);
+        for (int b = 0; b < B; ++b) {
+            int s_idx = 0;
+            for (int j = 0; j < Tp; ++j) {
+                TSHIP_REQUIRE(s_idx < c.max_segments, "TSHip_GptPrefill: a sequence holds more separator tokens than the model has segment embeddings");
+                sg[(size_t)b * Tp + j] = s_idx;
+                if (host_ids[(size_t)b * Tp + j] == c.sep_token_id) ++s_idx;
+            }
+        }
+        m->pw_seg.reserve((size_t)R * sizeof(int));
+        TSHIP_CHECK_HIP(hipMemcpyAsync(m->pw_seg.p, sg.data(), (size_t)R * sizeof(int), hipMemcpyHostToDevice, stream()));
+        TSHIP_CHECK_HIP(hipStreamSynchronize(stream()));       // (the host vector is a local)
+    }
     std::vector<int> map(B);             // row of every sequence's last position
     for (int b = 0; b < B; ++b) map[b] = Tp * (b + 1) - 1;
     rowmap.reserve(B * sizeof(int));
@@ -974,6 +997,7 @@ static void prefill(TSHipGpt* m, const int32_t* host_ids, int B, int Tp, const i
         FnPrepArgs a; std::memset(&a, 0, sizeof(a));
         a.x = px.as<float>(); a.ldx = h; a.h = h;
         a.ids = ids.as<int>(); a.emb = m->emb.p; a.emb_f16 = m->f16; a.emb_scale = (float)std::sqrt((double)h);
+        a.seg = m->seg.as<float>(); a.seg_ids = m->seg.p ? m->pw_seg.as<int>() : nullptr;
         a.gamma = m->L[0]->n1_g.as<float>(); a.xg16 = pxn.as<half_t>(); a.xg_kt = 0; a.xg_ld = m->ldh; a.ssq_out = pssq.as<float>(); a.ssq_ld = R;
         if (h <= 2048) launch(m, "p_embed_prepare", fn_prepare_kernel<8>, dim3((unsigned)R), dim3(256), a);
         else if (h <= 4096) launch(m, "p_embed_prepare", fn_prepare_kernel<16>, dim3((unsigned)R), dim3(256), a);
@@ -982,6 +1006,7 @@ static void prefill(TSHipGpt* m, const int32_t* host_ids, int B, int Tp, const i
     } else {
         ResidNormArgs a = rn;
         a.ids = ids.as<int>(); a.emb = m->emb.p; a.emb_f16 = m->f16; a.emb_scale = (float)std::sqrt((double)h);
+        a.seg = m->seg.as<float>(); a.seg_ids = m->seg.p ? m->pw_seg.as<int>() : nullptr;
         a.gamma = m->L[0]->n1_g.as<float>(); a.beta = m->L[0]->n1_b.as<float>();
         run_resid_norm(m, "p_embed_norm", (int)R, a);
     }
@@ -1132,6 +1157,7 @@ TSHIP_API int TSHip_GptCreate(const TSHipGptConfig* cfg, TSHipGpt** out) {
     TSHIP_REQUIRE(c.max_seq_len >= 2, "TSHip_GptCreate: max_seq_len too small");
     TSHIP_REQUIRE(c.act >= 0 && c.act <= 4, "TSHip_GptCreate: unknown activation");
     TSHIP_REQUIRE(c.norm_type == 0 || c.norm_type == 1, "TSHip_GptCreate: unknown norm type");
+    TSHIP_REQUIRE(c.max_segments >= 0 && c.max_segments <= 65536, "TSHip_GptCreate: max_segments out of range");
     std::unique_ptr<TSHipGpt> m(new TSHipGpt());
     m->c = c;
     m->f16 = c.dtype == TSHIP_F16;

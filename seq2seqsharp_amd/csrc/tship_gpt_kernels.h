@@ -1672,6 +1672,9 @@ __global__ void ffn_act_kernel(const float* __restrict__ part, int KS, long spli
 struct ResidNormArgs {
     float* x; long ldx; int h;
     const int* ids; const void* emb; int emb_f16; float emb_scale;
+    // segment embeddings (TensorUtils.CreateTokensEmbeddings, Seq2SeqSharp/Utils/TensorUtils.cs:147-152): fp32 table
+    // [segments][h], added to the scaled token embedding; seg_ids [rows] = segment of every row, null = segment 0
+    const float* seg; const int* seg_ids;
     const float* part; int KS; long split_stride; long ld_part; const float* bias;
     const float* gamma; const float* beta; float eps; int norm_type;
     void* xn; long ldxn;
@@ -1718,6 +1721,7 @@ __global__ __launch_bounds__(256) void resid_norm_kernel(ResidNormArgs a) {
             if (a.ids) {
                 float e = a.emb_f16 ? (float)((const half_t*)a.emb)[erow * a.h + c] : ((const float*)a.emb)[erow * a.h + c];
                 v[i] = e * a.emb_scale;
+                if (a.seg) v[i] = v[i] + a.seg[(long)(a.seg_ids ? a.seg_ids[r] : 0) * a.h + c];
             } else {
                 v[i] = xin[c];
             }
@@ -1912,6 +1916,7 @@ __global__ __launch_bounds__(256) void rinv_rows_kernel(const float* __restrict_
 struct FnPrepArgs {
     float* x; long ldx; int h;
     const int* ids; const void* emb; int emb_f16; float emb_scale;
+    const float* seg; const int* seg_ids;      // segment embeddings, as in ResidNormArgs
     const float* src; long ld_src; const int* row_map;
     const float* gamma; half_t* xg16; int xg_kt; float* ssq_out; long ssq_ld;
     long xg_ld;             // xg_kt == 0: xg16 is row-major with this leading dimension
@@ -1922,13 +1927,15 @@ template <int NPT, int NT>
 __device__ __forceinline__ void fn_prepare_row(const FnPrepArgs& a, int r, long erow, int t) {
     const long srow = a.row_map ? a.row_map[r] : r;
     // all requests first (unconditional, the column clamped), then the arithmetic and the stores
-    float vin[NPT], gmv[NPT];
+    float vin[NPT], gmv[NPT], sgv[NPT];
+    const long seg_row = (a.ids && a.seg && a.seg_ids) ? a.seg_ids[r] : 0;
 #pragma unroll
     for (int i = 0; i < NPT; ++i) {
         const int c = min(t + i * NT, a.h - 1);
         if (a.ids) vin[i] = a.emb_f16 ? (float)((const half_t*)a.emb)[erow * a.h + c] : ((const float*)a.emb)[erow * a.h + c];
         else vin[i] = a.src[srow * a.ld_src + c];
         gmv[i] = a.gamma[c];
+        sgv[i] = (a.ids && a.seg) ? a.seg[seg_row * a.h + c] : 0.0f;
     }
 #pragma unroll
     for (int i = 0; i < NPT; ++i) {
@@ -1936,6 +1943,7 @@ __device__ __forceinline__ void fn_prepare_row(const FnPrepArgs& a, int r, long 
         float v = 0.0f;
         if (c < a.h) {
             v = a.ids ? vin[i] * a.emb_scale : vin[i];
+            if (a.ids && a.seg) v = v + sgv[i];
             a.x[(long)r * a.ldx + c] = v;
             if (a.xg_kt > 0) a.xg16[xpack_index(r, c, a.xg_kt)] = (half_t)(gmv[i] * v);
             else a.xg16[(long)r * a.xg_ld + c] = (half_t)(gmv[i] * v);

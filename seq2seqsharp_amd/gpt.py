@@ -139,7 +139,7 @@ class HipGpt:
                            cfg["attn_type"], cfg["norm_type"], cfg["act"], cfg.get("n_experts", 1),
                            cfg.get("experts_per_token", 1), cfg.get("norm_eps", 1e-6), cfg.get("rope_base", 500000.0),
                            cfg.get("use_rope", 1), F16 if cfg.get("dtype", "f32") == "f16" else F32,
-                           self.max_batch, self.max_seq_len)
+                           self.max_batch, self.max_seq_len, cfg.get("max_segments", 0), cfg.get("sep_token_id", 3))
         h = C.c_void_p()
         check(L.TSHip_GptCreate(C.byref(c), C.byref(h)))
         self.h = h

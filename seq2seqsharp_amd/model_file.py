@@ -200,11 +200,20 @@ def gpt_config(m, dtype=None):
         raise ValueError("model file: DecoderType %d is not GPTDecoder" % m["DecoderType"])
     if m["PEType"] == PE_APE:
         raise ValueError("model file: absolute position embeddings (PEType APE) are outside the decode path built here (RoPE and NoPE are supported)")
+    max_segments, sep_id = 0, 3
     if m["EnableSegmentEmbeddings"]:
         # CreateTokensEmbeddings adds SegmentEmbedding[segment index] to every token embedding (Utils/TensorUtils.cs:147-152,
-        # table built by Misc.CreateAuxEmbeddings, Utils/Misc.cs:164-168); the fused path has no such table
-        raise ValueError("model file: segment embeddings (EnableSegmentEmbeddings, MaxSegmentNum %d) are not built into this decode path; "
-                         "its logits would differ from the reference's" % m["MaxSegmentNum"])
+        # table [MaxSegmentNum, EncoderEmbeddingDim] built by Misc.CreateAuxEmbeddings, Utils/Misc.cs:164-168); the segment index
+        # counts the vocabulary's "[SEP]" tokens (BuildInTokens.SEP)
+        max_segments = m["MaxSegmentNum"]
+        if max_segments < 1:
+            raise ValueError("model file: EnableSegmentEmbeddings with MaxSegmentNum %d" % max_segments)
+        if m["EncoderEmbeddingDim"] and m["EncoderEmbeddingDim"] != m["HiddenDim"]:
+            raise ValueError("model file: the segment embedding table is %d wide, the decoder's hidden size is %d" % (m["EncoderEmbeddingDim"], m["HiddenDim"]))
+        words = m["TgtVocab"]["word_to_index"] if m["TgtVocab"] else {}
+        if "[SEP]" not in words:
+            raise ValueError("model file: segment embeddings are enabled but the target vocabulary has no [SEP] token")
+        sep_id = int(words["[SEP]"])
     # EnableTagEmbeddings does not change GPTDecoder's results: Decoder.GPTDecode calls CreateTokensEmbeddings without
     # enableTagEmbedding (Applications/Decoder.cs:673,695; only Encoder.cs:102 passes it), so the flag is accepted
     vocab = len(m["TgtVocab"]["index_to_word"]) if m["TgtVocab"] else 0
@@ -216,7 +225,7 @@ def gpt_config(m, dtype=None):
                 ffn_dim=m["IntermediateDim"], vocab=vocab, attn_type=synth.GQA if gqa else synth.MHA,
                 norm_type=synth.RMSNORM if m["NormType"] == NORM_RMSNORM else synth.LAYERNORM, act=m["ActivateFunc"],
                 n_experts=max(m["ExpertNum"], 1), experts_per_token=max(m["ExpertsPerTokenFactor"], 1), norm_eps=1e-6, rope_base=500000.0,
-                use_rope=1 if m["PEType"] == PE_ROPE else 0, dtype=dtype)
+                use_rope=1 if m["PEType"] == PE_ROPE else 0, dtype=dtype, max_segments=max_segments, sep_token_id=sep_id)
 
 
 def load_gpt(path_or_bytes, dtype=None):
@@ -332,6 +341,8 @@ def save_gpt(cfg, weights, path=None, storage="f32", vocab_words=None):
              NormType=NORM_RMSNORM if cfg["norm_type"] == synth.RMSNORM else NORM_LAYERNORM,
              MultiHeadAttentionType=GQA if cfg["attn_type"] == synth.GQA else MHA, KVGroupNum=cfg["n_kv_heads"] if cfg["attn_type"] == synth.GQA else 0,
              Name2Weights={}, Name2WeightsHalf={}, Name2WeightsVQ={}, Name2CodeBook={})
+    if cfg.get("max_segments", 0) > 0:
+        m.update(EnableSegmentEmbeddings=1, MaxSegmentNum=cfg["max_segments"], EncoderEmbeddingDim=cfg["hidden"])
     for name, w in weights.items():
         flat = np.asarray(w, np.float32).reshape(-1)
         if storage == "f32":

@@ -53,6 +53,8 @@ def weight_shapes(cfg):
     d = h // H
     ln = cfg["norm_type"] == LAYERNORM
     out = [("TgtEmbeddings", (V, h), "normal")]
+    if cfg.get("max_segments", 0) > 0:          # Misc.CreateAuxEmbeddings: "SegmentEmbedding" [MaxSegmentNum, EncoderEmbeddingDim]
+        out.append(("SegmentEmbedding", (cfg["max_segments"], h), "normal"))
 
     def norm(prefix):
         out.append((prefix + ".m_alpha", (1, h), "ones"))

@@ -98,7 +98,7 @@ def test_marshalled_structs_follow_the_header():
         if d.startswith("public"):
             _, t, names = d.split(None, 2)
             types_cs += [t] * len(names.split(","))
-    assert len(fields_h) == len(types_cs) == 17
+    assert len(fields_h) == len(types_cs) == 19
     assert [{"int32_t": "int", "float": "float"}[t] for t in types_h] == types_cs
     ten = re.search(r"internal unsafe struct TSHipTensor\s*\{(.*?)public static", cs, flags=re.S).group(1)
     order = re.findall(r"public\s+(?:fixed\s+)?(\w+)\s+(\w+)", ten)

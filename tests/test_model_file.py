@@ -170,17 +170,27 @@ def test_loader_refuses_what_the_path_does_not_cover():
         mf.load_gpt(mf.write_model(m))
 
 
-def test_loader_refuses_segment_embeddings_and_unused_parameters():
-    """A file whose reference decode adds segment embeddings (Utils/TensorUtils.cs:147-152) must not load silently; neither
-    must one that stores parameters the path would ignore.  EnableTagEmbeddings is accepted: GPTDecode never passes it on."""
+def test_loader_segment_embeddings_and_unused_parameters():
+    """A file whose reference decode adds segment embeddings (Utils/TensorUtils.cs:147-152) loads with its table and its
+    separator id, or not at all; one that stores parameters the path would ignore must not load silently.
+    EnableTagEmbeddings is accepted: GPTDecode never passes it on."""
     cfg = synth.tiny_config()
     blob = mf.save_gpt(cfg, synth.make_weights(cfg, 1))
     m = mf.read_model(blob)
-    m["EnableSegmentEmbeddings"], m["MaxSegmentNum"] = 1, 16
-    with pytest.raises(ValueError, match="segment embeddings"):
+    m["EnableSegmentEmbeddings"], m["MaxSegmentNum"] = 1, 16      # the flag without the table: the table is then a missing weight
+    with pytest.raises(KeyError, match="SegmentEmbedding"):
         mf.load_gpt(mf.write_model(m))
-    with pytest.raises(ValueError, match="segment embeddings"):
-        mf.gpt_config(mf.read_model(mf.write_model(m)))
+    m["MaxSegmentNum"] = 0
+    with pytest.raises(ValueError, match="MaxSegmentNum"):
+        mf.gpt_config(m)
+    # with the table and a [SEP] word the model loads, and the configuration carries the table's height and the separator's id
+    cfg_s = synth.tiny_config(max_segments=5)
+    cfg2, w2, vocab = mf.load_gpt(mf.save_gpt(cfg_s, synth.make_weights(cfg_s, 2)))
+    assert cfg2["max_segments"] == 5 and cfg2["sep_token_id"] == vocab["word_to_index"]["[SEP]"] == 3
+    assert w2["SegmentEmbedding"].shape == (5, cfg_s["hidden"])
+    m = mf.read_model(mf.save_gpt(cfg_s, synth.make_weights(cfg_s, 2), vocab_words=["</s>", "<s>", "<unk>"] + ["w%d" % i for i in range(3, cfg_s["vocab"])]))
+    with pytest.raises(ValueError, match=r"no \[SEP\] token"):
+        mf.gpt_config(m)
     m = mf.read_model(blob)
     m["MaxSegmentNum"] = 16          # the number alone changes nothing in the reference either
     m["EnableTagEmbeddings"] = 1

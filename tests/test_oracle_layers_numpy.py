@@ -119,6 +119,14 @@ def gpt64(cfg, w, seqs, past=None, lens=None, mut=None):
     ids = seqs if past is None else seqs[:, -1:]
     Tq = ids.shape[1]
     x = w["TgtEmbeddings"].astype(F64)[ids.reshape(-1)] * F64(np.float32(np.sqrt(np.float32(h))))
+    if cfg.get("max_segments", 0) > 0:
+        # TensorUtils.CreateTokensEmbeddings (Utils/TensorUtils.cs:60-72, 147-152), written differently from the oracle's loop:
+        # the segment of a token is the count of separators strictly before it in the fed list, i.e. an exclusive running sum
+        is_sep = (ids == cfg.get("sep_token_id", 3)).astype(np.int64)
+        seg_idx = np.cumsum(is_sep, axis=1) - is_sep
+        if mut == "seg_inclusive":
+            seg_idx = np.cumsum(is_sep, axis=1)
+        x = x + w["SegmentEmbedding"].astype(F64)[seg_idx.reshape(-1)]
     new = []
     for layer in range(cfg["n_layers"]):
         x, kv = attention64(cfg, w, layer, x, B, Tq, None if past is None else past[layer], lens=lens, mut=mut)
@@ -207,6 +215,35 @@ def test_decoder_step_logits(oracle, name):
     # without a cache the whole sequence is recomputed under the mask: same logits
     lg_full, _, _ = gpt64(cfg, w, cur)
     assert np.abs(lg_full - lg64).max() <= 1e-9
+
+
+def test_segment_embeddings(oracle):
+    """EnableSegmentEmbeddings: every token's embedding gets the row of "SegmentEmbedding" that counts the [SEP] tokens before
+    it in the list that is fed: the whole prompt on the first call, the single new token (hence always row 0) on a cached
+    step, whatever separators the cache holds (Decoder.cs:661-673 feeds only the last token to CreateTokensEmbeddings)."""
+    cfg = synth.tiny_config(n_layers=2, max_segments=4, sep_token_id=3)
+    w = _sharpen(synth.make_weights(cfg, 31, random_bias=True))
+    w["SegmentEmbedding"] = (np.asarray(w["SegmentEmbedding"]) * 20).astype(np.float32)      # as large as the scaled token embeddings
+    seqs = synth.make_prompts(cfg, 32)
+    seqs[0, 2] = 3; seqs[0, 5] = 3; seqs[1, 0] = 3                                            # separators at different places per row
+    m = oracle.OracleGpt(cfg, w)
+    p, lg = m.step(seqs, use_cache=True)
+    lg64, _, past = gpt64(cfg, w, seqs)
+    assert np.abs(lg - lg64).max() <= 1e-5
+    # the checks must be able to fail: counting the separator itself, or leaving the table out, moves the logits
+    assert np.abs(lg - gpt64(cfg, w, seqs, mut="seg_inclusive")[0]).max() > 1e-3
+    assert np.abs(lg - gpt64(dict(cfg, max_segments=0), w, seqs)[0]).max() > 1e-3
+    cur = seqs
+    for tok in (3, 9):                                                                        # a separator as the new token, then an ordinary one
+        cur = np.concatenate([cur, np.full((cur.shape[0], 1), tok, np.int32)], 1)
+        p, lg = m.step(cur, use_cache=True)
+        lg64, _, past = gpt64(cfg, w, cur, past)
+        assert np.abs(lg - lg64).max() <= 1e-5
+    # a full recompute of the same tokens counts the separators of the whole sequence: different logits from the cached run
+    lg_full = gpt64(cfg, w, cur)[0]
+    assert np.abs(lg_full - lg64).max() > 1e-3
+    m2 = oracle.OracleGpt(cfg, w)
+    assert np.abs(m2.step(cur, use_cache=False)[1] - lg_full).max() <= 1e-5
 
 
 def test_temperature_divides_logits_only_when_sampling(oracle):
