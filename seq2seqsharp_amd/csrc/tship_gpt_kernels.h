@@ -2722,10 +2722,14 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(D == 64 ? (
     // blocks per compute unit the launch bounds ask for (waves per SIMD x 4 SIMDs / 8 wavefronts per block): their LDS must fit
     constexpr int BLOCKS_PER_CU = (D == 64 ? (NQ == 1 && !RAGGED ? 6 : 4) : 2) * 4 / NW;
     static_assert(sizeof(PrefillLds) * BLOCKS_PER_CU <= 160 * 1024, "the resident blocks' LDS fits the 160 KiB of a compute unit");
-    __shared__ PrefillLds lds;
-    half_t (&sbuf)[NW][D * 16] = lds.sbuf;
-    float (&sl)[NW][16] = lds.sl;
-    half_t* const sstage = &lds.sstage[0][0];
+    // (the struct above is the layout the assertions are about; the regions themselves are three objects of the same
+    // shapes, which the compiler keeps apart by construction: allocated as one object, the register allocator of this
+    // 80-register build put a spill reload into the chunk loops)
+    __shared__ __attribute__((aligned(16))) half_t sbuf[NW][D * 16];
+    __shared__ float sl[NW][16];
+    __shared__ __attribute__((aligned(16))) half_t sstage[STAGES * NF * 512];
+    static_assert(sizeof(sbuf) == sizeof(PrefillLds::sbuf) && sizeof(sl) == sizeof(PrefillLds::sl) && sizeof(sstage) == sizeof(PrefillLds::sstage),
+                  "the allocated regions have the asserted shapes");
     const int lane = threadIdx.x & 63, w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int r16 = lane & 15, q = lane >> 4;
     const int kvh = blockIdx.y, b = blockIdx.z;
