@@ -78,6 +78,13 @@ static std::string kernel_symbol(const void* host_fn) {
     if (!raw) { (void)hipGetLastError(); return std::string(); }
     int status = 0;
     char* dem = abi::__cxa_demangle(raw, nullptr, nullptr, &status);
+    if (status != 0 || !dem) {
+        // (this demangler does not know the _Float16 type code DF16_: spell it as the older half type Dh for the name's sake)
+        std::free(dem); dem = nullptr;
+        std::string alt(raw);
+        for (size_t i = alt.find("DF16_"); i != std::string::npos; i = alt.find("DF16_", i)) alt.replace(i, 5, "Dh");
+        dem = abi::__cxa_demangle(alt.c_str(), nullptr, nullptr, &status);
+    }
     std::string out = (status == 0 && dem) ? dem : raw;
     std::free(dem);
     return out;
