@@ -537,7 +537,7 @@ static void run_big_gemm(TSHipGpt* m, const char* name, const GemmW& w, const vo
             e.patch_rows = ph;
             grid.x = (unsigned)(round_up(patches, 8) * 4 * ph);
         }
-        if (n_problems > 1) { e.blocks_per_problem = (int)grid.x; grid.x *= (unsigned)n_problems; }
+        if (n_problems > 1 && !e.packed_problems) { e.blocks_per_problem = (int)grid.x; grid.x *= (unsigned)n_problems; }
         if (w.KT % 2 == 0) {      // asynchronous staging: four stages of two k-tiles, eight wavefronts
             if (epi == BEPI_F32_BIAS) launch_shm(m, name, big_gemm3_f16_kernel<BEPI_F32_BIAS>, grid, dim3(512), shm, e);
             else if (epi == BEPI_RESID) launch_shm(m, name, big_gemm3_f16_kernel<BEPI_RESID>, grid, dim3(512), shm, e);
@@ -705,7 +705,7 @@ static void launch_attn_decode(TSHipGpt* m, AttnArgs a, int B) {
 // MoE feed-forward at decode (MoEFeedForward.Process, Seq2SeqSharp/Layers/MoEFeedForward.cs:76-181)
 // ------------------------------------------------------------------------------------------------
 static void run_moe_ffn(TSHipGpt* m, LayerW& L, int rows, const ResidNormArgs& pre, const ResidNormArgs* next);
-static void run_moe_ffn_prefill(TSHipGpt* m, LayerW& L, int rows, const ResidNormArgs& pre, const int* last_rows, int n_last);
+static void run_moe_ffn_prefill(TSHipGpt* m, LayerW& L, int rows, const ResidNormArgs& pre, const int* last_rows, int n_last, const ResidNormArgs* next);
 static void moe_alloc(TSHipGpt* m);
 static void moe_get_routing(TSHipGpt* m, int layer, float* top_idx, float* top_val, float* probs);
 static void sample_tokens(TSHipGpt* m, int mode, float top_p, float temperature, const float* host_uniforms, const float* dev_uniforms, int B, int* gen_out, const int* d_step, bool record,
@@ -1081,10 +1081,12 @@ static void prefill(TSHipGpt* m, const int32_t* host_ids, int B, int Tp, const i
         ResidNormArgs a3 = rn;
         if (l + 1 < c.n_layers) { a3.gamma = m->L[l + 1]->n1_g.as<float>(); a3.beta = m->L[l + 1]->n1_b.as<float>(); }
         else a3.xn = nullptr;
+        const bool norm_after = !deferred && (l + 1 < c.n_layers || !m->f16);
         if (L.moe) {
             // the router kernel applies the pending attention output (fp32 models) and the layer's own LayerNorm; the
-            // combine kernel adds the experts' output to the residual stream
-            run_moe_ffn_prefill(m, L, (int)R, a2, rowmap.as<int>(), B);
+            // experts' output is added to the residual stream by the norm kernel that follows (a combine kernel of its own
+            // behind the last layer of an fp16 model, which no norm kernel follows)
+            run_moe_ffn_prefill(m, L, (int)R, a2, rowmap.as<int>(), B, norm_after ? &a3 : nullptr);
         } else if (deferred) make_rinv("p_rinv_ffn");
         else run_resid_norm(m, "p_norm_ffn", (int)R, a2);
         if (L.moe) {
@@ -1108,7 +1110,7 @@ static void prefill(TSHipGpt* m, const int32_t* host_ids, int B, int Tp, const i
             a3.part = pqkv.as<float>(); a3.KS = 1; a3.ld_part = qp; a3.bias = L.b2.as<float>();
         }
         if (deferred) { if (l + 1 < c.n_layers) make_rinv("p_rinv_attn"); }
-        else if (l + 1 < c.n_layers || !m->f16) run_resid_norm(m, "p_norm_attn", (int)R, a3);
+        else if (norm_after && !L.moe) run_resid_norm(m, "p_norm_attn", (int)R, a3);
     }
     // last position of every sequence (Decoder.cs:705-716) -> final norm -> vocabulary projection
     if (m->fused_norm && !m->ln) {

@@ -49,6 +49,9 @@ static void moe_get_routing(TSHipGpt* m, int layer, float* top_idx, float* top_v
 // many-row kernel, the host reads the experts' row counts (the reference builds its lists on the host as well,
 // MoEFeedForward.cs:92-105) and every expert with rows runs the prefill GEMMs on its gathered rows
 // next: when given, the norm kernel that follows adds the experts' outputs itself (no separate combine launch)
+// Prefills of fp16 models with 512 rows or more never read the counts back: the router writes the normalised rows as fp16,
+// one launch per projection covers every expert's row tiles packed one behind the other (found on the device from the
+// counts), and the up projection reads its rows through the token lists.
 static void run_moe_ffn_impl(TSHipGpt* m, LayerW& L, int rows, const ResidNormArgs& pre, bool batched, long cap, const int* last_rows, int n_last,
                              const ResidNormArgs* next = nullptr) {
     auto& c = m->c;
@@ -77,6 +80,9 @@ static void run_moe_ffn_impl(TSHipGpt* m, LayerW& L, int rows, const ResidNormAr
     // fp16 decode steps: the router kernel also takes the row's place in its experts' batches and writes the row there
     const bool fused_route = m->f16 && h % 4 == 0 && !batched && k <= 64;
     if (fused_route) { r.xg16 = (half_t*)(base + o.xg); r.xg_estride = xg_stride; r.packed_kt = (int)(m->ldh / 16); r.counts = counts; r.slot = slot; r.max_rows = (int)Bp; }
+    const bool packed = batched && m->f16 && h % 4 == 0 && rows >= 512 && big_gemm_batched_ok(*L.e1[0], rows) && big_gemm_batched_ok(*L.e2[0], rows) &&
+                        L.wtab1.p && L.wtab2.p && !g_hooks.no_moe_batch;
+    if (packed) { r.xn16 = (half_t*)(base + o.xg); r.ld_xn16 = m->ldh; }       // (the gathered rows' area holds them: E * cap rows are reserved)
     const unsigned router_shm = (unsigned)((2L * h + (r.router_lds ? (long)E * h : 0)) * sizeof(float));
     if (m->f16 && h % 4 == 0) {      // tree-order sums: an fp16 model's routing input is not the reference's to the last bit anyway
         if (h <= 1024) launch(m, "moe_router", moe_router_fast_kernel<1>, dim3(rows), dim3(256), r);
@@ -88,12 +94,27 @@ static void run_moe_ffn_impl(TSHipGpt* m, LayerW& L, int rows, const ResidNormAr
     if (batched) launch(m, "moe_lists", moe_lists_big_kernel, dim3(E), dim3(1024), (const float*)top_idx, rows, k, (int)Bp, counts, lists, slot);
     else if (!fused_lists && !fused_route) launch_shm(m, "moe_lists", moe_lists_kernel, dim3(1), dim3(64), (unsigned)(rows * k * sizeof(int)), (const float*)top_idx, rows, k, E, (int)Bp, counts, lists, slot);
     std::vector<int> n_e(E, rows);
-    if (batched) {
+    if (packed) {
+        half_t* xn16 = (half_t*)(base + o.xg); half_t* mid = (half_t*)(base + o.mid);
+        const int rt_bound = (int)((long)rows * k / 256 + E);      // >= the sum over the experts of ceil(count / 256)
+        BigArgs e1; std::memset(&e1, 0, sizeof(e1));
+        e1.bias = zero; e1.out16 = mid; e1.ld16 = (int)o.ld4h; e1.act = c.act; e1.gated = 0; e1.n_valid = 4 * h;
+        e1.Wtab = (const half_t* const*)L.wtab1.p; e1.rows_tab = counts; e1.x_estride = 0; e1.out16_estride = mid_stride;
+        e1.row_idx = lists; e1.idx_estride = Bp; e1.packed_problems = E; e1.packed_rt = rt_bound;
+        run_big_gemm(m, "moe_gemm1", *L.e1[0], xn16, m->ldh, (long)rt_bound * 256, BEPI_ACT16, e1, E);
+        BigArgs e2; std::memset(&e2, 0, sizeof(e2));
+        e2.bias = zero; e2.out = y; e2.ld_out = (int)o.ldy; e2.n_valid = h;
+        e2.Wtab = (const half_t* const*)L.wtab2.p; e2.rows_tab = counts; e2.x_estride = mid_stride; e2.out_estride = y_stride;
+        e2.packed_problems = E; e2.packed_rt = rt_bound;
+        run_big_gemm(m, "moe_gemm2", *L.e2[0], mid, o.ld4h, (long)rt_bound * 256, BEPI_F32_BIAS, e2, E);
+    } else if (batched) {
         TSHIP_CHECK_HIP(hipMemcpyAsync(n_e.data(), counts, E * sizeof(int), hipMemcpyDeviceToHost, stream()));
         TSHIP_CHECK_HIP(hipStreamSynchronize(stream()));
         for (int e = 0; e < E; ++e) TSHIP_REQUIRE(n_e[e] >= 0 && n_e[e] <= rows, "internal: expert row count out of range");
     }
-    if (m->f16 && batched) {
+    if (packed) {
+        // (done above)
+    } else if (m->f16 && batched) {
         half_t* xg = (half_t*)(base + o.xg); half_t* mid = (half_t*)(base + o.mid);
         launch(m, "moe_gather", moe_gather_kernel<half_t>, dim3(rows, E), dim3(256), (const float*)xn32, h, (const int*)counts, (const int*)lists, (int)Bp, xg,
                m->ldh, xg_stride, 0);
@@ -186,10 +207,10 @@ static void run_moe_ffn_impl(TSHipGpt* m, LayerW& L, int rows, const ResidNormAr
 
 static void run_moe_ffn(TSHipGpt* m, LayerW& L, int rows, const ResidNormArgs& pre, const ResidNormArgs* next) { run_moe_ffn_impl(m, L, rows, pre, false, m->Bpad, nullptr, 0, next); }
 
-static void run_moe_ffn_prefill(TSHipGpt* m, LayerW& L, int rows, const ResidNormArgs& pre, const int* last_rows, int n_last) {
+static void run_moe_ffn_prefill(TSHipGpt* m, LayerW& L, int rows, const ResidNormArgs& pre, const int* last_rows, int n_last, const ResidNormArgs* next) {
     const long cap = round_up(rows, 128);
     m->pw_moe.reserve(moe_layout(m, cap).total);
-    run_moe_ffn_impl(m, L, rows, pre, true, cap, last_rows, n_last);
+    run_moe_ffn_impl(m, L, rows, pre, true, cap, last_rows, n_last, next);
 }
 
 // next tokens from the logits on the device -> m->ids (and gen_out); greedy or top-p.

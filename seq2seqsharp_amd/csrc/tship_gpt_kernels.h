@@ -767,6 +767,15 @@ struct BigArgs {
     // e = blockIdx.x / blocks_per_problem takes its weights from Wtab[e], its row count from rows_tab[e] (read on the
     // device; blocks beyond it leave at once) and its activations / outputs at fixed strides.  0: one problem.
     int blocks_per_problem; const half_t* const* Wtab; const int* rows_tab; long x_estride, out_estride, out16_estride;
+    // The same with the problems' row tiles packed one behind the other (packed_problems > 0; blocks_per_problem unused): the
+    // launch covers packed_rt row tiles, an upper bound of the sum over the problems of ceil(rows_tab[e] / 256) that the host
+    // knows without reading the counts (the sum of the rows / 256 + the number of problems); every block finds its problem
+    // from the counts, blocks beyond the last problem's tiles leave at once.  Consecutive row tiles mostly belong to one
+    // problem, so a patch still shares its weight tiles.
+    int packed_problems; int packed_rt;
+    // Optional (LDS-tiled asynchronous kernel): row r of problem e is row row_idx[e * idx_estride + r] of X (the rows an
+    // expert was given, read where they lie instead of being copied together first)
+    const int* row_idx; long idx_estride;
     // LDS-tiled asynchronous kernel: row tiles per XCD patch (8, or fewer for launches that would otherwise fill fewer
     // than eight patches and leave XCDs idle); 0 means 8
     int patch_rows;
@@ -1377,20 +1386,37 @@ __global__ __launch_bounds__(512) void big_gemm3_f16_kernel(BigArgs a) {
     const int wr = w >> 1, wn = w & 1;                   // 4 x 2 wavefronts
     unsigned bid = blockIdx.x;
     int rot = 0;
-    if (a.blocks_per_problem) {
-        const int e = (int)(bid / (unsigned)a.blocks_per_problem);
-        bid -= (unsigned)e * (unsigned)a.blocks_per_problem;
+    auto take_problem = [&](int e) {
         a.R = a.rows_tab[e]; a.W = a.Wtab[e]; a.X += e * a.x_estride;
         if (a.out) a.out += e * a.out_estride;
         if (a.out16) a.out16 += e * a.out16_estride;
+        if (a.row_idx) a.row_idx += e * a.idx_estride;
+    };
+    if (a.blocks_per_problem && !a.packed_problems) {
+        const int e = (int)(bid / (unsigned)a.blocks_per_problem);
+        bid -= (unsigned)e * (unsigned)a.blocks_per_problem;
+        take_problem(e);
         rot = e;      // a problem with fewer than eight patches would leave XCDs idle: problem e starts on XCD e % 8
     }
-    const int CT = (a.NT + 7) / 8, RT = (int)((a.R + 255) / 256), PC = (CT + 3) / 4;
+    const int CT = (a.NT + 7) / 8, PC = (CT + 3) / 4;
+    const int RT = a.packed_problems ? a.packed_rt : (int)((a.R + 255) / 256);
     const int xcd = (int)((bid - (unsigned)rot) & 7), seq = (int)(bid >> 3);
     const int PH = a.patch_rows ? a.patch_rows : 8;          // a patch: PH row tiles x 4 column tiles
     const int patch = (seq / (4 * PH)) * 8 + xcd, q = seq % (4 * PH);
-    const int ctile = (patch % PC) * 4 + (q & 3), rtile = (patch / PC) * PH + (q >> 2);
+    const int ctile = (patch % PC) * 4 + (q & 3);
+    int rtile = (patch / PC) * PH + (q >> 2);
     if (ctile >= CT || rtile >= RT) return;
+    if (a.packed_problems) {
+        // the problem whose tiles hold packed row tile `rtile` (block-uniform: the counts sit in scalar registers)
+        int e = -1, first = 0;
+        for (int i = 0; i < a.packed_problems; ++i) {
+            const int tiles = (a.rows_tab[i] + 255) / 256;
+            if (e < 0 && rtile < first + tiles) { e = i; rtile -= first; }
+            first += tiles;
+        }
+        if (e < 0) return;
+        take_problem(e);
+    }
     const int nt0 = ctile * 8;
     const long row0 = (long)rtile * 256;
     floatx16 acc[4][2];
@@ -1412,7 +1438,8 @@ __global__ __launch_bounds__(512) void big_gemm3_f16_kernel(BigArgs a) {
         const int nt = min(nt0 + tl, a.NT - 1);
         wsrc[i] = a.W + (((long)nt * a.KT + ktl) * 64 + lane) * 8;
         const int rl = f * 16 + (lane >> 2);
-        const long row = min(row0 + rl, (long)a.R - 1);
+        long row = min(row0 + rl, (long)a.R - 1);
+        if (a.row_idx) row = a.row_idx[row];
         xsrc[i] = a.X + row * (long)a.ldx + 8 * ((lane & 3) ^ ((rl >> 2) & 3));
     }
     typedef const void __attribute__((address_space(1)))* gptr_t;

@@ -23,6 +23,9 @@ struct MoeRouterArgs {
     // fast kernel only, when xg16 is set: the row's place in each chosen expert's batch is taken from the expert's counter
     // and the normalised row is written there in fp16 (fragment packed), so that no list or gather launch follows
     half_t* xg16; long xg_estride; int packed_kt; int* counts; int* slot; int max_rows;
+    // fast kernel only, when xn16 is set (prefill): the normalised row leaves as fp16, row-major with ld_xn16 elements per
+    // row, where the experts' up projection reads it through the token lists; xn32 is not written
+    half_t* xn16; long ld_xn16;
 };
 
 __device__ __forceinline__ float tree8(float v) {
@@ -324,7 +327,10 @@ __global__ __launch_bounds__(256) void moe_router_fast_kernel(MoeRouterArgs a) {
         const int c = 4 * (t + i * 256);
 #pragma unroll
         for (int q = 0; q < 4; ++q) y[i][q] = c < h ? g[i][q] * ((v[i][q] - mean) / sigma) + bt[i][q] : 0.0f;
-        if (c < h && !a.xg16) *(floatx4*)(a.xn32 + (long)r * h + c) = y[i];
+        if (c < h && a.xn16) {
+            half4 hv = {(half_t)y[i][0], (half_t)y[i][1], (half_t)y[i][2], (half_t)y[i][3]};
+            *(half4*)(a.xn16 + (long)r * a.ld_xn16 + c) = hv;
+        } else if (c < h && !a.xg16) *(floatx4*)(a.xn32 + (long)r * h + c) = y[i];
     }
     // router logits: every thread's columns against all experts, then a tree over the block
     for (int e0 = 0; e0 < E; e0 += 8) {
