@@ -278,7 +278,8 @@ TSHIP_API int TSHip_GptStepBytes(TSHipGpt* m, int batch, double* weight_bytes, d
  *   TSHIP_PATCH_ROWS=1|2|4|8  prefill GEMM: row tiles per tile patch of an XCD
  *   TSHIP_ATTN_NQ=1|2         prefill attention: groups of 16 MFMA columns per wavefront
  *   TSHIP_NO_KV_FUSE=1        prefill: the QKV projection leaves the cache write to a kernel of its own
- *   TSHIP_NO_MOE_BATCH=1      prefill of MoE layers: one GEMM launch per expert instead of one per projection */
+ *   TSHIP_NO_MOE_BATCH=1      prefill of MoE layers: the experts' row counts are read back, the rows gathered and one GEMM
+ *                             launched per expert, instead of one launch per projection with everything on the device */
 
 #ifdef __cplusplus
 }

@@ -605,20 +605,38 @@ def test_argument_errors(G):
     gpu.close()
 
 
-def test_moe_prefill_one_launch_for_all_experts_equals_one_per_expert(G, monkeypatch):
-    """From 512 rows per expert on, the prefill runs each projection of all experts as one launch of the LDS-tiled kernel
-    (weights by pointer table, row counts read on the device).  Same logits, bit for bit, as one launch per expert
-    (TSHIP_NO_MOE_BATCH=1), also when an expert holds far fewer rows than the largest one."""
-    cfg = synth.tiny_config(n_layers=3, n_experts=4, experts_per_token=1, norm_type=synth.LAYERNORM, act=synth.RELU, dtype="f16",
-                            batch=5, prompt=520, vocab=300)
+@pytest.mark.parametrize("experts,k,batch,prompt,router_bias", [
+    (4, 1, 5, 520, None),                 # 2600 rows, one choice per token
+    (16, 4, 2, 300, None),                # 600 rows, 2400 (token, choice) pairs over 16 experts: about 150 rows each
+    (4, 2, 3, 200, (-60.0, 0.0, 0.0, 0.0)),       # expert 0 is never chosen: a problem with no rows
+    (4, 2, 3, 200, (60.0, 0.0, 0.0, 0.0)),        # expert 0 is chosen by every token: all 600 rows in one problem
+    (8, 2, 1, 777, None),                 # row counts that are no multiples of anything
+])
+def test_moe_prefill_one_launch_for_all_experts_equals_one_per_expert(G, oracle, monkeypatch, experts, k, batch, prompt, router_bias):
+    """From 512 prompt rows on, the prefill of an fp16 model never reads the experts' row counts back: each projection of
+    all experts is one launch of the LDS-tiled kernel over the experts' row tiles packed one behind the other (weights by
+    pointer table, the problem of a tile found on the device from the counts), and the up projection reads its rows
+    through the token lists.  Same logits, bit for bit, as the path with the counts on the host, gathered rows and one
+    launch per expert (TSHIP_NO_MOE_BATCH=1): with an expert that holds far fewer rows than the largest one, one with no
+    rows at all, one with every row, and row counts that fill no tile.  And the logits against the oracle."""
+    cfg = synth.tiny_config(n_layers=3, n_experts=experts, experts_per_token=k, norm_type=synth.LAYERNORM, act=synth.RELU, dtype="f16",
+                            batch=batch, prompt=prompt, vocab=300)
     w = synth.make_weights(cfg, 62, random_bias=True)
+    if router_bias is not None:
+        w = dict(w)
+        w["GPTDecoder.MoEFFN_2.m_RouterBias"] = np.asarray(router_bias, np.float32).reshape(1, experts)
     seqs = synth.make_prompts(cfg, 162)
-    gpu = G.HipGpt(cfg, w, max_batch=5, max_seq_len=530)
+    gpu = G.HipGpt(cfg, w, max_batch=batch, max_seq_len=prompt + 10)
     gpu.prefill(seqs)
     one = gpu.logits()
+    if router_bias is not None:
+        ti, _, _ = gpu.moe_routing(2)
+        assert (ti == 0).any(axis=1).all() if router_bias[0] > 0 else not (ti == 0).any()
     monkeypatch.setenv("TSHIP_NO_MOE_BATCH", "1")
     gpu.reset()
     gpu.prefill(seqs)
     monkeypatch.delenv("TSHIP_NO_MOE_BATCH")
     assert np.array_equal(one, gpu.logits())
+    _, lg = oracle.OracleGpt(cfg, w).step(seqs, use_cache=True)
+    assert np.abs(one - lg).max() <= FP16_ABS
     gpu.close()
