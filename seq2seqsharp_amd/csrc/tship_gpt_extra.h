@@ -199,9 +199,12 @@ static void run_moe_ffn_impl(TSHipGpt* m, LayerW& L, int rows, const ResidNormAr
     }
     if (batched && last_rows) {
         // what TSHip_GptGetMoeRouting reports after a prefill: the routing of every sequence's last position
-        launch(m, "moe_last_rows", moe_rows_kernel, dim3(n_last), dim3(64), (const float*)probs, last_rows, lroute, E);
-        launch(m, "moe_last_rows", moe_rows_kernel, dim3(n_last), dim3(64), (const float*)top_val, last_rows, lroute + (size_t)m->Bpad * E, k);
-        launch(m, "moe_last_rows", moe_rows_kernel, dim3(n_last), dim3(64), (const float*)top_idx, last_rows, lroute + (size_t)m->Bpad * (E + k), k);
+        MoeRowsArgs ra; std::memset(&ra, 0, sizeof(ra));
+        ra.row_map = last_rows;
+        ra.src[0] = probs; ra.dst[0] = lroute; ra.width[0] = E;
+        ra.src[1] = top_val; ra.dst[1] = lroute + (size_t)m->Bpad * E; ra.width[1] = k;
+        ra.src[2] = top_idx; ra.dst[2] = lroute + (size_t)m->Bpad * (E + k); ra.width[2] = k;
+        launch(m, "moe_last_rows", moe_rows_kernel, dim3(n_last, 3), dim3(64), ra);
     }
 }
 

@@ -465,34 +465,51 @@ __global__ __launch_bounds__(64) void moe_lists_kernel(const float* __restrict__
 // wavefront totals through LDS), so the lists come out in ascending token order like the serial kernel's.
 __global__ __launch_bounds__(1024) void moe_lists_big_kernel(const float* __restrict__ top_idx, int rows, int k, int max_rows, int* __restrict__ counts,
                                                               int* __restrict__ lists, int* __restrict__ slot) {
-    __shared__ int s_wave[16];
-    __shared__ int s_base;
+    __shared__ int s_wave[2][16];
     const int e = blockIdx.x, t = threadIdx.x, lane = t & 63, w = t >> 6;
-    if (t == 0) s_base = 0;
-    __syncthreads();
     const int n_pairs = rows * k;
-    for (int i0 = 0; i0 < n_pairs; i0 += 1024) {
-        const int i = i0 + t;
-        const bool hit = i < n_pairs && (int)top_idx[i] == e;
-        const unsigned long long bal = __ballot(hit);
-        const int before = __popcll(bal & ((1ull << lane) - 1ull));
-        if (lane == 0) s_wave[w] = __popcll(bal);
+    int base = 0;            // the expert's pairs before this round (every thread keeps its own copy)
+    // a thread takes four consecutive pairs per round (4096 pairs per round and block); the rounds alternate between
+    // two sets of wavefront totals, so one barrier per round is enough
+    int par = 0;
+    for (int i0 = 0; i0 < n_pairs; i0 += 4096, par ^= 1) {
+        const int i = i0 + 4 * t;
+        float tv[4];
+        if (i + 3 < n_pairs) { const floatx4 q = *(const floatx4*)(top_idx + i); tv[0] = q[0]; tv[1] = q[1]; tv[2] = q[2]; tv[3] = q[3]; }
+        else {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) tv[j] = i + j < n_pairs ? top_idx[i + j] : -1.0f;
+        }
+        bool hit[4];
+        int before = 0, total = 0;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            hit[j] = (int)tv[j] == e;
+            const unsigned long long bal = __ballot(hit[j]);
+            before += __popcll(bal & ((1ull << lane) - 1ull));          // the lower lanes' pairs all come first
+            total += __popcll(bal);
+        }
+        if (lane == 0) s_wave[par][w] = total;
         __syncthreads();
-        int off = s_base;
-        for (int j = 0; j < w; ++j) off += s_wave[j];
-        if (hit) { const int n = off + before; lists[(long)e * max_rows + n] = i / k; slot[i] = n; }
-        __syncthreads();
-        if (t == 0) { int tot = 0; for (int j = 0; j < 16; ++j) tot += s_wave[j]; s_base += tot; }
-        __syncthreads();
+        int off = base, all = 0;
+#pragma unroll
+        for (int j = 0; j < 16; ++j) { const int c = s_wave[par][j]; off += j < w ? c : 0; all += c; }
+        int n = off + before;
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            if (hit[j]) { lists[(long)e * max_rows + n] = (i + j) / k; slot[i + j] = n; ++n; }
+        base += all;
     }
-    if (t == 0) counts[e] = s_base;
+    if (t == 0) counts[e] = base;
 }
 
-// rows row_map[b] of a [.., width] table -> rows b of another (the routing of each sequence's last prompt position, kept
-// where the decode step keeps its routing): grid (batch)
-__global__ void moe_rows_kernel(const float* __restrict__ src, const int* __restrict__ row_map, float* __restrict__ dst, int width) {
-    const int b = blockIdx.x;
-    for (int c = threadIdx.x; c < width; c += blockDim.x) dst[(long)b * width + c] = src[(long)row_map[b] * width + c];
+// rows row_map[b] of up to three [.., width] tables -> rows b of others (the routing of each sequence's last prompt
+// position, kept where the decode step keeps its routing): grid (batch, tables)
+struct MoeRowsArgs { const float* src[3]; float* dst[3]; int width[3]; const int* row_map; };
+__global__ void moe_rows_kernel(MoeRowsArgs a) {
+    const int b = blockIdx.x, q = blockIdx.y;
+    const float* src = a.src[q]; float* dst = a.dst[q]; const int width = a.width[q];
+    for (int c = threadIdx.x; c < width; c += blockDim.x) dst[(long)b * width + c] = src[(long)a.row_map[b] * width + c];
 }
 
 // IndexSelect(inputNorm, tokenIdx_e) for every expert (MoEFeedForward.cs:155): grid (max_rows, E)
