@@ -563,7 +563,11 @@ static AttnKernel pick_attn_g(int G, bool prefill) {
         case 2: return prefill ? attn_prefill_kernel<CT, AT, D, 2> : attn_decode_kernel<CT, AT, D, 2>;
         case 4: return prefill ? attn_prefill_kernel<CT, AT, D, 4> : attn_decode_kernel<CT, AT, D, 4>;
         case 8: return prefill ? attn_prefill_kernel<CT, AT, D, 8> : attn_decode_kernel<CT, AT, D, 8>;
-        default: throw Error("query heads per KV head must be 1, 2, 4 or 8");
+        case 3: return prefill ? attn_prefill_kernel<CT, AT, D, 3> : attn_decode_kernel<CT, AT, D, 3>;
+        case 5: return prefill ? attn_prefill_kernel<CT, AT, D, 5> : attn_decode_kernel<CT, AT, D, 5>;
+        case 6: return prefill ? attn_prefill_kernel<CT, AT, D, 6> : attn_decode_kernel<CT, AT, D, 6>;
+        case 7: return prefill ? attn_prefill_kernel<CT, AT, D, 7> : attn_decode_kernel<CT, AT, D, 7>;
+        default: throw Error("query heads per KV head must be 1 to 8");
     }
 }
 template <typename CT, typename AT>
@@ -585,7 +589,7 @@ static AttnKernel pick_attn_mfma(int G, bool prefill, bool split, bool ragged, i
                 case 2: return attn_mfma_prefill_kernel<D, 2, true, 2>;
                 case 4: return attn_mfma_prefill_kernel<D, 4, true, 2>;
                 case 8: return attn_mfma_prefill_kernel<D, 8, true, 2>;
-                default: throw Error("query heads per KV head must be 1, 2, 4 or 8");
+                default: throw Error("internal: two column groups per wavefront are for 1, 2, 4 or 8 query heads per KV head");
             }
         }
         switch (G) {
@@ -593,7 +597,7 @@ static AttnKernel pick_attn_mfma(int G, bool prefill, bool split, bool ragged, i
             case 2: return attn_mfma_prefill_kernel<D, 2, false, 2>;
             case 4: return attn_mfma_prefill_kernel<D, 4, false, 2>;
             case 8: return attn_mfma_prefill_kernel<D, 8, false, 2>;
-            default: throw Error("query heads per KV head must be 1, 2, 4 or 8");
+            default: throw Error("internal: two column groups per wavefront are for 1, 2, 4 or 8 query heads per KV head");
         }
     }
     if (prefill && ragged) {
@@ -602,7 +606,11 @@ static AttnKernel pick_attn_mfma(int G, bool prefill, bool split, bool ragged, i
             case 2: return attn_mfma_prefill_kernel<D, 2, true>;
             case 4: return attn_mfma_prefill_kernel<D, 4, true>;
             case 8: return attn_mfma_prefill_kernel<D, 8, true>;
-            default: throw Error("query heads per KV head must be 1, 2, 4 or 8");
+            case 3: return attn_mfma_prefill_kernel<D, 3, true>;
+            case 5: return attn_mfma_prefill_kernel<D, 5, true>;
+            case 6: return attn_mfma_prefill_kernel<D, 6, true>;
+            case 7: return attn_mfma_prefill_kernel<D, 7, true>;
+            default: throw Error("query heads per KV head must be 1 to 8");
         }
     }
     TSHIP_REQUIRE(prefill, "internal: the MFMA decode kernels are picked by pick_attn_mfma_decode");
@@ -612,7 +620,11 @@ static AttnKernel pick_attn_mfma(int G, bool prefill, bool split, bool ragged, i
         case 2: return attn_mfma_prefill_kernel<D, 2>;
         case 4: return attn_mfma_prefill_kernel<D, 4>;
         case 8: return attn_mfma_prefill_kernel<D, 8>;
-        default: throw Error("query heads per KV head must be 1, 2, 4 or 8");
+        case 3: return attn_mfma_prefill_kernel<D, 3>;
+        case 5: return attn_mfma_prefill_kernel<D, 5>;
+        case 6: return attn_mfma_prefill_kernel<D, 6>;
+        case 7: return attn_mfma_prefill_kernel<D, 7>;
+        default: throw Error("query heads per KV head must be 1 to 8");
     }
 }
 // MFMA decode attention: leading scalar arguments (preloaded at wavefront start) in front of the struct
@@ -642,7 +654,11 @@ static AttnDecodeKernel pick_attn_mfma_decode(int G, bool split) {
         case 2: return split ? attn_mfma_kernel<D, 2, true> : attn_mfma_kernel<D, 2, false>;
         case 4: return split ? attn_mfma_kernel<D, 4, true> : attn_mfma_kernel<D, 4, false>;
         case 8: return split ? attn_mfma_kernel<D, 8, true> : attn_mfma_kernel<D, 8, false>;
-        default: throw Error("query heads per KV head must be 1, 2, 4 or 8");
+        case 3: return split ? attn_mfma_kernel<D, 3, true> : attn_mfma_kernel<D, 3, false>;
+        case 5: return split ? attn_mfma_kernel<D, 5, true> : attn_mfma_kernel<D, 5, false>;
+        case 6: return split ? attn_mfma_kernel<D, 6, true> : attn_mfma_kernel<D, 6, false>;
+        case 7: return split ? attn_mfma_kernel<D, 7, true> : attn_mfma_kernel<D, 7, false>;
+        default: throw Error("query heads per KV head must be 1 to 8");
     }
 }
 static AttnKernel pick_attn(TSHipGpt* m, bool prefill, bool split = false, bool ragged = false, int nq = 1) {
@@ -1061,8 +1077,8 @@ static void prefill(TSHipGpt* m, const int32_t* host_ids, int B, int Tp, const i
             // Two groups of 16 MFMA columns per wavefront (half the LDS fragment reads per score) at head size 128,
             // once the prompt is long enough for the coarser blocks to fill the chip.  (At head size 64 the second
             // group costs the second block per compute unit its registers and measured the same.)
-            int nq = (m->D == 128 && (long)ceil_div(Tp, (16 / m->G) * 16) * c.n_kv_heads * B >= 2048) ? 2 : 1;
-            if (g_hooks.attn_nq) nq = g_hooks.attn_nq;
+            int nq = (m->D == 128 && 16 % m->G == 0 && (long)ceil_div(Tp, (16 / m->G) * 16) * c.n_kv_heads * B >= 2048) ? 2 : 1;
+            if (g_hooks.attn_nq && 16 % m->G == 0) nq = g_hooks.attn_nq;
             const int per_block = (16 / m->G) * 8 * nq;
             launch(m, "p_attn", pick_attn(m, true, false, host_lens != nullptr, nq), dim3((unsigned)ceil_div(Tp, per_block), c.n_kv_heads, B), dim3(512), aa);
         }
@@ -1173,7 +1189,7 @@ TSHIP_API int TSHip_GptCreate(const TSHipGptConfig* cfg, TSHipGpt** out) {
     m->D = c.hidden / c.n_heads;
     m->G = c.n_heads / c.n_kv_heads;
     TSHIP_REQUIRE(m->D == 16 || m->D == 32 || m->D == 64 || m->D == 128, "TSHip_GptCreate: head_dim must be 16, 32, 64 or 128");
-    TSHIP_REQUIRE(m->G == 1 || m->G == 2 || m->G == 4 || m->G == 8, "TSHip_GptCreate: query heads per KV head must be 1, 2, 4 or 8");
+    TSHIP_REQUIRE(m->G >= 1 && m->G <= 8, "TSHip_GptCreate: query heads per KV head must be 1 to 8");
     m->Nqkv = (c.n_heads + 2 * c.n_kv_heads) * m->D;
     m->BT = c.max_batch <= 32 ? 1 : (c.max_batch <= 64 ? 2 : 4);
     m->Bpad = m->BT * 32;

@@ -2804,7 +2804,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(D == 64 ? (
                 const int p = lane + 64 * (b0 + u);
                 const int col = p / (D / 4), i4 = p % (D / 4);
                 const int qi = col / G, g = col % G;
-                ok[u] = active && tq0 + g2 * QB + qi < a.Tq;
+                ok[u] = active && qi < QB && tq0 + g2 * QB + qi < a.Tq;      // (G that does not divide 16: the last 16 - QB G columns stay empty)
                 const int qic = ok[u] ? g2 * QB + qi : 0;        // (a valid address either way; the value is dropped)
                 const long row = (long)b * a.Tq + min(tq0, a.Tq - 1) + qic;
                 const int c0 = (kvh * G + g) * D + 4 * i4;
@@ -3081,7 +3081,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(D == 64 ? (
             // four lanes per column: lane (col, part) divides and writes D / 8 consecutive outputs of its column as 16-byte pieces
             const int col = lane >> 2, part = lane & 3;
             const int qi = g2 * QB + col / G, g = col % G;
-            if (tq0 + qi < a.Tq) {
+            if (col / G < QB && tq0 + qi < a.Tq) {
                 half_t* out = (half_t*)a.out + ((long)b * a.Tq + tq0 + qi) * a.ld_out + (kvh * G + g) * D + hf * (D / 2) + part * (D / 8);
                 const float inv = 1.0f / sl[w][col];
 #pragma unroll

@@ -1,4 +1,4 @@
-"""Seeded sweep over model shapes the fused path accepts: head sizes 16-128, 1/2/4/8 query heads per KV head, both
+"""Seeded sweep over model shapes the fused path accepts: head sizes 16-128, 1 to 8 query heads per KV head, both
 attention layers, both norms, all activations, MoE layers, odd vocabulary sizes and feed-forward widths, batches on both
 sides of the 32- and 64-row tiles, prompts on both sides of the 32-position cache chunks.  Prefill and three decode steps
 against the CPU oracle, fp32 and fp16 bars as everywhere else."""
@@ -68,6 +68,65 @@ def test_random_shape_against_oracle(oracle, seed):
         p, lg = orc.step(cur, use_cache=True)
         gpu.decode(nxt)
     gpu.close()
+
+
+@pytest.mark.parametrize("g,d,hkv,dtype,batch,prompt,padded", [
+    (3, 64, 2, "f16", 3, 21, False),        # 24 query heads on 8 KV heads is a real shape; here 6 on 2
+    (3, 128, 1, "f16", 2, 70, True),
+    (5, 64, 1, "f16", 33, 5, False),
+    (6, 128, 1, "f16", 2, 33, False),
+    (6, 64, 2, "f16", 4, 47, True),
+    (7, 64, 1, "f16", 5, 40, False),        # 28 on 4 likewise; here 7 on 1
+    (7, 128, 1, "f16", 1, 9, False),
+    (3, 16, 2, "f16", 4, 12, False),        # small heads: the kernels without matrix instructions
+    (7, 32, 1, "f32", 3, 35, True),
+    (5, 64, 2, "f32", 2, 10, False),
+    (6, 16, 1, "f32", 40, 3, False),
+])
+def test_group_sizes_that_do_not_divide_sixteen(oracle, g, d, hkv, dtype, batch, prompt, padded):
+    """GroupQueryAttention.cs:156-159 expands the KV heads by any whole factor.  3, 5, 6 and 7 query heads per KV head: the
+    matrix-instruction prefill kernel gives a wavefront floor(16 / g) positions and leaves the last 16 - g floor(16 / g)
+    columns empty, the decode kernel uses g of its 16 columns.  Prefill (with and without padded rows) and five decode
+    steps against the oracle."""
+    from seq2seqsharp_amd import gpt as G
+    heads = hkv * g
+    cfg = synth._cfg(n_layers=2, hidden=heads * d, n_heads=heads, n_kv_heads=hkv, ffn_dim=96, vocab=257, attn_type=synth.GQA,
+                     norm_type=synth.RMSNORM, act=synth.SWIGLU, batch=batch, prompt=prompt, steps=5, dtype=dtype)
+    w = synth.make_weights(cfg, 900 + g, random_bias=True)
+    orc = oracle.OracleGpt(cfg, w)
+    gpu = G.HipGpt(cfg, w, max_batch=batch, max_seq_len=prompt + 8)
+    cur = synth.make_prompts(cfg, 950 + g)
+    lens = None
+    if padded:
+        lens = np.random.default_rng(g).integers(1, prompt + 1, batch).astype(np.int32)
+        lens[0] = prompt
+        for b in range(batch):
+            cur[b, lens[b]:] = 0
+    p, lg = orc.step(cur, use_cache=True, lens=lens)
+    gpu.prefill(cur, lens)
+    for step in range(6):
+        gl = gpu.logits()
+        if dtype == "f32":
+            assert float(np.abs(gl - lg).max() / max(np.abs(lg).max(), 1e-6)) <= 1e-4, step
+        else:
+            assert np.abs(gl - lg).max() <= 3e-2, step
+        if step == 5:
+            break
+        nxt = oracle.argmax(p).astype(np.int32)
+        cur = np.concatenate([cur, nxt[:, None]], 1)
+        p, lg = orc.step(cur, use_cache=True)
+        gpu.decode(nxt)
+    gpu.close()
+
+
+def test_group_size_limits_are_refused():
+    from seq2seqsharp_amd import gpt as G
+    from seq2seqsharp_amd._lib import TSHipError
+    for heads, hkv in ((9, 1), (6, 4)):
+        cfg = synth._cfg(n_layers=1, hidden=heads * 16, n_heads=heads, n_kv_heads=hkv, ffn_dim=48, vocab=61, attn_type=synth.GQA,
+                         norm_type=synth.RMSNORM, act=synth.RELU, batch=1, prompt=2, steps=1, dtype="f32")
+        with pytest.raises(TSHipError, match="query heads per KV head|divisible by n_kv_heads"):
+            G.HipGpt(cfg, {}, max_batch=1, max_seq_len=8)
 
 
 @pytest.mark.parametrize("experts,k,batch,dtype", [(16, 4, 9, "f16"), (12, 3, 40, "f16"), (16, 4, 33, "f32"), (3, 3, 5, "f16"), (64, 2, 7, "f16")])
