@@ -340,7 +340,7 @@ __global__ __launch_bounds__(NW * 64) void skinny_gemm_f16_kernel(const half_t* 
         for (int u = 0; u < U; ++u) {
             const int kk = min(kt + u, klast);
 #pragma unroll
-            for (int j = 0; j < NJ; ++j) wf0[u][j] = *(const half8*)(wp[j] + (long)kk * 512);
+            for (int j = 0; j < NJ; ++j) wf0[u][j] = load_once((const half8*)(wp[j] + (long)kk * 512));
 #pragma unroll
             for (int bt = 0; bt < BT; ++bt) xf0[u][bt] = *(const half8*)(xp[bt] + (long)kk * 512);
         }
@@ -413,7 +413,7 @@ __global__ __launch_bounds__(NW * 64) void skinny_gemm_f16_kernel(const half_t* 
 #pragma unroll
         for (int u = 0; u < U; ++u) {
 #pragma unroll
-            for (int j = 0; j < NJ; ++j) wf[u][j] = *(const half8*)(wp[j] + (long)(kt + u) * 512);
+            for (int j = 0; j < NJ; ++j) wf[u][j] = load_once((const half8*)(wp[j] + (long)(kt + u) * 512));
 #pragma unroll
             for (int bt = 0; bt < BT; ++bt) xf[u][bt] = *(const half8*)(xp[bt] + (long)(kt + u) * 512);
         }
@@ -433,7 +433,7 @@ __global__ __launch_bounds__(NW * 64) void skinny_gemm_f16_kernel(const half_t* 
         for (int u = 0; u < U; ++u) {
             if (kt + u < wk1) {
 #pragma unroll
-                for (int j = 0; j < NJ; ++j) wf[u][j] = *(const half8*)(wp[j] + (long)(kt + u) * 512);
+                for (int j = 0; j < NJ; ++j) wf[u][j] = load_once((const half8*)(wp[j] + (long)(kt + u) * 512));
 #pragma unroll
                 for (int bt = 0; bt < BT; ++bt) xf[u][bt] = *(const half8*)(xp[bt] + (long)(kt + u) * 512);
             }
@@ -1570,7 +1570,7 @@ __global__ __launch_bounds__(256) void skinny_gemm_f32_kernel(F32GemmArgs a) {
             for (int u = 0; u < U; ++u) {
                 const int kk = k + 16 * u;
                 const float* src = a.B + (long)(k0 + kk) * a.ldb + col0;
-                if (kk < kn && vec) wv[u] = *(const floatx4*)src;
+                if (kk < kn && vec) wv[u] = load_once((const floatx4*)src);
                 else {
 #pragma unroll
                     for (int c = 0; c < 4; ++c) wv[u][c] = (kk < kn && col0 + c < a.N) ? src[c] : 0.0f;
@@ -2026,7 +2026,8 @@ struct AttnArgs {
 // Every lane group keeps its own online-softmax state over the rows it visits; the groups of a wavefront are
 // merged with lane shuffles and the NW wavefronts through LDS.
 // sQ: LDS [G][D] queries, already rotated and scaled.  Result (fp32) is written to sOut [G][D] in LDS.
-template <typename CT, int D, int G, int NW>
+// ONCE: the launch reads every cached row once (a decode step), see load_once; a prefill's blocks share them through L2.
+template <typename CT, int D, int G, int NW, bool ONCE = false>
 __device__ __forceinline__ void attn_core(const float* sQ, const CT* Kb, const CT* Vb, int T, float* sM, float* sL, float* sAcc,
                                           float* sOut, bool quant = false) {
     constexpr int EPL = 16 / (int)sizeof(CT);
@@ -2037,6 +2038,7 @@ __device__ __forceinline__ void attn_core(const float* sQ, const CT* Kb, const C
     typedef CT vec_t __attribute__((ext_vector_type(EPL)));
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int sub = lane % LPR, rg = lane / LPR;
+    auto kv_load = [](const vec_t* p) { if constexpr (ONCE) return load_once(p); else return *p; };
 
     // fp16 cache: queries are kept as packed halves and the dot product uses v_dot2_f32_f16 (fp32 accumulate);
     // fp32 cache: plain fp32 multiply-add
@@ -2071,8 +2073,8 @@ __device__ __forceinline__ void attn_core(const float* sQ, const CT* Kb, const C
 #pragma unroll
         for (int e = 0; e < EPL; ++e) { kv[u][e] = (CT)0.0f; vv[u][e] = (CT)0.0f; }
         if (tt[u] < T) {
-            kv[u] = *(const vec_t*)(Kb + (long)tt[u] * D + sub * EPL);
-            vv[u] = *(const vec_t*)(Vb + (long)tt[u] * D + sub * EPL);
+            kv[u] = kv_load((const vec_t*)(Kb + (long)tt[u] * D + sub * EPL));
+            vv[u] = kv_load((const vec_t*)(Vb + (long)tt[u] * D + sub * EPL));
         }
     }
     for (int base = 0; base < T; base += SWEEP) {
@@ -2085,8 +2087,8 @@ __device__ __forceinline__ void attn_core(const float* sQ, const CT* Kb, const C
             for (int e = 0; e < EPL; ++e) vf[e] = (float)vv[u][e];
             tt[u] += SWEEP;
             if (tt[u] < T) {
-                kv[u] = *(const vec_t*)(Kb + (long)tt[u] * D + sub * EPL);
-                vv[u] = *(const vec_t*)(Vb + (long)tt[u] * D + sub * EPL);
+                kv[u] = kv_load((const vec_t*)(Kb + (long)tt[u] * D + sub * EPL));
+                vv[u] = kv_load((const vec_t*)(Vb + (long)tt[u] * D + sub * EPL));
             }
             float s[G];
 #pragma unroll
@@ -2223,7 +2225,7 @@ __global__ __launch_bounds__(1024) void attn_decode_kernel(AttnArgs a) {
     for (int d = t; d < D; d += NTH) Vb[(long)pos * D + d] = (CT)sm.in[(G + 1) * D + d];
     __threadfence_block();
     __syncthreads();
-    attn_core<CT, D, G, NW>(sm.q, Kb, Vb, pos + 1, sm.m, sm.l, sm.acc, sm.out);
+    attn_core<CT, D, G, NW, true>(sm.q, Kb, Vb, pos + 1, sm.m, sm.l, sm.acc, sm.out);
     if (a.out_kt > 0) {
         for (int idx = t; idx < G * D; idx += NTH) ((AT*)a.out)[xpack_index(b, kvh * G * D + idx, a.out_kt)] = (AT)sm.out[idx];
     } else {
@@ -2416,9 +2418,9 @@ __global__ __launch_bounds__(D == 128 ? 256 : 512) void attn_mfma_kernel(void* k
 #pragma unroll
         for (int tile = 0; tile < 2; ++tile)
 #pragma unroll
-            for (int kd = 0; kd < KD; ++kd) kf[tile][kd] = *(const half8*)(kc + (tile * KD + kd) * 512);
+            for (int kd = 0; kd < KD; ++kd) kf[tile][kd] = load_once((const half8*)(kc + (tile * KD + kd) * 512));
 #pragma unroll
-        for (int dt = 0; dt < DT; ++dt) vf[dt] = *(const half8*)(vc + dt * 512);
+        for (int dt = 0; dt < DT; ++dt) vf[dt] = load_once((const half8*)(vc + dt * 512));
     };
     // Chunks of this wavefront: gw, gw + GS, ...  A CU accepts about 64 KiB of outstanding loads; a wavefront that
     // requests more stalls at the request, and loads that hit in L2 come back behind the misses queued before them.
