@@ -879,7 +879,8 @@ __device__ __forceinline__ void resid_store_lines(const BigArgs& a, const floatx
     const int lh = lane >> 5, r = lane & 31, piece = lane & 7, rr = lane >> 3;
     floatx4 old[8];
 #pragma unroll
-    for (int ps = 0; ps < 8; ++ps) old[ps] = RESID ? *(const floatx4*)(a.out + (row_first + 8 * ps + rr) * a.ld_out + (long)nt * 32 + 4 * piece) : floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+    // (the old values were written a whole GEMM ago and are read once here; the new ones are read a whole GEMM from now)
+    for (int ps = 0; ps < 8; ++ps) old[ps] = RESID ? load_once((const floatx4*)(a.out + (row_first + 8 * ps + rr) * a.ld_out + (long)nt * 32 + 4 * piece)) : floatx4{0.0f, 0.0f, 0.0f, 0.0f};
     float bb[16];
 #pragma unroll
     for (int v = 0; v < 16; ++v) bb[v] = a.bias[nt * 32 + 8 * (v / 4) + 4 * lh + (v % 4)];
@@ -904,7 +905,7 @@ __device__ __forceinline__ void resid_store_lines(const BigArgs& a, const floatx
         floatx4 sv;
 #pragma unroll
         for (int e = 0; e < 4; ++e) sv[e] = RESID ? v[ps][e] + old[ps][e] : v[ps][e];
-        *(floatx4*)(a.out + row * a.ld_out + (long)nt * 32 + 4 * piece) = sv;
+        __builtin_nontemporal_store(sv, (floatx4*)(a.out + row * a.ld_out + (long)nt * 32 + 4 * piece));
         if (RESID && a.xg16) {
             half4v xg;
             float q = 0.0f;
