@@ -29,7 +29,12 @@ def algorithmic_prefill_flops(cfg, B, Tp):
     h, H, G, F, V, L = cfg["hidden"], cfg["n_heads"], cfg["n_kv_heads"], cfg["ffn_dim"], cfg["vocab"], cfg["n_layers"]
     d = h // H
     nW = 3 if cfg["act"] in (3, 4) else 2
-    per_tok = L * (h * H * d + 2 * h * G * d + H * d * h + nW * h * F)
+    # MoE layers (every layer after the second when the model has experts, GPTDecoder.cs:83-91): a token runs through
+    # experts_per_token experts of two matrices h x 4h and 4h x h each, plus the router (MoEFeedForward.cs:76-181)
+    E, k = cfg.get("n_experts", 1), cfg.get("experts_per_token", 1)
+    n_moe = max(L - 2, 0) if E > 1 else 0
+    ffn = (L - n_moe) * nW * h * F + n_moe * (k * 2 * h * 4 * h + h * E)
+    per_tok = L * (h * H * d + 2 * h * G * d + H * d * h) + ffn
     return 2.0 * B * Tp * per_tok + 2.0 * B * h * V + L * B * H * d * float(Tp) * Tp * 2.0
 
 
