@@ -103,7 +103,8 @@ using namespace tship;
 struct TSHipGpt {
     TSHipGptConfig c;
     bool f16;
-    int D, G, Nqkv, Bpad, BT;
+    int D, G, Nqkv, Bpad, BT;      // G: query heads per block of the attention kernels (all of a KV head's, or a group of them)
+    int SG = 1, Hv = 0;            // groups of G query heads per KV head (more than eight heads per KV head), and n_kv_heads * SG
     long ldh, ldF;                 // leading dims of activation buffers (elements)
     int F13;                       // columns of the first FFN GEMM output (F or 2F)
     bool gated;
@@ -638,28 +639,35 @@ static AttnPacked attn_pack_args(const AttnArgs& a) {
         return (int)(d >> 8);
     };
     TSHIP_REQUIRE(a.max_len < (1L << 31) && a.ldq < (1L << 31) && a.split_stride < (1L << 31), "internal: attention strides beyond 32 bits");
-    TSHIP_REQUIRE(a.H < 256 && a.Hkv < 256 && a.KS < 256 && a.ssq_nt < 65536 && a.ssq_ld < 65536, "internal: attention counts beyond their packed fields");
+    TSHIP_REQUIRE(a.H < 256 && a.Hkv < 256 && a.KS < 256 && a.ssq_nt < 65536 && a.ssq_ld < 65536 && a.kv_sub >= 0 && a.kv_sub < 32,
+                  "internal: attention counts beyond their packed fields");
     AttnPacked p;
     p.kcache = a.kcache; p.d_vcache = off(a.vcache, "values"); p.d_qkv = off(a.qkv, "projection"); p.d_pos = off(a.d_pos, "position");
     p.d_bias = off(a.bias, "bias"); p.d_ssq = off(a.ssq, "tile sums"); p.d_rope_cos = off(a.rope_cos, "cosines"); p.d_rope_sin = off(a.rope_sin, "sines");
     p.max_len = (int)a.max_len;
-    p.counts = (unsigned)a.H | ((unsigned)a.Hkv << 8) | ((unsigned)a.KS << 16) | (a.ssq ? 1u << 24 : 0u) | (a.rope_cos ? 1u << 25 : 0u) | (a.ln ? 1u << 26 : 0u);
+    p.counts = (unsigned)a.H | ((unsigned)a.Hkv << 8) | ((unsigned)a.KS << 16) | (a.ssq ? 1u << 24 : 0u) | (a.rope_cos ? 1u << 25 : 0u) | (a.ln ? 1u << 26 : 0u) |
+               ((unsigned)a.kv_sub << 27);
     p.ldq = (int)a.ldq; p.split_stride = (int)a.split_stride; p.ssq_dims = (unsigned)a.ssq_nt | ((unsigned)a.ssq_ld << 16);
     return p;
 }
-template <int D>
-static AttnDecodeKernel pick_attn_mfma_decode(int G, bool split) {
+template <int D, bool SUB>
+static AttnDecodeKernel pick_attn_mfma_decode_s(int G, bool split) {
     switch (G) {
-        case 1: return split ? attn_mfma_kernel<D, 1, true> : attn_mfma_kernel<D, 1, false>;
-        case 2: return split ? attn_mfma_kernel<D, 2, true> : attn_mfma_kernel<D, 2, false>;
-        case 4: return split ? attn_mfma_kernel<D, 4, true> : attn_mfma_kernel<D, 4, false>;
-        case 8: return split ? attn_mfma_kernel<D, 8, true> : attn_mfma_kernel<D, 8, false>;
-        case 3: return split ? attn_mfma_kernel<D, 3, true> : attn_mfma_kernel<D, 3, false>;
-        case 5: return split ? attn_mfma_kernel<D, 5, true> : attn_mfma_kernel<D, 5, false>;
-        case 6: return split ? attn_mfma_kernel<D, 6, true> : attn_mfma_kernel<D, 6, false>;
-        case 7: return split ? attn_mfma_kernel<D, 7, true> : attn_mfma_kernel<D, 7, false>;
+        case 1: return split ? attn_mfma_kernel<D, 1, true, SUB> : attn_mfma_kernel<D, 1, false, SUB>;
+        case 2: return split ? attn_mfma_kernel<D, 2, true, SUB> : attn_mfma_kernel<D, 2, false, SUB>;
+        case 4: return split ? attn_mfma_kernel<D, 4, true, SUB> : attn_mfma_kernel<D, 4, false, SUB>;
+        case 8: return split ? attn_mfma_kernel<D, 8, true, SUB> : attn_mfma_kernel<D, 8, false, SUB>;
+        case 3: return split ? attn_mfma_kernel<D, 3, true, SUB> : attn_mfma_kernel<D, 3, false, SUB>;
+        case 5: return split ? attn_mfma_kernel<D, 5, true, SUB> : attn_mfma_kernel<D, 5, false, SUB>;
+        case 6: return split ? attn_mfma_kernel<D, 6, true, SUB> : attn_mfma_kernel<D, 6, false, SUB>;
+        case 7: return split ? attn_mfma_kernel<D, 7, true, SUB> : attn_mfma_kernel<D, 7, false, SUB>;
         default: throw Error("query heads per KV head must be 1 to 8");
     }
+}
+// sub: the query heads of a KV head come in several groups (more than eight per KV head)
+template <int D>
+static AttnDecodeKernel pick_attn_mfma_decode(int G, bool split, bool sub) {
+    return sub ? pick_attn_mfma_decode_s<D, true>(G, split) : pick_attn_mfma_decode_s<D, false>(G, split);
 }
 static AttnKernel pick_attn(TSHipGpt* m, bool prefill, bool split = false, bool ragged = false, int nq = 1) {
     if (m->vt) return m->D == 64 ? pick_attn_mfma<64>(m->G, prefill, split, ragged, nq) : pick_attn_mfma<128>(m->G, prefill, split, ragged, nq);
@@ -679,7 +687,7 @@ static AttnKernel pick_kvw(TSHipGpt* m) { return m->f16 ? pick_kvw_t<half_t>(m->
 
 static AttnArgs attn_args(TSHipGpt* m, LayerW& L) {
     AttnArgs a; std::memset(&a, 0, sizeof(a));
-    a.bias = L.bqkv.as<float>(); a.H = m->c.n_heads; a.Hkv = m->c.n_kv_heads;
+    a.bias = L.bqkv.as<float>(); a.H = m->c.n_heads; a.Hkv = m->c.n_kv_heads; a.kv_sub = m->SG;
     a.kcache = L.kc.p; a.vcache = L.vc.p; a.max_len = m->ML; a.vt = m->vt ? 1 : 0;
     if (m->c.use_rope) { a.rope_cos = m->rope_cos.as<float>(); a.rope_sin = m->rope_sin.as<float>(); }
     a.d_pos = m->d_pos.as<int>();
@@ -691,7 +699,7 @@ static AttnArgs attn_args(TSHipGpt* m, LayerW& L) {
 static int attn_splits(TSHipGpt* m, int B) {
     if (!m->vt) return 1;
     const int NW = m->D == 128 ? 4 : 8;
-    const long pairs = (long)B * m->c.n_kv_heads;
+    const long pairs = (long)B * m->Hv;
     long S = n_compute_units() / std::max<long>(pairs, 1);                  // fill the CUs
     // Splitting pays when a wavefront still walks many chunks: at a context of 1 k the launch is bound by its fixed
     // costs and the exchange adds 0.7 us (measured: 16.8 vs 15.9 us at 4 rows); at 8 k it gains 2.5 %.
@@ -700,18 +708,19 @@ static int attn_splits(TSHipGpt* m, int B) {
     return (int)std::max<long>(1, std::min<long>(S, TSHipGpt::MAX_ATTN_SPLITS));
 }
 static void launch_attn_decode(TSHipGpt* m, AttnArgs a, int B) {
-    if (!m->vt) { launch(m, "attn_decode", pick_attn(m, false), dim3(m->c.n_kv_heads, B), dim3(1024), a); return; }
+    if (!m->vt) { launch(m, "attn_decode", pick_attn(m, false), dim3(m->Hv, B), dim3(1024), a); return; }
     const int S = attn_splits(m, B);
     const unsigned threads = m->D == 128 ? 256 : 512;
-    dim3 grid(m->c.n_kv_heads, B);
+    dim3 grid(m->c.n_kv_heads, B, m->SG);       // (one block per pair: the groups of a KV head's query heads on z)
     if (S > 1) {
-        const long pairs = (long)B * m->c.n_kv_heads, per = (long)m->G * m->D + 2 * m->G;
+        grid = dim3(m->Hv, B);
+        const long pairs = (long)B * m->Hv, per = (long)m->G * m->D + 2 * m->G;
         TSHIP_REQUIRE((size_t)(pairs * S * per) * sizeof(float) <= m->attn_xchg.bytes && (size_t)pairs * sizeof(int) <= m->attn_count.bytes,
                       "internal: attention exchange area too small");
         a.S = S; a.xchg = m->attn_xchg.as<float>(); a.xcount = m->attn_count.as<int>();
         grid.z = (unsigned)S;
     }
-    AttnDecodeKernel k = m->D == 64 ? pick_attn_mfma_decode<64>(m->G, S > 1) : pick_attn_mfma_decode<128>(m->G, S > 1);
+    AttnDecodeKernel k = m->D == 64 ? pick_attn_mfma_decode<64>(m->G, S > 1, m->SG > 1) : pick_attn_mfma_decode<128>(m->G, S > 1, m->SG > 1);
     const AttnPacked p = attn_pack_args(a);
     launch(m, "attn_decode", k, grid, dim3(threads), p.kcache, p.d_vcache, p.d_qkv, p.d_pos, p.d_bias, p.d_ssq, p.d_rope_cos, p.d_rope_sin, p.max_len, p.counts,
            p.ldq, p.split_stride, p.ssq_dims, a);
@@ -1077,12 +1086,12 @@ static void prefill(TSHipGpt* m, const int32_t* host_ids, int B, int Tp, const i
             // Two groups of 16 MFMA columns per wavefront (half the LDS fragment reads per score) at head size 128,
             // once the prompt is long enough for the coarser blocks to fill the chip.  (At head size 64 the second
             // group costs the second block per compute unit its registers and measured the same.)
-            int nq = (m->D == 128 && 16 % m->G == 0 && (long)ceil_div(Tp, (16 / m->G) * 16) * c.n_kv_heads * B >= 2048) ? 2 : 1;
+            int nq = (m->D == 128 && 16 % m->G == 0 && (long)ceil_div(Tp, (16 / m->G) * 16) * m->Hv * B >= 2048) ? 2 : 1;
             if (g_hooks.attn_nq && 16 % m->G == 0) nq = g_hooks.attn_nq;
             const int per_block = (16 / m->G) * 8 * nq;
-            launch(m, "p_attn", pick_attn(m, true, false, host_lens != nullptr, nq), dim3((unsigned)ceil_div(Tp, per_block), c.n_kv_heads, B), dim3(512), aa);
+            launch(m, "p_attn", pick_attn(m, true, false, host_lens != nullptr, nq), dim3((unsigned)ceil_div(Tp, per_block), m->Hv, B), dim3(512), aa);
         }
-        else launch(m, "p_attn", pick_attn(m, true), dim3(Tp, c.n_kv_heads, B), dim3(256), aa);
+        else launch(m, "p_attn", pick_attn(m, true), dim3(Tp, m->Hv, B), dim3(256), aa);
         ResidNormArgs a2 = rn;
         a2.gamma = L.n2_g.as<float>(); a2.beta = L.n2_b.as<float>();
         if (m->f16) {
@@ -1187,9 +1196,17 @@ TSHIP_API int TSHip_GptCreate(const TSHipGptConfig* cfg, TSHipGpt** out) {
     m->c = c;
     m->f16 = c.dtype == TSHIP_F16;
     m->D = c.hidden / c.n_heads;
-    m->G = c.n_heads / c.n_kv_heads;
+    {
+        // GroupQueryAttention.cs:156-159 expands the KV heads by any whole factor.  The attention kernels take up to eight
+        // query heads per block: a larger factor is served as groups of its largest divisor up to eight.
+        const int per_kv = c.n_heads / c.n_kv_heads;
+        m->G = 1;
+        for (int g = 2; g <= 8; ++g) if (per_kv % g == 0) m->G = g;
+        m->SG = per_kv / m->G;
+        m->Hv = c.n_kv_heads * m->SG;
+    }
     TSHIP_REQUIRE(m->D == 16 || m->D == 32 || m->D == 64 || m->D == 128, "TSHip_GptCreate: head_dim must be 16, 32, 64 or 128");
-    TSHIP_REQUIRE(m->G >= 1 && m->G <= 8, "TSHip_GptCreate: query heads per KV head must be 1 to 8");
+    TSHIP_REQUIRE(m->SG < 32, "TSHip_GptCreate: the query heads of a KV head must split into fewer than 32 groups of up to eight (at most 248 per KV head, no large prime counts)");
     m->Nqkv = (c.n_heads + 2 * c.n_kv_heads) * m->D;
     m->BT = c.max_batch <= 32 ? 1 : (c.max_batch <= 64 ? 2 : 4);
     m->Bpad = m->BT * 32;
@@ -1243,7 +1260,7 @@ TSHIP_API int TSHip_GptCreate(const TSHipGptConfig* cfg, TSHipGpt** out) {
     m->ids.alloc((size_t)m->Bpad * sizeof(int));
     m->d_pos.alloc(2 * sizeof(int));      // [0] cached positions, [1] step counter of the running generate call
     if (m->vt) {
-        const long pairs = (long)c.max_batch * c.n_kv_heads, per = (long)m->G * m->D + 2 * m->G;
+        const long pairs = (long)c.max_batch * m->Hv, per = (long)m->G * m->D + 2 * m->G;
         // at most as many blocks as CUs (or one per pair) ever share the area
         const long blocks = std::max<long>(pairs, std::min<long>(pairs * TSHipGpt::MAX_ATTN_SPLITS, 2L * n_compute_units()));
         m->attn_xchg.alloc((size_t)(blocks * per) * sizeof(float));

@@ -2033,6 +2033,11 @@ struct AttnArgs {
     // from lens[b] on has every column masked, which after the softmax means: it attends to ALL columns of the padded
     // sequence, with scores rounded to multiples of 2^-9 by the float32 addition of -30000.
     const int* lens;
+    // More than eight query heads per KV head: the heads of a KV head are served in kv_sub groups of G (the kernels'
+    // template argument) heads each, a block per group.  The grid then counts Hkv * kv_sub "KV heads"; block index v
+    // takes query heads v G ... v G + G - 1 and the cache and projection columns of KV head v / kv_sub.  At decode every
+    // group of a KV head appends the same new row (the same values to the same place).  0 or 1: one group.
+    int kv_sub;
 };
 
 // Single-query attention of G query heads that share one KV head over T cached positions.
@@ -2195,6 +2200,7 @@ __global__ __launch_bounds__(1024) void attn_decode_kernel(AttnArgs a) {
     constexpr int NW = 16, NTH = NW * 64;
     __shared__ AttnSmem<CT, D, G, NW> sm;
     const int kvh = blockIdx.x, b = blockIdx.y, t = threadIdx.x;
+    const int kvc = a.kv_sub > 1 ? kvh / a.kv_sub : kvh;       // the KV head whose cache this group of query heads reads
     const int pos = *a.d_pos;
     const int HD = a.H * D, GD = a.Hkv * D;
     float rinv = 1.0f, mean = 0.0f;
@@ -2214,8 +2220,8 @@ __global__ __launch_bounds__(1024) void attn_decode_kernel(AttnArgs a) {
     for (int idx = t; idx < (G + 2) * D; idx += NTH) {
         int col;
         if (idx < G * D) col = kvh * G * D + idx;
-        else if (idx < (G + 1) * D) col = HD + kvh * D + (idx - G * D);
-        else col = HD + GD + kvh * D + (idx - (G + 1) * D);
+        else if (idx < (G + 1) * D) col = HD + kvc * D + (idx - G * D);
+        else col = HD + GD + kvc * D + (idx - (G + 1) * D);
         // split-K partials in index order, eight requested at a time (unconditionally, the index clamped to the last split)
         float s = a.qkv[(long)b * a.ldq + col];
         for (int k = 1; k < a.KS; k += 8) {
@@ -2228,8 +2234,8 @@ __global__ __launch_bounds__(1024) void attn_decode_kernel(AttnArgs a) {
         sm.in[idx] = a.ln ? (s - mean * a.bias[a.ldq + col]) * rinv + a.bias[col] : s * rinv + a.bias[col];
     }
     __syncthreads();
-    CT* Kb = (CT*)a.kcache + ((long)b * a.Hkv + kvh) * a.max_len * D;
-    CT* Vb = (CT*)a.vcache + ((long)b * a.Hkv + kvh) * a.max_len * D;
+    CT* Kb = (CT*)a.kcache + ((long)b * a.Hkv + kvc) * a.max_len * D;
+    CT* Vb = (CT*)a.vcache + ((long)b * a.Hkv + kvc) * a.max_len * D;
     for (int p = t; p < (G + 1) * D / 2; p += NTH) {
         int vec = p / (D / 2), i = p % (D / 2);
         float x0 = sm.in[vec * D + 2 * i], x1 = sm.in[vec * D + 2 * i + 1], y0 = x0, y1 = x1;
@@ -2352,6 +2358,7 @@ template <typename CT, typename AT, int D, int G>
 __global__ __launch_bounds__(256) void attn_prefill_kernel(AttnArgs a) {
     __shared__ AttnSmem<CT, D, G, 4> sm;
     const int tq = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z, t = threadIdx.x;
+    const int kvc = a.kv_sub > 1 ? kvh / a.kv_sub : kvh;
     const long row = (long)b * a.Tq + tq;
     const int pos = a.pos0 + tq;
     for (int p = t; p < G * D / 2; p += 256) {
@@ -2362,8 +2369,8 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(AttnArgs a) {
         sm.q[vec * D + 2 * i] = a.scale * y0; sm.q[vec * D + 2 * i + 1] = a.scale * y1;
     }
     __syncthreads();
-    const CT* Kb = (const CT*)a.kcache + ((long)b * a.Hkv + kvh) * a.max_len * D;
-    const CT* Vb = (const CT*)a.vcache + ((long)b * a.Hkv + kvh) * a.max_len * D;
+    const CT* Kb = (const CT*)a.kcache + ((long)b * a.Hkv + kvc) * a.max_len * D;
+    const CT* Vb = (const CT*)a.vcache + ((long)b * a.Hkv + kvc) * a.max_len * D;
     const bool all_masked = a.lens && tq >= a.lens[b];          // (padded prompts start an empty cache: pos0 = 0)
     attn_core<CT, D, G, 4>(sm.q, Kb, Vb, all_masked ? a.pos0 + a.Tq : pos + 1, sm.m, sm.l, sm.acc, sm.out, all_masked);
     AT* out = (AT*)a.out + row * a.ld_out + kvh * G * D;
@@ -2394,7 +2401,7 @@ struct AttnPacked {
     int max_len; unsigned counts;     // H | Hkv << 8 | KS << 16 | (ssq ? 1 : 0) << 24 | (rope ? 1 : 0) << 25 | (ln ? 1 : 0) << 26
     int ldq, split_stride; unsigned ssq_dims;   // ssq_nt | ssq_ld << 16
 };
-template <int D, int G, bool SPLIT>
+template <int D, int G, bool SPLIT, bool SUB = false>      // SUB: groups of query heads share a KV head (AttnArgs::kv_sub > 1)
 __global__ __launch_bounds__(D == 128 ? 256 : 512) void attn_mfma_kernel(void* kcache_, int d_vcache, int d_qkv, int d_pos, int d_bias, int d_ssq, int d_rope_cos,
                                                                        int d_rope_sin, int max_len_, unsigned counts, int ldq_, int split_stride_,
                                                                        unsigned ssq_dims, AttnArgs a) {
@@ -2404,7 +2411,7 @@ __global__ __launch_bounds__(D == 128 ? 256 : 512) void attn_mfma_kernel(void* k
         a.kcache = kcache_; a.vcache = at(d_vcache); a.qkv = (const float*)at(d_qkv); a.d_pos = (const int*)at(d_pos); a.bias = (const float*)at(d_bias);
         a.ssq = (counts >> 24) & 1 ? (const float*)at(d_ssq) : nullptr; a.ln = (counts >> 26) & 1;
         a.rope_cos = (counts >> 25) & 1 ? (const float*)at(d_rope_cos) : nullptr; a.rope_sin = (counts >> 25) & 1 ? (const float*)at(d_rope_sin) : nullptr;
-        a.max_len = max_len_; a.H = counts & 255; a.Hkv = (counts >> 8) & 255; a.KS = (counts >> 16) & 255;
+        a.max_len = max_len_; a.H = counts & 255; a.Hkv = (counts >> 8) & 255; a.KS = (counts >> 16) & 255; a.kv_sub = SUB ? counts >> 27 : 1;
         a.ldq = ldq_; a.split_stride = split_stride_; a.ssq_nt = ssq_dims & 0xffff; a.ssq_ld = ssq_dims >> 16;
     }
     constexpr int NW = D == 128 ? 4 : 8, NTH = NW * 64;
@@ -2420,12 +2427,26 @@ __global__ __launch_bounds__(D == 128 ? 256 : 512) void attn_mfma_kernel(void* k
     const int gw = SPLIT ? (int)blockIdx.z * NW + w : w, GS = SPLIT ? a.S * NW : NW;
     const int r16 = lane & 15, q = lane >> 4;
     const int HD = a.H * D, GD = a.Hkv * D;
-    const int kvh = blockIdx.x, b = blockIdx.y;
+    // Groups of query heads that share a KV head (AttnArgs::kv_sub).  One block per pair: grid (Hkv, batch, kv_sub), so
+    // that the cache addresses, which the first requests need, depend on blockIdx.x alone.  Several blocks per pair: grid
+    // (Hkv * kv_sub, batch, blocks); kvh + 0.5 lies at least 1 / (2 kv_sub) from a multiple of kv_sub, far more than the
+    // reciprocal's error.
+    const int b = blockIdx.y;
+    int kvh, kvc;
+    if constexpr (!SUB) {
+        kvh = kvc = blockIdx.x;
+    } else if constexpr (SPLIT) {
+        kvh = blockIdx.x;
+        kvc = (int)(((float)kvh + 0.5f) * __builtin_amdgcn_rcpf((float)a.kv_sub));
+    } else {
+        kvc = blockIdx.x;
+        kvh = kvc * a.kv_sub + (int)blockIdx.z;
+    }
     // (the position is requested here and first used behind the prologue's other requests, which do not depend on it:
     // one memory round trip for both instead of one after the other)
     const int pos_base = *a.d_pos;
-    half_t* Kb = (half_t*)a.kcache + ((long)b * a.Hkv + kvh) * a.max_len * D;
-    half_t* Vt = (half_t*)a.vcache + ((long)b * a.Hkv + kvh) * (long)D * a.max_len;
+    half_t* Kb = (half_t*)a.kcache + ((long)b * a.Hkv + kvc) * a.max_len * D;
+    half_t* Vt = (half_t*)a.vcache + ((long)b * a.Hkv + kvc) * (long)D * a.max_len;
     half8 kfA[2][KD], vfA[DT];
     auto load_chunk = [&](int c, half8 (&kf)[2][KD], half8 (&vf)[DT]) {
         const half_t* kc = Kb + (long)c * (32 * D) + lane * 8;
@@ -2474,8 +2495,8 @@ __global__ __launch_bounds__(D == 128 ? 256 : 512) void attn_mfma_kernel(void* k
             if (idx < (G + 2) * D) {
                 int col;
                 if (idx < G * D) col = kvh * G * D + idx;
-                else if (idx < (G + 1) * D) col = HD + kvh * D + (idx - G * D);
-                else col = HD + GD + kvh * D + (idx - (G + 1) * D);
+                else if (idx < (G + 1) * D) col = HD + kvc * D + (idx - G * D);
+                else col = HD + GD + kvc * D + (idx - (G + 1) * D);
                 pcol[ci] = col;
 #pragma unroll
                 for (int k = 0; k < 8; ++k) if (k < a.KS) part[ci][k] = a.qkv[k * a.split_stride + (long)b * a.ldq + col];
@@ -2650,7 +2671,7 @@ __global__ __launch_bounds__(D == 128 ? 256 : 512) void attn_mfma_kernel(void* k
     if constexpr (SPLIT) {
         // block sums relative to the block maximum -> exchange area [pair][block][NCOL D + 2 NCOL] floats
         __shared__ int s_last;
-        const int pair = b * a.Hkv + kvh;
+        const int pair = b * (int)gridDim.x + kvh;
         const long per = (long)NCOL * D + 2 * NCOL;
         float* mine = a.xchg + ((long)pair * a.S + blockIdx.z) * per;
         for (int idx = t; idx < NCOL * D; idx += NTH) {
@@ -2777,6 +2798,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(D == 64 ? (
     const int lane = threadIdx.x & 63, w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int r16 = lane & 15, q = lane >> 4;
     const int kvh = blockIdx.y, b = blockIdx.z;
+    const int kvc = a.kv_sub > 1 ? kvh / a.kv_sub : kvh;       // (groups of query heads that share a KV head, see AttnArgs::kv_sub)
     const int tq0 = (blockIdx.x * NW + w) * (QB * NQ);
     const bool active = tq0 < a.Tq;          // wavefronts beyond the prompt still fetch their share of every chunk
     const int pos_base = a.pos0 + tq0, T = min(pos_base + QB * NQ, a.pos0 + a.Tq);
@@ -2785,8 +2807,8 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(D == 64 ? (
     const int len_b = RAGGED ? a.lens[b] : 0x7fffffff;
     const int Ttot = a.pos0 + a.Tq;
     const int nchunks = (RAGGED && tq_last > len_b) ? (Ttot + 31) / 32 : (a.pos0 + tq_last + 31) / 32;
-    const half_t* Kb = (const half_t*)a.kcache + ((long)b * a.Hkv + kvh) * a.max_len * D;
-    const half_t* Vt = (const half_t*)a.vcache + ((long)b * a.Hkv + kvh) * (long)D * a.max_len;
+    const half_t* Kb = (const half_t*)a.kcache + ((long)b * a.Hkv + kvc) * a.max_len * D;
+    const half_t* Vt = (const half_t*)a.vcache + ((long)b * a.Hkv + kvc) * (long)D * a.max_len;
     typedef const void __attribute__((address_space(1)))* gptr_t;
     typedef void __attribute__((address_space(3)))* lptr_t;
     auto stage_of = [&](int c) -> half_t* { return sstage + (c & (STAGES - 1)) * (NF * 512); };

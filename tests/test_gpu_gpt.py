@@ -439,11 +439,12 @@ def test_head_dim_128_against_oracle(G, oracle, kv_heads, batch, prompt):
 
 
 @pytest.mark.parametrize("hidden,heads,kv_heads,batch,prompt,splits", [(256, 4, 2, 2, 300, 2), (512, 4, 1, 1, 200, 2), (256, 4, 4, 1, 530, 3),
-                                                                      (256, 4, 2, 3, 90, 16)])
+                                                                      (256, 4, 2, 3, 90, 16), (1024, 16, 1, 1, 200, 2)])
 def test_decode_attention_split_over_blocks(G, oracle, monkeypatch, hidden, heads, kv_heads, batch, prompt, splits):
     """Few (row, KV head) pairs and a long context: several blocks share a pair and the last one to arrive merges their
     sums.  The library only splits at contexts of several thousand positions; the environment variable forces it here
-    (head_dim 64 and 128, two and three blocks, and sixteen blocks most of which have no chunk at all).  fp16, against
+    (head_dim 64 and 128, two and three blocks, sixteen blocks most of which have no chunk at all, and sixteen query heads
+    on one KV head, served as two groups of eight that each split in two).  fp16, against
     the oracle, with decode steps across a 32-position chunk boundary; then decode against the prefill path, which does
     not split."""
     monkeypatch.setenv("TSHIP_ATTN_SPLITS", str(splits))

@@ -82,12 +82,22 @@ def test_random_shape_against_oracle(oracle, seed):
     (7, 32, 1, "f32", 3, 35, True),
     (5, 64, 2, "f32", 2, 10, False),
     (6, 16, 1, "f32", 40, 3, False),
+    # more than eight query heads per KV head: groups of the largest divisor up to eight, a block per group
+    (16, 64, 1, "f16", 3, 37, False),       # two groups of eight
+    (12, 64, 1, "f16", 2, 70, True),        # two groups of six
+    (9, 64, 1, "f16", 33, 5, False),        # three groups of three
+    (32, 16, 1, "f16", 2, 12, False),       # multi-query attention, 32 heads on one: four groups of eight
+    (11, 64, 1, "f16", 2, 9, False),        # a prime: eleven groups of one
+    (16, 128, 1, "f16", 1, 40, False),
+    (10, 32, 2, "f32", 3, 35, True),        # two groups of five on each of two KV heads
+    (16, 16, 1, "f32", 40, 3, False),
 ])
 def test_group_sizes_that_do_not_divide_sixteen(oracle, g, d, hkv, dtype, batch, prompt, padded):
     """GroupQueryAttention.cs:156-159 expands the KV heads by any whole factor.  3, 5, 6 and 7 query heads per KV head: the
     matrix-instruction prefill kernel gives a wavefront floor(16 / g) positions and leaves the last 16 - g floor(16 / g)
-    columns empty, the decode kernel uses g of its 16 columns.  Prefill (with and without padded rows) and five decode
-    steps against the oracle."""
+    columns empty, the decode kernel uses g of its 16 columns.  More than eight: the heads of a KV head are served in
+    groups (of the largest divisor up to eight), a block per group, all groups reading the KV head's cache.  Prefill (with
+    and without padded rows) and five decode steps against the oracle."""
     from seq2seqsharp_amd import gpt as G
     heads = hkv * g
     cfg = synth._cfg(n_layers=2, hidden=heads * d, n_heads=heads, n_kv_heads=hkv, ffn_dim=96, vocab=257, attn_type=synth.GQA,
@@ -122,10 +132,10 @@ def test_group_sizes_that_do_not_divide_sixteen(oracle, g, d, hkv, dtype, batch,
 def test_group_size_limits_are_refused():
     from seq2seqsharp_amd import gpt as G
     from seq2seqsharp_amd._lib import TSHipError
-    for heads, hkv in ((9, 1), (6, 4)):
+    for heads, hkv in ((37, 1), (6, 4)):            # 37 groups of one; no whole ratio
         cfg = synth._cfg(n_layers=1, hidden=heads * 16, n_heads=heads, n_kv_heads=hkv, ffn_dim=48, vocab=61, attn_type=synth.GQA,
                          norm_type=synth.RMSNORM, act=synth.RELU, batch=1, prompt=2, steps=1, dtype="f32")
-        with pytest.raises(TSHipError, match="query heads per KV head|divisible by n_kv_heads"):
+        with pytest.raises(TSHipError, match="query heads of a KV head|divisible by n_kv_heads"):
             G.HipGpt(cfg, {}, max_batch=1, max_seq_len=8)
 
 
