@@ -23,7 +23,8 @@ def _sharp(cfg, seed):
     return w
 
 
-@pytest.mark.parametrize("beam,kw", [(3, dict()), (4, dict(attn_type=synth.MHA, n_kv_heads=4, norm_type=synth.LAYERNORM, act=synth.RELU)), (2, dict(batch=3))])
+@pytest.mark.parametrize("beam,kw", [(3, dict()), (4, dict(attn_type=synth.MHA, n_kv_heads=4, norm_type=synth.LAYERNORM, act=synth.RELU)), (2, dict(batch=3)),
+                                     (3, dict(hidden=160, n_heads=10, n_kv_heads=1))])      # ten heads on one KV head: two groups of five
 def test_greedy_beam_search_matches_the_reference_loop(G, oracle, beam, kw):
     cfg = synth.tiny_config(prompt=5, vocab=61, **kw)
     w = _sharp(cfg, 3)

@@ -12,6 +12,7 @@ CASES = [
     dict(dtype="f16"),                                                          # fp16, row-major cache (head size 16)
     dict(dtype="f16", hidden=128, n_heads=2, n_kv_heads=1, ffn_dim=256),        # fp16, head size 64: fragment-major cache, MFMA attention
     dict(dtype="f16", norm_type=synth.LAYERNORM, act=synth.RELU, attn_type=synth.MHA, n_kv_heads=4),
+    dict(dtype="f16", hidden=768, n_heads=12, n_kv_heads=1, ffn_dim=128),       # twelve query heads on one KV head: two groups of six
 ]
 
 
